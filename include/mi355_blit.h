@@ -1,0 +1,169 @@
+/*
+ * mi355_blit -- C ABI of the gfx950 blit engine (linear copy, dword fill and
+ * batched small copies done by compute kernels on one MI355X).
+ *
+ * This is the boundary a ROCr build binds to in place of the body of
+ * AMD::BlitKernel.  Citations are relative to
+ * projects/rocr-runtime/runtime/hsa-runtime/ in ROCm/rocm-systems.
+ *
+ * Conventions: plain C, opaque handle, every call returns an int status whose
+ * values equal the hsa_status_t values of the same meaning (inc/hsa.h), so a
+ * caller inside ROCr can return them unchanged.  Every entry point may be
+ * called from any thread; calls on one handle are submitted in call order per
+ * stream.  Pointers must be device-accessible on the handle's GPU and stay
+ * valid until the work has completed; overlapping source and destination are
+ * undefined, as in inc/hsa_ext_amd.h:1712-1714.
+ */
+#ifndef MI355_BLIT_H_
+#define MI355_BLIT_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_BLIT_ABI_VERSION 1
+
+/* Same numeric values as HSA_STATUS_* (inc/hsa.h). */
+enum {
+  MI355_BLIT_SUCCESS = 0x0,
+  MI355_BLIT_ERROR = 0x1000,                  /* HSA_STATUS_ERROR */
+  MI355_BLIT_ERROR_INVALID_ARGUMENT = 0x1001, /* HSA_STATUS_ERROR_INVALID_ARGUMENT */
+  MI355_BLIT_ERROR_OUT_OF_RESOURCES = 0x1008, /* HSA_STATUS_ERROR_OUT_OF_RESOURCES */
+  MI355_BLIT_ERROR_NOT_INITIALIZED = 0x100B   /* HSA_STATUS_ERROR_NOT_INITIALIZED */
+};
+
+/* Kernel families.  The reference picks between CopyAligned and CopyMisaligned
+ * on (src & 3) == (dst & 3) (core/runtime/amd_blit_kernel.cpp:716); here the
+ * same predicate picks between the plain vector copy and the one that realigns
+ * source dwords in registers. */
+enum {
+  MI355_BLIT_KERNEL_COPY = 0,         /* (src - dst) % 4 == 0 */
+  MI355_BLIT_KERNEL_COPY_REALIGN = 1, /* (src - dst) % 4 != 0 */
+  MI355_BLIT_KERNEL_FILL = 2,
+  MI355_BLIT_KERNEL_COPY_BATCH = 3
+};
+
+typedef struct mi355_blit mi355_blit_t;
+
+/* How one command is cut up and launched.  Replaces the phase bounds the
+ * reference writes into BlitKernel::KernelArgs (core/inc/amd_blit_kernel.h:
+ * 122-154) and its fixed grids (amd_blit_kernel.cpp:723, 759, 797).
+ *   bytes == head_bytes + 16 * body_vecs + tail_bytes
+ *   (dst + head_bytes) % 16 == 0 whenever body_vecs > 0
+ *   head_bytes <= 15 and tail_bytes <= 15
+ * For a fill the same fields count bytes of whole dwords. */
+typedef struct {
+  uint32_t kernel;      /* MI355_BLIT_KERNEL_* */
+  uint32_t wg_size;     /* work-items per workgroup, multiple of 64 */
+  uint32_t grid;        /* workgroups */
+  uint32_t unroll;      /* 16-byte vectors each lane keeps in flight */
+  uint32_t nt_load;     /* non-temporal loads */
+  uint32_t store_policy;/* MI355_BLIT_STORE_* */
+  uint32_t byte_shift;  /* (src - dst) & 3 */
+  uint32_t reserved;
+  uint64_t head_bytes;
+  uint64_t body_vecs;
+  uint64_t tail_bytes;
+} mi355_blit_plan_t;
+
+/* Cache policy of the body's 16-byte stores. */
+enum {
+  MI355_BLIT_STORE_CACHED = 0,    /* write-back L2 */
+  MI355_BLIT_STORE_NT = 1,        /* non-temporal hint */
+  MI355_BLIT_STORE_AGENT_WT = 2,  /* sc1: written through L2 */
+  MI355_BLIT_STORE_SYSTEM_WT = 3  /* sc0 sc1: written through, system scope */
+};
+
+/* Overrides for the sizing heuristics; 0 in a field keeps the heuristic.
+ * nt_load: 0 = heuristic, 1 = force off, 2 = force on.
+ * store_policy: 0 = heuristic, otherwise MI355_BLIT_STORE_* + 1. */
+typedef struct {
+  uint32_t wg_size;
+  uint32_t unroll;
+  uint32_t max_grid;   /* cap on workgroups; beyond it waves stride over tiles */
+  uint32_t nt_load;
+  uint32_t store_policy;
+  uint32_t reserved[3];
+} mi355_blit_tuning_t;
+
+/* One element of a batched submission.  No counterpart in the reference. */
+typedef struct {
+  void* dst;
+  const void* src;
+  uint64_t bytes;
+} mi355_blit_desc_t;
+
+/* Replaces BlitKernel::BlitKernel + Initialize (core/runtime/amd_blit_kernel.cpp:
+ * 538-591): binds to a GPU, reads its CU count, loads the kernels' code object
+ * (what GpuAgent::AssembleShader does for the reference,
+ * core/runtime/amd_gpu_agent.cpp:251-426) and creates the submission stream. */
+int mi355_blit_create(int device_ordinal, mi355_blit_t** out);
+
+/* Replaces BlitKernel::Destroy (amd_blit_kernel.cpp:593-612).  Blocks until all
+ * submitted commands have executed. */
+int mi355_blit_destroy(mi355_blit_t* h);
+
+/* Replaces the dispatch half of BlitKernel::SubmitLinearCopyCommand
+ * (amd_blit_kernel.cpp:641-785) and the CopyAligned / CopyMisaligned shaders
+ * (core/runtime/blit_shaders/blit_copyAligned.s, blit_copyMisaligned.s).
+ * Non-blocking.  stream is a hipStream_t, or NULL for the handle's own stream.
+ * dst or src NULL -> INVALID_ARGUMENT; bytes == 0 -> SUCCESS without a launch
+ * (core/runtime/hsa.cpp:1170-1184). */
+int mi355_blit_copy(mi355_blit_t* h, void* dst, const void* src, size_t bytes, void* stream);
+
+/* Replaces the dispatch half of BlitKernel::SubmitLinearFillCommand
+ * (amd_blit_kernel.cpp:787-837) and the Fill shader (blit_shaders/blit_fill.s).
+ * Non-blocking.  ptr NULL or not 4-byte aligned -> INVALID_ARGUMENT;
+ * num_dwords == 0 -> SUCCESS without a launch
+ * (core/runtime/hsa_ext_amd.cpp:237-251). */
+int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwords, void* stream);
+
+/* Batched small-copy descriptor path: n independent copies in one submission.
+ * No counterpart in the reference (it submits one AQL packet per copy).
+ * descs may live in host memory (descs_on_device == 0: the library stages
+ * them) or be device-resident (descs_on_device != 0: read in place, must stay
+ * valid until completion).  Regions must not overlap one another. */
+int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n,
+                          int descs_on_device, void* stream);
+
+/* Blocks until every command submitted on the handle's own stream is done;
+ * the wait BlitKernel does on its completion signal
+ * (amd_blit_kernel.cpp:632, 830). */
+int mi355_blit_synchronize(mi355_blit_t* h);
+
+/* Replaces BlitKernel::PendingBytes (amd_blit_kernel.cpp:943-970): approximate
+ * bytes not yet copied or filled; a return of 0 is exact. */
+uint64_t mi355_blit_pending_bytes(mi355_blit_t* h);
+
+/* The plan used by the most recent copy / fill / batch on this handle. */
+int mi355_blit_last_launch_info(mi355_blit_t* h, mi355_blit_plan_t* out);
+
+/* Dispatch sizing heuristics as pure host functions (no GPU needed): replace
+ * the phase arithmetic of amd_blit_kernel.cpp:714-775 and 796-813.  num_cus is
+ * the compute-unit count (amd_blit_kernel.cpp:572); tuning may be NULL. */
+int mi355_blit_plan_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t num_cus,
+                         const mi355_blit_tuning_t* tuning, mi355_blit_plan_t* out);
+int mi355_blit_plan_fill(uint64_t ptr, uint64_t num_dwords, uint32_t num_cus,
+                         const mi355_blit_tuning_t* tuning, mi355_blit_plan_t* out);
+
+/* Installs overrides used by every later command on the handle (NULL clears).
+ * For tuning sweeps; replaces the reference's string-parsed kernel parameters
+ * (amd_blit_kernel.cpp:499-532). */
+int mi355_blit_set_tuning(mi355_blit_t* h, const mi355_blit_tuning_t* tuning);
+
+/* Compute units of the handle's GPU (amd_blit_kernel.cpp:572). */
+int mi355_blit_num_cus(mi355_blit_t* h);
+
+/* The handle's own stream as a hipStream_t. */
+void* mi355_blit_stream(mi355_blit_t* h);
+
+const char* mi355_blit_status_string(int status);
+int mi355_blit_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_BLIT_H_ */

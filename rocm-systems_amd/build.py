@@ -1,0 +1,89 @@
+"""Compile recipe for the native parts.  Everything is built in-tree with
+hipcc / gcc; nothing is fetched."""
+import os
+import shutil
+import subprocess
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG_DIR)
+CSRC = os.path.join(PKG_DIR, "csrc")
+LIB_DIR = os.path.join(PKG_DIR, "lib")
+INCLUDE = os.path.join(ROOT, "include")
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+
+BLIT_LIB = os.path.join(LIB_DIR, "libmi355blit.so")
+ROCR_LIB = os.path.join(LIB_DIR, "libmi355blit_rocr.so")
+ROCR_TEST = os.path.join(LIB_DIR, "test_rocr_blit")
+ORACLE_LIB = os.path.join(ORACLE_DIR, "libblit_oracle.so")
+
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+
+HIPCC_FLAGS = [
+    "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC",
+    # hipcc may pair float ops into packed-FP32 instructions; keep them scalar
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _hipcc():
+    exe = shutil.which("hipcc") or os.path.join(ROCM, "bin", "hipcc")
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; cannot build the gfx950 blit library")
+    return exe
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("build step failed: %s\n%s" % (" ".join(cmd), proc.stdout))
+    return proc.stdout
+
+
+def build_blit():
+    """HIP kernels + C ABI -> lib/libmi355blit.so"""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    _run([_hipcc()] + HIPCC_FLAGS + [
+        "-shared", "-I", INCLUDE, "-I", CSRC,
+        "-o", BLIT_LIB, os.path.join(CSRC, "blit_capi.hip"),
+    ])
+    return BLIT_LIB
+
+
+def build_rocr_adapter():
+    """C++ core::Blit adapter over the C ABI + public HSA signals ->
+    lib/libmi355blit_rocr.so, and its native test driver."""
+    src = os.path.join(CSRC, "rocr_blit.cpp")
+    if not os.path.exists(src):
+        return None
+    os.makedirs(LIB_DIR, exist_ok=True)
+    common = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-I", INCLUDE, "-I", CSRC,
+              "-I", os.path.join(ROCM, "include")]
+    link = ["-L", LIB_DIR, "-lmi355blit", "-L", os.path.join(ROCM, "lib"), "-lhsa-runtime64",
+            "-lpthread", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(ROCM, "lib")]
+    _run(["g++"] + common + ["-shared", "-o", ROCR_LIB, src] + link)
+    test_src = os.path.join(ROOT, "tests", "cpp", "test_rocr_blit.cpp")
+    if os.path.exists(test_src):
+        _run(["g++"] + common + ["-o", ROCR_TEST, test_src, "-lmi355blit_rocr"] + link
+             + ["-L", os.path.join(ROCM, "lib"), "-lamdhip64"])
+    return ROCR_LIB
+
+
+def build_oracle():
+    """CPU oracle (test infrastructure) -> oracle/libblit_oracle.so"""
+    _run(["make", "-C", ORACLE_DIR, "-B", "libblit_oracle.so"])
+    return ORACLE_LIB
+
+
+def build_all():
+    out = [build_blit()]
+    r = build_rocr_adapter()
+    if r:
+        out.append(r)
+    out.append(build_oracle())
+    return out
+
+
+if __name__ == "__main__":
+    for path in build_all():
+        print("built", path)

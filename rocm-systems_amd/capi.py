@@ -1,0 +1,182 @@
+"""ctypes binding of include/mi355_blit.h.  Thin on purpose: tests and the
+benchmark call the C ABI itself, this file only declares signatures.
+
+There is no CPU fallback: if the library is missing, loading raises."""
+import ctypes as C
+import os
+
+from . import build as _build
+
+SUCCESS = 0x0
+ERROR = 0x1000
+ERROR_INVALID_ARGUMENT = 0x1001
+ERROR_OUT_OF_RESOURCES = 0x1008
+ERROR_NOT_INITIALIZED = 0x100B
+
+KERNEL_COPY = 0
+KERNEL_COPY_REALIGN = 1
+KERNEL_FILL = 2
+KERNEL_COPY_BATCH = 3
+
+STORE_CACHED = 0
+STORE_NT = 1
+STORE_AGENT_WT = 2
+STORE_SYSTEM_WT = 3
+
+
+class Plan(C.Structure):
+    _fields_ = [
+        ("kernel", C.c_uint32), ("wg_size", C.c_uint32), ("grid", C.c_uint32),
+        ("unroll", C.c_uint32), ("nt_load", C.c_uint32), ("store_policy", C.c_uint32),
+        ("byte_shift", C.c_uint32), ("reserved", C.c_uint32),
+        ("head_bytes", C.c_uint64), ("body_vecs", C.c_uint64), ("tail_bytes", C.c_uint64),
+    ]
+
+    def as_dict(self):
+        return {n: getattr(self, n) for n, _ in self._fields_ if n != "reserved"}
+
+
+class Tuning(C.Structure):
+    _fields_ = [
+        ("wg_size", C.c_uint32), ("unroll", C.c_uint32), ("max_grid", C.c_uint32),
+        ("nt_load", C.c_uint32), ("store_policy", C.c_uint32), ("reserved", C.c_uint32 * 3),
+    ]
+
+
+class Desc(C.Structure):
+    _fields_ = [("dst", C.c_void_p), ("src", C.c_void_p), ("bytes", C.c_uint64)]
+
+
+# every symbol include/mi355_blit.h declares: name -> (restype, argtypes)
+SIGNATURES = {
+    "mi355_blit_create": (C.c_int, [C.c_int, C.POINTER(C.c_void_p)]),
+    "mi355_blit_destroy": (C.c_int, [C.c_void_p]),
+    "mi355_blit_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "mi355_blit_fill32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t, C.c_void_p]),
+    "mi355_blit_copy_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]),
+    "mi355_blit_synchronize": (C.c_int, [C.c_void_p]),
+    "mi355_blit_pending_bytes": (C.c_uint64, [C.c_void_p]),
+    "mi355_blit_last_launch_info": (C.c_int, [C.c_void_p, C.POINTER(Plan)]),
+    "mi355_blit_plan_copy": (C.c_int, [C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint32,
+                                       C.POINTER(Tuning), C.POINTER(Plan)]),
+    "mi355_blit_plan_fill": (C.c_int, [C.c_uint64, C.c_uint64, C.c_uint32,
+                                       C.POINTER(Tuning), C.POINTER(Plan)]),
+    "mi355_blit_set_tuning": (C.c_int, [C.c_void_p, C.POINTER(Tuning)]),
+    "mi355_blit_num_cus": (C.c_int, [C.c_void_p]),
+    "mi355_blit_stream": (C.c_void_p, [C.c_void_p]),
+    "mi355_blit_status_string": (C.c_char_p, [C.c_int]),
+    "mi355_blit_abi_version": (C.c_int, []),
+}
+
+_lib = None
+
+
+def library_path():
+    return _build.BLIT_LIB
+
+
+def load():
+    """dlopen lib/libmi355blit.so and declare its signatures.  Import torch
+    before calling this in a process that also uses torch, so that both share
+    one HIP runtime."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = library_path()
+    if not os.path.exists(path):
+        raise RuntimeError(
+            "%s is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'`"
+            % path)
+    lib = C.CDLL(path, mode=C.RTLD_GLOBAL)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+class BlitError(RuntimeError):
+    def __init__(self, status, what):
+        self.status = status
+        msg = load().mi355_blit_status_string(status).decode()
+        super().__init__("%s failed: 0x%x (%s)" % (what, status, msg))
+
+
+def check(status, what):
+    if status != SUCCESS:
+        raise BlitError(status, what)
+
+
+class Blit:
+    """Owner of one mi355_blit_t handle; methods map 1:1 to the C ABI and take
+    raw device addresses (ints)."""
+
+    def __init__(self, device=0):
+        self.lib = load()
+        h = C.c_void_p()
+        check(self.lib.mi355_blit_create(device, C.byref(h)), "mi355_blit_create")
+        self.handle = h
+
+    def close(self):
+        if self.handle:
+            st = self.lib.mi355_blit_destroy(self.handle)
+            self.handle = None
+            check(st, "mi355_blit_destroy")
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def copy(self, dst, src, nbytes, stream=None):
+        return self.lib.mi355_blit_copy(self.handle, dst, src, nbytes, stream)
+
+    def fill32(self, ptr, value, num_dwords, stream=None):
+        return self.lib.mi355_blit_fill32(self.handle, ptr, value, num_dwords, stream)
+
+    def copy_batch(self, descs, n, on_device=False, stream=None):
+        addr = descs if isinstance(descs, int) else C.cast(descs, C.c_void_p)
+        return self.lib.mi355_blit_copy_batch(self.handle, addr, n, 1 if on_device else 0, stream)
+
+    def synchronize(self):
+        return self.lib.mi355_blit_synchronize(self.handle)
+
+    def pending_bytes(self):
+        return self.lib.mi355_blit_pending_bytes(self.handle)
+
+    def last_plan(self):
+        p = Plan()
+        check(self.lib.mi355_blit_last_launch_info(self.handle, C.byref(p)), "last_launch_info")
+        return p
+
+    def set_tuning(self, **kw):
+        if not kw:
+            return self.lib.mi355_blit_set_tuning(self.handle, None)
+        t = Tuning()
+        for k, v in kw.items():
+            setattr(t, k, v)
+        return self.lib.mi355_blit_set_tuning(self.handle, C.byref(t))
+
+    @property
+    def num_cus(self):
+        return self.lib.mi355_blit_num_cus(self.handle)
+
+    @property
+    def stream(self):
+        return self.lib.mi355_blit_stream(self.handle)
+
+
+def plan_copy(dst, src, nbytes, num_cus=256, tuning=None):
+    p = Plan()
+    st = load().mi355_blit_plan_copy(dst, src, nbytes, num_cus,
+                                     C.byref(tuning) if tuning is not None else None, C.byref(p))
+    return st, p
+
+
+def plan_fill(ptr, num_dwords, num_cus=256, tuning=None):
+    p = Plan()
+    st = load().mi355_blit_plan_fill(ptr, num_dwords, num_cus,
+                                     C.byref(tuning) if tuning is not None else None, C.byref(p))
+    return st, p

@@ -1,0 +1,428 @@
+// C ABI of the gfx950 blit engine over HIP (declarations and the reference
+// interfaces they replace: include/mi355_blit.h).  Host work per command is
+// O(1): one plan, one kernel launch, one ledger record -- like the ~100 bytes
+// of kernargs plus one AQL packet ROCr's BlitKernel writes per command
+// (projects/rocr-runtime/runtime/hsa-runtime/core/runtime/amd_blit_kernel.cpp:
+// 641-785).
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+
+#include "blit_kernels.h"
+#include "blit_plan.h"
+#include "mi355_blit.h"
+
+namespace {
+
+using namespace mi355;
+
+// Commands remembered for PendingBytes; ROCr's ledger has one record per AQL
+// queue slot and its utility queue has 64 (amd_gpu_agent.h:507-508).
+constexpr unsigned kLedgerSlots = 64;
+
+struct LedgerSlot {
+  hipEvent_t done = nullptr;
+  uint64_t bytes = 0;
+  bool in_flight = false;
+};
+
+}  // namespace
+
+struct mi355_blit {
+  int device = 0;
+  int num_cus = 0;
+  hipStream_t stream = nullptr;
+
+  std::mutex lock;  // guards everything below
+  mi355_blit_tuning_t tuning{};
+  bool has_tuning = false;
+  mi355_blit_plan_t last_plan{};
+
+  LedgerSlot ledger[kLedgerSlots];
+  uint64_t ledger_head = 0;  // next slot to use
+
+  // batched path staging (grown on demand, never shrunk)
+  BatchDesc* descs_host = nullptr;  // pinned
+  BatchDesc* descs_dev = nullptr;
+  uint32_t* chunk_start_dev = nullptr;
+  size_t batch_capacity = 0;
+  hipEvent_t staging_free = nullptr;  // previous batch has consumed the staging buffers
+  bool staging_busy = false;
+};
+
+namespace {
+
+int status_of(hipError_t e) {
+  switch (e) {
+    case hipSuccess: return MI355_BLIT_SUCCESS;
+    case hipErrorOutOfMemory: return MI355_BLIT_ERROR_OUT_OF_RESOURCES;
+    case hipErrorInvalidValue: return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+    default: return MI355_BLIT_ERROR;
+  }
+}
+
+#define BLIT_HIP(expr)                       \
+  do {                                       \
+    hipError_t e_ = (expr);                  \
+    if (e_ != hipSuccess) return status_of(e_); \
+  } while (0)
+
+struct DeviceScope {
+  int prev = -1;
+  bool switched = false;
+  hipError_t err = hipSuccess;
+  explicit DeviceScope(int dev) {
+    err = hipGetDevice(&prev);
+    if (err == hipSuccess && prev != dev) {
+      err = hipSetDevice(dev);
+      switched = (err == hipSuccess);
+    }
+  }
+  ~DeviceScope() {
+    if (switched) (void)hipSetDevice(prev);
+  }
+};
+
+typedef void (*copy_kernel_t)(CopyArgs);
+typedef void (*fill_kernel_t)(FillArgs);
+
+template <int U, bool NTL, bool SHIFT>
+copy_kernel_t copy_kernel_st(unsigned policy) {
+  switch (policy) {
+    case MI355_BLIT_STORE_CACHED: return k_copy<U, NTL, kStoreCached, SHIFT>;
+    case MI355_BLIT_STORE_NT: return k_copy<U, NTL, kStoreNt, SHIFT>;
+    case MI355_BLIT_STORE_AGENT_WT: return k_copy<U, NTL, kStoreAgentWt, SHIFT>;
+    case MI355_BLIT_STORE_SYSTEM_WT: return k_copy<U, NTL, kStoreSystemWt, SHIFT>;
+    default: return nullptr;
+  }
+}
+
+template <bool SHIFT>
+copy_kernel_t copy_kernel_u(unsigned u, bool ntl, unsigned policy) {
+  switch (u) {
+    case 1: return ntl ? copy_kernel_st<1, true, SHIFT>(policy) : copy_kernel_st<1, false, SHIFT>(policy);
+    case 2: return ntl ? copy_kernel_st<2, true, SHIFT>(policy) : copy_kernel_st<2, false, SHIFT>(policy);
+    case 4: return ntl ? copy_kernel_st<4, true, SHIFT>(policy) : copy_kernel_st<4, false, SHIFT>(policy);
+    default: return nullptr;
+  }
+}
+
+copy_kernel_t select_copy_kernel(const mi355_blit_plan_t& p) {
+  return p.byte_shift ? copy_kernel_u<true>(p.unroll, p.nt_load, p.store_policy)
+                      : copy_kernel_u<false>(p.unroll, p.nt_load, p.store_policy);
+}
+
+template <int U>
+fill_kernel_t fill_kernel_st(unsigned policy) {
+  switch (policy) {
+    case MI355_BLIT_STORE_CACHED: return k_fill<U, kStoreCached>;
+    case MI355_BLIT_STORE_NT: return k_fill<U, kStoreNt>;
+    case MI355_BLIT_STORE_AGENT_WT: return k_fill<U, kStoreAgentWt>;
+    case MI355_BLIT_STORE_SYSTEM_WT: return k_fill<U, kStoreSystemWt>;
+    default: return nullptr;
+  }
+}
+
+fill_kernel_t select_fill_kernel(const mi355_blit_plan_t& p) {
+  switch (p.unroll) {
+    case 1: return fill_kernel_st<1>(p.store_policy);
+    case 2: return fill_kernel_st<2>(p.store_policy);
+    case 4: return fill_kernel_st<4>(p.store_policy);
+    default: return nullptr;
+  }
+}
+
+// Which waves of the launch take the partial last tile and the edges.
+void set_tail_waves(const mi355_blit_plan_t& p, uint32_t* partial_wave, uint32_t* edge_wave) {
+  const uint64_t n_waves = static_cast<uint64_t>(p.grid) * (p.wg_size / 64);
+  const uint64_t n_full = p.body_vecs / (64ull * p.unroll);
+  *partial_wave = static_cast<uint32_t>(n_full % n_waves);
+  *edge_wave = static_cast<uint32_t>((n_full + 1) % n_waves);
+}
+
+// Records `bytes` as queued behind everything already on `s`.  Caller holds
+// h->lock.  When the ledger is full the oldest command is waited for, the
+// back-pressure ROCr applies when its AQL ring is full
+// (amd_blit_kernel.cpp:844-854).
+int ledger_record(mi355_blit* h, hipStream_t s, uint64_t bytes) {
+  LedgerSlot& slot = h->ledger[h->ledger_head % kLedgerSlots];
+  if (slot.in_flight) {
+    BLIT_HIP(hipEventSynchronize(slot.done));
+    slot.in_flight = false;
+  }
+  BLIT_HIP(hipEventRecord(slot.done, s));
+  slot.bytes = bytes;
+  slot.in_flight = true;
+  ++h->ledger_head;
+  return MI355_BLIT_SUCCESS;
+}
+
+int ensure_batch_capacity(mi355_blit* h, size_t n) {
+  if (n <= h->batch_capacity) return MI355_BLIT_SUCCESS;
+  // the old buffers may still be read by a batch in flight
+  if (h->staging_busy) {
+    BLIT_HIP(hipEventSynchronize(h->staging_free));
+    h->staging_busy = false;
+  }
+  size_t cap = h->batch_capacity ? h->batch_capacity : 1024;
+  while (cap < n) cap *= 2;
+  if (h->descs_host) (void)hipHostFree(h->descs_host);
+  if (h->descs_dev) (void)hipFree(h->descs_dev);
+  if (h->chunk_start_dev) (void)hipFree(h->chunk_start_dev);
+  h->descs_host = nullptr;
+  h->descs_dev = nullptr;
+  h->chunk_start_dev = nullptr;
+  h->batch_capacity = 0;
+  BLIT_HIP(hipHostMalloc(reinterpret_cast<void**>(&h->descs_host), cap * sizeof(BatchDesc), hipHostMallocDefault));
+  BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->descs_dev), cap * sizeof(BatchDesc)));
+  BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->chunk_start_dev), (cap + 1) * sizeof(uint32_t)));
+  h->batch_capacity = cap;
+  return MI355_BLIT_SUCCESS;
+}
+
+}  // namespace
+
+static_assert(sizeof(mi355_blit_desc_t) == sizeof(mi355::BatchDesc), "descriptor layout");
+static_assert(mi355::kBatchChunkVecs == mi355::kChunkVecs, "chunk size");
+static_assert(MI355_BLIT_STORE_SYSTEM_WT == mi355::kStoreSystemWt && MI355_BLIT_STORE_NT == mi355::kStoreNt &&
+              MI355_BLIT_STORE_AGENT_WT == mi355::kStoreAgentWt, "store policy values");
+
+extern "C" {
+
+int mi355_blit_abi_version(void) { return MI355_BLIT_ABI_VERSION; }
+
+const char* mi355_blit_status_string(int status) {
+  switch (status) {
+    case MI355_BLIT_SUCCESS: return "success";
+    case MI355_BLIT_ERROR: return "error";
+    case MI355_BLIT_ERROR_INVALID_ARGUMENT: return "invalid argument";
+    case MI355_BLIT_ERROR_OUT_OF_RESOURCES: return "out of resources";
+    case MI355_BLIT_ERROR_NOT_INITIALIZED: return "not initialized";
+    default: return "unknown status";
+  }
+}
+
+int mi355_blit_plan_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t num_cus,
+                         const mi355_blit_tuning_t* tuning, mi355_blit_plan_t* out) {
+  return plan_copy(dst, src, bytes, num_cus, tuning, out);
+}
+
+int mi355_blit_plan_fill(uint64_t ptr, uint64_t num_dwords, uint32_t num_cus,
+                         const mi355_blit_tuning_t* tuning, mi355_blit_plan_t* out) {
+  return plan_fill(ptr, num_dwords, num_cus, tuning, out);
+}
+
+int mi355_blit_create(int device_ordinal, mi355_blit_t** out) {
+  if (!out) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  *out = nullptr;
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) return MI355_BLIT_ERROR_NOT_INITIALIZED;
+  if (device_ordinal < 0 || device_ordinal >= count) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  DeviceScope scope(device_ordinal);
+  if (scope.err != hipSuccess) return status_of(scope.err);
+
+  mi355_blit* h = new (std::nothrow) mi355_blit;
+  if (!h) return MI355_BLIT_ERROR_OUT_OF_RESOURCES;
+  h->device = device_ordinal;
+  int cus = 0;
+  hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device_ordinal);
+  if (e == hipSuccess && cus > 0) e = hipStreamCreateWithFlags(&h->stream, hipStreamNonBlocking);
+  for (unsigned i = 0; e == hipSuccess && i < kLedgerSlots; ++i)
+    e = hipEventCreateWithFlags(&h->ledger[i].done, hipEventDisableTiming);
+  if (e == hipSuccess) e = hipEventCreateWithFlags(&h->staging_free, hipEventDisableTiming);
+  if (e != hipSuccess || cus <= 0) {
+    mi355_blit_destroy(h);
+    return e == hipSuccess ? MI355_BLIT_ERROR : status_of(e);
+  }
+  h->num_cus = cus;
+  *out = h;
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_blit_destroy(mi355_blit_t* h) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  int rc = MI355_BLIT_SUCCESS;
+  {
+    std::lock_guard<std::mutex> g(h->lock);
+    DeviceScope scope(h->device);
+    // every command, on whichever stream it went, has a ledger record
+    for (unsigned i = 0; i < kLedgerSlots; ++i) {
+      LedgerSlot& s = h->ledger[i];
+      if (s.done) {
+        if (s.in_flight && hipEventSynchronize(s.done) != hipSuccess) rc = MI355_BLIT_ERROR;
+        (void)hipEventDestroy(s.done);
+      }
+    }
+    if (h->stream) {
+      if (hipStreamSynchronize(h->stream) != hipSuccess) rc = MI355_BLIT_ERROR;
+      (void)hipStreamDestroy(h->stream);
+    }
+    if (h->staging_free) (void)hipEventDestroy(h->staging_free);
+    if (h->descs_host) (void)hipHostFree(h->descs_host);
+    if (h->descs_dev) (void)hipFree(h->descs_dev);
+    if (h->chunk_start_dev) (void)hipFree(h->chunk_start_dev);
+  }
+  delete h;
+  return rc;
+}
+
+int mi355_blit_num_cus(mi355_blit_t* h) { return h ? h->num_cus : 0; }
+
+void* mi355_blit_stream(mi355_blit_t* h) { return h ? static_cast<void*>(h->stream) : nullptr; }
+
+int mi355_blit_set_tuning(mi355_blit_t* h, const mi355_blit_tuning_t* tuning) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> g(h->lock);
+  h->has_tuning = tuning != nullptr;
+  if (tuning) h->tuning = *tuning;
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_blit_last_launch_info(mi355_blit_t* h, mi355_blit_plan_t* out) {
+  if (!h || !out) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> g(h->lock);
+  *out = h->last_plan;
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_blit_copy(mi355_blit_t* h, void* dst, const void* src, size_t bytes, void* stream) {
+  if (!h || !dst || !src) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (bytes == 0) return MI355_BLIT_SUCCESS;
+  std::lock_guard<std::mutex> g(h->lock);
+  DeviceScope scope(h->device);
+  if (scope.err != hipSuccess) return status_of(scope.err);
+  mi355_blit_plan_t p;
+  int rc = plan_copy(reinterpret_cast<uint64_t>(dst), reinterpret_cast<uint64_t>(src), bytes,
+                     h->num_cus, h->has_tuning ? &h->tuning : nullptr, &p);
+  if (rc != MI355_BLIT_SUCCESS) return rc;
+  copy_kernel_t k = select_copy_kernel(p);
+  if (!k) return MI355_BLIT_ERROR;
+  CopyArgs a;
+  a.dst = static_cast<uint8_t*>(dst);
+  a.src = static_cast<const uint8_t*>(src);
+  a.bytes = bytes;
+  a.n_vec = p.body_vecs;
+  a.head = static_cast<uint32_t>(p.head_bytes);
+  set_tail_waves(p, &a.partial_wave, &a.edge_wave);
+  hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
+  hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
+  BLIT_HIP(hipGetLastError());
+  h->last_plan = p;
+  return ledger_record(h, s, bytes);
+}
+
+int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwords, void* stream) {
+  if (!h || !ptr || (reinterpret_cast<uintptr_t>(ptr) & 3)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (num_dwords == 0) return MI355_BLIT_SUCCESS;
+  std::lock_guard<std::mutex> g(h->lock);
+  DeviceScope scope(h->device);
+  if (scope.err != hipSuccess) return status_of(scope.err);
+  mi355_blit_plan_t p;
+  int rc = plan_fill(reinterpret_cast<uint64_t>(ptr), num_dwords, h->num_cus,
+                     h->has_tuning ? &h->tuning : nullptr, &p);
+  if (rc != MI355_BLIT_SUCCESS) return rc;
+  fill_kernel_t k = select_fill_kernel(p);
+  if (!k) return MI355_BLIT_ERROR;
+  FillArgs a;
+  a.dst = static_cast<uint32_t*>(ptr);
+  a.n_dwords = num_dwords;
+  a.n_vec = p.body_vecs;
+  a.head = static_cast<uint32_t>(p.head_bytes / 4);
+  a.value = value;
+  set_tail_waves(p, &a.partial_wave, &a.edge_wave);
+  hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
+  hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
+  BLIT_HIP(hipGetLastError());
+  h->last_plan = p;
+  return ledger_record(h, s, num_dwords * 4);
+}
+
+int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n,
+                          int descs_on_device, void* stream) {
+  if (!h || (!descs && n)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (n == 0) return MI355_BLIT_SUCCESS;
+  std::lock_guard<std::mutex> g(h->lock);
+  DeviceScope scope(h->device);
+  if (scope.err != hipSuccess) return status_of(scope.err);
+  hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
+
+  int rc = ensure_batch_capacity(h, n);
+  if (rc != MI355_BLIT_SUCCESS) return rc;
+  // chunk_start_dev (and the staging pair) are shared by consecutive batches
+  if (h->staging_busy) {
+    BLIT_HIP(hipStreamWaitEvent(s, h->staging_free, 0));
+  }
+  uint64_t total_bytes = 0;
+  const BatchDesc* dev_descs;
+  if (descs_on_device) {
+    dev_descs = reinterpret_cast<const BatchDesc*>(descs);
+    total_bytes = n;  // lengths are only known on the device; keep the record non-zero
+  } else {
+    for (size_t i = 0; i < n; ++i) {
+      if (descs[i].bytes && (!descs[i].dst || !descs[i].src)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+      total_bytes += descs[i].bytes;
+    }
+    // the pinned buffer is rewritten by the host: the previous upload must be over
+    if (h->staging_busy) {
+      BLIT_HIP(hipEventSynchronize(h->staging_free));
+      h->staging_busy = false;
+    }
+    std::memcpy(h->descs_host, descs, n * sizeof(BatchDesc));
+    BLIT_HIP(hipMemcpyAsync(h->descs_dev, h->descs_host, n * sizeof(BatchDesc), hipMemcpyHostToDevice, s));
+    dev_descs = h->descs_dev;
+  }
+  hipLaunchKernelGGL(k_batch_scan, dim3(1), dim3(1024), 0, s, dev_descs, static_cast<uint64_t>(n),
+                     h->chunk_start_dev);
+  BLIT_HIP(hipGetLastError());
+  mi355_blit_plan_t p{};
+  p.kernel = MI355_BLIT_KERNEL_COPY_BATCH;
+  p.wg_size = 256;
+  p.unroll = kBatchChunkVecs / 64;
+  uint32_t max_grid = h->num_cus * kWgPerCu;
+  if (h->has_tuning && h->tuning.max_grid) max_grid = h->tuning.max_grid;
+  // A copy has at least one chunk and, at the sizes this path is meant for,
+  // at most a few dozen; with few copies a full-device grid would be mostly
+  // idle waves.
+  const uint64_t wgs = static_cast<uint64_t>(n) * 16;
+  p.grid = static_cast<uint32_t>(wgs < max_grid ? wgs : max_grid);
+  hipLaunchKernelGGL(k_batch_copy, dim3(p.grid), dim3(p.wg_size), 0, s, dev_descs,
+                     static_cast<uint64_t>(n), h->chunk_start_dev);
+  BLIT_HIP(hipGetLastError());
+  BLIT_HIP(hipEventRecord(h->staging_free, s));
+  h->staging_busy = true;
+  h->last_plan = p;
+  return ledger_record(h, s, total_bytes);
+}
+
+int mi355_blit_synchronize(mi355_blit_t* h) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  hipStream_t s;
+  {
+    std::lock_guard<std::mutex> g(h->lock);
+    s = h->stream;
+  }
+  DeviceScope scope(h->device);
+  if (scope.err != hipSuccess) return status_of(scope.err);
+  BLIT_HIP(hipStreamSynchronize(s));
+  return MI355_BLIT_SUCCESS;
+}
+
+uint64_t mi355_blit_pending_bytes(mi355_blit_t* h) {
+  if (!h) return 0;
+  std::lock_guard<std::mutex> g(h->lock);
+  DeviceScope scope(h->device);
+  uint64_t pending = 0;
+  for (unsigned i = 0; i < kLedgerSlots; ++i) {
+    LedgerSlot& s = h->ledger[i];
+    if (!s.in_flight) continue;
+    if (hipEventQuery(s.done) == hipSuccess) s.in_flight = false;
+    else pending += s.bytes;
+  }
+  return pending;
+}
+
+}  // extern "C"

@@ -1,0 +1,362 @@
+// Device kernels of the gfx950 blit engine: linear copy, dword fill, batched
+// small copies.  They take the place of ROCr's CopyAligned, CopyMisaligned and
+// Fill shaders (projects/rocr-runtime/runtime/hsa-runtime/core/runtime/
+// blit_shaders/blit_copyAligned.s:76-259, blit_copyMisaligned.s:90-182,
+// blit_fill.s:91-185) but share none of their structure:
+//
+//  * Every global access in the body is a 16-byte global_load/store_dwordx4;
+//    one wave instruction moves a contiguous 1 KiB.
+//  * A wave owns a contiguous tile of 64 * U vectors and issues all U loads
+//    before its first store, so U KiB per wave are in flight.  By default the
+//    grid has one wave per tile: the hardware dispatcher hands tiles out in
+//    address order as waves retire, which keeps the set of DRAM pages in use
+//    small; measured on MI355X this beats a persistent grid-stride loop by
+//    ~10 % at 1 GiB.  The grid-stride loop remains for capped grids.
+//  * Large transfers bypass the caches: loads carry nt, stores are written
+//    through L2 (sc1 / sc0 sc1), chosen per size by the host.
+//  * Stores are always 16-byte aligned: the destination is aligned first and
+//    the source takes whatever alignment is left.  When source and destination
+//    differ by a multiple of 4 the loads are dword-aligned dwordx4.  Otherwise
+//    each lane loads the dword-aligned 16 bytes that contain its source bytes,
+//    takes the 17th..20th byte from the next lane with a DPP wave rotate, and
+//    rebuilds its vector with four v_alignbyte_b32.  No sub-dword access is
+//    made outside the <=15-byte head and tail of a copy.
+//  * The source is never read outside the aligned dwords that contain at
+//    least one requested byte, so no access can touch a page the copy does
+//    not own.
+#ifndef MI355_BLIT_KERNELS_H_
+#define MI355_BLIT_KERNELS_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mi355 {
+
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+// Same vector with only dword alignment promised: the compiler still emits one
+// global_load_dwordx4, which the memory pipeline accepts at any dword address.
+typedef v4u v4u_a4 __attribute__((aligned(4)));
+
+constexpr unsigned kWave = 64;
+
+struct CopyArgs {
+  uint8_t* dst;
+  const uint8_t* src;
+  uint64_t bytes;
+  uint64_t n_vec;  // 16-byte vectors in the body
+  uint32_t head;   // bytes in front of the body, <= 15
+  // Waves that take the partial last tile and the head/tail bytes: the two
+  // after the wave of the last full tile, n_full % n_waves and
+  // (n_full + 1) % n_waves, worked out on the host.
+  uint32_t partial_wave;
+  uint32_t edge_wave;
+};
+
+struct FillArgs {
+  uint32_t* dst;
+  uint64_t n_dwords;
+  uint64_t n_vec;  // 16-byte vectors in the body
+  uint32_t head;   // dwords in front of the body, <= 3
+  uint32_t value;
+  uint32_t partial_wave;  // as in CopyArgs
+  uint32_t edge_wave;
+};
+
+template <bool NT>
+__device__ __forceinline__ v4u ld_v4(const v4u_a4* p) {
+  if constexpr (NT) return __builtin_nontemporal_load(p);
+  else return *p;
+}
+template <bool NT>
+__device__ __forceinline__ unsigned ld_u32(const unsigned* p) {
+  if constexpr (NT) return __builtin_nontemporal_load(p);
+  else return *p;
+}
+// Store cache policies (values of mi355_blit_plan_t::store_policy).
+constexpr int kStoreCached = 0;   // plain write-back L2
+constexpr int kStoreNt = 1;       // non-temporal hint
+constexpr int kStoreAgentWt = 2;  // sc1: written through L2 at agent scope
+constexpr int kStoreSystemWt = 3; // sc0 sc1: written through at system scope
+
+// The write-through forms have no builtin for a 16-byte store, hence the asm.
+// A store needs no wait of its own, and on gfx9 the extra outstanding store
+// only makes a compiler-placed s_waitcnt vmcnt(n) wait longer, never shorter.
+// A store of more than 8 bytes reads its data registers after issue: a VALU
+// write to them within the next 2 wait states (gfx940 and later) corrupts the
+// data.  The compiler pads its own stores but cannot see into the asm, so the
+// s_nop is part of it.
+template <int POLICY>
+__device__ __forceinline__ void st_v4(v4u* p, v4u v) {
+  if constexpr (POLICY == kStoreNt) {
+    __builtin_nontemporal_store(v, p);
+  } else if constexpr (POLICY == kStoreAgentWt) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
+  } else if constexpr (POLICY == kStoreSystemWt) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
+  } else {
+    *p = v;
+  }
+}
+
+// Lane i receives the value lane (i + 1) % 64 passed in (DPP wave_rol:1).
+__device__ __forceinline__ unsigned wave_rotate_down1(unsigned v) {
+  return __builtin_amdgcn_update_dpp(0u, v, 0x134, 0xf, 0xf, false);
+}
+
+// Bytes r..r+3 of the little-endian pair {hi:lo}, r in 0..3.
+__device__ __forceinline__ unsigned shift_bytes(unsigned hi, unsigned lo, unsigned r) {
+  return __builtin_amdgcn_alignbyte(hi, lo, r);
+}
+
+__device__ __forceinline__ v4u realign(v4u x, unsigned w4, unsigned r) {
+  v4u o;
+  o.x = shift_bytes(x.y, x.x, r);
+  o.y = shift_bytes(x.z, x.y, r);
+  o.z = shift_bytes(x.w, x.z, r);
+  o.w = shift_bytes(w4, x.w, r);
+  return o;
+}
+
+// Copies n_vec 16-byte vectors to the 16-byte aligned d.  Source vector v
+// starts r bytes after s + v, where s is dword aligned; r != 0 only when
+// SHIFT.  Called by whole waves: wave w of n_waves takes tiles w, w + n_waves,
+// ...; wave partial_wave takes the vectors after the last full tile.
+template <int U, bool NTL, int NTS, bool SHIFT>
+__device__ __forceinline__ void copy_vectors(v4u* __restrict__ d, const v4u_a4* __restrict__ s,
+                                             unsigned r, uint64_t n_vec, uint64_t wave,
+                                             uint64_t n_waves, uint64_t partial_wave,
+                                             unsigned lane) {
+  constexpr uint64_t kTile = kWave * U;
+  const uint64_t n_full = n_vec / kTile;
+  for (uint64_t t = wave; t < n_full; t += n_waves) {
+    const uint64_t base = t * kTile + lane;
+    v4u x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) x[u] = ld_v4<NTL>(s + base + u * kWave);
+    if constexpr (SHIFT) {
+      // Lane 0 fetches the first dword after the tile: with r != 0 it holds
+      // the last r bytes the tile needs, so it is always a wanted dword.
+      unsigned e = 0;
+      if (lane == 0) e = ld_u32<NTL>(reinterpret_cast<const unsigned*>(s + t * kTile + kTile));
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const unsigned nxt = (u + 1 < U) ? x[u + 1 < U ? u + 1 : u].x : e;
+        const unsigned w4 = wave_rotate_down1(lane == 0 ? nxt : x[u].x);
+        st_v4<NTS>(d + base + u * kWave, realign(x[u], w4, r));
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) st_v4<NTS>(d + base + u * kWave, x[u]);
+    }
+  }
+  if (wave == partial_wave) {
+    for (uint64_t v = n_full * kTile + lane; v < n_vec; v += kWave) {
+      v4u x = ld_v4<NTL>(s + v);
+      if constexpr (SHIFT) {
+        const unsigned w4 = ld_u32<NTL>(reinterpret_cast<const unsigned*>(s + v + 1));
+        x = realign(x, w4, r);
+      }
+      st_v4<NTS>(d + v, x);
+    }
+  }
+}
+
+// Head (< 16 bytes in front of the first aligned vector) and tail (< 16 bytes
+// after the last one), one byte per lane: lanes 0..15 head, 16..31 tail.
+__device__ __forceinline__ void copy_edges(uint8_t* dst, const uint8_t* src, uint64_t bytes,
+                                           unsigned head, uint64_t n_vec, unsigned lane) {
+  const uint64_t tail_off = head + 16 * n_vec;
+  const unsigned tail = static_cast<unsigned>(bytes - tail_off);
+  if (lane < head) {
+    dst[lane] = src[lane];
+  } else if (lane >= 16 && lane - 16 < tail) {
+    dst[tail_off + lane - 16] = src[tail_off + lane - 16];
+  }
+}
+
+template <int U, bool NTL, int NTS, bool SHIFT>
+__global__ void __launch_bounds__(1024) k_copy(CopyArgs a) {
+  const unsigned lane = threadIdx.x & (kWave - 1);
+  const unsigned waves_per_wg = blockDim.x / kWave;
+  const uint64_t wave =
+      __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
+  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * waves_per_wg;
+  const uint8_t* sb = a.src + a.head;
+  const unsigned r = SHIFT ? static_cast<unsigned>(reinterpret_cast<uintptr_t>(sb) & 3) : 0;
+  copy_vectors<U, NTL, NTS, SHIFT>(reinterpret_cast<v4u*>(a.dst + a.head),
+                                   reinterpret_cast<const v4u_a4*>(sb - r), r, a.n_vec, wave,
+                                   n_waves, a.partial_wave, lane);
+  if (wave == a.edge_wave) copy_edges(a.dst, a.src, a.bytes, a.head, a.n_vec, lane);
+}
+
+template <int U, int NTS>
+__global__ void __launch_bounds__(1024) k_fill(FillArgs a) {
+  const unsigned lane = threadIdx.x & (kWave - 1);
+  const unsigned waves_per_wg = blockDim.x / kWave;
+  const uint64_t wave =
+      __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
+  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * waves_per_wg;
+  const v4u val = {a.value, a.value, a.value, a.value};
+  v4u* d = reinterpret_cast<v4u*>(a.dst + a.head);
+  constexpr uint64_t kTile = kWave * U;
+  const uint64_t n_full = a.n_vec / kTile;
+  for (uint64_t t = wave; t < n_full; t += n_waves) {
+    const uint64_t base = t * kTile + lane;
+#pragma unroll
+    for (int u = 0; u < U; ++u) st_v4<NTS>(d + base + u * kWave, val);
+  }
+  if (wave == a.partial_wave) {
+    for (uint64_t v = n_full * kTile + lane; v < a.n_vec; v += kWave) st_v4<NTS>(d + v, val);
+  }
+  if (wave == a.edge_wave) {
+    // whole dwords outside the vector body: lanes 0..3 head, 4..7 tail
+    const uint64_t tail_off = a.head + 4 * a.n_vec;
+    const unsigned tail = static_cast<unsigned>(a.n_dwords - tail_off);
+    if (lane < a.head) a.dst[lane] = a.value;
+    else if (lane >= 4 && lane - 4 < tail) a.dst[tail_off + lane - 4] = a.value;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Batched small copies: n descriptors {dst, src, bytes}, one submission.
+// Each copy is cut into chunks of kChunkVecs body vectors (the first chunk
+// also moves the head bytes, the last one the tail bytes); a prefix sum over
+// the chunk counts lets every wave take an equal, contiguous share of all
+// chunks, so a 64-byte copy and a 256 KiB copy load the device evenly.
+// ---------------------------------------------------------------------------
+
+struct BatchDesc {
+  uint8_t* dst;
+  const uint8_t* src;
+  uint64_t bytes;
+};
+
+constexpr unsigned kChunkVecs = 256;  // 4 KiB: one wave, four vectors per lane
+
+__device__ __forceinline__ unsigned desc_head(const BatchDesc& d) {
+  const unsigned h = (16 - (static_cast<unsigned>(reinterpret_cast<uintptr_t>(d.dst)) & 15)) & 15;
+  return h > d.bytes ? static_cast<unsigned>(d.bytes) : h;
+}
+
+__device__ __forceinline__ unsigned desc_chunks(const BatchDesc& d) {
+  if (d.bytes == 0) return 0;
+  const uint64_t n_vec = (d.bytes - desc_head(d)) / 16;
+  const uint64_t c = (n_vec + kChunkVecs - 1) / kChunkVecs;
+  return c ? static_cast<unsigned>(c) : 1u;
+}
+
+// chunk_start[i] = chunks of copies 0..i-1, chunk_start[n] = all chunks.
+// One workgroup of 1024 lanes; lane t owns a contiguous run of descriptors.
+__global__ void __launch_bounds__(1024) k_batch_scan(const BatchDesc* __restrict__ descs, uint64_t n,
+                                                     uint32_t* __restrict__ chunk_start) {
+  __shared__ uint32_t part[1024];
+  const unsigned t = threadIdx.x;
+  const uint64_t per = (n + 1023) / 1024;
+  const uint64_t lo = t * per < n ? t * per : n;
+  const uint64_t hi = lo + per < n ? lo + per : n;
+  uint32_t sum = 0;
+  for (uint64_t i = lo; i < hi; ++i) sum += desc_chunks(descs[i]);
+  part[t] = sum;
+  __syncthreads();
+  for (unsigned off = 1; off < 1024; off <<= 1) {
+    const uint32_t add = t >= off ? part[t - off] : 0;
+    __syncthreads();
+    part[t] += add;
+    __syncthreads();
+  }
+  uint32_t run = part[t] - sum;  // exclusive prefix of this lane's run
+  for (uint64_t i = lo; i < hi; ++i) {
+    chunk_start[i] = run;
+    run += desc_chunks(descs[i]);
+  }
+  if (t == 1023) chunk_start[n] = part[1023];
+}
+
+// One chunk of one copy, done by one wave.
+template <bool NTL, int NTS, bool SHIFT>
+__device__ __forceinline__ void copy_chunk(v4u* __restrict__ d, const v4u_a4* __restrict__ s,
+                                           unsigned r, unsigned n_vec, unsigned lane) {
+  constexpr int U = kChunkVecs / kWave;
+  if (n_vec == kChunkVecs) {
+    v4u x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) x[u] = ld_v4<NTL>(s + lane + u * kWave);
+    if constexpr (SHIFT) {
+      unsigned e = 0;
+      if (lane == 0) e = ld_u32<NTL>(reinterpret_cast<const unsigned*>(s + kChunkVecs));
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const unsigned nxt = (u + 1 < U) ? x[u + 1 < U ? u + 1 : u].x : e;
+        const unsigned w4 = wave_rotate_down1(lane == 0 ? nxt : x[u].x);
+        st_v4<NTS>(d + lane + u * kWave, realign(x[u], w4, r));
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) st_v4<NTS>(d + lane + u * kWave, x[u]);
+    }
+  } else {
+    for (unsigned v = lane; v < n_vec; v += kWave) {
+      v4u x = ld_v4<NTL>(s + v);
+      if constexpr (SHIFT) {
+        const unsigned w4 = ld_u32<NTL>(reinterpret_cast<const unsigned*>(s + v + 1));
+        x = realign(x, w4, r);
+      }
+      st_v4<NTS>(d + v, x);
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256) k_batch_copy(const BatchDesc* __restrict__ descs, uint64_t n,
+                                                    const uint32_t* __restrict__ chunk_start) {
+  const unsigned lane = threadIdx.x & (kWave - 1);
+  const unsigned waves_per_wg = blockDim.x / kWave;
+  const uint64_t wave =
+      __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
+  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * waves_per_wg;
+  const uint64_t total = chunk_start[n];
+  const uint64_t c0 = total * wave / n_waves;
+  const uint64_t c1 = total * (wave + 1) / n_waves;
+  if (c0 >= c1) return;
+  // largest i with chunk_start[i] <= c0 (copies without chunks share a start
+  // with their successor; they are stepped over below)
+  uint64_t lo = 0, hi = n;
+  while (lo < hi) {
+    const uint64_t mid = (lo + hi + 1) / 2;
+    if (chunk_start[mid] <= c0) lo = mid; else hi = mid - 1;
+  }
+  uint64_t i = lo;
+  uint64_t c = c0;
+  while (c < c1 && i < n) {
+    const uint64_t cs = chunk_start[i];
+    const uint64_t ce = chunk_start[i + 1];
+    if (ce <= c) { ++i; continue; }
+    const BatchDesc dsc = descs[i];
+    const unsigned head = desc_head(dsc);
+    const uint64_t n_vec = (dsc.bytes - head) / 16;
+    const uint8_t* sb = dsc.src + head;
+    const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(sb)) & 3;
+    v4u* d = reinterpret_cast<v4u*>(dsc.dst + head);
+    const v4u_a4* s = reinterpret_cast<const v4u_a4*>(sb - r);
+    const uint64_t stop = ce < c1 ? ce : c1;
+    for (; c < stop; ++c) {
+      const uint64_t k = c - cs;
+      const uint64_t v0 = k * kChunkVecs;
+      const uint64_t left = n_vec > v0 ? n_vec - v0 : 0;
+      const unsigned nv = left < kChunkVecs ? static_cast<unsigned>(left) : kChunkVecs;
+      if (r) copy_chunk<false, kStoreCached, true>(d + v0, s + v0, r, nv, lane);
+      else copy_chunk<false, kStoreCached, false>(d + v0, s + v0, 0, nv, lane);
+      // first chunk moves the head bytes, last chunk the tail bytes
+      if (k == 0 && lane < head) dsc.dst[lane] = dsc.src[lane];
+      if (c + 1 == ce) {
+        const uint64_t tail_off = head + 16 * n_vec;
+        const unsigned tail = static_cast<unsigned>(dsc.bytes - tail_off);
+        if (lane >= 16 && lane - 16 < tail) dsc.dst[tail_off + lane - 16] = dsc.src[tail_off + lane - 16];
+      }
+    }
+    ++i;
+  }
+}
+
+}  // namespace mi355
+
+#endif  // MI355_BLIT_KERNELS_H_

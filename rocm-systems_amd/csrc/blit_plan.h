@@ -1,0 +1,121 @@
+// Dispatch sizing for the gfx950 blit kernels: how a copy or fill is cut into
+// head / 16-byte body / tail, and which workgroup size, grid, unroll and cache
+// policy it is launched with.  Pure host arithmetic, no HIP.
+//
+// Takes the place of the phase arithmetic and fixed grids in ROCr's
+// BlitKernel (projects/rocr-runtime/runtime/hsa-runtime/core/runtime/
+// amd_blit_kernel.cpp:714-775 for copies, :796-813 for fills): there the grid
+// is always 64*4*num_cus (copy) or 64*num_cus (fill) single-wave workgroups
+// with one vector per lane in flight, whatever the size.
+#ifndef MI355_BLIT_PLAN_H_
+#define MI355_BLIT_PLAN_H_
+
+#include <stdint.h>
+
+#include "mi355_blit.h"
+
+namespace mi355 {
+
+// Vectors of one batched-copy chunk: one wave, four loads per lane.
+constexpr uint32_t kBatchChunkVecs = 256;
+// Workgroups of 256 lanes that fill one CU's wave slots (8 waves per SIMD);
+// used where a kernel wants a device-filling persistent grid.
+constexpr uint32_t kWgPerCu = 8;
+// The grid dimension is a 32-bit count of work-items in an AQL packet.
+constexpr uint64_t kMaxGridWorkItems = 0x7fffffc0ull;
+
+struct SizeClass {
+  uint64_t min_bytes;  // applies from this size up
+  uint32_t wg_size;
+  uint32_t unroll;
+  uint32_t nt_load;
+  uint32_t store_policy;
+};
+
+// Measured on MI355X (256 CUs): one 1 KiB tile per single-wave workgroup is
+// the fastest copy shape once the transfer streams from HBM; fills are store
+// issue bound in the dispatcher at that size and want 4-wave workgroups.
+// Transfers that cannot stay in cache bypass it.  Last match wins.
+constexpr SizeClass kCopyClasses[] = {
+    {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
+    {8ull << 20, 64, 1, 1, MI355_BLIT_STORE_AGENT_WT},
+};
+constexpr SizeClass kFillClasses[] = {
+    {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
+    {8ull << 20, 256, 1, 0, MI355_BLIT_STORE_SYSTEM_WT},
+};
+
+inline bool valid_unroll(uint32_t u) { return u == 1 || u == 2 || u == 4; }
+
+template <unsigned N>
+inline const SizeClass& pick_class(const SizeClass (&tbl)[N], uint64_t bytes) {
+  const SizeClass* c = &tbl[0];
+  for (unsigned i = 0; i < N; ++i)
+    if (bytes >= tbl[i].min_bytes) c = &tbl[i];
+  return *c;
+}
+
+inline void apply_launch_shape(mi355_blit_plan_t* p, const SizeClass& cls, uint32_t num_cus,
+                               const mi355_blit_tuning_t* t) {
+  (void)num_cus;
+  p->wg_size = cls.wg_size;
+  p->unroll = cls.unroll;
+  p->nt_load = cls.nt_load;
+  p->store_policy = cls.store_policy;
+  uint64_t max_grid = 0;
+  if (t) {
+    if (t->wg_size >= 64 && t->wg_size <= 1024 && (t->wg_size % 64) == 0) p->wg_size = t->wg_size;
+    if (valid_unroll(t->unroll)) p->unroll = t->unroll;
+    if (t->nt_load) p->nt_load = (t->nt_load == 2);
+    if (t->store_policy >= 1 && t->store_policy <= 4) p->store_policy = t->store_policy - 1;
+    max_grid = t->max_grid;
+  }
+  const uint64_t hw_max = kMaxGridWorkItems / p->wg_size;
+  if (max_grid == 0 || max_grid > hw_max) max_grid = hw_max;
+  // One wave per tile of 64*unroll vectors plus one for the edges; a capped
+  // grid makes the waves stride over the tiles instead.
+  const uint64_t tile_vecs = 64ull * p->unroll;
+  const uint64_t tiles = (p->body_vecs + tile_vecs - 1) / tile_vecs;
+  const uint64_t waves = tiles + 1;
+  const uint64_t waves_per_wg = p->wg_size / 64;
+  uint64_t wgs = (waves + waves_per_wg - 1) / waves_per_wg;
+  if (wgs > max_grid) wgs = max_grid;
+  if (wgs == 0) wgs = 1;
+  p->grid = static_cast<uint32_t>(wgs);
+}
+
+inline int plan_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t num_cus,
+                     const mi355_blit_tuning_t* t, mi355_blit_plan_t* p) {
+  if (!p) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  *p = mi355_blit_plan_t{};
+  uint64_t head = (16 - (dst & 15)) & 15;
+  if (head > bytes) head = bytes;
+  p->head_bytes = head;
+  p->body_vecs = (bytes - head) / 16;
+  p->tail_bytes = bytes - head - 16 * p->body_vecs;
+  p->byte_shift = static_cast<uint32_t>((src - dst) & 3);
+  p->kernel = p->byte_shift ? MI355_BLIT_KERNEL_COPY_REALIGN : MI355_BLIT_KERNEL_COPY;
+  apply_launch_shape(p, pick_class(kCopyClasses, bytes), num_cus, t);
+  return MI355_BLIT_SUCCESS;
+}
+
+inline int plan_fill(uint64_t ptr, uint64_t num_dwords, uint32_t num_cus,
+                     const mi355_blit_tuning_t* t, mi355_blit_plan_t* p) {
+  if (!p) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (ptr & 3) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  *p = mi355_blit_plan_t{};
+  const uint64_t bytes = num_dwords * 4;
+  uint64_t head = (16 - (ptr & 15)) & 15;
+  if (head > bytes) head = bytes;
+  p->head_bytes = head;
+  p->body_vecs = (bytes - head) / 16;
+  p->tail_bytes = bytes - head - 16 * p->body_vecs;
+  p->kernel = MI355_BLIT_KERNEL_FILL;
+  apply_launch_shape(p, pick_class(kFillClasses, bytes), num_cus, t);
+  p->nt_load = 0;
+  return MI355_BLIT_SUCCESS;
+}
+
+}  // namespace mi355
+
+#endif  // MI355_BLIT_PLAN_H_

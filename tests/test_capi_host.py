@@ -1,0 +1,146 @@
+"""Host-only checks of the C ABI: the library loads, exports every symbol the
+header declares, validates arguments, and its dispatch-sizing functions obey
+the plan's invariants.  No compute calls: there is no GPU here."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _has_gpu():
+    import torch
+    return torch.cuda.is_available()
+
+
+@pytest.fixture(scope="module")
+def capi_host(pkg):
+    import torch  # noqa: F401  (one HIP runtime per process: torch's first)
+    pkg.capi.load()
+    return pkg.capi
+
+
+def test_library_exports_every_declared_symbol(capi_host):
+    header = open(os.path.join(ROOT, "include", "mi355_blit.h")).read()
+    declared = set(re.findall(r"\b(mi355_blit_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    lib = C.CDLL(capi_host.library_path())
+    for name in sorted(declared):
+        assert hasattr(lib, name), "library does not export %s" % name
+    # and the ctypes binding declares exactly the same set
+    assert declared == set(capi_host.SIGNATURES)
+
+
+def test_abi_version_and_status_strings(capi_host):
+    lib = capi_host.load()
+    assert lib.mi355_blit_abi_version() == 1
+    assert lib.mi355_blit_status_string(0) == b"success"
+    assert lib.mi355_blit_status_string(capi_host.ERROR_INVALID_ARGUMENT) == b"invalid argument"
+    assert lib.mi355_blit_status_string(12345) == b"unknown status"
+
+
+def test_struct_layouts_match_header(capi_host):
+    assert C.sizeof(capi_host.Plan) == 8 * 4 + 3 * 8
+    assert C.sizeof(capi_host.Tuning) == 32
+    assert C.sizeof(capi_host.Desc) == 24
+
+
+def test_null_handle_is_rejected(capi_host):
+    lib = capi_host.load()
+    inv = capi_host.ERROR_INVALID_ARGUMENT
+    assert lib.mi355_blit_destroy(None) == inv
+    assert lib.mi355_blit_copy(None, 16, 32, 8, None) == inv
+    assert lib.mi355_blit_fill32(None, 16, 0, 8, None) == inv
+    assert lib.mi355_blit_copy_batch(None, None, 0, 0, None) == inv
+    assert lib.mi355_blit_synchronize(None) == inv
+    assert lib.mi355_blit_pending_bytes(None) == 0
+    assert lib.mi355_blit_create(0, None) == inv
+
+
+def test_create_without_gpu_fails_loudly(capi_host):
+    if _has_gpu():
+        pytest.skip("a GPU is present")
+    h = C.c_void_p()
+    st = capi_host.load().mi355_blit_create(0, C.byref(h))
+    assert st == capi_host.ERROR_NOT_INITIALIZED and not h.value
+    with pytest.raises(capi_host.BlitError):
+        capi_host.Blit(0)
+
+
+def _check_copy_plan(p, dst, src, n):
+    assert p.head_bytes + 16 * p.body_vecs + p.tail_bytes == n
+    assert p.head_bytes <= 15 and p.tail_bytes <= 15
+    if p.body_vecs:
+        assert (dst + p.head_bytes) % 16 == 0
+    assert p.byte_shift == (src - dst) % 4
+    assert p.kernel == (1 if p.byte_shift else 0)
+    assert p.wg_size % 64 == 0 and 64 <= p.wg_size <= 1024
+    assert p.unroll in (1, 2, 4)
+    assert p.grid >= 1 and p.grid * p.wg_size < 2 ** 31
+    # uncapped: one wave per tile plus one for the edges
+    tiles = -(-p.body_vecs // (64 * p.unroll))
+    assert p.grid * (p.wg_size // 64) >= min(tiles + 1, p.grid * (p.wg_size // 64))
+
+
+def test_plan_copy_invariants(capi_host):
+    sizes = list(range(0, 70)) + [255, 256, 257, 1023, 1024, 1025, 4096, 65537, (1 << 20) + 3,
+                                  (8 << 20) - 1, 8 << 20, (1 << 30), (1 << 32), (1 << 32) + 17]
+    for d_off in range(16):
+        for s_off in range(16):
+            dst, src = 0x7f0000001000 + d_off, 0x7e0000002000 + s_off
+            for n in sizes:
+                st, p = capi_host.plan_copy(dst, src, n)
+                assert st == 0
+                _check_copy_plan(p, dst, src, n)
+
+
+def test_plan_copy_covers_every_tile_when_uncapped(capi_host):
+    for n in (1 << 30, (1 << 32) + 5, 12345678):
+        st, p = capi_host.plan_copy(0x7f0000000000, 0x7e0000000000, n)
+        tiles = -(-p.body_vecs // (64 * p.unroll))
+        assert p.grid * (p.wg_size // 64) >= tiles + 1
+
+
+def test_plan_copy_tuning_overrides(capi_host):
+    t = capi_host.Tuning(wg_size=512, unroll=4, max_grid=100, nt_load=2, store_policy=capi_host.STORE_NT + 1)
+    st, p = capi_host.plan_copy(0x1000, 0x9000, 1 << 30, 256, t)
+    assert st == 0 and (p.wg_size, p.unroll, p.grid, p.nt_load, p.store_policy) == (512, 4, 100, 1, capi_host.STORE_NT)
+    # nonsense values are ignored rather than launched
+    t = capi_host.Tuning(wg_size=100, unroll=3, store_policy=9)
+    st, q = capi_host.plan_copy(0x1000, 0x9000, 1 << 30, 256, t)
+    st, d = capi_host.plan_copy(0x1000, 0x9000, 1 << 30, 256)
+    assert (q.wg_size, q.unroll, q.store_policy) == (d.wg_size, d.unroll, d.store_policy)
+    t = capi_host.Tuning(nt_load=1, store_policy=capi_host.STORE_CACHED + 1)
+    st, p = capi_host.plan_copy(0x1000, 0x9000, 1 << 30, 256, t)
+    assert p.nt_load == 0 and p.store_policy == capi_host.STORE_CACHED
+
+
+def test_plan_fill_invariants(capi_host):
+    for off in (0, 4, 8, 12):
+        ptr = 0x7f0000000000 + off
+        for count in list(range(0, 40)) + [1023, 1024, 1 << 18, (1 << 28), (1 << 30) + 3]:
+            st, p = capi_host.plan_fill(ptr, count)
+            assert st == 0 and p.kernel == 2
+            assert p.head_bytes + 16 * p.body_vecs + p.tail_bytes == 4 * count
+            assert p.head_bytes % 4 == 0 and p.tail_bytes % 4 == 0
+            assert p.head_bytes <= 12 and p.tail_bytes <= 12
+            if p.body_vecs:
+                assert (ptr + p.head_bytes) % 16 == 0
+    for off in (1, 2, 3):
+        st, _ = capi_host.plan_fill(0x1000 + off, 4)
+        assert st == capi_host.ERROR_INVALID_ARGUMENT
+    assert capi_host.load().mi355_blit_plan_fill(0x1000, 4, 256, None, None) == capi_host.ERROR_INVALID_ARGUMENT
+    assert capi_host.load().mi355_blit_plan_copy(0x1000, 0x2000, 4, 256, None, None) == capi_host.ERROR_INVALID_ARGUMENT
+
+
+def test_kernel_choice_matches_reference_predicate(capi_host, oracle):
+    """Same split as amd_blit_kernel.cpp:716: (src & 3) == (dst & 3)."""
+    from conftest import KernArgs
+    ka = KernArgs()
+    for d in range(16):
+        for s in range(16):
+            st, p = capi_host.plan_copy(0x10000 + d, 0x90000 + s, 4096)
+            ref = oracle.oracle_ref_plan_copy(0x10000 + d, 0x90000 + s, 4096, 256, C.byref(ka))
+            assert p.kernel == ref

@@ -1,0 +1,520 @@
+"""Parity of the gfx950 blit kernels with the CPU oracle, through the C ABI.
+Bit-exact: every byte of the destination, guard bands included, must equal
+what the oracle (host memcpy / dword fill) leaves on the same seeded inputs."""
+import ctypes as C
+import threading
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+GUARD = 256
+GUARD_BYTE = 0xEE
+FILL_VALUE = 0xA5C30F1E  # the benchmark's pattern
+MIB = 1 << 20
+
+
+class Arena:
+    """A device buffer with a host mirror.  Offsets are relative to a 256-byte
+    aligned device address, so `off & 15` is the device pointer's alignment."""
+
+    def __init__(self, torch, nbytes, fill=None, host=None):
+        self.torch = torch
+        self.nbytes = nbytes
+        self.t = torch.empty(nbytes + 256, dtype=torch.uint8, device="cuda:0")
+        self.shift = (-self.t.data_ptr()) % 256
+        self.base = self.t.data_ptr() + self.shift
+        self.view = self.t[self.shift:self.shift + nbytes]
+        if host is not None:
+            self.view.copy_(torch.from_numpy(host))
+        elif fill is not None:
+            self.view.fill_(fill)
+        torch.cuda.synchronize()
+
+    def fill(self, lo, hi, value):
+        """Set bytes on torch's stream and wait: the blit runs on its own stream."""
+        self.view[lo:hi].fill_(value)
+        self.torch.cuda.synchronize()
+
+    def host(self, lo=0, hi=None):
+        hi = self.nbytes if hi is None else hi
+        return self.view[lo:hi].cpu().numpy()
+
+
+def check_ok(capi, st, what):
+    assert st == capi.SUCCESS, "%s returned 0x%x" % (what, st)
+
+
+def run_copy_case(capi, blit, oracle, src_arena, src_host, dst_arena, s_off, d_off, n):
+    """Copy n bytes; compare [d_off-GUARD, d_off+n+GUARD) with the oracle."""
+    lo, hi = d_off - GUARD, d_off + n + GUARD
+    assert lo >= 0 and hi <= dst_arena.nbytes and s_off + n <= src_arena.nbytes
+    dst_arena.fill(lo, hi, GUARD_BYTE)
+    check_ok(capi, blit.copy(dst_arena.base + d_off, src_arena.base + s_off, n), "copy")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    got = dst_arena.host(lo, hi)
+    want = np.full(hi - lo, GUARD_BYTE, dtype=np.uint8)
+    oracle.oracle_copy(want.ctypes.data + GUARD, src_host.ctypes.data + s_off, n)
+    if not np.array_equal(got, want):
+        bad = np.nonzero(got != want)[0]
+        raise AssertionError("copy mismatch s_off=%d d_off=%d n=%d: %d bytes differ, first at %d "
+                             "(relative to dst start: %d), plan=%s"
+                             % (s_off, d_off, n, bad.size, bad[0], bad[0] - GUARD,
+                                blit.last_plan().as_dict()))
+
+
+@pytest.fixture(scope="module")
+def arenas(torch_cuda, rand):
+    """64 MiB (+ slack) source with seeded bytes and a destination of the same size."""
+    n = 64 * MIB + 2 * MIB
+    src_host = rand(n, 0xB1170004)
+    src = Arena(torch_cuda, n, host=src_host)
+    dst = Arena(torch_cuda, n, fill=GUARD_BYTE)
+    return src, src_host, dst
+
+
+# ---------------------------------------------------------------- aligned copy
+
+@pytest.mark.parametrize("n", [4096 * 4 ** k for k in range(8)])  # 4 KiB .. 64 MiB
+def test_aligned_copy_sweep(capi, blit, oracle, arenas, n):
+    src, src_host, dst = arenas
+    run_copy_case(capi, blit, oracle, src, src_host, dst, 0, GUARD, n)
+    p = blit.last_plan()
+    assert p.kernel == capi.KERNEL_COPY and p.head_bytes == 0 and p.tail_bytes == 0
+
+
+def test_reference_perf_sizes(capi, blit, oracle, arenas):
+    """Sizes of rocrtst's Memory_Async_Copy (memory_async_copy.h:207-216), to 32 MiB."""
+    src, src_host, dst = arenas
+    for k in range(16):
+        run_copy_case(capi, blit, oracle, src, src_host, dst, 0, GUARD, 1024 << k)
+
+
+@pytest.mark.parametrize("n", [256 * MIB, 1 << 30])
+def test_aligned_copy_large_full_compare(capi, blit, oracle, rand, torch_cuda, n):
+    """Headline size, every byte against the oracle."""
+    torch = torch_cuda
+    src_host = rand(n, 0xB1170003)
+    src = Arena(torch, n, host=src_host)
+    dst = Arena(torch, n + 2 * GUARD, fill=GUARD_BYTE)
+    check_ok(capi, blit.copy(dst.base + GUARD, src.base, n), "copy")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    got = dst.host()
+    want = np.full(n + 2 * GUARD, GUARD_BYTE, dtype=np.uint8)
+    oracle.oracle_copy(want.ctypes.data + GUARD, src_host.ctypes.data, n)
+    assert np.array_equal(got, want)
+
+
+def test_copy_4gib_properties(capi, blit, oracle, rand, torch_cuda):
+    """Maximum sweep size.  A host compare of 4 GiB is slow, so: the source is a
+    64 MiB seeded block repeated 64 times; after the copy every 64 MiB slice of
+    the destination must hash like the oracle's copy of that block, the device
+    compare dst == src must hold, and the guards must be intact."""
+    torch = torch_cuda
+    n = 4 << 30
+    blk = 64 * MIB
+    block_host = rand(blk, 0xB1170033)
+    src = Arena(torch, n)
+    block_dev = torch.from_numpy(block_host).to("cuda:0")
+    for i in range(n // blk):
+        src.view[i * blk:(i + 1) * blk].copy_(block_dev)
+    torch.cuda.synchronize()
+    dst = Arena(torch, n + 2 * GUARD, fill=GUARD_BYTE)
+    check_ok(capi, blit.copy(dst.base + GUARD, src.base, n), "copy")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert bool((dst.view[:GUARD] == GUARD_BYTE).all()) and bool((dst.view[GUARD + n:] == GUARD_BYTE).all())
+    assert torch.equal(dst.view[GUARD:GUARD + n], src.view)
+    want = np.empty(blk, dtype=np.uint8)
+    oracle.oracle_copy(want.ctypes.data, block_host.ctypes.data, blk)
+    want_hash = oracle.oracle_fnv1a64(want.ctypes.data, 1 << 16)
+    for i in (0, 1, 31, 62, 63):
+        got = dst.host(GUARD + i * blk, GUARD + (i + 1) * blk)
+        assert np.array_equal(got, want), "slice %d differs" % i
+        assert oracle.oracle_fnv1a64(got.ctypes.data, 1 << 16) == want_hash
+    p = blit.last_plan()
+    assert p.grid * (p.wg_size // 64) >= -(-p.body_vecs // (64 * p.unroll))
+
+
+# -------------------------------------------------------------- misaligned copy
+
+def _log_uniform_lengths(rng, k, max_bytes):
+    return np.maximum(1, np.floor(2.0 ** (np.log2(max_bytes) * rng.random(k)))).astype(np.int64)
+
+
+def test_misaligned_all_256_offset_pairs(capi, blit, oracle, arenas):
+    """Every (src & 15, dst & 15) pair, 8 log-uniform lengths 1 B .. 64 MiB each
+    (most draws are capped at 4 MiB to keep the host compare short; each pair
+    class still meets lengths up to 64 MiB), guards checked."""
+    src, src_host, dst = arenas
+    rng = np.random.default_rng(0xB1170004)
+    for so in range(16):
+        for do in range(16):
+            lens = _log_uniform_lengths(rng, 8, 64 * MIB)
+            big_ok = (so * 16 + do) % 37 == 0
+            for n in lens:
+                n = int(n)
+                if n > 4 * MIB and not big_ok:
+                    n = int(n % (4 * MIB)) + 1
+                run_copy_case(capi, blit, oracle, src, src_host, dst, 512 + so, GUARD + 16 + do, n)
+                p = blit.last_plan()
+                assert p.byte_shift == (so - do) % 4
+
+
+def test_misaligned_tiny_lengths_every_pair(capi, blit, oracle, arenas):
+    """Lengths 1..40 for every offset pair: all head/tail/body splits near zero.
+    Each length has its own 128-byte slot, so one compare covers a pair."""
+    src, src_host, dst = arenas
+    slot = 128
+    span = GUARD + 41 * slot + GUARD
+    for so in range(16):
+        for do in range(16):
+            dst.fill(0, span, GUARD_BYTE)
+            want = np.full(span, GUARD_BYTE, dtype=np.uint8)
+            for n in range(1, 41):
+                d_off = GUARD + n * slot + do
+                s_off = 1024 + n * 64 + so
+                check_ok(capi, blit.copy(dst.base + d_off, src.base + s_off, n), "copy")
+                oracle.oracle_copy(want.ctypes.data + d_off, src_host.ctypes.data + s_off, n)
+            check_ok(capi, blit.synchronize(), "synchronize")
+            got = dst.host(0, span)
+            if not np.array_equal(got, want):
+                bad = np.nonzero(got != want)[0]
+                raise AssertionError("so=%d do=%d: first bad byte at %d (slot %d)"
+                                     % (so, do, bad[0], (bad[0] - GUARD) // slot))
+
+
+@pytest.mark.parametrize("so,do", [(0, 0), (4, 0), (0, 8), (1, 0), (0, 2), (3, 0), (7, 13), (15, 1), (5, 5)])
+def test_misaligned_1gib_headline(capi, blit, oracle, rand, torch_cuda, so, do):
+    """1 GiB per representative class of ((so-do) & 3, (so-do) & 12); every
+    byte against the oracle."""
+    torch = torch_cuda
+    n = (1 << 30) - 64
+    src_host = rand(n + 64, 0xB1170044 + so * 16 + do)
+    src = Arena(torch, n + 64, host=src_host)
+    dst = Arena(torch, n + 2 * GUARD + 64, fill=GUARD_BYTE)
+    check_ok(capi, blit.copy(dst.base + GUARD + do, src.base + so, n), "copy")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    got = dst.host()
+    want = np.full(dst.nbytes, GUARD_BYTE, dtype=np.uint8)
+    oracle.oracle_copy(want.ctypes.data + GUARD + do, src_host.ctypes.data + so, n)
+    assert np.array_equal(got, want)
+
+
+# ------------------------------------------------------------------------- fill
+
+def run_fill_case(capi, blit, oracle, dst, d_off, count, value):
+    lo, hi = d_off - GUARD, d_off + 4 * count + GUARD
+    dst.fill(lo, hi, GUARD_BYTE)
+    check_ok(capi, blit.fill32(dst.base + d_off, value, count), "fill32")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    got = dst.host(lo, hi)
+    want = np.full(hi - lo, GUARD_BYTE, dtype=np.uint8)
+    oracle.oracle_fill32(want.ctypes.data + GUARD, value, count)
+    if not np.array_equal(got, want):
+        bad = np.nonzero(got != want)[0]
+        raise AssertionError("fill mismatch d_off=%d count=%d: %d bytes differ, first at %d, plan=%s"
+                             % (d_off, count, bad.size, bad[0] - GUARD, blit.last_plan().as_dict()))
+
+
+@pytest.mark.parametrize("nbytes", [4096 * 4 ** k for k in range(8)])
+def test_fill_sweep(capi, blit, oracle, arenas, nbytes):
+    _, _, dst = arenas
+    run_fill_case(capi, blit, oracle, dst, GUARD, nbytes // 4, FILL_VALUE)
+
+
+@pytest.mark.parametrize("value", [0xabcdef12, 0xba5eba11, 0xfeed5a1e, 0xbaadf00d])
+def test_fill_reference_patterns(capi, blit, oracle, arenas, value):
+    """async_mem_copy.cc:62-65: fill, then every dword must equal the pattern."""
+    _, _, dst = arenas
+    run_fill_case(capi, blit, oracle, dst, GUARD, MIB // 4, value)
+
+
+def test_fill_offsets_and_odd_counts(capi, blit, oracle, arenas):
+    _, _, dst = arenas
+    for off in (0, 4, 8, 12):
+        for count in list(range(1, 20)) + [63, 64, 65, 255, 257, 1023, 1025, 65537, (MIB // 4) + 3, (9 * MIB // 4) + 1]:
+            run_fill_case(capi, blit, oracle, dst, GUARD + off, count, FILL_VALUE ^ count)
+
+
+def test_fill_1gib_headline(capi, blit, oracle, torch_cuda):
+    torch = torch_cuda
+    count = 1 << 28
+    dst = Arena(torch, 4 * count + 2 * GUARD, fill=GUARD_BYTE)
+    # pre-fill with the complement so that an unwritten dword shows
+    dst.view[GUARD:GUARD + 4 * count].view(torch.int32).fill_(~FILL_VALUE & 0x7fffffff)
+    torch.cuda.synchronize()
+    check_ok(capi, blit.fill32(dst.base + GUARD, FILL_VALUE, count), "fill32")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    got = dst.host()
+    want = np.full(dst.nbytes, GUARD_BYTE, dtype=np.uint8)
+    oracle.oracle_fill32(want.ctypes.data + GUARD, FILL_VALUE, count)
+    assert np.array_equal(got, want)
+
+
+def test_fill_4gib_properties(capi, blit, torch_cuda):
+    torch = torch_cuda
+    count = 1 << 30
+    dst = Arena(torch, 4 * count + 2 * GUARD, fill=GUARD_BYTE)
+    check_ok(capi, blit.fill32(dst.base + GUARD, FILL_VALUE, count), "fill32")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    body = dst.view[GUARD:GUARD + 4 * count].view(torch.int32)
+    want = FILL_VALUE - (1 << 32)  # as int32
+    assert int(body.min()) == want and int(body.max()) == want
+    assert bool((dst.view[:GUARD] == GUARD_BYTE).all()) and bool((dst.view[GUARD + 4 * count:] == GUARD_BYTE).all())
+
+
+# --------------------------------------------------------------- kernel variants
+
+@pytest.mark.parametrize("unroll", [1, 2, 4])
+@pytest.mark.parametrize("wg", [64, 256, 1024])
+def test_every_copy_variant_is_exact(capi, fresh_tuning, oracle, arenas, unroll, wg):
+    """Each instantiation (unroll x load policy x store policy x realign) and a
+    capped grid (waves striding over tiles) against the oracle."""
+    blit = fresh_tuning
+    src, src_host, dst = arenas
+    n = 3 * MIB + 4321
+    for nt_load in (1, 2):
+        for policy in range(4):
+            for max_grid in (0, 7):
+                blit.set_tuning(wg_size=wg, unroll=unroll, nt_load=nt_load, store_policy=policy + 1,
+                                max_grid=max_grid)
+                for so, do in ((0, 0), (4, 8), (1, 0), (6, 3)):
+                    run_copy_case(capi, blit, oracle, src, src_host, dst, 64 + so, GUARD + do, n)
+                    p = blit.last_plan()
+                    assert (p.wg_size, p.unroll, p.nt_load, p.store_policy) == (wg, unroll, nt_load - 1, policy)
+                    if max_grid:
+                        assert p.grid == max_grid
+
+
+@pytest.mark.parametrize("unroll", [1, 2, 4])
+def test_every_fill_variant_is_exact(capi, fresh_tuning, oracle, arenas, unroll):
+    blit = fresh_tuning
+    _, _, dst = arenas
+    for wg in (64, 256, 1024):
+        for policy in range(4):
+            for max_grid in (0, 5):
+                blit.set_tuning(wg_size=wg, unroll=unroll, store_policy=policy + 1, max_grid=max_grid)
+                for off in (0, 4):
+                    run_fill_case(capi, blit, oracle, dst, GUARD + off, (2 * MIB + 1236) // 4, FILL_VALUE)
+
+
+# ---------------------------------------------------------------------- batched
+
+def _make_batch(capi, rng, src, dst, n, min_len=64, max_len=256 << 10):
+    """Copies carved sequentially: stride = len rounded up to 256 + 256 guard."""
+    lens = np.floor(min_len * 2.0 ** (np.log2(max_len / min_len) * rng.random(n))).astype(np.int64)
+    so = rng.integers(0, 16, n)
+    do = rng.integers(0, 16, n)
+    stride = ((lens + 255) // 256) * 256 + 256
+    offs = np.concatenate([[0], np.cumsum(stride)[:-1]]) + 256
+    total = int(offs[-1] + stride[-1] + 256)
+    assert total <= src.nbytes and total <= dst.nbytes, total
+    descs = (capi.Desc * n)()
+    for i in range(n):
+        descs[i].dst = dst.base + int(offs[i] + do[i])
+        descs[i].src = src.base + int(offs[i] + so[i])
+        descs[i].bytes = int(lens[i])
+    return descs, lens, offs, so, do, total
+
+
+def _expect_batch(oracle, src_host, total, lens, offs, so, do):
+    want = np.full(total, GUARD_BYTE, dtype=np.uint8)
+    for i in range(len(lens)):
+        oracle.oracle_copy(want.ctypes.data + int(offs[i] + do[i]),
+                           src_host.ctypes.data + int(offs[i] + so[i]), int(lens[i]))
+    return want
+
+
+@pytest.mark.parametrize("n", [1, 2, 63, 1000])
+def test_batch_small(capi, blit, oracle, arenas, n):
+    src, src_host, dst = arenas
+    rng = np.random.default_rng(n)
+    descs, lens, offs, so, do, total = _make_batch(capi, rng, src, dst, n)
+    dst.fill(0, total, GUARD_BYTE)
+    check_ok(capi, blit.copy_batch(descs, n), "copy_batch")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert np.array_equal(dst.host(0, total), _expect_batch(oracle, src_host, total, lens, offs, so, do))
+    assert blit.last_plan().kernel == capi.KERNEL_COPY_BATCH
+
+
+def test_batch_edge_lengths(capi, blit, oracle, arenas):
+    """Zero-length entries, lengths 1..48 and lengths around the 4 KiB chunk."""
+    src, src_host, dst = arenas
+    lens = [0, 0] + list(range(1, 49)) + [0] + [4095, 4096, 4097, 4096 + 15, 8192, 8193, 12288 + 31, 0]
+    n = len(lens)
+    rng = np.random.default_rng(99)
+    so = rng.integers(0, 16, n)
+    do = rng.integers(0, 16, n)
+    lens = np.array(lens, dtype=np.int64)
+    stride = ((lens + 255) // 256) * 256 + 256
+    offs = np.concatenate([[0], np.cumsum(stride)[:-1]]) + 256
+    total = int(offs[-1] + stride[-1] + 256)
+    descs = (capi.Desc * n)()
+    for i in range(n):
+        descs[i].dst = dst.base + int(offs[i] + do[i])
+        descs[i].src = src.base + int(offs[i] + so[i])
+        descs[i].bytes = int(lens[i])
+    dst.fill(0, total, GUARD_BYTE)
+    check_ok(capi, blit.copy_batch(descs, n), "copy_batch")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert np.array_equal(dst.host(0, total), _expect_batch(oracle, src_host, total, lens, offs, so, do))
+
+
+def test_batch_device_resident_descriptors(capi, blit, oracle, arenas, torch_cuda):
+    torch = torch_cuda
+    src, src_host, dst = arenas
+    n = 777
+    rng = np.random.default_rng(4242)
+    descs, lens, offs, so, do, total = _make_batch(capi, rng, src, dst, n)
+    raw = np.frombuffer(bytes(descs), dtype=np.uint8).copy()
+    descs_dev = torch.from_numpy(raw).to("cuda:0")
+    dst.fill(0, total, GUARD_BYTE)
+    torch.cuda.synchronize()
+    check_ok(capi, blit.copy_batch(descs_dev.data_ptr(), n, on_device=True), "copy_batch")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert np.array_equal(dst.host(0, total), _expect_batch(oracle, src_host, total, lens, offs, so, do))
+
+
+def test_batch_65536_copies(capi, blit, oracle, rand, torch_cuda):
+    """The benchmark's batch: 65,536 copies, 64 B .. 256 KiB log-uniform, offsets
+    0..15 on both sides, carved sequentially out of one arena; all bytes and
+    all guards against the oracle."""
+    torch = torch_cuda
+    n = 65536
+    rng = np.random.default_rng(0xB1170005)
+    lens = np.floor(64 * 2.0 ** (12 * rng.random(n))).astype(np.int64)
+    stride = ((lens + 255) // 256) * 256 + 256
+    total = int(stride.sum() + 512)
+    src_host = rand(total, 0xB1170005)
+    src = Arena(torch, total, host=src_host)
+    dst = Arena(torch, total, fill=GUARD_BYTE)
+    rng = np.random.default_rng(0xB1170005)
+    descs, lens, offs, so, do, total2 = _make_batch(capi, rng, src, dst, n)
+    assert total2 <= total
+    check_ok(capi, blit.copy_batch(descs, n), "copy_batch")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    got = dst.host()
+    want = np.full(total, GUARD_BYTE, dtype=np.uint8)
+    want[:total2] = _expect_batch(oracle, src_host, total2, lens, offs, so, do)
+    assert np.array_equal(got, want)
+
+
+def test_batch_back_to_back_reuses_staging(capi, blit, oracle, arenas):
+    """Two host-descriptor batches in a row share the staging buffers."""
+    src, src_host, dst = arenas
+    rng = np.random.default_rng(31337)
+    d1, l1, o1, s1, e1, t1 = _make_batch(capi, rng, src, dst, 300)
+    dst.fill(0, t1, GUARD_BYTE)
+    check_ok(capi, blit.copy_batch(d1, 300), "copy_batch")
+    # second batch: same regions shifted by a fixed distance past the first
+    shift = ((t1 + 255) // 256) * 256
+    d2 = (capi.Desc * 200)()
+    for i in range(200):
+        d2[i].dst = d1[i].dst + shift
+        d2[i].src = d1[i].src
+        d2[i].bytes = d1[i].bytes
+    dst.fill(shift, shift + t1, GUARD_BYTE)
+    check_ok(capi, blit.copy_batch(d2, 200), "copy_batch")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert np.array_equal(dst.host(0, t1), _expect_batch(oracle, src_host, t1, l1, o1, s1, e1))
+    want2 = np.full(t1, GUARD_BYTE, dtype=np.uint8)
+    for i in range(200):
+        oracle.oracle_copy(want2.ctypes.data + int(o1[i] + e1[i]), src_host.ctypes.data + int(o1[i] + s1[i]), int(l1[i]))
+    assert np.array_equal(dst.host(shift, shift + t1), want2)
+
+
+# ---------------------------------------------------------- API edge behaviour
+
+def test_argument_validation(capi, blit, arenas):
+    """Same answers as hsa_memory_copy / hsa_amd_memory_fill give at the API
+    edge (hsa.cpp:1170-1184, hsa_ext_amd.cpp:237-251)."""
+    src, _, dst = arenas
+    inv = capi.ERROR_INVALID_ARGUMENT
+    assert blit.copy(None, src.base, 16) == inv
+    assert blit.copy(dst.base, None, 16) == inv
+    assert blit.fill32(None, 1, 4) == inv
+    for off in (1, 2, 3):
+        assert blit.fill32(dst.base + off, 1, 4) == inv
+    # zero size succeeds without touching memory
+    dst.fill(0, 64, GUARD_BYTE)
+    assert blit.copy(dst.base, src.base, 0) == capi.SUCCESS
+    assert blit.fill32(dst.base, 1, 0) == capi.SUCCESS
+    assert blit.copy_batch(None, 0) == capi.SUCCESS
+    assert blit.lib.mi355_blit_copy_batch(blit.handle, None, 3, 0, None) == inv
+    bad = (capi.Desc * 1)()
+    bad[0].dst, bad[0].src, bad[0].bytes = None, src.base, 8
+    assert blit.copy_batch(bad, 1) == inv
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert bool((dst.view[:64] == GUARD_BYTE).all())
+
+
+def test_pending_bytes_zero_is_exact(capi, blit, arenas):
+    src, _, dst = arenas
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert blit.pending_bytes() == 0
+    n = 32 * MIB
+    for _ in range(100):  # more commands than ledger slots: back-pressure path
+        check_ok(capi, blit.copy(dst.base, src.base, n), "copy")
+    pending = blit.pending_bytes()
+    assert pending % n == 0 and pending <= 100 * n
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert blit.pending_bytes() == 0
+
+
+def test_external_stream_and_ordering(capi, blit, oracle, arenas, torch_cuda):
+    """Commands on a caller's stream run in order with that stream's other work."""
+    torch = torch_cuda
+    src, src_host, dst = arenas
+    s = torch.cuda.Stream()
+    n = 5 * MIB + 3
+    with torch.cuda.stream(s):
+        dst.view[:n + 2 * GUARD].fill_(GUARD_BYTE)
+        check_ok(capi, blit.fill32(dst.base + GUARD, 0x01020304, n // 4, s.cuda_stream), "fill32")
+        check_ok(capi, blit.copy(dst.base + GUARD + 1, src.base + 2, n - 2, s.cuda_stream), "copy")
+    s.synchronize()
+    want = np.full(n + 2 * GUARD, GUARD_BYTE, dtype=np.uint8)
+    oracle.oracle_fill32(want.ctypes.data + GUARD, 0x01020304, n // 4)
+    oracle.oracle_copy(want.ctypes.data + GUARD + 1, src_host.ctypes.data + 2, n - 2)
+    assert np.array_equal(dst.host(0, n + 2 * GUARD), want)
+
+
+def test_concurrent_submitters(capi, blit, oracle, arenas):
+    """Several host threads submit to one handle, as several callers of
+    hsa_memory_copy would (the reference serialises them on a mutex)."""
+    src, src_host, dst = arenas
+    n = MIB + 17
+    nthreads, per = 4, 8
+    region = ((n + 2 * GUARD + 255) // 256) * 256
+    dst.fill(0, nthreads * per * region, GUARD_BYTE)
+    errs = []
+
+    def worker(t):
+        for j in range(per):
+            slot = t * per + j
+            st = blit.copy(dst.base + slot * region + GUARD + (slot % 16), src.base + slot * 4096 + (slot % 7), n)
+            if st != capi.SUCCESS:
+                errs.append(st)
+
+    ths = [threading.Thread(target=worker, args=(t,)) for t in range(nthreads)]
+    for t in ths:
+        t.start()
+    for t in ths:
+        t.join()
+    assert not errs
+    check_ok(capi, blit.synchronize(), "synchronize")
+    got = dst.host(0, nthreads * per * region)
+    want = np.full(got.size, GUARD_BYTE, dtype=np.uint8)
+    for slot in range(nthreads * per):
+        oracle.oracle_copy(want.ctypes.data + slot * region + GUARD + (slot % 16),
+                           src_host.ctypes.data + slot * 4096 + (slot % 7), n)
+    assert np.array_equal(got, want)
+
+
+def test_create_destroy_many(capi):
+    for _ in range(5):
+        b = capi.Blit(0)
+        assert b.num_cus > 0 and b.stream
+        b.close()
+    h = C.c_void_p()
+    assert capi.load().mi355_blit_create(10_000, C.byref(h)) == capi.ERROR_INVALID_ARGUMENT

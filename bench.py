@@ -1,0 +1,341 @@
+#!/usr/bin/env python3
+"""Benchmark of the gfx950 blit engine on one MI355X.
+
+One "step" is one pass of the hot path over one batch of synthetic input: for
+the default workload, one aligned device-to-device copy of 1 GiB of seeded
+random bytes (source and destination 256-byte aligned, resident in HBM before
+the clock starts).  The metric is algorithmic GB/s, read + written bytes
+(copy of N bytes = 2 N, fill of N bytes = N), and its fraction of the 8 TB/s
+HBM3E peak.  Prints ONE JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+Workloads: copy (default, the headline), fill, misaligned, batch, and calib (a
+plain torch copy_ of the same size: not this library, only the known-size
+kernel that scales the profiler's HBM counters).  Whatever the
+workload, the line also carries the other configurations' figures under
+"also" (measured outside the timed region), the roofline of the dominant
+kernel, and the CPU baseline (the reference's host path: memcpy / dword fill,
+timed on this box's cores on a bounded sample).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+GIB = 1 << 30
+MIB = 1 << 20
+FILL_VALUE = 0xA5C30F1E
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="copy", choices=["copy", "fill", "misaligned", "batch", "calib"])
+    ap.add_argument("--bytes", type=int, default=GIB, help="transfer size of the copy/fill workloads")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-also", action="store_true", help="skip the secondary configurations")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget")
+    return ap.parse_args()
+
+
+def aligned_ptr(t, a=256):
+    p = t.data_ptr()
+    return p + (-p) % a
+
+
+class Runner:
+    def __init__(self, torch, pkg, ora):
+        self.torch = torch
+        self.capi = pkg.capi
+        self.ora = ora
+        self.blit = pkg.capi.Blit(0)
+        # a stream torch can time: events are recorded on the stream the
+        # kernels are launched on
+        self.tstream = torch.cuda.Stream()
+        self.stream = self.tstream.cuda_stream
+        assert self.stream, "need a non-null stream"
+
+    def device_bytes(self, n, seed=None):
+        import numpy as np
+        t = self.torch.empty(n + 512, dtype=self.torch.uint8, device="cuda:0")
+        if seed is not None:
+            # seeded on the host by the shared generator, in 64 MiB pieces
+            step = 64 * MIB
+            host = np.empty(min(step, n), dtype=np.uint8)
+            off = (-t.data_ptr()) % 256
+            for lo in range(0, n, step):
+                m = min(step, n - lo)
+                self.ora.oracle_fill_random(host.ctypes.data, m, seed + lo // step)
+                t[off + lo:off + lo + m].copy_(self.torch.from_numpy(host[:m]))
+        self.torch.cuda.synchronize()
+        return t
+
+    def time_launches(self, fn, steps, warmup):
+        """W untimed + K timed back-to-back launches.  Returns (wall seconds for
+        the K steps, average device microseconds per launch from HIP events on
+        the launch stream)."""
+        torch = self.torch
+        for _ in range(warmup):
+            fn()
+        self.tstream.synchronize()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record(self.tstream)
+        for _ in range(steps):
+            fn()
+        e1.record(self.tstream)
+        self.tstream.synchronize()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        return t1 - t0, e0.elapsed_time(e1) * 1e3 / steps
+
+    def check(self, st, what):
+        self.capi.check(st, what)
+
+
+def make_copy(r, nbytes, s_off=0, d_off=0):
+    src = r.device_bytes(nbytes + 64, seed=0xB1170003)
+    dst = r.device_bytes(nbytes + 64)
+    S, D = aligned_ptr(src) + s_off, aligned_ptr(dst) + d_off
+    fn = lambda: r.check(r.blit.copy(D, S, nbytes, r.stream), "copy")
+
+    def verify():
+        # device compare of the whole range, oracle compare of a 64 MiB sample
+        import numpy as np
+        so = (-src.data_ptr()) % 256 + s_off
+        do = (-dst.data_ptr()) % 256 + d_off
+        assert r.torch.equal(dst[do:do + nbytes], src[so:so + nbytes]), "copy result differs"
+        m = min(nbytes, 64 * MIB)
+        hs = src[so:so + m].cpu().numpy()
+        want = np.empty(m, dtype=np.uint8)
+        r.ora.oracle_copy(want.ctypes.data, hs.ctypes.data, m)
+        assert np.array_equal(dst[do:do + m].cpu().numpy(), want), "copy differs from oracle"
+    return fn, verify, 2 * nbytes, (src, dst)
+
+
+def make_calib(r, nbytes):
+    """torch's own elementwise copy kernel: nbytes read + nbytes written."""
+    src = r.device_bytes(nbytes + 64, seed=0xB1170003)
+    dst = r.device_bytes(nbytes + 64)
+    a, b = src[:nbytes], dst[:nbytes]
+
+    def fn():
+        with r.torch.cuda.stream(r.tstream):
+            b.copy_(a)
+    return fn, (lambda: None), 2 * nbytes, (src, dst)
+
+
+def make_fill(r, nbytes):
+    dst = r.device_bytes(nbytes + 64)
+    D = aligned_ptr(dst)
+    fn = lambda: r.check(r.blit.fill32(D, FILL_VALUE, nbytes // 4, r.stream), "fill32")
+
+    def verify():
+        do = (-dst.data_ptr()) % 256
+        body = dst[do:do + nbytes].view(r.torch.int32)
+        want = FILL_VALUE - (1 << 32)
+        assert int(body.min()) == want and int(body.max()) == want, "fill result differs"
+    return fn, verify, nbytes, (dst,)
+
+
+def make_batch(r, n=65536, arena=8 * GIB):
+    """65,536 copies, 64 B .. 256 KiB log-uniform, byte offsets 0..15 on both
+    sides, non-overlapping regions spread over an `arena`-byte source and an
+    `arena`-byte destination (16 GiB in all)."""
+    import numpy as np
+    rng = np.random.default_rng(0xB1170005)
+    lens = np.floor(64 * 2.0 ** (12 * rng.random(n))).astype(np.int64)
+    so = rng.integers(0, 16, n)
+    do = rng.integers(0, 16, n)
+    need = ((lens + 255) // 256) * 256 + 256
+    scale = (arena - 4096) / float(need.sum())
+    stride = (np.floor(need * scale).astype(np.int64) // 256) * 256
+    offs = np.concatenate([[0], np.cumsum(stride)[:-1]]) + 256
+    src = r.torch.empty(arena + 512, dtype=r.torch.uint8, device="cuda:0")
+    dst = r.torch.empty(arena + 512, dtype=r.torch.uint8, device="cuda:0")
+    # seeded 64 MiB block repeated: cheap to make, every region still has varied bytes
+    blk = np.empty(64 * MIB, dtype=np.uint8)
+    r.ora.oracle_fill_random(blk.ctypes.data, blk.size, 0xB1170005)
+    blk_d = r.torch.from_numpy(blk).to("cuda:0")
+    for lo in range(0, arena, blk.size):
+        src[lo:lo + blk.size].copy_(blk_d[:min(blk.size, arena - lo)])
+    dst.zero_()
+    r.torch.cuda.synchronize()
+    S, D = aligned_ptr(src), aligned_ptr(dst)
+    descs = (r.capi.Desc * n)()
+    for i in range(n):
+        descs[i].dst = D + int(offs[i] + do[i])
+        descs[i].src = S + int(offs[i] + so[i])
+        descs[i].bytes = int(lens[i])
+    fn = lambda: r.check(r.blit.copy_batch(descs, n, False, r.stream), "copy_batch")
+
+    def verify():
+        sh = (-src.data_ptr()) % 256
+        dh = (-dst.data_ptr()) % 256
+        for i in list(range(0, n, 997)) + [n - 1]:
+            a = dst[dh + int(offs[i] + do[i]):dh + int(offs[i] + do[i] + lens[i])]
+            b = src[sh + int(offs[i] + so[i]):sh + int(offs[i] + so[i] + lens[i])]
+            assert r.torch.equal(a, b), "batched copy %d differs" % i
+    return fn, verify, int(2 * lens.sum()), (src, dst, descs)
+
+
+def small_copy_latency(r, sizes=(4096, 65536, MIB)):
+    """Host-observed microseconds per blocking copy (submit -> completion seen),
+    the way rocrtst times hsa_amd_memory_async_copy (memory_async_copy.cc:396-405)."""
+    out = {}
+    src = r.device_bytes(max(sizes) + 64, seed=0xB1170003)
+    dst = r.device_bytes(max(sizes) + 64)
+    S, D = aligned_ptr(src), aligned_ptr(dst)
+    for n in sizes:
+        for _ in range(20):
+            r.check(r.blit.copy(D, S, n), "copy")
+            r.check(r.blit.synchronize(), "synchronize")
+        ts = []
+        for _ in range(200):
+            t0 = time.perf_counter()
+            r.check(r.blit.copy(D, S, n), "copy")
+            r.check(r.blit.synchronize(), "synchronize")
+            ts.append(time.perf_counter() - t0)
+        ts.sort()
+        out[str(n)] = round(ts[len(ts) // 2] * 1e6, 2)
+    return out
+
+
+def cpu_baseline(ora, budget_s):
+    """The reference's host path on this box's cores: memcpy of 256 MiB
+    (BASELINE config 1; what hsa_memory_copy does for host pointers), single
+    thread and T threads, on a bounded number of repetitions."""
+    import numpy as np
+    n = 256 * MIB
+    T = min(16, os.cpu_count() or 1)
+    src = np.empty(n, dtype=np.uint8)
+    dst = np.empty(n, dtype=np.uint8)
+    ora.oracle_fill_random(src.ctypes.data, 16 * MIB, 0xB1170001)
+    for lo in range(16 * MIB, n, 16 * MIB):
+        src[lo:lo + 16 * MIB] = src[:16 * MIB]
+    dst[:] = 0  # pages touched
+
+    def best_of(fn, seconds):
+        best, reps, t_end = 1e9, 0, time.perf_counter() + seconds
+        while reps < 3 or (time.perf_counter() < t_end and reps < 200):
+            t0 = time.perf_counter()
+            fn()
+            best = min(best, time.perf_counter() - t0)
+            reps += 1
+        return best, reps
+
+    b1, r1 = best_of(lambda: ora.oracle_copy(dst.ctypes.data, src.ctypes.data, n), budget_s * 0.35)
+    assert np.array_equal(dst[:MIB], src[:MIB]) and np.array_equal(dst[-MIB:], src[-MIB:])
+    bt, rt = best_of(lambda: ora.oracle_copy_mt(dst.ctypes.data, src.ctypes.data, n, T), budget_s * 0.35)
+    bf, rf = best_of(lambda: ora.oracle_fill32_mt(dst.ctypes.data, FILL_VALUE, n // 4, T), budget_s * 0.3)
+    assert int(dst.view("<u4")[12345]) == FILL_VALUE
+    return {
+        "value": round(2 * n / bt / 1e9, 2), "unit": "GB/s", "cores": T, "kind": "port",
+        "sample": "host memcpy of 256 MiB seeded bytes (oracle_copy_mt, %d threads, best of %d); "
+                  "read+write bytes" % (T, rt),
+        "copy_1thread_gbs": round(2 * n / b1 / 1e9, 2),
+        "fill_gbs": round(n / bf / 1e9, 2),
+        "reps": {"copy_1thread": r1, "copy_mt": rt, "fill_mt": rf},
+    }
+
+
+def load_traffic(kernel_key):
+    """HBM bytes per launch from committed rocprofv3 --pmc runs (FETCH_SIZE +
+    WRITE_SIZE, scaled by a plain copy kernel of known size), if recorded."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        return json.load(f).get(kernel_key, {}).get("bytes_per_launch")
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus)
+    import torch
+    import __graft_entry__ as entry
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    pkg = entry.load_package()
+    ora = entry.load_oracle()
+    r = Runner(torch, pkg, ora)
+    nbytes = args.bytes
+
+    if args.workload == "copy":
+        fn, verify, algo, keep = make_copy(r, nbytes)
+        name = "aligned D2D copy, %d MiB seeded random bytes, src/dst 256-byte aligned" % (nbytes // MIB)
+        traffic_key = "copy_1GiB" if nbytes == GIB else None
+    elif args.workload == "fill":
+        fn, verify, algo, keep = make_fill(r, nbytes)
+        name = "dword fill 0x%08X, %d MiB, 256-byte aligned" % (FILL_VALUE, nbytes // MIB)
+        traffic_key = "fill_1GiB" if nbytes == GIB else None
+    elif args.workload == "misaligned":
+        fn, verify, algo, keep = make_copy(r, nbytes - 64, s_off=3, d_off=9)
+        name = "misaligned D2D copy, %d MiB - 64 B, src&15=3 dst&15=9" % (nbytes // MIB)
+        traffic_key = "misaligned_1GiB" if nbytes == GIB else None
+    elif args.workload == "calib":
+        fn, verify, algo, keep = make_calib(r, nbytes)
+        name = "calibration: torch copy_ of %d MiB (not this library)" % (nbytes // MIB)
+        traffic_key = None
+    else:
+        fn, verify, algo, keep = make_batch(r)
+        name = "65536 batched D2D copies, 64 B..256 KiB log-uniform, offsets 0..15, 16 GiB arena"
+        traffic_key = "batch_65536"
+
+    wall, dev_us = r.time_launches(fn, args.steps, args.warmup)
+    verify()
+    plan = r.blit.last_plan().as_dict()
+    value = algo * args.steps / wall / 1e9
+    achieved = algo / dev_us / 1e3
+
+    also = {}
+    if not args.no_also:
+        del keep
+        torch.cuda.empty_cache()
+        for key, maker in (("copy_1GiB", lambda: make_copy(r, GIB)),
+                           ("fill_1GiB", lambda: make_fill(r, GIB)),
+                           ("misaligned_1GiB", lambda: make_copy(r, GIB - 64, s_off=3, d_off=9)),
+                           ("batch_65536", lambda: make_batch(r))):
+            f2, v2, a2, k2 = maker()
+            w2, us2 = r.time_launches(f2, 20, 3)
+            v2()
+            also[key] = {"gbs": round(a2 / us2 / 1e3, 1), "frac_of_peak": round(a2 / us2 / 1e3 / HBM_PEAK_GBS, 4),
+                         "us_per_launch": round(us2, 2)}
+            del f2, v2, k2
+            torch.cuda.empty_cache()
+        also["small_copy_us"] = small_copy_latency(r)
+
+    line = {
+        "metric": "D2D copy & fill GB/s (R+W) at 1 GiB on 1 MI355X",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall / args.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": name, "bytes_per_step": algo, "plan": plan,
+                   "device": torch.cuda.get_device_name(0), "cus": r.blit.num_cus},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": load_traffic(traffic_key) if traffic_key else None,
+                     "kernel_us": round(dev_us, 2), "algorithmic_bytes_per_launch": algo},
+        "also": also,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(ora, args.cpu_seconds)
+    r.blit.close()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

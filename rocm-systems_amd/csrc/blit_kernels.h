@@ -245,31 +245,85 @@ __device__ __forceinline__ unsigned desc_chunks(const BatchDesc& d) {
   return c ? static_cast<unsigned>(c) : 1u;
 }
 
-// chunk_start[i] = chunks of copies 0..i-1, chunk_start[n] = all chunks.
-// One workgroup of 1024 lanes; lane t owns a contiguous run of descriptors.
-__global__ void __launch_bounds__(1024) k_batch_scan(const BatchDesc* __restrict__ descs, uint64_t n,
-                                                     uint32_t* __restrict__ chunk_start) {
-  __shared__ uint32_t part[1024];
-  const unsigned t = threadIdx.x;
-  const uint64_t per = (n + 1023) / 1024;
-  const uint64_t lo = t * per < n ? t * per : n;
-  const uint64_t hi = lo + per < n ? lo + per : n;
-  uint32_t sum = 0;
-  for (uint64_t i = lo; i < hi; ++i) sum += desc_chunks(descs[i]);
-  part[t] = sum;
+// Exclusive prefix sum over the 1024 lanes of a workgroup; *total gets the sum.
+// lds holds 16 words.
+__device__ __forceinline__ uint32_t block_scan_1024(uint32_t v, uint32_t* lds, uint32_t* total) {
+  const unsigned lane = threadIdx.x & (kWave - 1);
+  const unsigned w = threadIdx.x / kWave;
+  uint32_t incl = v;
+#pragma unroll
+  for (unsigned off = 1; off < kWave; off <<= 1) {
+    const uint32_t x = __shfl_up(incl, off, kWave);
+    if (lane >= off) incl += x;
+  }
+  if (lane == kWave - 1) lds[w] = incl;
   __syncthreads();
-  for (unsigned off = 1; off < 1024; off <<= 1) {
-    const uint32_t add = t >= off ? part[t - off] : 0;
-    __syncthreads();
-    part[t] += add;
-    __syncthreads();
+  if (w == 0) {
+    uint32_t s = lane < 16 ? lds[lane] : 0;
+#pragma unroll
+    for (unsigned off = 1; off < 16; off <<= 1) {
+      const uint32_t x = __shfl_up(s, off, kWave);
+      if (lane >= off) s += x;
+    }
+    if (lane < 16) lds[lane] = s;
   }
-  uint32_t run = part[t] - sum;  // exclusive prefix of this lane's run
-  for (uint64_t i = lo; i < hi; ++i) {
-    chunk_start[i] = run;
-    run += desc_chunks(descs[i]);
+  __syncthreads();
+  *total = lds[15];
+  return (w ? lds[w - 1] : 0) + incl - v;
+}
+
+// Prefix sum of the chunk counts in three small launches (no workgroup ever
+// waits for another):
+//  1. k_batch_scan_local, one workgroup per 1024 copies: chunk_start[i] =
+//     chunks of the copies before i in the same workgroup, block_sum[b] = all
+//     chunks of workgroup b;
+//  2. k_batch_scan_top, one workgroup: block_sum becomes its own exclusive
+//     prefix, chunk_start[n] = all chunks;
+//  3. k_batch_expand, one lane per copy: chunk_start[i] += block_sum[i / 1024]
+//     and, when owner != nullptr, owner[c] = i for every chunk c of copy i.
+__global__ void __launch_bounds__(1024) k_batch_scan_local(const BatchDesc* __restrict__ descs,
+                                                           uint64_t n,
+                                                           uint32_t* __restrict__ chunk_start,
+                                                           uint32_t* __restrict__ block_sum) {
+  __shared__ uint32_t lds[16];
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 1024 + threadIdx.x;
+  const uint32_t c = i < n ? desc_chunks(descs[i]) : 0;
+  uint32_t total;
+  const uint32_t excl = block_scan_1024(c, lds, &total);
+  if (i < n) chunk_start[i] = excl;
+  if (threadIdx.x == 0) block_sum[blockIdx.x] = total;
+}
+
+__global__ void __launch_bounds__(1024) k_batch_scan_top(uint32_t* __restrict__ block_sum,
+                                                         uint32_t n_blocks,
+                                                         uint32_t* __restrict__ chunk_start,
+                                                         uint64_t n) {
+  __shared__ uint32_t lds[16];
+  uint32_t carry = 0;
+  for (uint32_t base = 0; base < n_blocks; base += 1024) {
+    const uint32_t j = base + threadIdx.x;
+    const uint32_t v = j < n_blocks ? block_sum[j] : 0;
+    uint32_t total;
+    const uint32_t excl = block_scan_1024(v, lds, &total);
+    if (j < n_blocks) block_sum[j] = carry + excl;
+    carry += total;
+    __syncthreads();  // lds is reused by the next round
   }
-  if (t == 1023) chunk_start[n] = part[1023];
+  if (threadIdx.x == 0) chunk_start[n] = carry;
+}
+
+__global__ void __launch_bounds__(256) k_batch_expand(const BatchDesc* __restrict__ descs, uint64_t n,
+                                                      uint32_t* __restrict__ chunk_start,
+                                                      const uint32_t* __restrict__ block_sum,
+                                                      uint32_t* __restrict__ owner) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint32_t base = chunk_start[i] + block_sum[i / 1024];
+  chunk_start[i] = base;
+  if (owner) {
+    const uint32_t cnt = desc_chunks(descs[i]);
+    for (uint32_t k = 0; k < cnt; ++k) owner[base + k] = static_cast<uint32_t>(i);
+  }
 }
 
 // One chunk of one copy, done by one wave.
@@ -306,8 +360,56 @@ __device__ __forceinline__ void copy_chunk(v4u* __restrict__ d, const v4u_a4* __
   }
 }
 
-__global__ void __launch_bounds__(256) k_batch_copy(const BatchDesc* __restrict__ descs, uint64_t n,
-                                                    const uint32_t* __restrict__ chunk_start) {
+// Chunk k of one copy, with the head bytes on the first chunk and the tail
+// bytes on the last.
+template <bool NTL, int NTS>
+__device__ __forceinline__ void copy_desc_chunk(const BatchDesc& dsc, uint64_t k, bool last,
+                                                unsigned lane) {
+  const unsigned head = desc_head(dsc);
+  const uint64_t n_vec = (dsc.bytes - head) / 16;
+  const uint8_t* sb = dsc.src + head;
+  const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(sb)) & 3;
+  v4u* d = reinterpret_cast<v4u*>(dsc.dst + head);
+  const v4u_a4* s = reinterpret_cast<const v4u_a4*>(sb - r);
+  const uint64_t v0 = k * kChunkVecs;
+  const uint64_t left = n_vec > v0 ? n_vec - v0 : 0;
+  const unsigned nv = left < kChunkVecs ? static_cast<unsigned>(left) : kChunkVecs;
+  if (r) copy_chunk<NTL, NTS, true>(d + v0, s + v0, r, nv, lane);
+  else copy_chunk<NTL, NTS, false>(d + v0, s + v0, 0, nv, lane);
+  if (k == 0 && lane < head) dsc.dst[lane] = dsc.src[lane];
+  if (last) {
+    const uint64_t tail_off = head + 16 * n_vec;
+    const unsigned tail = static_cast<unsigned>(dsc.bytes - tail_off);
+    if (lane >= 16 && lane - 16 < tail) dsc.dst[tail_off + lane - 16] = dsc.src[tail_off + lane - 16];
+  }
+}
+
+// One wave per chunk, chunks in global order (the shape that streams best for
+// a single large copy); owner[c] names the copy chunk c belongs to.  Needs the
+// chunk total on the host to size the grid.
+template <bool NTL, int NTS>
+__global__ void __launch_bounds__(1024) k_batch_copy_mapped(const BatchDesc* __restrict__ descs,
+                                                            const uint32_t* __restrict__ chunk_start,
+                                                            const uint32_t* __restrict__ owner,
+                                                            uint64_t total_chunks) {
+  const unsigned lane = threadIdx.x & (kWave - 1);
+  const unsigned waves_per_wg = blockDim.x / kWave;
+  const uint64_t c =
+      __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
+  if (c >= total_chunks) return;
+  const uint32_t i = owner[c];
+  const BatchDesc dsc = descs[i];
+  const uint64_t k = c - chunk_start[i];
+  copy_desc_chunk<NTL, NTS>(dsc, k, k + 1 == desc_chunks(dsc), lane);
+}
+
+// Device-filling grid, every wave takes an equal contiguous share of all
+// chunks and finds its first copy by bisection.  Used when the descriptors
+// are device-resident and the host cannot know the chunk total.
+template <bool NTL, int NTS>
+__global__ void __launch_bounds__(256) k_batch_copy_strided(const BatchDesc* __restrict__ descs,
+                                                            uint64_t n,
+                                                            const uint32_t* __restrict__ chunk_start) {
   const unsigned lane = threadIdx.x & (kWave - 1);
   const unsigned waves_per_wg = blockDim.x / kWave;
   const uint64_t wave =
@@ -331,28 +433,8 @@ __global__ void __launch_bounds__(256) k_batch_copy(const BatchDesc* __restrict_
     const uint64_t ce = chunk_start[i + 1];
     if (ce <= c) { ++i; continue; }
     const BatchDesc dsc = descs[i];
-    const unsigned head = desc_head(dsc);
-    const uint64_t n_vec = (dsc.bytes - head) / 16;
-    const uint8_t* sb = dsc.src + head;
-    const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(sb)) & 3;
-    v4u* d = reinterpret_cast<v4u*>(dsc.dst + head);
-    const v4u_a4* s = reinterpret_cast<const v4u_a4*>(sb - r);
     const uint64_t stop = ce < c1 ? ce : c1;
-    for (; c < stop; ++c) {
-      const uint64_t k = c - cs;
-      const uint64_t v0 = k * kChunkVecs;
-      const uint64_t left = n_vec > v0 ? n_vec - v0 : 0;
-      const unsigned nv = left < kChunkVecs ? static_cast<unsigned>(left) : kChunkVecs;
-      if (r) copy_chunk<false, kStoreCached, true>(d + v0, s + v0, r, nv, lane);
-      else copy_chunk<false, kStoreCached, false>(d + v0, s + v0, 0, nv, lane);
-      // first chunk moves the head bytes, last chunk the tail bytes
-      if (k == 0 && lane < head) dsc.dst[lane] = dsc.src[lane];
-      if (c + 1 == ce) {
-        const uint64_t tail_off = head + 16 * n_vec;
-        const unsigned tail = static_cast<unsigned>(dsc.bytes - tail_off);
-        if (lane >= 16 && lane - 16 < tail) dsc.dst[tail_off + lane - 16] = dsc.src[tail_off + lane - 16];
-      }
-    }
+    for (; c < stop; ++c) copy_desc_chunk<NTL, NTS>(dsc, c - cs, c + 1 == ce, lane);
     ++i;
   }
 }

@@ -32,13 +32,27 @@ struct SizeClass {
   uint32_t store_policy;
 };
 
-// Measured on MI355X (256 CUs): one 1 KiB tile per single-wave workgroup is
-// the fastest copy shape once the transfer streams from HBM; fills are store
-// issue bound in the dispatcher at that size and want 4-wave workgroups.
-// Transfers that cannot stay in cache bypass it.  Last match wins.
-constexpr SizeClass kCopyClasses[] = {
+// Measured on MI355X (256 CUs) at 1 GiB.  Source and destination equally
+// aligned mod 16: one 1 KiB tile per single-wave workgroup is the fastest
+// shape once the transfer streams from HBM.  A dword offset between them makes
+// every wave's 1 KiB of loads straddle a cache line shared with its
+// neighbour, and 4-wave workgroups share that line in one CU.  A byte offset
+// adds one extra dword fetch per tile (the bytes that spill past the last
+// lane), which 2 KiB tiles in 8-wave workgroups amortise best.  Fills are
+// bound by the dispatcher's workgroup rate at one wave per workgroup and want
+// 4-wave workgroups.  Transfers that cannot stay in cache bypass it: loads
+// non-temporal, stores written through.  Last match wins.
+constexpr SizeClass kCopyClasses[] = {      // (src - dst) % 16 == 0
     {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
     {8ull << 20, 64, 1, 1, MI355_BLIT_STORE_AGENT_WT},
+};
+constexpr SizeClass kCopyDwordOffsetClasses[] = {  // (src - dst) % 4 == 0
+    {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
+    {8ull << 20, 256, 1, 1, MI355_BLIT_STORE_AGENT_WT},
+};
+constexpr SizeClass kCopyRealignClasses[] = {  // (src - dst) % 4 != 0
+    {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
+    {8ull << 20, 512, 2, 1, MI355_BLIT_STORE_NT},
 };
 constexpr SizeClass kFillClasses[] = {
     {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
@@ -95,7 +109,11 @@ inline int plan_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t num_cu
   p->tail_bytes = bytes - head - 16 * p->body_vecs;
   p->byte_shift = static_cast<uint32_t>((src - dst) & 3);
   p->kernel = p->byte_shift ? MI355_BLIT_KERNEL_COPY_REALIGN : MI355_BLIT_KERNEL_COPY;
-  apply_launch_shape(p, pick_class(kCopyClasses, bytes), num_cus, t);
+  const uint64_t delta = (src - dst) & 15;
+  const SizeClass& cls = delta == 0         ? pick_class(kCopyClasses, bytes)
+                         : (delta & 3) == 0 ? pick_class(kCopyDwordOffsetClasses, bytes)
+                                            : pick_class(kCopyRealignClasses, bytes);
+  apply_launch_shape(p, cls, num_cus, t);
   return MI355_BLIT_SUCCESS;
 }
 

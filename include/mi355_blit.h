@@ -129,6 +129,21 @@ int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwo
 int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n,
                           int descs_on_device, void* stream);
 
+/* Decrements an HSA signal by 1 from the GPU once every command submitted
+ * before it on the stream has completed, and wakes its waiters: replaces the
+ * completion_signal field of the reference's dispatch packet
+ * (amd_blit_kernel.cpp:777-779, 884).  hsa_signal_handle is hsa_signal_t.handle
+ * of a signal created by hsa_signal_create / hsa_amd_signal_create (its memory
+ * is visible to every GPU); it must stay alive until it has been decremented. */
+int mi355_blit_signal_complete(mi355_blit_t* h, uint64_t hsa_signal_handle, void* stream);
+
+/* Runs fn(user) on a host thread once every command submitted before it on the
+ * stream has completed: the host-side alternative to
+ * mi355_blit_signal_complete, slower by a thread wake-up.  fn must not call
+ * back into this library. */
+typedef void (*mi355_blit_callback_t)(void* user);
+int mi355_blit_add_callback(mi355_blit_t* h, mi355_blit_callback_t fn, void* user, void* stream);
+
 /* Blocks until every command submitted on the handle's own stream is done;
  * the wait BlitKernel does on its completion signal
  * (amd_blit_kernel.cpp:632, 830). */

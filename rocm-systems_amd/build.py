@@ -62,11 +62,23 @@ def build_rocr_adapter():
     link = ["-L", LIB_DIR, "-lmi355blit", "-L", os.path.join(ROCM, "lib"), "-lhsa-runtime64",
             "-lpthread", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(ROCM, "lib")]
     _run(["g++"] + common + ["-shared", "-o", ROCR_LIB, src] + link)
-    test_src = os.path.join(ROOT, "tests", "cpp", "test_rocr_blit.cpp")
-    if os.path.exists(test_src):
-        _run(["g++"] + common + ["-o", ROCR_TEST, test_src, "-lmi355blit_rocr"] + link
-             + ["-L", os.path.join(ROCM, "lib"), "-lamdhip64"])
     return ROCR_LIB
+
+
+def build_rocr_test():
+    """Native test driver of the adapter (links the CPU oracle as its checker)."""
+    test_src = os.path.join(ROOT, "tests", "cpp", "test_rocr_blit.cpp")
+    if not (os.path.exists(test_src) and os.path.exists(ROCR_LIB)):
+        return None
+    _run(["g++", "-O2", "-std=c++17", "-Wall", "-D__HIP_PLATFORM_AMD__",
+          "-I", INCLUDE, "-I", CSRC, "-I", os.path.join(ROCM, "include"),
+          "-o", ROCR_TEST, test_src,
+          "-L", LIB_DIR, "-lmi355blit_rocr", "-lmi355blit",
+          "-L", ORACLE_DIR, "-lblit_oracle",
+          "-L", os.path.join(ROCM, "lib"), "-lhsa-runtime64", "-lamdhip64", "-lpthread",
+          "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,$ORIGIN/../../oracle",
+          "-Wl,-rpath," + os.path.join(ROCM, "lib")])
+    return ROCR_TEST
 
 
 def build_oracle():
@@ -81,6 +93,9 @@ def build_all():
     if r:
         out.append(r)
     out.append(build_oracle())
+    t = build_rocr_test()
+    if t:
+        out.append(t)
     return out
 
 

@@ -54,6 +54,8 @@ SIGNATURES = {
     "mi355_blit_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "mi355_blit_fill32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t, C.c_void_p]),
     "mi355_blit_copy_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]),
+    "mi355_blit_signal_complete": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p]),
+    "mi355_blit_add_callback": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "mi355_blit_synchronize": (C.c_int, [C.c_void_p]),
     "mi355_blit_pending_bytes": (C.c_uint64, [C.c_void_p]),
     "mi355_blit_last_launch_info": (C.c_int, [C.c_void_p, C.POINTER(Plan)]),

@@ -487,6 +487,28 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
   return ledger_record(h, s, total_bytes);
 }
 
+int mi355_blit_signal_complete(mi355_blit_t* h, uint64_t hsa_signal_handle, void* stream) {
+  if (!h || !hsa_signal_handle || (hsa_signal_handle & 63)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> g(h->lock);
+  DeviceScope scope(h->device);
+  if (scope.err != hipSuccess) return status_of(scope.err);
+  hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
+  hipLaunchKernelGGL(k_signal_complete, dim3(1), dim3(64), 0, s,
+                     reinterpret_cast<HsaSignalAbi*>(hsa_signal_handle));
+  BLIT_HIP(hipGetLastError());
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_blit_add_callback(mi355_blit_t* h, mi355_blit_callback_t fn, void* user, void* stream) {
+  if (!h || !fn) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> g(h->lock);
+  DeviceScope scope(h->device);
+  if (scope.err != hipSuccess) return status_of(scope.err);
+  hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
+  BLIT_HIP(hipLaunchHostFunc(s, fn, user));
+  return MI355_BLIT_SUCCESS;
+}
+
 int mi355_blit_synchronize(mi355_blit_t* h) {
   if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   hipStream_t s;

@@ -439,6 +439,44 @@ __global__ void __launch_bounds__(256) k_batch_copy_strided(const BatchDesc* __r
   }
 }
 
+// ---------------------------------------------------------------------------
+// Completion of an HSA signal from the device, queued behind a command.  In
+// the reference the packet processor does this with the dispatch packet's
+// completion_signal field (core/runtime/amd_blit_kernel.cpp:884); an agent
+// other than the packet processor follows the protocol ROCr's SDMA engine
+// uses (core/runtime/amd_blit_sdma.cpp:478-514): atomically decrement the
+// value and, when the signal has an event mailbox, post the event id there
+// and raise the interrupt that wakes waiters sleeping in the kernel driver.
+// ---------------------------------------------------------------------------
+
+// Layout of amd_signal_t (inc/amd_hsa_signal.h, struct amd_signal_s).
+struct HsaSignalAbi {
+  int64_t kind;
+  int64_t value;
+  uint64_t event_mailbox_ptr;
+  uint32_t event_id;
+  uint32_t reserved1;
+  uint64_t start_ts;
+  uint64_t end_ts;
+  uint64_t queue_ptr;
+  uint32_t reserved3[2];
+};
+static_assert(sizeof(HsaSignalAbi) == 64, "amd_signal_t is 64 bytes");
+
+__global__ void __launch_bounds__(64) k_signal_complete(HsaSignalAbi* sig) {
+  if (threadIdx.x != 0) return;
+  __hip_atomic_fetch_sub(&sig->value, static_cast<int64_t>(1), __ATOMIC_RELEASE,
+                         __HIP_MEMORY_SCOPE_SYSTEM);
+  uint64_t* mailbox = reinterpret_cast<uint64_t*>(sig->event_mailbox_ptr);
+  if (mailbox) {
+    const uint32_t id = sig->event_id;
+    __hip_atomic_store(mailbox, static_cast<uint64_t>(id), __ATOMIC_RELEASE,
+                       __HIP_MEMORY_SCOPE_SYSTEM);
+    // MSG_INTERRUPT with the event id's low byte in m0
+    __builtin_amdgcn_s_sendmsg(1, __builtin_amdgcn_readfirstlane(id) & 0xff);
+  }
+}
+
 }  // namespace mi355
 
 #endif  // MI355_BLIT_KERNELS_H_

@@ -1,0 +1,185 @@
+// The gfx950 blit engine behind ROCr's blit interface.
+//
+// rocr::core::Blit below repeats, member for member, the abstract interface of
+// projects/rocr-runtime/runtime/hsa-runtime/core/inc/blit.h:52-122, and
+// rocr::AMD::BlitKernelGfx950 is shaped like AMD::BlitKernel
+// (core/inc/amd_blit_kernel.h:56-118): constructed over a queue, Initialize()d
+// with the agent, owned by GpuAgent through lazy_ptr<core::Blit>
+// (core/runtime/amd_gpu_agent.cpp:749-759, 858-863).
+//
+// ROCr's internal headers are not installed with ROCm, so the three internal
+// types the interface mentions are given minimal stand-ins here: core::Agent
+// (only the GPU ordinal and the profiling flag are needed), core::Queue (an
+// opaque pointer, unused: commands go through a HIP stream inside the C ABI)
+// and core::Signal, a thin view of an hsa_signal_t driven through the public
+// hsa_signal_* API.  Inside a ROCr tree the stand-ins are replaced by the real
+// classes; core::Signal::Convert() yields the same hsa_signal_t handle there.
+#ifndef MI355_ROCR_BLIT_H_
+#define MI355_ROCR_BLIT_H_
+
+#include <hsa/hsa.h>
+#include <stdint.h>
+
+#include <atomic>
+#include <condition_variable>
+#include <deque>
+#include <mutex>
+#include <thread>
+#include <vector>
+
+struct mi355_blit;
+
+namespace rocr {
+namespace core {
+
+class Agent {
+ public:
+  explicit Agent(int gpu_ordinal, bool profiling = false)
+      : gpu_ordinal_(gpu_ordinal), profiling_enabled_(profiling) {}
+  virtual ~Agent() {}
+  int gpu_ordinal() const { return gpu_ordinal_; }
+  bool profiling_enabled() const { return profiling_enabled_; }
+
+ private:
+  int gpu_ordinal_;
+  bool profiling_enabled_;
+};
+
+class Queue;  // opaque
+
+class Signal {
+ public:
+  explicit Signal(hsa_signal_t handle) : handle_(handle) {}
+  static hsa_signal_t Convert(const Signal* s) { return s->handle_; }
+  hsa_signal_t handle() const { return handle_; }
+  hsa_signal_value_t LoadRelaxed() const { return hsa_signal_load_relaxed(handle_); }
+  void StoreRelaxed(hsa_signal_value_t v) { hsa_signal_store_relaxed(handle_, v); }
+  void SubRelease(hsa_signal_value_t v) { hsa_signal_subtract_screlease(handle_, v); }
+
+ private:
+  hsa_signal_t handle_;
+};
+
+// core/inc/blit.h:52-122
+class Blit {
+ public:
+  explicit Blit() {}
+  virtual ~Blit() {}
+
+  /// Blocks until all commands have executed, then releases the engine.
+  virtual hsa_status_t Destroy(const core::Agent& agent) = 0;
+
+  /// Blocking linear copy.
+  virtual hsa_status_t SubmitLinearCopyCommand(void* dst, const void* src, size_t size) = 0;
+
+  /// Non-blocking linear copy: starts after every dependent signal is 0,
+  /// decrements out_signal once when done.
+  virtual hsa_status_t SubmitLinearCopyCommand(void* dst, const void* src, size_t size,
+                                               std::vector<core::Signal*>& dep_signals,
+                                               core::Signal& out_signal,
+                                               std::vector<core::Signal*>& gang_signals) = 0;
+
+  /// Blocking fill of num uint32_t with value.
+  virtual hsa_status_t SubmitLinearFillCommand(void* ptr, uint32_t value, size_t num) = 0;
+
+  virtual hsa_status_t EnableProfiling(bool enable) = 0;
+
+  virtual bool isSDMA() const { return false; }
+
+  /// Approximate bytes still to copy or fill; a return of zero is exact.
+  virtual uint64_t PendingBytes() = 0;
+
+  virtual void GangLeader(bool gang_leader) = 0;
+  virtual bool GangLeader() const { return false; }
+};
+
+}  // namespace core
+
+namespace AMD {
+
+class BlitKernelGfx950 : public core::Blit {
+ public:
+  /// How out_signal is decremented when a command has finished.
+  enum class Completion {
+    kDeviceSignal,  ///< by a one-wave kernel queued behind the command
+    kHostCallback,  ///< by hsa_signal_subtract_screlease from a host callback
+  };
+
+  explicit BlitKernelGfx950(core::Queue* queue, Completion completion = Completion::kDeviceSignal);
+  ~BlitKernelGfx950() override;
+
+  /// Binds to the agent's GPU, loads the kernels, creates the completion
+  /// signal used by the blocking calls (amd_blit_kernel.cpp:553-591).
+  hsa_status_t Initialize(const core::Agent& agent);
+
+  hsa_status_t Destroy(const core::Agent& agent) override;
+
+  hsa_status_t SubmitLinearCopyCommand(void* dst, const void* src, size_t size) override;
+
+  hsa_status_t SubmitLinearCopyCommand(void* dst, const void* src, size_t size,
+                                       std::vector<core::Signal*>& dep_signals,
+                                       core::Signal& out_signal,
+                                       std::vector<core::Signal*>& gang_signals) override;
+
+  hsa_status_t SubmitLinearFillCommand(void* ptr, uint32_t value, size_t count) override;
+
+  /// Batched small copies: n independent copies in one submission, out_signal
+  /// decremented once when all are done.  No counterpart in core::Blit.
+  hsa_status_t SubmitBatchCopyCommand(const void* descs, size_t n, bool descs_on_device,
+                                      std::vector<core::Signal*>& dep_signals,
+                                      core::Signal& out_signal);
+
+  hsa_status_t EnableProfiling(bool enable) override;
+
+  uint64_t PendingBytes() override;
+
+  void GangLeader(bool) override {}
+  bool GangLeader() const override { return false; }
+
+  /// The C ABI handle underneath (for the test driver).
+  mi355_blit* c_handle() const { return blit_; }
+
+ private:
+  enum class Op { Copy, Fill, Batch };
+  struct Command {
+    Op op;
+    void* dst;
+    const void* src;
+    size_t size;     // bytes, dwords (Fill) or descriptors (Batch)
+    uint32_t value;  // Fill pattern / Batch: descriptors are device-resident
+    std::vector<hsa_signal_t> deps;
+    hsa_signal_t out;
+  };
+
+  static bool DepsSatisfied(const std::vector<hsa_signal_t>& deps);
+  hsa_status_t Launch(const Command& cmd);
+  hsa_status_t Submit(Command&& cmd);
+  void WorkerLoop();
+  void DrainWorker();
+  static void OnComplete(void* user);
+
+  core::Queue* queue_;
+  mi355_blit* blit_;
+  Completion completion_;
+
+  /// Completion signal of the blocking calls; guarded by lock_.
+  hsa_signal_t completion_signal_;
+  std::mutex lock_;
+
+  /// Commands whose dependencies were not yet satisfied at submission, and
+  /// everything submitted behind them: executed in order by worker_.
+  std::mutex queue_lock_;
+  std::condition_variable queue_cv_;
+  std::deque<Command> waiting_;
+  bool worker_busy_;
+  bool stopping_;
+  std::thread worker_;
+  uint64_t waiting_bytes_;
+
+  std::atomic<bool> profiling_;
+};
+
+}  // namespace AMD
+}  // namespace rocr
+
+#endif  // MI355_ROCR_BLIT_H_

@@ -1,0 +1,423 @@
+// Native test driver for rocr::AMD::BlitKernelGfx950 (the core::Blit adapter).
+// Runs on a GPU box; prints one "PASS <name>" or "FAIL <name>: why" line per
+// case and exits non-zero if any case fails.  Expected bytes come from the CPU
+// oracle (oracle/blit_oracle.h); the cases follow what the reference's own
+// tests do with this interface through the HSA API: fill, copy, wait on the
+// completion signal, compare every element
+// (rocrtst/samples/async_mem_copy/async_mem_copy.cc:269-357).
+#include <hip/hip_runtime_api.h>
+#include <hsa/hsa.h>
+
+#include <algorithm>
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "../../oracle/blit_oracle.h"
+#include "mi355_blit.h"
+#include "rocr_blit.h"
+
+using rocr::AMD::BlitKernelGfx950;
+using rocr::core::Signal;
+
+namespace {
+
+int g_failures = 0;
+constexpr size_t kGuard = 256;
+constexpr uint8_t kGuardByte = 0xEE;
+
+#define REQUIRE(cond, ...)                         \
+  do {                                             \
+    if (!(cond)) {                                 \
+      std::printf("FAIL %s: ", name);              \
+      std::printf(__VA_ARGS__);                    \
+      std::printf(" (line %d)\n", __LINE__);       \
+      std::fflush(stdout);                         \
+      ++g_failures;                                \
+      return;                                      \
+    }                                              \
+  } while (0)
+
+#define HIP_OK(expr) REQUIRE((expr) == hipSuccess, "%s failed", #expr)
+
+struct DeviceBuf {
+  uint8_t* p = nullptr;
+  size_t n = 0;
+  explicit DeviceBuf(size_t bytes) : n(bytes) {
+    if (hipMalloc(reinterpret_cast<void**>(&p), bytes) != hipSuccess) p = nullptr;
+  }
+  ~DeviceBuf() {
+    if (p) (void)hipFree(p);
+  }
+  bool upload(const std::vector<uint8_t>& h) { return hipMemcpy(p, h.data(), h.size(), hipMemcpyHostToDevice) == hipSuccess; }
+  bool download(std::vector<uint8_t>& h) {
+    h.resize(n);
+    return hipMemcpy(h.data(), p, n, hipMemcpyDeviceToHost) == hipSuccess;
+  }
+};
+
+hsa_signal_t make_signal(hsa_signal_value_t v) {
+  hsa_signal_t s{0};
+  if (hsa_signal_create(v, 0, nullptr, &s) != HSA_STATUS_SUCCESS) s.handle = 0;
+  return s;
+}
+
+bool wait_zero(hsa_signal_t s, hsa_wait_state_t state, uint64_t timeout_ms = 20000) {
+  // timeout in the system timestamp's units; read its frequency
+  uint64_t freq = 0;
+  hsa_system_get_info(HSA_SYSTEM_INFO_TIMESTAMP_FREQUENCY, &freq);
+  const uint64_t ticks = freq ? freq / 1000 * timeout_ms : UINT64_MAX;
+  const auto deadline = std::chrono::steady_clock::now() + std::chrono::milliseconds(timeout_ms);
+  while (std::chrono::steady_clock::now() < deadline) {
+    if (hsa_signal_wait_scacquire(s, HSA_SIGNAL_CONDITION_LT, 1, ticks, state) < 1) return true;
+  }
+  return false;
+}
+
+std::vector<uint8_t> seeded(size_t n, uint64_t seed) {
+  std::vector<uint8_t> v(n);
+  oracle_fill_random(v.data(), n, seed);
+  return v;
+}
+
+// ---------------------------------------------------------------------------
+
+void test_blocking_copy(BlitKernelGfx950& blit) {
+  const char* name = "blocking_copy_offsets_and_sizes";
+  const size_t max_n = (3u << 20) + 77;
+  std::vector<uint8_t> src_h = seeded(max_n + 64, 0xB1170003);
+  DeviceBuf src(src_h.size()), dst(max_n + 2 * kGuard + 64);
+  REQUIRE(src.p && dst.p, "hipMalloc");
+  REQUIRE(src.upload(src_h), "upload");
+  const size_t sizes[] = {1, 3, 4, 15, 16, 17, 255, 4096, 65537, (1u << 20), max_n};
+  for (size_t n : sizes) {
+    for (int pair = 0; pair < 4; ++pair) {
+      const size_t so = (pair * 5 + 1) & 15, dof = (pair * 11 + 2) & 15;
+      std::vector<uint8_t> want(dst.n, kGuardByte), got;
+      REQUIRE(dst.upload(want), "upload");
+      hsa_status_t st = blit.SubmitLinearCopyCommand(dst.p + kGuard + dof, src.p + so, n);
+      REQUIRE(st == HSA_STATUS_SUCCESS, "status 0x%x", st);
+      oracle_copy(want.data() + kGuard + dof, src_h.data() + so, n);
+      REQUIRE(dst.download(got), "download");
+      REQUIRE(got == want, "bytes differ n=%zu so=%zu do=%zu", n, so, dof);
+    }
+  }
+  std::printf("PASS %s\n", name);
+}
+
+void test_blocking_fill(BlitKernelGfx950& blit) {
+  const char* name = "blocking_fill_reference_patterns";
+  // rocrtst/samples/async_mem_copy/async_mem_copy.cc:62-65
+  const uint32_t values[] = {0xabcdef12, 0xba5eba11, 0xfeed5a1e, 0xbaadf00d, 0xA5C30F1E};
+  const size_t counts[] = {1, 3, 4, 5, 1023, 262144 + 3};
+  DeviceBuf dst(4 * (262144 + 3) + 2 * kGuard + 16);
+  REQUIRE(dst.p, "hipMalloc");
+  for (uint32_t v : values) {
+    for (size_t c : counts) {
+      for (size_t off : {size_t(0), size_t(4), size_t(12)}) {
+        std::vector<uint8_t> want(dst.n, kGuardByte), got;
+        REQUIRE(dst.upload(want), "upload");
+        hsa_status_t st = blit.SubmitLinearFillCommand(dst.p + kGuard + off, v, c);
+        REQUIRE(st == HSA_STATUS_SUCCESS, "status 0x%x", st);
+        oracle_fill32(want.data() + kGuard + off, v, c);
+        REQUIRE(dst.download(got), "download");
+        REQUIRE(got == want, "bytes differ value=%x count=%zu off=%zu", v, c, off);
+      }
+    }
+  }
+  // amd_blit_kernel.cpp:791-794: misaligned pointer -> HSA_STATUS_ERROR, nothing written
+  std::vector<uint8_t> want(dst.n, kGuardByte), got;
+  REQUIRE(dst.upload(want), "upload");
+  for (size_t off : {size_t(1), size_t(2), size_t(3)}) {
+    hsa_status_t st = blit.SubmitLinearFillCommand(dst.p + kGuard + off, 1, 4);
+    REQUIRE(st == HSA_STATUS_ERROR, "misaligned fill returned 0x%x", st);
+    REQUIRE(oracle_ref_blit_fill_status(reinterpret_cast<uintptr_t>(dst.p + kGuard + off)) == ORACLE_STATUS_ERROR,
+            "oracle disagrees");
+  }
+  REQUIRE(dst.download(got), "download");
+  REQUIRE(got == want, "rejected fill wrote memory");
+  std::printf("PASS %s\n", name);
+}
+
+void test_async_copy_signal(BlitKernelGfx950& blit, hsa_wait_state_t state, const char* name) {
+  const size_t n = (8u << 20) + 5;
+  std::vector<uint8_t> src_h = seeded(n + 16, 0xB1170002);
+  DeviceBuf src(src_h.size()), dst(n + 2 * kGuard + 16);
+  REQUIRE(src.p && dst.p, "hipMalloc");
+  REQUIRE(src.upload(src_h), "upload");
+  std::vector<uint8_t> want(dst.n, kGuardByte), got;
+  REQUIRE(dst.upload(want), "upload");
+  hsa_signal_t done = make_signal(1);
+  REQUIRE(done.handle, "signal");
+  Signal out(done);
+  std::vector<Signal*> deps, gang;
+  hsa_status_t st = blit.SubmitLinearCopyCommand(dst.p + kGuard + 3, src.p + 1, n, deps, out, gang);
+  REQUIRE(st == HSA_STATUS_SUCCESS, "status 0x%x", st);
+  REQUIRE(wait_zero(done, state), "completion signal never reached 0");
+  REQUIRE(hsa_signal_load_relaxed(done) == 0, "signal value %ld", (long)hsa_signal_load_relaxed(done));
+  oracle_copy(want.data() + kGuard + 3, src_h.data() + 1, n);
+  REQUIRE(dst.download(got), "download");
+  REQUIRE(got == want, "bytes differ");
+  // the blit reports idle once everything has completed
+  uint64_t pending = 1;
+  for (int i = 0; i < 1000 && pending; ++i) {
+    pending = blit.PendingBytes();
+    if (pending) std::this_thread::sleep_for(std::chrono::milliseconds(1));
+  }
+  REQUIRE(pending == 0, "PendingBytes stuck at %llu", (unsigned long long)pending);
+  hsa_signal_destroy(done);
+  std::printf("PASS %s\n", name);
+}
+
+void test_dependencies(BlitKernelGfx950& blit, size_t n_deps, const char* name) {
+  const size_t n = (1u << 20) + 9;
+  std::vector<uint8_t> src_h = seeded(n, 0xB1170004);
+  DeviceBuf src(n), dst(n + 2 * kGuard);
+  REQUIRE(src.p && dst.p, "hipMalloc");
+  REQUIRE(src.upload(src_h), "upload");
+  std::vector<uint8_t> before(dst.n, kGuardByte), got;
+  REQUIRE(dst.upload(before), "upload");
+  std::vector<hsa_signal_t> dep_handles;
+  std::vector<Signal> dep_objs;
+  for (size_t i = 0; i < n_deps; ++i) dep_handles.push_back(make_signal(1));
+  for (hsa_signal_t h : dep_handles) {
+    REQUIRE(h.handle, "signal");
+    dep_objs.emplace_back(h);
+  }
+  std::vector<Signal*> deps, gang;
+  for (Signal& s : dep_objs) deps.push_back(&s);
+  hsa_signal_t done = make_signal(1);
+  Signal out(done);
+  hsa_status_t st = blit.SubmitLinearCopyCommand(dst.p + kGuard, src.p, n, deps, out, gang);
+  REQUIRE(st == HSA_STATUS_SUCCESS, "status 0x%x", st);
+  // a command submitted behind a blocked one must not overtake it
+  hsa_signal_t done2 = make_signal(1);
+  Signal out2(done2);
+  std::vector<Signal*> no_deps;
+  st = blit.SubmitLinearCopyCommand(dst.p + kGuard, src.p + 1, 16, no_deps, out2, gang);
+  REQUIRE(st == HSA_STATUS_SUCCESS, "status 0x%x", st);
+  REQUIRE(blit.PendingBytes() != 0, "PendingBytes is 0 with blocked commands");
+  // satisfy all but the last dependency: nothing may run
+  for (size_t i = 0; i + 1 < n_deps; ++i) hsa_signal_store_screlease(dep_handles[i], 0);
+  std::this_thread::sleep_for(std::chrono::milliseconds(100));
+  REQUIRE(hsa_signal_load_scacquire(done) == 1, "copy completed before its dependencies");
+  REQUIRE(hsa_signal_load_scacquire(done2) == 1, "a later command overtook a blocked one");
+  REQUIRE(dst.download(got), "download");
+  REQUIRE(got == before, "destination written before dependencies were satisfied");
+  hsa_signal_store_screlease(dep_handles[n_deps - 1], 0);
+  REQUIRE(wait_zero(done, HSA_WAIT_STATE_BLOCKED), "copy never completed");
+  REQUIRE(wait_zero(done2, HSA_WAIT_STATE_BLOCKED), "second copy never completed");
+  std::vector<uint8_t> want(before);
+  oracle_copy(want.data() + kGuard, src_h.data(), n);
+  oracle_copy(want.data() + kGuard, src_h.data() + 1, 16);  // second command, in order
+  REQUIRE(dst.download(got), "download");
+  REQUIRE(got == want, "bytes differ");
+  for (hsa_signal_t h : dep_handles) hsa_signal_destroy(h);
+  hsa_signal_destroy(done);
+  hsa_signal_destroy(done2);
+  std::printf("PASS %s\n", name);
+}
+
+void test_chain(BlitKernelGfx950& blit) {
+  const char* name = "chain_a_to_b_to_c";
+  const size_t n = (2u << 20) + 11;
+  std::vector<uint8_t> a_h = seeded(n, 0xB1170005);
+  DeviceBuf a(n), b(n + 32), c(n + 2 * kGuard + 32);
+  REQUIRE(a.p && b.p && c.p, "hipMalloc");
+  REQUIRE(a.upload(a_h), "upload");
+  std::vector<uint8_t> want(c.n, kGuardByte), got;
+  REQUIRE(c.upload(want), "upload");
+  HIP_OK(hipMemset(b.p, 0, b.n));
+  hsa_signal_t s1 = make_signal(1), s2 = make_signal(1);
+  Signal sig1(s1), sig2(s2);
+  std::vector<Signal*> none, after1{&sig1}, gang;
+  REQUIRE(blit.SubmitLinearCopyCommand(b.p + 5, a.p, n, none, sig1, gang) == HSA_STATUS_SUCCESS, "submit 1");
+  REQUIRE(blit.SubmitLinearCopyCommand(c.p + kGuard + 2, b.p + 5, n, after1, sig2, gang) == HSA_STATUS_SUCCESS,
+          "submit 2");
+  REQUIRE(wait_zero(s2, HSA_WAIT_STATE_BLOCKED), "chain never completed");
+  REQUIRE(hsa_signal_load_relaxed(s1) == 0, "first signal not 0");
+  oracle_copy(want.data() + kGuard + 2, a_h.data(), n);
+  REQUIRE(c.download(got), "download");
+  REQUIRE(got == want, "bytes differ");
+  hsa_signal_destroy(s1);
+  hsa_signal_destroy(s2);
+  std::printf("PASS %s\n", name);
+}
+
+void test_zero_size_and_bad_args(BlitKernelGfx950& blit) {
+  const char* name = "zero_size_and_bad_arguments";
+  DeviceBuf d(4096);
+  REQUIRE(d.p, "hipMalloc");
+  hsa_signal_t s = make_signal(1);
+  Signal sig(s);
+  std::vector<Signal*> none, gang;
+  REQUIRE(blit.SubmitLinearCopyCommand(nullptr, d.p, 16, none, sig, gang) == HSA_STATUS_ERROR_INVALID_ARGUMENT, "null dst");
+  REQUIRE(blit.SubmitLinearCopyCommand(d.p, nullptr, 16, none, sig, gang) == HSA_STATUS_ERROR_INVALID_ARGUMENT, "null src");
+  REQUIRE(hsa_signal_load_relaxed(s) == 1, "signal touched by a rejected command");
+  // size 0 completes the signal without moving anything
+  REQUIRE(blit.SubmitLinearCopyCommand(d.p, d.p + 64, 0, none, sig, gang) == HSA_STATUS_SUCCESS, "zero size");
+  REQUIRE(wait_zero(s, HSA_WAIT_STATE_BLOCKED), "zero-size copy never completed");
+  REQUIRE(blit.SubmitLinearCopyCommand(d.p, d.p + 64, 0) == HSA_STATUS_SUCCESS, "blocking zero size");
+  REQUIRE(blit.SubmitLinearFillCommand(d.p, 7, 0) == HSA_STATUS_SUCCESS, "zero-count fill");
+  REQUIRE(!blit.isSDMA() && !blit.GangLeader(), "engine kind");
+  REQUIRE(blit.EnableProfiling(true) == HSA_STATUS_SUCCESS && blit.EnableProfiling(false) == HSA_STATUS_SUCCESS,
+          "EnableProfiling");
+  hsa_signal_destroy(s);
+  std::printf("PASS %s\n", name);
+}
+
+void test_batch(BlitKernelGfx950& blit) {
+  const char* name = "batched_copies_with_signal";
+  const size_t ncopy = 500;
+  std::vector<size_t> len(ncopy), off(ncopy), so(ncopy), dof(ncopy);
+  std::vector<uint8_t> rnd = seeded(ncopy * 4, 0xB1170055);
+  size_t total = 256;
+  for (size_t i = 0; i < ncopy; ++i) {
+    len[i] = 1 + (size_t(rnd[4 * i]) | (size_t(rnd[4 * i + 1]) << 8)) % 40000;
+    so[i] = rnd[4 * i + 2] & 15;
+    dof[i] = rnd[4 * i + 3] & 15;
+    off[i] = total;
+    total += ((len[i] + 255) / 256) * 256 + 256;
+  }
+  std::vector<uint8_t> src_h = seeded(total, 0xB1170056);
+  DeviceBuf src(total), dst(total);
+  REQUIRE(src.p && dst.p, "hipMalloc");
+  REQUIRE(src.upload(src_h), "upload");
+  std::vector<uint8_t> want(total, kGuardByte), got;
+  REQUIRE(dst.upload(want), "upload");
+  std::vector<mi355_blit_desc_t> descs(ncopy);
+  for (size_t i = 0; i < ncopy; ++i) {
+    descs[i].dst = dst.p + off[i] + dof[i];
+    descs[i].src = src.p + off[i] + so[i];
+    descs[i].bytes = len[i];
+    oracle_copy(want.data() + off[i] + dof[i], src_h.data() + off[i] + so[i], len[i]);
+  }
+  hsa_signal_t s = make_signal(1);
+  Signal sig(s);
+  std::vector<Signal*> none;
+  REQUIRE(blit.SubmitBatchCopyCommand(descs.data(), ncopy, false, none, sig) == HSA_STATUS_SUCCESS, "submit");
+  REQUIRE(wait_zero(s, HSA_WAIT_STATE_BLOCKED), "batch never completed");
+  REQUIRE(dst.download(got), "download");
+  REQUIRE(got == want, "bytes differ");
+  hsa_signal_destroy(s);
+  std::printf("PASS %s\n", name);
+}
+
+void test_threads(BlitKernelGfx950& blit) {
+  const char* name = "concurrent_submitters";
+  const int kThreads = 4, kPer = 6;
+  const size_t n = (1u << 18) + 13, region = ((n + 2 * kGuard + 255) / 256) * 256;
+  std::vector<uint8_t> src_h = seeded(n + 64, 0xB1170077);
+  DeviceBuf src(src_h.size()), dst(region * kThreads * kPer);
+  REQUIRE(src.p && dst.p, "hipMalloc");
+  REQUIRE(src.upload(src_h), "upload");
+  std::vector<uint8_t> want(dst.n, kGuardByte), got;
+  REQUIRE(dst.upload(want), "upload");
+  std::vector<hsa_status_t> status(kThreads * kPer, HSA_STATUS_SUCCESS);
+  std::vector<std::thread> ths;
+  for (int t = 0; t < kThreads; ++t) {
+    ths.emplace_back([&, t] {
+      for (int j = 0; j < kPer; ++j) {
+        const int slot = t * kPer + j;
+        // alternate blocking copies and blocking fills followed by copies
+        if (j & 1) status[slot] = blit.SubmitLinearFillCommand(dst.p + slot * region + kGuard, 0x01020304u * (slot + 1), n / 4);
+        else status[slot] = blit.SubmitLinearCopyCommand(dst.p + slot * region + kGuard + (slot & 15), src.p + (slot % 7), n);
+      }
+    });
+  }
+  for (auto& th : ths) th.join();
+  for (int slot = 0; slot < kThreads * kPer; ++slot) {
+    REQUIRE(status[slot] == HSA_STATUS_SUCCESS, "slot %d status 0x%x", slot, status[slot]);
+    if ((slot % kPer) & 1) oracle_fill32(want.data() + slot * region + kGuard, 0x01020304u * (slot + 1), n / 4);
+    else oracle_copy(want.data() + slot * region + kGuard + (slot & 15), src_h.data() + (slot % 7), n);
+  }
+  REQUIRE(dst.download(got), "download");
+  REQUIRE(got == want, "bytes differ");
+  std::printf("PASS %s\n", name);
+}
+
+void latency_report(BlitKernelGfx950& blit, const char* mode) {
+  // host-observed time per blocking call, submit -> completion seen
+  // (the way memory_async_copy.cc:396-405 times a copy)
+  DeviceBuf a(1 << 20), b(1 << 20);
+  if (!a.p || !b.p) return;
+  for (size_t n : {size_t(4096), size_t(65536), size_t(1 << 20)}) {
+    std::vector<double> us;
+    for (int i = 0; i < 120; ++i) {
+      auto t0 = std::chrono::steady_clock::now();
+      blit.SubmitLinearCopyCommand(b.p, a.p, n);
+      auto t1 = std::chrono::steady_clock::now();
+      if (i >= 20) us.push_back(std::chrono::duration<double, std::micro>(t1 - t0).count());
+    }
+    std::sort(us.begin(), us.end());
+    std::printf("INFO blocking_copy_us mode=%s bytes=%zu median=%.2f min=%.2f\n", mode, n, us[us.size() / 2], us[0]);
+  }
+}
+
+}  // namespace
+
+int main(int argc, char** argv) {
+  if (argc > 1 && std::string(argv[1]) == "--list") {
+    std::printf("blocking_copy_offsets_and_sizes\nblocking_fill_reference_patterns\nasync_copy_active_wait\n"
+                "async_copy_blocked_wait\ndependencies_1\ndependencies_6\nchain_a_to_b_to_c\n"
+                "zero_size_and_bad_arguments\nbatched_copies_with_signal\nconcurrent_submitters\n"
+                "host_callback_async_copy\n");
+    return 0;
+  }
+  if (hsa_init() != HSA_STATUS_SUCCESS) {
+    std::printf("FAIL setup: hsa_init failed (no GPU?)\n");
+    return 2;
+  }
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count < 1) {
+    std::printf("FAIL setup: no HIP device\n");
+    return 2;
+  }
+  rocr::core::Agent agent(0);
+  {
+    // the host-callback completion mode: one asynchronous and one blocking case
+    BlitKernelGfx950 cb(nullptr, BlitKernelGfx950::Completion::kHostCallback);
+    if (cb.Initialize(agent) != HSA_STATUS_SUCCESS) {
+      std::printf("FAIL setup: Initialize (host callback)\n");
+      return 2;
+    }
+    test_async_copy_signal(cb, HSA_WAIT_STATE_BLOCKED, "host_callback_async_copy");
+    test_chain(cb);
+    latency_report(cb, "host_callback");
+    if (cb.Destroy(agent) != HSA_STATUS_SUCCESS) {
+      std::printf("FAIL destroy (host callback)\n");
+      ++g_failures;
+    }
+  }
+  BlitKernelGfx950* blit = new BlitKernelGfx950(nullptr);
+  if (blit->Initialize(agent) != HSA_STATUS_SUCCESS) {
+    std::printf("FAIL setup: Initialize\n");
+    return 2;
+  }
+  test_blocking_copy(*blit);
+  test_blocking_fill(*blit);
+  test_async_copy_signal(*blit, HSA_WAIT_STATE_ACTIVE, "async_copy_active_wait");
+  test_async_copy_signal(*blit, HSA_WAIT_STATE_BLOCKED, "async_copy_blocked_wait");
+  test_dependencies(*blit, 1, "dependencies_1");
+  test_dependencies(*blit, 6, "dependencies_6");  // more than one barrier packet's worth in the reference
+  test_chain(*blit);
+  test_zero_size_and_bad_args(*blit);
+  test_batch(*blit);
+  test_threads(*blit);
+  latency_report(*blit, "device_signal");
+  hsa_status_t st = blit->Destroy(agent);
+  if (st != HSA_STATUS_SUCCESS) {
+    std::printf("FAIL destroy: status 0x%x\n", st);
+    ++g_failures;
+  } else {
+    std::printf("PASS destroy\n");
+  }
+  delete blit;
+  hsa_shut_down();
+  std::printf("%s (%d failures)\n", g_failures ? "FAILED" : "OK", g_failures);
+  return g_failures ? 1 : 0;
+}

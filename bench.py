@@ -212,6 +212,58 @@ def small_copy_latency(r, sizes=(4096, 65536, MIB)):
     return out
 
 
+def reference_gpu_path(r):
+    """The reference's own blit kernels on this GPU, for orientation: the ROCr
+    this process already runs on (libhsa-runtime64, the binary build of the same
+    component) serves hsa_memory_copy / hsa_amd_memory_fill on same-GPU device
+    pointers with AMD::BlitKernel (runtime.cpp:513, amd_gpu_agent.cpp:951, 1285).
+    Blocking calls timed with the host clock, best of a few."""
+    try:
+        hsa = C.CDLL("libhsa-runtime64.so.1")
+        hsa.hsa_init.restype = C.c_int
+        hsa.hsa_memory_copy.restype = C.c_int
+        hsa.hsa_memory_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        hsa.hsa_amd_memory_fill.restype = C.c_int
+        hsa.hsa_amd_memory_fill.argtypes = [C.c_void_p, C.c_uint32, C.c_size_t]
+        if hsa.hsa_init() != 0:
+            return None
+    except (OSError, AttributeError):
+        return None
+    src = r.device_bytes(GIB + 64, seed=0xB1170003)
+    dst = r.device_bytes(GIB + 64)
+    S, D = aligned_ptr(src), aligned_ptr(dst)
+
+    def best(fn, reps):
+        b = 1e9
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            st = fn()
+            b = min(b, time.perf_counter() - t0)
+            if st != 0:
+                return None
+        return b
+
+    out = {}
+    t = best(lambda: hsa.hsa_memory_copy(D, S, GIB), 6)
+    if t:
+        assert r.torch.equal(dst[(-dst.data_ptr()) % 256:][:GIB], src[(-src.data_ptr()) % 256:][:GIB])
+        out["copy_1GiB_gbs"] = round(2 * GIB / t / 1e9, 1)
+    t = best(lambda: hsa.hsa_memory_copy(D + 9, S + 3, GIB - 64), 3)
+    if t:
+        out["misaligned_1GiB_gbs"] = round(2 * (GIB - 64) / t / 1e9, 1)
+    t = best(lambda: hsa.hsa_amd_memory_fill(D, FILL_VALUE, GIB // 4), 6)
+    if t:
+        out["fill_1GiB_gbs"] = round(GIB / t / 1e9, 1)
+    t = best(lambda: hsa.hsa_memory_copy(D, S, 4096), 200)
+    if t:
+        out["copy_4KiB_us"] = round(t * 1e6, 2)
+    t = best(lambda: hsa.hsa_memory_copy(D, S, MIB), 200)
+    if t:
+        out["copy_1MiB_us"] = round(t * 1e6, 2)
+    out["how"] = "blocking hsa_memory_copy / hsa_amd_memory_fill of the loaded libhsa-runtime64, host clock, best of n"
+    return out or None
+
+
 def cpu_baseline(ora, budget_s):
     """The reference's host path on this box's cores: memcpy of 256 MiB
     (BASELINE config 1; what hsa_memory_copy does for host pointers), single
@@ -316,6 +368,7 @@ def main():
             del f2, v2, k2
             torch.cuda.empty_cache()
         also["small_copy_us"] = small_copy_latency(r)
+        also["reference_gpu_path"] = reference_gpu_path(r)
 
     line = {
         "metric": "D2D copy & fill GB/s (R+W) at 1 GiB on 1 MI355X",

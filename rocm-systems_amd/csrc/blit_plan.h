@@ -32,31 +32,36 @@ struct SizeClass {
   uint32_t store_policy;
 };
 
-// Measured on MI355X (256 CUs) at 1 GiB.  Source and destination equally
-// aligned mod 16: one 1 KiB tile per single-wave workgroup is the fastest
-// shape once the transfer streams from HBM.  A dword offset between them makes
-// every wave's 1 KiB of loads straddle a cache line shared with its
-// neighbour, and 4-wave workgroups share that line in one CU.  A byte offset
-// adds one extra dword fetch per tile (the bytes that spill past the last
-// lane), which 2 KiB tiles in 8-wave workgroups amortise best.  Fills are
-// bound by the dispatcher's workgroup rate at one wave per workgroup and want
-// 4-wave workgroups.  Transfers that cannot stay in cache bypass it: loads
-// non-temporal, stores written through.  Last match wins.
+// Measured on MI355X (256 CUs), sweeps of 4 KiB .. 4 GiB in powers of 4.
+// Up to a few MiB a launch is bound by its fixed cost (~3.5 us back to back)
+// and the shape does not matter.  From there on transfers bypass the caches:
+// loads non-temporal, stores written through L2.  Source and destination
+// equally aligned mod 16: one 1 KiB tile per single-wave workgroup is the
+// fastest shape once the transfer streams from HBM (>= 512 MiB); while the
+// 256 MiB last-level cache still absorbs part of it, 4-wave workgroups are.
+// A dword offset between the two makes every wave's 1 KiB of loads straddle a
+// cache line shared with its neighbour; 4-wave workgroups share that line
+// within one CU.  A byte offset adds one dword fetch per tile (the bytes that
+// spill past the last lane), which 2 KiB tiles amortise best.  Fills at one
+// wave per workgroup are bound by the dispatcher's workgroup rate and want
+// 4-wave workgroups.  Last match wins.
 constexpr SizeClass kCopyClasses[] = {      // (src - dst) % 16 == 0
     {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
-    {8ull << 20, 64, 1, 1, MI355_BLIT_STORE_AGENT_WT},
+    {4ull << 20, 256, 1, 1, MI355_BLIT_STORE_AGENT_WT},
+    {512ull << 20, 64, 1, 1, MI355_BLIT_STORE_AGENT_WT},
 };
 constexpr SizeClass kCopyDwordOffsetClasses[] = {  // (src - dst) % 4 == 0
     {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
-    {8ull << 20, 256, 1, 1, MI355_BLIT_STORE_AGENT_WT},
+    {4ull << 20, 256, 1, 1, MI355_BLIT_STORE_AGENT_WT},
 };
 constexpr SizeClass kCopyRealignClasses[] = {  // (src - dst) % 4 != 0
-    {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
-    {8ull << 20, 512, 2, 1, MI355_BLIT_STORE_NT},
+    {0, 512, 1, 0, MI355_BLIT_STORE_CACHED},
+    {4ull << 20, 256, 2, 1, MI355_BLIT_STORE_AGENT_WT},
+    {512ull << 20, 256, 2, 1, MI355_BLIT_STORE_NT},
 };
 constexpr SizeClass kFillClasses[] = {
     {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
-    {8ull << 20, 256, 1, 0, MI355_BLIT_STORE_SYSTEM_WT},
+    {16ull << 20, 256, 1, 0, MI355_BLIT_STORE_SYSTEM_WT},
 };
 
 inline bool valid_unroll(uint32_t u) { return u == 1 || u == 2 || u == 4; }

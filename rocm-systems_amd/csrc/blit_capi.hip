@@ -28,6 +28,10 @@ using namespace mi355;
 // queue has 64 (amd_gpu_agent.h:507-508).
 constexpr unsigned kLedgerSlots = 64;
 
+// Waves that share one 4 KiB chunk of the batched copy: with 4, a 4-wave
+// workgroup moves one chunk, 1 KiB per wave (measured best on MI355X).
+constexpr unsigned kBatchSplit = 4;
+
 struct LedgerSlot {
   hipEvent_t done = nullptr;
   uint64_t bytes = 0;  // submitted between the previous marker and this one
@@ -53,12 +57,15 @@ struct mi355_blit {
   hipStream_t last_stream = nullptr;
 
   // batched path staging (grown on demand, never shrunk)
-  BatchDesc* descs_host = nullptr;  // pinned
+  BatchDesc* descs_host[2] = {nullptr, nullptr};  // pinned, used alternately
+  hipEvent_t upload_done[2] = {nullptr, nullptr};  // the upload from descs_host[i] has finished
+  bool upload_busy[2] = {false, false};
+  unsigned next_host = 0;
   BatchDesc* descs_dev = nullptr;
   uint32_t* chunk_start_dev = nullptr;
   uint32_t* block_sum_dev = nullptr;
-  uint32_t* owner_dev = nullptr;  // chunk -> copy map
-  size_t owner_capacity = 0;
+  ChunkRecord* records_dev = nullptr;  // one per chunk
+  size_t records_capacity = 0;
   size_t batch_capacity = 0;
   hipEvent_t staging_free = nullptr;  // previous batch has consumed the staging buffers
   bool staging_busy = false;
@@ -146,6 +153,28 @@ fill_kernel_t select_fill_kernel(const mi355_blit_plan_t& p) {
   }
 }
 
+typedef void (*batch_kernel_t)(const ChunkRecord*, uint64_t);
+
+template <int SPLIT, bool NTL>
+batch_kernel_t batch_kernel_st(unsigned policy) {
+  switch (policy) {
+    case MI355_BLIT_STORE_CACHED: return k_batch_copy_records<SPLIT, NTL, kStoreCached>;
+    case MI355_BLIT_STORE_NT: return k_batch_copy_records<SPLIT, NTL, kStoreNt>;
+    case MI355_BLIT_STORE_AGENT_WT: return k_batch_copy_records<SPLIT, NTL, kStoreAgentWt>;
+    case MI355_BLIT_STORE_SYSTEM_WT: return k_batch_copy_records<SPLIT, NTL, kStoreSystemWt>;
+    default: return nullptr;
+  }
+}
+
+batch_kernel_t select_batch_kernel(unsigned split, bool ntl, unsigned policy) {
+  switch (split) {
+    case 1: return ntl ? batch_kernel_st<1, true>(policy) : batch_kernel_st<1, false>(policy);
+    case 2: return ntl ? batch_kernel_st<2, true>(policy) : batch_kernel_st<2, false>(policy);
+    case 4: return ntl ? batch_kernel_st<4, true>(policy) : batch_kernel_st<4, false>(policy);
+    default: return nullptr;
+  }
+}
+
 // Which waves of the launch take the partial last tile and the edges.
 void set_tail_waves(const mi355_blit_plan_t& p, uint32_t* partial_wave, uint32_t* edge_wave) {
   const uint64_t n_waves = static_cast<uint64_t>(p.grid) * (p.wg_size / 64);
@@ -187,21 +216,23 @@ int ledger_record(mi355_blit* h, hipStream_t s, uint64_t bytes) {
 }
 
 void free_batch_buffers(mi355_blit* h) {
-  if (h->descs_host) (void)hipHostFree(h->descs_host);
+  for (int i = 0; i < 2; ++i) {
+    if (h->descs_host[i]) (void)hipHostFree(h->descs_host[i]);
+    h->descs_host[i] = nullptr;
+  }
   if (h->descs_dev) (void)hipFree(h->descs_dev);
   if (h->chunk_start_dev) (void)hipFree(h->chunk_start_dev);
   if (h->block_sum_dev) (void)hipFree(h->block_sum_dev);
-  h->descs_host = nullptr;
   h->descs_dev = nullptr;
   h->chunk_start_dev = nullptr;
   h->block_sum_dev = nullptr;
   h->batch_capacity = 0;
 }
 
-// Buffers for n descriptors and, when owner_entries != 0, a chunk map of that
-// many entries.  Caller holds h->lock.
-int ensure_batch_capacity(mi355_blit* h, size_t n, size_t owner_entries) {
-  if (n <= h->batch_capacity && owner_entries <= h->owner_capacity) return MI355_BLIT_SUCCESS;
+// Buffers for n descriptors and, when n_records != 0, that many chunk records.
+// Caller holds h->lock.
+int ensure_batch_capacity(mi355_blit* h, size_t n, size_t n_records) {
+  if (n <= h->batch_capacity && n_records <= h->records_capacity) return MI355_BLIT_SUCCESS;
   // the old buffers may still be read by a batch in flight
   if (h->staging_busy) {
     BLIT_HIP(hipEventSynchronize(h->staging_free));
@@ -211,20 +242,24 @@ int ensure_batch_capacity(mi355_blit* h, size_t n, size_t owner_entries) {
     size_t cap = h->batch_capacity ? h->batch_capacity : 1024;
     while (cap < n) cap *= 2;
     free_batch_buffers(h);
-    BLIT_HIP(hipHostMalloc(reinterpret_cast<void**>(&h->descs_host), cap * sizeof(BatchDesc), hipHostMallocDefault));
+    for (int i = 0; i < 2; ++i) {
+      // uploads from the old pinned buffers are over: staging_free was waited for above
+      h->upload_busy[i] = false;
+      BLIT_HIP(hipHostMalloc(reinterpret_cast<void**>(&h->descs_host[i]), cap * sizeof(BatchDesc), hipHostMallocDefault));
+    }
     BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->descs_dev), cap * sizeof(BatchDesc)));
     BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->chunk_start_dev), (cap + 1) * sizeof(uint32_t)));
     BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->block_sum_dev), (cap / 1024 + 1) * sizeof(uint32_t)));
     h->batch_capacity = cap;
   }
-  if (owner_entries > h->owner_capacity) {
-    size_t cap = h->owner_capacity ? h->owner_capacity : 65536;
-    while (cap < owner_entries) cap *= 2;
-    if (h->owner_dev) (void)hipFree(h->owner_dev);
-    h->owner_dev = nullptr;
-    h->owner_capacity = 0;
-    BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->owner_dev), cap * sizeof(uint32_t)));
-    h->owner_capacity = cap;
+  if (n_records > h->records_capacity) {
+    size_t cap = h->records_capacity ? h->records_capacity : 65536;
+    while (cap < n_records) cap *= 2;
+    if (h->records_dev) (void)hipFree(h->records_dev);
+    h->records_dev = nullptr;
+    h->records_capacity = 0;
+    BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->records_dev), cap * sizeof(ChunkRecord)));
+    h->records_capacity = cap;
   }
   return MI355_BLIT_SUCCESS;
 }
@@ -289,6 +324,8 @@ int mi355_blit_create(int device_ordinal, mi355_blit_t** out) {
   for (unsigned i = 0; e == hipSuccess && i < kLedgerSlots; ++i)
     e = hipEventCreateWithFlags(&h->ledger[i].done, hipEventDisableTiming);
   if (e == hipSuccess) e = hipEventCreateWithFlags(&h->staging_free, hipEventDisableTiming);
+  for (int i = 0; e == hipSuccess && i < 2; ++i)
+    e = hipEventCreateWithFlags(&h->upload_done[i], hipEventDisableTiming);
   if (e != hipSuccess || cus <= 0) {
     mi355_blit_destroy(h);
     return e == hipSuccess ? MI355_BLIT_ERROR : status_of(e);
@@ -318,8 +355,10 @@ int mi355_blit_destroy(mi355_blit_t* h) {
       (void)hipStreamDestroy(h->stream);
     }
     if (h->staging_free) (void)hipEventDestroy(h->staging_free);
+    for (int i = 0; i < 2; ++i)
+      if (h->upload_done[i]) (void)hipEventDestroy(h->upload_done[i]);
     free_batch_buffers(h);
-    if (h->owner_dev) (void)hipFree(h->owner_dev);
+    if (h->records_dev) (void)hipFree(h->records_dev);
   }
   delete h;
   return rc;
@@ -422,19 +461,26 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
   int rc = ensure_batch_capacity(h, n, descs_on_device ? 0 : total_chunks);
   if (rc != MI355_BLIT_SUCCESS) return rc;
 
-  // The staging buffers are shared by consecutive batches: device-side reuse
-  // waits on the stream, the host-written pinned buffer on the host.
+  // The device-side staging buffers are shared by consecutive batches: the
+  // next batch waits for the previous one on the stream.  The host writes the
+  // pinned descriptor copies alternately, so preparing one batch overlaps the
+  // execution of the one before; a pinned buffer is only waited for until its
+  // own upload, two batches ago, has finished.
   if (h->staging_busy) BLIT_HIP(hipStreamWaitEvent(s, h->staging_free, 0));
   const BatchDesc* dev_descs;
   if (descs_on_device) {
     dev_descs = reinterpret_cast<const BatchDesc*>(descs);
   } else {
-    if (h->staging_busy) {
-      BLIT_HIP(hipEventSynchronize(h->staging_free));
-      h->staging_busy = false;
+    const unsigned b = h->next_host;
+    h->next_host ^= 1;
+    if (h->upload_busy[b]) {
+      BLIT_HIP(hipEventSynchronize(h->upload_done[b]));
+      h->upload_busy[b] = false;
     }
-    std::memcpy(h->descs_host, descs, n * sizeof(BatchDesc));
-    BLIT_HIP(hipMemcpyAsync(h->descs_dev, h->descs_host, n * sizeof(BatchDesc), hipMemcpyHostToDevice, s));
+    std::memcpy(h->descs_host[b], descs, n * sizeof(BatchDesc));
+    BLIT_HIP(hipMemcpyAsync(h->descs_dev, h->descs_host[b], n * sizeof(BatchDesc), hipMemcpyHostToDevice, s));
+    BLIT_HIP(hipEventRecord(h->upload_done[b], s));
+    h->upload_busy[b] = true;
     dev_descs = h->descs_dev;
   }
 
@@ -443,9 +489,6 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
                      static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev);
   hipLaunchKernelGGL(k_batch_scan_top, dim3(1), dim3(1024), 0, s, h->block_sum_dev, n_blocks,
                      h->chunk_start_dev, static_cast<uint64_t>(n));
-  hipLaunchKernelGGL(k_batch_expand, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, s,
-                     dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev,
-                     descs_on_device ? nullptr : h->owner_dev);
   BLIT_HIP(hipGetLastError());
 
   mi355_blit_plan_t p{};
@@ -453,21 +496,35 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
   p.unroll = kBatchChunkVecs / 64;
   p.body_vecs = total_chunks;  // chunks, when known
   const mi355_blit_tuning_t* t = h->has_tuning ? &h->tuning : nullptr;
-  // Measured on MI355X with 65,536 copies of 64 B..256 KiB: bypassing the
-  // caches (nt loads, write-through stores) costs ~15 % here, unlike for one
-  // large copy; it stays selectable for sweeps.
-  bool streaming = false;
+  // Measured on MI355X with 65,536 copies of 64 B..256 KiB: non-temporal loads
+  // and stores are best (739 us against 824 us cached); written-through
+  // stores are worst (958 us), because a chunk's first and last cache line
+  // are shared with its neighbours and written through in halves.
+  bool streaming = descs_on_device || total_bytes >= (4ull << 20);
   if (t && t->nt_load) streaming = (t->nt_load == 2);
   p.nt_load = streaming;
-  p.store_policy = streaming ? MI355_BLIT_STORE_AGENT_WT : MI355_BLIT_STORE_CACHED;
+  p.store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
+  if (t && t->store_policy >= 1 && t->store_policy <= 4) p.store_policy = t->store_policy - 1;
   if (!descs_on_device) {
-    p.wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size : 512;
+    // the host knows the chunk total: one record per chunk
+    hipLaunchKernelGGL(k_batch_make_records, dim3(static_cast<uint32_t>((total_chunks + 255) / 256)),
+                       dim3(256), 0, s, dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev,
+                       h->block_sum_dev, n_blocks, total_chunks, h->records_dev);
+    p.wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size : 256;
     const uint64_t waves_per_wg = p.wg_size / 64;
-    p.grid = static_cast<uint32_t>((total_chunks + waves_per_wg - 1) / waves_per_wg);
-    auto k = streaming ? k_batch_copy_mapped<true, kStoreAgentWt> : k_batch_copy_mapped<false, kStoreCached>;
-    hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, dev_descs, h->chunk_start_dev,
-                       h->owner_dev, total_chunks);
+    unsigned split = kBatchSplit;
+    if (t && (t->unroll == 1 || t->unroll == 2 || t->unroll == 4)) split = 4 / t->unroll;
+    const uint64_t waves = total_chunks * split;
+    uint64_t wgs = (waves + waves_per_wg - 1) / waves_per_wg;
+    if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
+    p.grid = static_cast<uint32_t>(wgs);
+    p.unroll = 4 / split;
+    void (*k)(const ChunkRecord*, uint64_t) = select_batch_kernel(split, streaming, p.store_policy);
+    if (!k) return MI355_BLIT_ERROR;
+    hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, h->records_dev, total_chunks);
   } else {
+    hipLaunchKernelGGL(k_batch_finalize, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, s,
+                       static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev);
     p.wg_size = 256;
     uint32_t max_grid = h->num_cus * kWgPerCu;
     if (t && t->max_grid) max_grid = t->max_grid;
@@ -476,7 +533,8 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
     // idle waves.
     const uint64_t wgs = static_cast<uint64_t>(n) * 16;
     p.grid = static_cast<uint32_t>(wgs < max_grid ? wgs : max_grid);
-    auto k = streaming ? k_batch_copy_strided<true, kStoreAgentWt> : k_batch_copy_strided<false, kStoreCached>;
+    auto k = streaming ? k_batch_copy_strided<true, kStoreNt> : k_batch_copy_strided<false, kStoreCached>;
+    p.store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
     hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, dev_descs, static_cast<uint64_t>(n),
                        h->chunk_start_dev);
   }

@@ -279,8 +279,11 @@ __device__ __forceinline__ uint32_t block_scan_1024(uint32_t v, uint32_t* lds, u
 //     chunks of workgroup b;
 //  2. k_batch_scan_top, one workgroup: block_sum becomes its own exclusive
 //     prefix, chunk_start[n] = all chunks;
-//  3. k_batch_expand, one lane per copy: chunk_start[i] += block_sum[i / 1024]
-//     and, when owner != nullptr, owner[c] = i for every chunk c of copy i.
+//  3. either k_batch_make_records, one lane per chunk: finds the chunk's copy
+//     by bisecting block_sum and then that workgroup's chunk_start, and
+//     writes the chunk's record; or k_batch_finalize, one lane per copy:
+//     chunk_start[i] += block_sum[i / 1024], for the kernel that walks
+//     chunk_start itself.
 __global__ void __launch_bounds__(1024) k_batch_scan_local(const BatchDesc* __restrict__ descs,
                                                            uint64_t n,
                                                            uint32_t* __restrict__ chunk_start,
@@ -312,18 +315,62 @@ __global__ void __launch_bounds__(1024) k_batch_scan_top(uint32_t* __restrict__ 
   if (threadIdx.x == 0) chunk_start[n] = carry;
 }
 
-__global__ void __launch_bounds__(256) k_batch_expand(const BatchDesc* __restrict__ descs, uint64_t n,
-                                                      uint32_t* __restrict__ chunk_start,
-                                                      const uint32_t* __restrict__ block_sum,
-                                                      uint32_t* __restrict__ owner) {
+__global__ void __launch_bounds__(256) k_batch_finalize(uint64_t n, uint32_t* __restrict__ chunk_start,
+                                                        const uint32_t* __restrict__ block_sum) {
   const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const uint32_t base = chunk_start[i] + block_sum[i / 1024];
-  chunk_start[i] = base;
-  if (owner) {
-    const uint32_t cnt = desc_chunks(descs[i]);
-    for (uint32_t k = 0; k < cnt; ++k) owner[base + k] = static_cast<uint32_t>(i);
+  if (i < n) chunk_start[i] += block_sum[i / 1024];
+}
+
+// Everything a wave needs to move one chunk, so that it reads one record
+// instead of a map entry, a descriptor and two prefix sums in sequence.
+struct __attribute__((aligned(32))) ChunkRecord {
+  uint8_t* dst;        // first 16-byte vector of the chunk (16-byte aligned)
+  const uint8_t* src;  // source byte that lands on dst[0]
+  uint32_t n_vec;      // vectors in the chunk, <= kChunkVecs
+  uint16_t head;       // bytes in front of dst, first chunk of a copy only
+  uint16_t tail;       // bytes behind the last vector, last chunk only
+  uint64_t pad;
+};
+static_assert(sizeof(ChunkRecord) == 32, "one s_load_dwordx8");
+
+__global__ void __launch_bounds__(256) k_batch_make_records(const BatchDesc* __restrict__ descs,
+                                                            uint64_t n,
+                                                            const uint32_t* __restrict__ chunk_start,
+                                                            const uint32_t* __restrict__ block_sum,
+                                                            uint32_t n_blocks, uint64_t total_chunks,
+                                                            ChunkRecord* __restrict__ records) {
+  const uint64_t c = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (c >= total_chunks) return;
+  // last workgroup-of-1024 b with block_sum[b] <= c
+  uint32_t lo = 0, hi = n_blocks - 1;
+  while (lo < hi) {
+    const uint32_t mid = (lo + hi + 1) / 2;
+    if (block_sum[mid] <= c) lo = mid; else hi = mid - 1;
   }
+  const uint32_t local = static_cast<uint32_t>(c - block_sum[lo]);
+  // last copy i of that workgroup with chunk_start[i] <= local; copies
+  // without chunks share a start with their successor and lose to it
+  const uint64_t first = static_cast<uint64_t>(lo) * 1024;
+  uint64_t a = first, b = first + 1023 < n - 1 ? first + 1023 : n - 1;
+  while (a < b) {
+    const uint64_t mid = (a + b + 1) / 2;
+    if (chunk_start[mid] <= local) a = mid; else b = mid - 1;
+  }
+  const BatchDesc d = descs[a];
+  const uint32_t k = local - chunk_start[a];
+  const unsigned head = desc_head(d);
+  const uint64_t n_vec = (d.bytes - head) / 16;
+  const uint64_t v0 = static_cast<uint64_t>(k) * kChunkVecs;
+  const uint64_t left = n_vec > v0 ? n_vec - v0 : 0;
+  ChunkRecord r;
+  r.dst = d.dst + head + 16 * v0;
+  r.src = d.src + head + 16 * v0;
+  r.n_vec = left < kChunkVecs ? static_cast<uint32_t>(left) : kChunkVecs;
+  r.head = k == 0 ? static_cast<uint16_t>(head) : 0;
+  const bool last = v0 + kChunkVecs >= n_vec;
+  r.tail = last ? static_cast<uint16_t>(d.bytes - head - 16 * n_vec) : 0;
+  r.pad = 0;
+  records[c] = r;
 }
 
 // One chunk of one copy, done by one wave.
@@ -384,23 +431,76 @@ __device__ __forceinline__ void copy_desc_chunk(const BatchDesc& dsc, uint64_t k
   }
 }
 
-// One wave per chunk, chunks in global order (the shape that streams best for
-// a single large copy); owner[c] names the copy chunk c belongs to.  Needs the
-// chunk total on the host to size the grid.
-template <bool NTL, int NTS>
-__global__ void __launch_bounds__(1024) k_batch_copy_mapped(const BatchDesc* __restrict__ descs,
-                                                            const uint32_t* __restrict__ chunk_start,
-                                                            const uint32_t* __restrict__ owner,
-                                                            uint64_t total_chunks) {
+// Loads of one wave's share of a chunk, vectors [v0, v0 + 64 U) cut at n_vec:
+// up to U vectors per lane and, when the source is not dword aligned, the
+// dword behind the share's last vector.
+template <int U, bool NTL>
+__device__ __forceinline__ void record_load(const ChunkRecord& rec, unsigned v0, unsigned lane,
+                                            v4u (&x)[U], unsigned& e) {
+  const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(rec.src)) & 3;
+  const v4u_a4* s = reinterpret_cast<const v4u_a4*>(rec.src - r);
+  const unsigned end = rec.n_vec < v0 + kWave * U ? rec.n_vec : v0 + kWave * U;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const unsigned idx = v0 + lane + u * kWave;
+    if (idx < end) x[u] = ld_v4<NTL>(s + idx);
+  }
+  e = 0;
+  if (r && end > v0) e = ld_u32<NTL>(reinterpret_cast<const unsigned*>(s + end));
+}
+
+// Realign and store what record_load fetched.  With a dword-aligned source
+// the realignment is the identity (shift 0).
+template <int U, int NTS>
+__device__ __forceinline__ void record_store(const ChunkRecord& rec, unsigned v0, unsigned lane,
+                                             const v4u (&x)[U], unsigned e) {
+  const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(rec.src)) & 3;
+  v4u* d = reinterpret_cast<v4u*>(rec.dst);
+  const unsigned end = rec.n_vec < v0 + kWave * U ? rec.n_vec : v0 + kWave * U;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const unsigned idx = v0 + lane + u * kWave;
+    const unsigned nxt = x[u + 1 < U ? u + 1 : u].x;  // lane 0's copy is what lane 63 needs
+    unsigned w4 = wave_rotate_down1(lane == 0 ? nxt : x[u].x);
+    if (idx + 1 == end) w4 = e;
+    if (idx < end) st_v4<NTS>(d + idx, realign(x[u], w4, r));
+  }
+}
+
+// Head bytes in front of the chunk's first vector, tail bytes behind its last.
+__device__ __forceinline__ void record_edges(const ChunkRecord& rec, bool do_head, bool do_tail,
+                                             unsigned lane) {
+  if (do_head && lane < rec.head) {
+    (rec.dst - rec.head)[lane] = (rec.src - rec.head)[lane];
+  } else if (do_tail && lane >= 16 && lane - 16 < rec.tail) {
+    const uint64_t off = 16ull * rec.n_vec + lane - 16;
+    rec.dst[off] = rec.src[off];
+  }
+}
+
+// SPLIT waves per 4 KiB chunk, chunks in global order and waves in address
+// order within a chunk: the dispatcher then walks memory densely, the shape
+// that streams best for a single large copy.  Each wave reads its chunk's
+// record (one 32-byte scalar load) and then moves 256 / SPLIT vectors.
+template <int SPLIT, bool NTL, int NTS>
+__global__ void __launch_bounds__(1024) k_batch_copy_records(const ChunkRecord* __restrict__ records,
+                                                             uint64_t total_chunks) {
+  constexpr int U = kChunkVecs / kWave / SPLIT;
   const unsigned lane = threadIdx.x & (kWave - 1);
   const unsigned waves_per_wg = blockDim.x / kWave;
-  const uint64_t c =
+  const uint64_t wave =
       __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
-  if (c >= total_chunks) return;
-  const uint32_t i = owner[c];
-  const BatchDesc dsc = descs[i];
-  const uint64_t k = c - chunk_start[i];
-  copy_desc_chunk<NTL, NTS>(dsc, k, k + 1 == desc_chunks(dsc), lane);
+  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * waves_per_wg;
+  for (uint64_t w = wave; w < total_chunks * SPLIT; w += n_waves) {
+    const ChunkRecord rec = records[w / SPLIT];
+    const unsigned q = static_cast<unsigned>(w % SPLIT);
+    const unsigned v0 = q * (kChunkVecs / SPLIT);
+    v4u x[U];
+    unsigned e;
+    record_load<U, NTL>(rec, v0, lane, x, e);
+    record_store<U, NTS>(rec, v0, lane, x, e);
+    record_edges(rec, q == 0, q == SPLIT - 1, lane);
+  }
 }
 
 // Device-filling grid, every wave takes an equal contiguous share of all

@@ -63,7 +63,9 @@ typedef struct {
   uint32_t nt_load;     /* non-temporal loads */
   uint32_t store_policy;/* MI355_BLIT_STORE_* */
   uint32_t byte_shift;  /* (src - dst) & 3 */
-  uint32_t reserved;
+  uint32_t lead_vecs;   /* ((dst + head_bytes) & 255) / 16: tiles are anchored at
+                           256-byte boundaries of the destination, the first one
+                           starts this many vector slots below the body */
   uint64_t head_bytes;
   uint64_t body_vecs;
   uint64_t tail_bytes;

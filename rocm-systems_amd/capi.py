@@ -28,12 +28,12 @@ class Plan(C.Structure):
     _fields_ = [
         ("kernel", C.c_uint32), ("wg_size", C.c_uint32), ("grid", C.c_uint32),
         ("unroll", C.c_uint32), ("nt_load", C.c_uint32), ("store_policy", C.c_uint32),
-        ("byte_shift", C.c_uint32), ("reserved", C.c_uint32),
+        ("byte_shift", C.c_uint32), ("lead_vecs", C.c_uint32),
         ("head_bytes", C.c_uint64), ("body_vecs", C.c_uint64), ("tail_bytes", C.c_uint64),
     ]
 
     def as_dict(self):
-        return {n: getattr(self, n) for n, _ in self._fields_ if n != "reserved"}
+        return {n: getattr(self, n) for n, _ in self._fields_}
 
 
 class Tuning(C.Structure):

@@ -178,7 +178,10 @@ batch_kernel_t select_batch_kernel(unsigned split, bool ntl, unsigned policy) {
 // Which waves of the launch take the partial last tile and the edges.
 void set_tail_waves(const mi355_blit_plan_t& p, uint32_t* partial_wave, uint32_t* edge_wave) {
   const uint64_t n_waves = static_cast<uint64_t>(p.grid) * (p.wg_size / 64);
-  const uint64_t n_full = p.body_vecs / (64ull * p.unroll);
+  // full tiles, as tile_range() counts them on the device
+  const uint64_t first_full = p.lead_vecs ? 1 : 0;
+  const uint64_t end_full = (p.body_vecs + p.lead_vecs) / (64ull * p.unroll);
+  const uint64_t n_full = end_full > first_full ? end_full - first_full : 0;
   *partial_wave = static_cast<uint32_t>(n_full % n_waves);
   *edge_wave = static_cast<uint32_t>((n_full + 1) % n_waves);
 }
@@ -270,7 +273,8 @@ inline uint64_t host_desc_chunks(const mi355_blit_desc_t& d) {
   uint64_t head = (16 - (reinterpret_cast<uintptr_t>(d.dst) & 15)) & 15;
   if (head > d.bytes) head = d.bytes;
   const uint64_t n_vec = (d.bytes - head) / 16;
-  const uint64_t c = (n_vec + kBatchChunkVecs - 1) / kBatchChunkVecs;
+  const uint64_t lead = ((reinterpret_cast<uintptr_t>(d.dst) + head) & 255) / 16;
+  const uint64_t c = (n_vec + lead + kBatchChunkVecs - 1) / kBatchChunkVecs;
   return c ? c : 1;
 }
 
@@ -401,6 +405,7 @@ int mi355_blit_copy(mi355_blit_t* h, void* dst, const void* src, size_t bytes, v
   a.bytes = bytes;
   a.n_vec = p.body_vecs;
   a.head = static_cast<uint32_t>(p.head_bytes);
+  a.lead = p.lead_vecs;
   set_tail_waves(p, &a.partial_wave, &a.edge_wave);
   hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
   hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
@@ -426,6 +431,7 @@ int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwo
   a.n_dwords = num_dwords;
   a.n_vec = p.body_vecs;
   a.head = static_cast<uint32_t>(p.head_bytes / 4);
+  a.lead = p.lead_vecs;
   a.value = value;
   set_tail_waves(p, &a.partial_wave, &a.edge_wave);
   hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;

@@ -14,8 +14,10 @@
 //    ~10 % at 1 GiB.  The grid-stride loop remains for capped grids.
 //  * Large transfers bypass the caches: loads carry nt, stores are written
 //    through L2 (sc1 / sc0 sc1), chosen per size by the host.
-//  * Stores are always 16-byte aligned: the destination is aligned first and
-//    the source takes whatever alignment is left.  When source and destination
+//  * Stores are always 16-byte aligned, and tiles are anchored at 256-byte
+//    boundaries of the destination so that a wave stores whole cache lines:
+//    the destination is aligned first and the source takes whatever
+//    alignment is left.  When source and destination
 //    differ by a multiple of 4 the loads are dword-aligned dwordx4.  Otherwise
 //    each lane loads the dword-aligned 16 bytes that contain its source bytes,
 //    takes the 17th..20th byte from the next lane with a DPP wave rotate, and
@@ -45,9 +47,9 @@ struct CopyArgs {
   uint64_t bytes;
   uint64_t n_vec;  // 16-byte vectors in the body
   uint32_t head;   // bytes in front of the body, <= 15
-  // Waves that take the partial last tile and the head/tail bytes: the two
-  // after the wave of the last full tile, n_full % n_waves and
-  // (n_full + 1) % n_waves, worked out on the host.
+  uint32_t lead;   // ((dst + head) & 255) / 16: vector slots below the body in its first tile
+  // Waves that take the cut tiles at both ends and the head/tail bytes: the
+  // two after the wave of the last full tile, worked out on the host.
   uint32_t partial_wave;
   uint32_t edge_wave;
 };
@@ -57,6 +59,7 @@ struct FillArgs {
   uint64_t n_dwords;
   uint64_t n_vec;  // 16-byte vectors in the body
   uint32_t head;   // dwords in front of the body, <= 3
+  uint32_t lead;   // as in CopyArgs
   uint32_t value;
   uint32_t partial_wave;  // as in CopyArgs
   uint32_t edge_wave;
@@ -117,46 +120,92 @@ __device__ __forceinline__ v4u realign(v4u x, unsigned w4, unsigned r) {
   return o;
 }
 
-// Copies n_vec 16-byte vectors to the 16-byte aligned d.  Source vector v
-// starts r bytes after s + v, where s is dword aligned; r != 0 only when
-// SHIFT.  Called by whole waves: wave w of n_waves takes tiles w, w + n_waves,
-// ...; wave partial_wave takes the vectors after the last full tile.
+// ---------------------------------------------------------------------------
+// Tiling.  The body of a transfer is n_vec 16-byte vectors starting at a
+// 16-byte aligned destination address.  Tiles of 64*U vectors are anchored at
+// 256-byte boundaries of the DESTINATION: with lead = (address of vector 0 &
+// 255) / 16, vector v sits at virtual index v + lead and tile t covers virtual
+// indices [t*64U, (t+1)*64U).  Every wave's stores then cover whole cache lines
+// (the first and last tile excepted), whatever the destination's alignment;
+// unanchored, each wave would share its first and last line with a neighbour
+// and the memory side would see half-line writes.
+// ---------------------------------------------------------------------------
+
+struct TileRange {
+  uint64_t n_virtual;   // n_vec + lead
+  uint64_t first_full;  // first tile wholly inside [lead, n_virtual)
+  uint64_t end_full;    // one past the last such tile
+};
+
+template <int U>
+__device__ __forceinline__ TileRange tile_range(uint64_t n_vec, unsigned lead) {
+  constexpr uint64_t kTile = kWave * U;
+  TileRange t;
+  t.n_virtual = n_vec + lead;
+  t.first_full = lead ? 1 : 0;
+  t.end_full = t.n_virtual / kTile;
+  return t;
+}
+
+// Copies n_vec vectors to d (16-byte aligned).  Source vector v starts r bytes
+// after s + v, where s is dword aligned; r != 0 only when SHIFT.  Called by
+// whole waves: wave w of n_waves takes full tiles first_full + w, + n_waves,
+// ...; wave partial_wave takes the cut tiles at either end.
 template <int U, bool NTL, int NTS, bool SHIFT>
 __device__ __forceinline__ void copy_vectors(v4u* __restrict__ d, const v4u_a4* __restrict__ s,
-                                             unsigned r, uint64_t n_vec, uint64_t wave,
-                                             uint64_t n_waves, uint64_t partial_wave,
-                                             unsigned lane) {
+                                             unsigned r, uint64_t n_vec, unsigned lead,
+                                             uint64_t wave, uint64_t n_waves,
+                                             uint64_t partial_wave, unsigned lane) {
   constexpr uint64_t kTile = kWave * U;
-  const uint64_t n_full = n_vec / kTile;
-  for (uint64_t t = wave; t < n_full; t += n_waves) {
+  const TileRange tr = tile_range<U>(n_vec, lead);
+  // virtual bases: index v + lead; never dereferenced below index lead
+  v4u* dv = d - lead;
+  const v4u_a4* sv = s - lead;
+  for (uint64_t t = tr.first_full + wave; t < tr.end_full; t += n_waves) {
     const uint64_t base = t * kTile + lane;
     v4u x[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) x[u] = ld_v4<NTL>(s + base + u * kWave);
+    for (int u = 0; u < U; ++u) x[u] = ld_v4<NTL>(sv + base + u * kWave);
     if constexpr (SHIFT) {
       // Lane 0 fetches the first dword after the tile: with r != 0 it holds
       // the last r bytes the tile needs, so it is always a wanted dword.
       unsigned e = 0;
-      if (lane == 0) e = ld_u32<NTL>(reinterpret_cast<const unsigned*>(s + t * kTile + kTile));
+      if (lane == 0) e = ld_u32<NTL>(reinterpret_cast<const unsigned*>(sv + t * kTile + kTile));
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const unsigned nxt = (u + 1 < U) ? x[u + 1 < U ? u + 1 : u].x : e;
         const unsigned w4 = wave_rotate_down1(lane == 0 ? nxt : x[u].x);
-        st_v4<NTS>(d + base + u * kWave, realign(x[u], w4, r));
+        st_v4<NTS>(dv + base + u * kWave, realign(x[u], w4, r));
       }
     } else {
 #pragma unroll
-      for (int u = 0; u < U; ++u) st_v4<NTS>(d + base + u * kWave, x[u]);
+      for (int u = 0; u < U; ++u) st_v4<NTS>(dv + base + u * kWave, x[u]);
     }
   }
   if (wave == partial_wave) {
-    for (uint64_t v = n_full * kTile + lane; v < n_vec; v += kWave) {
-      v4u x = ld_v4<NTL>(s + v);
-      if constexpr (SHIFT) {
-        const unsigned w4 = ld_u32<NTL>(reinterpret_cast<const unsigned*>(s + v + 1));
-        x = realign(x, w4, r);
+    // virtual ranges of the cut tiles: [lead, end of tile 0) and
+    // [start of the last tile, n_virtual); one range when they coincide
+    uint64_t lo[2], hi[2];
+    int n_ranges = 0;
+    if (lead) {
+      lo[n_ranges] = lead;
+      hi[n_ranges] = tr.n_virtual < kTile ? tr.n_virtual : kTile;
+      ++n_ranges;
+    }
+    if (tr.n_virtual % kTile != 0 && (tr.end_full > 0 || !lead)) {
+      lo[n_ranges] = tr.end_full * kTile > lead ? tr.end_full * kTile : lead;
+      hi[n_ranges] = tr.n_virtual;
+      ++n_ranges;
+    }
+    for (int i = 0; i < n_ranges; ++i) {
+      for (uint64_t v = lo[i] + lane; v < hi[i]; v += kWave) {
+        v4u x = ld_v4<NTL>(sv + v);
+        if constexpr (SHIFT) {
+          const unsigned w4 = ld_u32<NTL>(reinterpret_cast<const unsigned*>(sv + v + 1));
+          x = realign(x, w4, r);
+        }
+        st_v4<NTS>(dv + v, x);
       }
-      st_v4<NTS>(d + v, x);
     }
   }
 }
@@ -184,8 +233,8 @@ __global__ void __launch_bounds__(1024) k_copy(CopyArgs a) {
   const uint8_t* sb = a.src + a.head;
   const unsigned r = SHIFT ? static_cast<unsigned>(reinterpret_cast<uintptr_t>(sb) & 3) : 0;
   copy_vectors<U, NTL, NTS, SHIFT>(reinterpret_cast<v4u*>(a.dst + a.head),
-                                   reinterpret_cast<const v4u_a4*>(sb - r), r, a.n_vec, wave,
-                                   n_waves, a.partial_wave, lane);
+                                   reinterpret_cast<const v4u_a4*>(sb - r), r, a.n_vec, a.lead,
+                                   wave, n_waves, a.partial_wave, lane);
   if (wave == a.edge_wave) copy_edges(a.dst, a.src, a.bytes, a.head, a.n_vec, lane);
 }
 
@@ -197,16 +246,23 @@ __global__ void __launch_bounds__(1024) k_fill(FillArgs a) {
       __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
   const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * waves_per_wg;
   const v4u val = {a.value, a.value, a.value, a.value};
-  v4u* d = reinterpret_cast<v4u*>(a.dst + a.head);
   constexpr uint64_t kTile = kWave * U;
-  const uint64_t n_full = a.n_vec / kTile;
-  for (uint64_t t = wave; t < n_full; t += n_waves) {
+  const TileRange tr = tile_range<U>(a.n_vec, a.lead);
+  v4u* dv = reinterpret_cast<v4u*>(a.dst + a.head) - a.lead;
+  for (uint64_t t = tr.first_full + wave; t < tr.end_full; t += n_waves) {
     const uint64_t base = t * kTile + lane;
 #pragma unroll
-    for (int u = 0; u < U; ++u) st_v4<NTS>(d + base + u * kWave, val);
+    for (int u = 0; u < U; ++u) st_v4<NTS>(dv + base + u * kWave, val);
   }
   if (wave == a.partial_wave) {
-    for (uint64_t v = n_full * kTile + lane; v < a.n_vec; v += kWave) st_v4<NTS>(d + v, val);
+    if (a.lead) {
+      const uint64_t hi = tr.n_virtual < kTile ? tr.n_virtual : kTile;
+      for (uint64_t v = a.lead + lane; v < hi; v += kWave) st_v4<NTS>(dv + v, val);
+    }
+    if (tr.n_virtual % kTile != 0 && (tr.end_full > 0 || !a.lead)) {
+      const uint64_t lo = tr.end_full * kTile > a.lead ? tr.end_full * kTile : a.lead;
+      for (uint64_t v = lo + lane; v < tr.n_virtual; v += kWave) st_v4<NTS>(dv + v, val);
+    }
   }
   if (wave == a.edge_wave) {
     // whole dwords outside the vector body: lanes 0..3 head, 4..7 tail
@@ -219,10 +275,11 @@ __global__ void __launch_bounds__(1024) k_fill(FillArgs a) {
 
 // ---------------------------------------------------------------------------
 // Batched small copies: n descriptors {dst, src, bytes}, one submission.
-// Each copy is cut into chunks of kChunkVecs body vectors (the first chunk
-// also moves the head bytes, the last one the tail bytes); a prefix sum over
-// the chunk counts lets every wave take an equal, contiguous share of all
-// chunks, so a 64-byte copy and a 256 KiB copy load the device evenly.
+// Each copy is cut into chunks of up to kChunkVecs body vectors, anchored at
+// 256-byte boundaries of its destination like the tiles above (the first
+// chunk also moves the head bytes, the last one the tail bytes).  A prefix sum
+// over the chunk counts orders all chunks of the batch; a chunk is the unit of
+// work, so a 64-byte copy and a 256 KiB copy load the device evenly.
 // ---------------------------------------------------------------------------
 
 struct BatchDesc {
@@ -231,17 +288,29 @@ struct BatchDesc {
   uint64_t bytes;
 };
 
-constexpr unsigned kChunkVecs = 256;  // 4 KiB: one wave, four vectors per lane
+constexpr unsigned kChunkVecs = 256;  // 4 KiB
 
-__device__ __forceinline__ unsigned desc_head(const BatchDesc& d) {
-  const unsigned h = (16 - (static_cast<unsigned>(reinterpret_cast<uintptr_t>(d.dst)) & 15)) & 15;
-  return h > d.bytes ? static_cast<unsigned>(d.bytes) : h;
+// The head / body split of one descriptor.
+struct DescShape {
+  unsigned head;    // bytes in front of the first 16-byte aligned destination address
+  unsigned lead;    // vector slots between the 256-byte boundary below and that address
+  uint64_t n_vec;   // body vectors
+};
+
+__device__ __forceinline__ DescShape desc_shape(const BatchDesc& d) {
+  DescShape sh;
+  const unsigned a = static_cast<unsigned>(reinterpret_cast<uintptr_t>(d.dst));
+  const unsigned h = (16 - (a & 15)) & 15;
+  sh.head = h > d.bytes ? static_cast<unsigned>(d.bytes) : h;
+  sh.lead = ((a + sh.head) & 255) / 16;
+  sh.n_vec = (d.bytes - sh.head) / 16;
+  return sh;
 }
 
 __device__ __forceinline__ unsigned desc_chunks(const BatchDesc& d) {
   if (d.bytes == 0) return 0;
-  const uint64_t n_vec = (d.bytes - desc_head(d)) / 16;
-  const uint64_t c = (n_vec + kChunkVecs - 1) / kChunkVecs;
+  const DescShape sh = desc_shape(d);
+  const uint64_t c = (sh.n_vec + sh.lead + kChunkVecs - 1) / kChunkVecs;
   return c ? static_cast<unsigned>(c) : 1u;
 }
 
@@ -326,12 +395,33 @@ __global__ void __launch_bounds__(256) k_batch_finalize(uint64_t n, uint32_t* __
 struct __attribute__((aligned(32))) ChunkRecord {
   uint8_t* dst;        // first 16-byte vector of the chunk (16-byte aligned)
   const uint8_t* src;  // source byte that lands on dst[0]
-  uint32_t n_vec;      // vectors in the chunk, <= kChunkVecs
+  uint32_t n_vec;      // vectors in the chunk, <= kChunkVecs - lead
   uint16_t head;       // bytes in front of dst, first chunk of a copy only
   uint16_t tail;       // bytes behind the last vector, last chunk only
-  uint64_t pad;
+  uint32_t lead;       // (dst & 255) / 16: non-zero on a copy's first chunk only
+  uint32_t pad;
 };
 static_assert(sizeof(ChunkRecord) == 32, "one s_load_dwordx8");
+
+// Chunk k of a copy.
+__device__ __forceinline__ ChunkRecord make_record(const BatchDesc& d, uint32_t k) {
+  const DescShape sh = desc_shape(d);
+  const uint64_t n_virtual = sh.n_vec + sh.lead;
+  uint64_t lo = static_cast<uint64_t>(k) * kChunkVecs;
+  uint64_t hi = lo + kChunkVecs;
+  if (lo < sh.lead) lo = sh.lead;
+  if (hi > n_virtual) hi = n_virtual;
+  if (hi < lo) hi = lo;  // a copy without body vectors still has one chunk
+  ChunkRecord r;
+  r.dst = d.dst + sh.head + 16 * (lo - sh.lead);
+  r.src = d.src + sh.head + 16 * (lo - sh.lead);
+  r.n_vec = static_cast<uint32_t>(hi - lo);
+  r.head = k == 0 ? static_cast<uint16_t>(sh.head) : 0;
+  r.tail = hi == n_virtual ? static_cast<uint16_t>(d.bytes - sh.head - 16 * sh.n_vec) : 0;
+  r.lead = k == 0 ? sh.lead : 0;
+  r.pad = 0;
+  return r;
+}
 
 __global__ void __launch_bounds__(256) k_batch_make_records(const BatchDesc* __restrict__ descs,
                                                             uint64_t n,
@@ -356,97 +446,26 @@ __global__ void __launch_bounds__(256) k_batch_make_records(const BatchDesc* __r
     const uint64_t mid = (a + b + 1) / 2;
     if (chunk_start[mid] <= local) a = mid; else b = mid - 1;
   }
-  const BatchDesc d = descs[a];
-  const uint32_t k = local - chunk_start[a];
-  const unsigned head = desc_head(d);
-  const uint64_t n_vec = (d.bytes - head) / 16;
-  const uint64_t v0 = static_cast<uint64_t>(k) * kChunkVecs;
-  const uint64_t left = n_vec > v0 ? n_vec - v0 : 0;
-  ChunkRecord r;
-  r.dst = d.dst + head + 16 * v0;
-  r.src = d.src + head + 16 * v0;
-  r.n_vec = left < kChunkVecs ? static_cast<uint32_t>(left) : kChunkVecs;
-  r.head = k == 0 ? static_cast<uint16_t>(head) : 0;
-  const bool last = v0 + kChunkVecs >= n_vec;
-  r.tail = last ? static_cast<uint16_t>(d.bytes - head - 16 * n_vec) : 0;
-  r.pad = 0;
-  records[c] = r;
+  records[c] = make_record(descs[a], local - chunk_start[a]);
 }
 
-// One chunk of one copy, done by one wave.
-template <bool NTL, int NTS, bool SHIFT>
-__device__ __forceinline__ void copy_chunk(v4u* __restrict__ d, const v4u_a4* __restrict__ s,
-                                           unsigned r, unsigned n_vec, unsigned lane) {
-  constexpr int U = kChunkVecs / kWave;
-  if (n_vec == kChunkVecs) {
-    v4u x[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) x[u] = ld_v4<NTL>(s + lane + u * kWave);
-    if constexpr (SHIFT) {
-      unsigned e = 0;
-      if (lane == 0) e = ld_u32<NTL>(reinterpret_cast<const unsigned*>(s + kChunkVecs));
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const unsigned nxt = (u + 1 < U) ? x[u + 1 < U ? u + 1 : u].x : e;
-        const unsigned w4 = wave_rotate_down1(lane == 0 ? nxt : x[u].x);
-        st_v4<NTS>(d + lane + u * kWave, realign(x[u], w4, r));
-      }
-    } else {
-#pragma unroll
-      for (int u = 0; u < U; ++u) st_v4<NTS>(d + lane + u * kWave, x[u]);
-    }
-  } else {
-    for (unsigned v = lane; v < n_vec; v += kWave) {
-      v4u x = ld_v4<NTL>(s + v);
-      if constexpr (SHIFT) {
-        const unsigned w4 = ld_u32<NTL>(reinterpret_cast<const unsigned*>(s + v + 1));
-        x = realign(x, w4, r);
-      }
-      st_v4<NTS>(d + v, x);
-    }
-  }
-}
-
-// Chunk k of one copy, with the head bytes on the first chunk and the tail
-// bytes on the last.
-template <bool NTL, int NTS>
-__device__ __forceinline__ void copy_desc_chunk(const BatchDesc& dsc, uint64_t k, bool last,
-                                                unsigned lane) {
-  const unsigned head = desc_head(dsc);
-  const uint64_t n_vec = (dsc.bytes - head) / 16;
-  const uint8_t* sb = dsc.src + head;
-  const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(sb)) & 3;
-  v4u* d = reinterpret_cast<v4u*>(dsc.dst + head);
-  const v4u_a4* s = reinterpret_cast<const v4u_a4*>(sb - r);
-  const uint64_t v0 = k * kChunkVecs;
-  const uint64_t left = n_vec > v0 ? n_vec - v0 : 0;
-  const unsigned nv = left < kChunkVecs ? static_cast<unsigned>(left) : kChunkVecs;
-  if (r) copy_chunk<NTL, NTS, true>(d + v0, s + v0, r, nv, lane);
-  else copy_chunk<NTL, NTS, false>(d + v0, s + v0, 0, nv, lane);
-  if (k == 0 && lane < head) dsc.dst[lane] = dsc.src[lane];
-  if (last) {
-    const uint64_t tail_off = head + 16 * n_vec;
-    const unsigned tail = static_cast<unsigned>(dsc.bytes - tail_off);
-    if (lane >= 16 && lane - 16 < tail) dsc.dst[tail_off + lane - 16] = dsc.src[tail_off + lane - 16];
-  }
-}
-
-// Loads of one wave's share of a chunk, vectors [v0, v0 + 64 U) cut at n_vec:
-// up to U vectors per lane and, when the source is not dword aligned, the
-// dword behind the share's last vector.
+// Loads of one wave's share of a chunk: virtual vector indices [v0, v0 + 64 U)
+// cut to [lead, lead + n_vec); up to U vectors per lane and, when the source
+// is not dword aligned, the dword behind the share's last vector.
 template <int U, bool NTL>
 __device__ __forceinline__ void record_load(const ChunkRecord& rec, unsigned v0, unsigned lane,
                                             v4u (&x)[U], unsigned& e) {
   const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(rec.src)) & 3;
-  const v4u_a4* s = reinterpret_cast<const v4u_a4*>(rec.src - r);
-  const unsigned end = rec.n_vec < v0 + kWave * U ? rec.n_vec : v0 + kWave * U;
+  const v4u_a4* sv = reinterpret_cast<const v4u_a4*>(rec.src - r) - rec.lead;
+  const unsigned all = rec.lead + rec.n_vec;
+  const unsigned end = all < v0 + kWave * U ? all : v0 + kWave * U;
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const unsigned idx = v0 + lane + u * kWave;
-    if (idx < end) x[u] = ld_v4<NTL>(s + idx);
+    if (idx >= rec.lead && idx < end) x[u] = ld_v4<NTL>(sv + idx);
   }
   e = 0;
-  if (r && end > v0) e = ld_u32<NTL>(reinterpret_cast<const unsigned*>(s + end));
+  if (r && end > v0 && end > rec.lead) e = ld_u32<NTL>(reinterpret_cast<const unsigned*>(sv + end));
 }
 
 // Realign and store what record_load fetched.  With a dword-aligned source
@@ -455,15 +474,16 @@ template <int U, int NTS>
 __device__ __forceinline__ void record_store(const ChunkRecord& rec, unsigned v0, unsigned lane,
                                              const v4u (&x)[U], unsigned e) {
   const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(rec.src)) & 3;
-  v4u* d = reinterpret_cast<v4u*>(rec.dst);
-  const unsigned end = rec.n_vec < v0 + kWave * U ? rec.n_vec : v0 + kWave * U;
+  v4u* dv = reinterpret_cast<v4u*>(rec.dst) - rec.lead;
+  const unsigned all = rec.lead + rec.n_vec;
+  const unsigned end = all < v0 + kWave * U ? all : v0 + kWave * U;
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const unsigned idx = v0 + lane + u * kWave;
     const unsigned nxt = x[u + 1 < U ? u + 1 : u].x;  // lane 0's copy is what lane 63 needs
     unsigned w4 = wave_rotate_down1(lane == 0 ? nxt : x[u].x);
     if (idx + 1 == end) w4 = e;
-    if (idx < end) st_v4<NTS>(d + idx, realign(x[u], w4, r));
+    if (idx >= rec.lead && idx < end) st_v4<NTS>(dv + idx, realign(x[u], w4, r));
   }
 }
 
@@ -510,6 +530,7 @@ template <bool NTL, int NTS>
 __global__ void __launch_bounds__(256) k_batch_copy_strided(const BatchDesc* __restrict__ descs,
                                                             uint64_t n,
                                                             const uint32_t* __restrict__ chunk_start) {
+  constexpr int U = kChunkVecs / kWave;
   const unsigned lane = threadIdx.x & (kWave - 1);
   const unsigned waves_per_wg = blockDim.x / kWave;
   const uint64_t wave =
@@ -534,7 +555,14 @@ __global__ void __launch_bounds__(256) k_batch_copy_strided(const BatchDesc* __r
     if (ce <= c) { ++i; continue; }
     const BatchDesc dsc = descs[i];
     const uint64_t stop = ce < c1 ? ce : c1;
-    for (; c < stop; ++c) copy_desc_chunk<NTL, NTS>(dsc, c - cs, c + 1 == ce, lane);
+    for (; c < stop; ++c) {
+      const ChunkRecord rec = make_record(dsc, static_cast<uint32_t>(c - cs));
+      v4u x[U];
+      unsigned e;
+      record_load<U, NTL>(rec, 0, lane, x, e);
+      record_store<U, NTS>(rec, 0, lane, x, e);
+      record_edges(rec, true, true, lane);
+    }
     ++i;
   }
 }

@@ -91,10 +91,11 @@ inline void apply_launch_shape(mi355_blit_plan_t* p, const SizeClass& cls, uint3
   }
   const uint64_t hw_max = kMaxGridWorkItems / p->wg_size;
   if (max_grid == 0 || max_grid > hw_max) max_grid = hw_max;
-  // One wave per tile of 64*unroll vectors plus one for the edges; a capped
-  // grid makes the waves stride over the tiles instead.
+  // One wave per tile of 64*unroll vectors (tiles anchored at 256-byte
+  // boundaries of the destination) plus one for the edges; a capped grid
+  // makes the waves stride over the tiles instead.
   const uint64_t tile_vecs = 64ull * p->unroll;
-  const uint64_t tiles = (p->body_vecs + tile_vecs - 1) / tile_vecs;
+  const uint64_t tiles = (p->body_vecs + p->lead_vecs + tile_vecs - 1) / tile_vecs;
   const uint64_t waves = tiles + 1;
   const uint64_t waves_per_wg = p->wg_size / 64;
   uint64_t wgs = (waves + waves_per_wg - 1) / waves_per_wg;
@@ -112,6 +113,7 @@ inline int plan_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t num_cu
   p->head_bytes = head;
   p->body_vecs = (bytes - head) / 16;
   p->tail_bytes = bytes - head - 16 * p->body_vecs;
+  p->lead_vecs = static_cast<uint32_t>(((dst + head) & 255) / 16);
   p->byte_shift = static_cast<uint32_t>((src - dst) & 3);
   p->kernel = p->byte_shift ? MI355_BLIT_KERNEL_COPY_REALIGN : MI355_BLIT_KERNEL_COPY;
   const uint64_t delta = (src - dst) & 15;
@@ -133,6 +135,7 @@ inline int plan_fill(uint64_t ptr, uint64_t num_dwords, uint32_t num_cus,
   p->head_bytes = head;
   p->body_vecs = (bytes - head) / 16;
   p->tail_bytes = bytes - head - 16 * p->body_vecs;
+  p->lead_vecs = static_cast<uint32_t>(((ptr + head) & 255) / 16);
   p->kernel = MI355_BLIT_KERNEL_FILL;
   apply_launch_shape(p, pick_class(kFillClasses, bytes), num_cus, t);
   p->nt_load = 0;

@@ -43,6 +43,7 @@ def test_abi_version_and_status_strings(capi_host):
 
 def test_struct_layouts_match_header(capi_host):
     assert C.sizeof(capi_host.Plan) == 8 * 4 + 3 * 8
+    assert capi_host.Plan.lead_vecs.offset == 28
     assert C.sizeof(capi_host.Tuning) == 32
     assert C.sizeof(capi_host.Desc) == 24
 
@@ -79,9 +80,10 @@ def _check_copy_plan(p, dst, src, n):
     assert p.wg_size % 64 == 0 and 64 <= p.wg_size <= 1024
     assert p.unroll in (1, 2, 4)
     assert p.grid >= 1 and p.grid * p.wg_size < 2 ** 31
-    # uncapped: one wave per tile plus one for the edges
-    tiles = -(-p.body_vecs // (64 * p.unroll))
-    assert p.grid * (p.wg_size // 64) >= min(tiles + 1, p.grid * (p.wg_size // 64))
+    assert p.lead_vecs == ((dst + p.head_bytes) % 256) // 16
+    # uncapped: one wave per 256-byte anchored tile plus one for the edges
+    tiles = -(-(p.body_vecs + p.lead_vecs) // (64 * p.unroll))
+    assert p.grid * (p.wg_size // 64) >= tiles + 1
 
 
 def test_plan_copy_invariants(capi_host):
@@ -98,9 +100,10 @@ def test_plan_copy_invariants(capi_host):
 
 def test_plan_copy_covers_every_tile_when_uncapped(capi_host):
     for n in (1 << 30, (1 << 32) + 5, 12345678):
-        st, p = capi_host.plan_copy(0x7f0000000000, 0x7e0000000000, n)
-        tiles = -(-p.body_vecs // (64 * p.unroll))
-        assert p.grid * (p.wg_size // 64) >= tiles + 1
+        for d_off in (0, 16, 48, 240, 251):
+            st, p = capi_host.plan_copy(0x7f0000000000 + d_off, 0x7e0000000000, n)
+            tiles = -(-(p.body_vecs + p.lead_vecs) // (64 * p.unroll))
+            assert p.grid * (p.wg_size // 64) >= tiles + 1
 
 
 def test_plan_copy_tuning_overrides(capi_host):
@@ -128,6 +131,7 @@ def test_plan_fill_invariants(capi_host):
             assert p.head_bytes <= 12 and p.tail_bytes <= 12
             if p.body_vecs:
                 assert (ptr + p.head_bytes) % 16 == 0
+            assert p.lead_vecs == ((ptr + p.head_bytes) % 256) // 16
     for off in (1, 2, 3):
         st, _ = capi_host.plan_fill(0x1000 + off, 4)
         assert st == capi_host.ERROR_INVALID_ARGUMENT

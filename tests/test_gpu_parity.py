@@ -184,6 +184,38 @@ def test_misaligned_tiny_lengths_every_pair(capi, blit, oracle, arenas):
                                      % (so, do, bad[0], (bad[0] - GUARD) // slot))
 
 
+@pytest.mark.parametrize("unroll,wg", [(0, 0), (1, 64), (2, 256), (4, 128)])
+def test_every_destination_offset_within_256_bytes(capi, fresh_tuning, oracle, arenas, unroll, wg):
+    """Tiles are anchored at 256-byte boundaries of the destination: every
+    16-byte step of (dst & 255), plus byte offsets, with lengths around one and
+    several tiles, so that the cut first and last tiles meet every shape."""
+    blit = fresh_tuning
+    src, src_host, dst = arenas
+    if unroll:
+        blit.set_tuning(unroll=unroll, wg_size=wg)
+    tile = 1024 * (unroll or 1)
+    lengths = [1, 17, 200, 255, 256, 257, tile - 16, tile, tile + 16, 2 * tile + 5, 5 * tile - 1, 33 * tile + 100]
+    for step in range(16):
+        for extra, so in ((0, 0), (0, 4), (5, 0), (11, 2)):
+            d_off = 2 * GUARD + 16 * step + extra
+            for n in lengths:
+                run_copy_case(capi, blit, oracle, src, src_host, dst, 2048 + so, d_off, n)
+                p = blit.last_plan()
+                assert p.lead_vecs == ((dst.base + d_off + p.head_bytes) % 256) // 16
+
+
+def test_fill_every_destination_offset_within_256_bytes(capi, fresh_tuning, oracle, arenas):
+    blit = fresh_tuning
+    _, _, dst = arenas
+    for unroll in (0, 2, 4):
+        if unroll:
+            blit.set_tuning(unroll=unroll, wg_size=128)
+        tile = 256 * (unroll or 1)  # dwords
+        for off in range(0, 256, 4):
+            for count in (1, 5, 63, tile - 4, tile, tile + 4, 3 * tile + 7):
+                run_fill_case(capi, blit, oracle, dst, 2 * GUARD + off, count, FILL_VALUE ^ off)
+
+
 @pytest.mark.parametrize("so,do", [(0, 0), (4, 0), (0, 8), (1, 0), (0, 2), (3, 0), (7, 13), (15, 1), (5, 5)])
 def test_misaligned_1gib_headline(capi, blit, oracle, rand, torch_cuda, so, do):
     """1 GiB per representative class of ((so-do) & 3, (so-do) & 12); every
@@ -305,8 +337,8 @@ def _make_batch(capi, rng, src, dst, n, min_len=64, max_len=256 << 10):
     """Copies carved sequentially: stride = len rounded up to 256 + 256 guard."""
     lens = np.floor(min_len * 2.0 ** (np.log2(max_len / min_len) * rng.random(n))).astype(np.int64)
     so = rng.integers(0, 16, n)
-    do = rng.integers(0, 16, n)
-    stride = ((lens + 255) // 256) * 256 + 256
+    do = rng.integers(0, 16, n) + 16 * rng.integers(0, 16, n)  # any destination offset within 256 bytes
+    stride = ((lens + 255) // 256) * 256 + 512
     offs = np.concatenate([[0], np.cumsum(stride)[:-1]]) + 256
     total = int(offs[-1] + stride[-1] + 256)
     assert total <= src.nbytes and total <= dst.nbytes, total
@@ -384,7 +416,7 @@ def test_batch_65536_copies(capi, blit, oracle, rand, torch_cuda):
     n = 65536
     rng = np.random.default_rng(0xB1170005)
     lens = np.floor(64 * 2.0 ** (12 * rng.random(n))).astype(np.int64)
-    stride = ((lens + 255) // 256) * 256 + 256
+    stride = ((lens + 255) // 256) * 256 + 512
     total = int(stride.sum() + 512)
     src_host = rand(total, 0xB1170005)
     src = Arena(torch, total, host=src_host)

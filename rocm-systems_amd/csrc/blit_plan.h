@@ -39,25 +39,26 @@ struct SizeClass {
 // equally aligned mod 16: one 1 KiB tile per single-wave workgroup is the
 // fastest shape once the transfer streams from HBM (>= 512 MiB); while the
 // 256 MiB last-level cache still absorbs part of it, 4-wave workgroups are.
-// A dword offset between the two makes every wave's 1 KiB of loads straddle a
-// cache line shared with its neighbour; 4-wave workgroups share that line
-// within one CU.  A byte offset adds one dword fetch per tile (the bytes that
+// Tiles are anchored at the destination's 256-byte boundaries, so when source
+// and destination differ mod 128 every wave's 1 KiB of loads straddles a cache
+// line shared with its neighbour; 4-wave workgroups share that line within
+// one CU instead of fetching it twice.  A byte offset adds one dword fetch per tile (the bytes that
 // spill past the last lane), which 2 KiB tiles amortise best.  Fills at one
 // wave per workgroup are bound by the dispatcher's workgroup rate and want
 // 4-wave workgroups.  Last match wins.
-constexpr SizeClass kCopyClasses[] = {      // (src - dst) % 16 == 0
+constexpr SizeClass kCopyClasses[] = {      // (src - dst) % 128 == 0
     {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
     {4ull << 20, 256, 1, 1, MI355_BLIT_STORE_AGENT_WT},
     {512ull << 20, 64, 1, 1, MI355_BLIT_STORE_AGENT_WT},
 };
-constexpr SizeClass kCopyDwordOffsetClasses[] = {  // (src - dst) % 4 == 0
+constexpr SizeClass kCopyDwordOffsetClasses[] = {  // (src - dst) % 4 == 0, not % 128
     {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
     {4ull << 20, 256, 1, 1, MI355_BLIT_STORE_AGENT_WT},
 };
 constexpr SizeClass kCopyRealignClasses[] = {  // (src - dst) % 4 != 0
     {0, 512, 1, 0, MI355_BLIT_STORE_CACHED},
     {4ull << 20, 256, 2, 1, MI355_BLIT_STORE_AGENT_WT},
-    {512ull << 20, 256, 2, 1, MI355_BLIT_STORE_NT},
+    {512ull << 20, 512, 2, 1, MI355_BLIT_STORE_NT},
 };
 constexpr SizeClass kFillClasses[] = {
     {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
@@ -116,7 +117,7 @@ inline int plan_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t num_cu
   p->lead_vecs = static_cast<uint32_t>(((dst + head) & 255) / 16);
   p->byte_shift = static_cast<uint32_t>((src - dst) & 3);
   p->kernel = p->byte_shift ? MI355_BLIT_KERNEL_COPY_REALIGN : MI355_BLIT_KERNEL_COPY;
-  const uint64_t delta = (src - dst) & 15;
+  const uint64_t delta = (src - dst) & 127;
   const SizeClass& cls = delta == 0         ? pick_class(kCopyClasses, bytes)
                          : (delta & 3) == 0 ? pick_class(kCopyDwordOffsetClasses, bytes)
                                             : pick_class(kCopyRealignClasses, bytes);

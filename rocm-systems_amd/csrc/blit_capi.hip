@@ -106,78 +106,46 @@ struct DeviceScope {
 
 typedef void (*copy_kernel_t)(CopyArgs);
 typedef void (*fill_kernel_t)(FillArgs);
+typedef void (*batch_kernel_t)(BatchCopyArgs);
 
-template <int U, bool NTL, bool SHIFT>
-copy_kernel_t copy_kernel_st(unsigned policy) {
-  switch (policy) {
-    case MI355_BLIT_STORE_CACHED: return k_copy<U, NTL, kStoreCached, SHIFT>;
-    case MI355_BLIT_STORE_NT: return k_copy<U, NTL, kStoreNt, SHIFT>;
-    case MI355_BLIT_STORE_AGENT_WT: return k_copy<U, NTL, kStoreAgentWt, SHIFT>;
-    case MI355_BLIT_STORE_SYSTEM_WT: return k_copy<U, NTL, kStoreSystemWt, SHIFT>;
-    default: return nullptr;
-  }
-}
+// One row per kernel variant, generated from the same list as the kernels.
+struct CopyVariant { unsigned unroll, nt_load, store, realign; copy_kernel_t fn; };
+struct FillVariant { unsigned unroll, store; fill_kernel_t fn; };
+struct BatchVariant { unsigned split, nt_load, store; batch_kernel_t fn; };
 
-template <bool SHIFT>
-copy_kernel_t copy_kernel_u(unsigned u, bool ntl, unsigned policy) {
-  switch (u) {
-    case 1: return ntl ? copy_kernel_st<1, true, SHIFT>(policy) : copy_kernel_st<1, false, SHIFT>(policy);
-    case 2: return ntl ? copy_kernel_st<2, true, SHIFT>(policy) : copy_kernel_st<2, false, SHIFT>(policy);
-    case 4: return ntl ? copy_kernel_st<4, true, SHIFT>(policy) : copy_kernel_st<4, false, SHIFT>(policy);
-    default: return nullptr;
-  }
-}
+#define MI355_COPY_ROW(U, L, S, R) {U, L, S, R, mi355_copy_u##U##_l##L##_s##S##_r##R},
+const CopyVariant kCopyVariants[] = {MI355_FOR_EACH_COPY_KERNEL(MI355_COPY_ROW)};
+#define MI355_FILL_ROW(U, S) {U, S, mi355_fill_u##U##_s##S},
+const FillVariant kFillVariants[] = {MI355_FOR_EACH_FILL_KERNEL(MI355_FILL_ROW)};
+#define MI355_BATCH_ROW(P, L, S) {P, L, S, mi355_batch_records_p##P##_l##L##_s##S},
+const BatchVariant kBatchVariants[] = {MI355_FOR_EACH_BATCH_RECORDS_KERNEL(MI355_BATCH_ROW)};
 
 copy_kernel_t select_copy_kernel(const mi355_blit_plan_t& p) {
-  return p.byte_shift ? copy_kernel_u<true>(p.unroll, p.nt_load, p.store_policy)
-                      : copy_kernel_u<false>(p.unroll, p.nt_load, p.store_policy);
-}
-
-template <int U>
-fill_kernel_t fill_kernel_st(unsigned policy) {
-  switch (policy) {
-    case MI355_BLIT_STORE_CACHED: return k_fill<U, kStoreCached>;
-    case MI355_BLIT_STORE_NT: return k_fill<U, kStoreNt>;
-    case MI355_BLIT_STORE_AGENT_WT: return k_fill<U, kStoreAgentWt>;
-    case MI355_BLIT_STORE_SYSTEM_WT: return k_fill<U, kStoreSystemWt>;
-    default: return nullptr;
-  }
+  for (const CopyVariant& v : kCopyVariants)
+    if (v.unroll == p.unroll && v.nt_load == p.nt_load && v.store == p.store_policy &&
+        v.realign == (p.byte_shift ? 1u : 0u))
+      return v.fn;
+  return nullptr;
 }
 
 fill_kernel_t select_fill_kernel(const mi355_blit_plan_t& p) {
-  switch (p.unroll) {
-    case 1: return fill_kernel_st<1>(p.store_policy);
-    case 2: return fill_kernel_st<2>(p.store_policy);
-    case 4: return fill_kernel_st<4>(p.store_policy);
-    default: return nullptr;
-  }
-}
-
-typedef void (*batch_kernel_t)(const ChunkRecord*, uint64_t);
-
-template <int SPLIT, bool NTL>
-batch_kernel_t batch_kernel_st(unsigned policy) {
-  switch (policy) {
-    case MI355_BLIT_STORE_CACHED: return k_batch_copy_records<SPLIT, NTL, kStoreCached>;
-    case MI355_BLIT_STORE_NT: return k_batch_copy_records<SPLIT, NTL, kStoreNt>;
-    case MI355_BLIT_STORE_AGENT_WT: return k_batch_copy_records<SPLIT, NTL, kStoreAgentWt>;
-    case MI355_BLIT_STORE_SYSTEM_WT: return k_batch_copy_records<SPLIT, NTL, kStoreSystemWt>;
-    default: return nullptr;
-  }
+  for (const FillVariant& v : kFillVariants)
+    if (v.unroll == p.unroll && v.store == p.store_policy) return v.fn;
+  return nullptr;
 }
 
 batch_kernel_t select_batch_kernel(unsigned split, bool ntl, unsigned policy) {
-  switch (split) {
-    case 1: return ntl ? batch_kernel_st<1, true>(policy) : batch_kernel_st<1, false>(policy);
-    case 2: return ntl ? batch_kernel_st<2, true>(policy) : batch_kernel_st<2, false>(policy);
-    case 4: return ntl ? batch_kernel_st<4, true>(policy) : batch_kernel_st<4, false>(policy);
-    default: return nullptr;
-  }
+  for (const BatchVariant& v : kBatchVariants)
+    if (v.split == split && v.nt_load == (ntl ? 1u : 0u) && v.store == policy) return v.fn;
+  return nullptr;
 }
 
 // Which waves of the launch take the partial last tile and the edges.
-void set_tail_waves(const mi355_blit_plan_t& p, uint32_t* partial_wave, uint32_t* edge_wave) {
+void set_tail_waves(const mi355_blit_plan_t& p, uint32_t* partial_wave, uint32_t* edge_wave,
+                    uint32_t* waves_per_wg, uint32_t* n_waves_out) {
   const uint64_t n_waves = static_cast<uint64_t>(p.grid) * (p.wg_size / 64);
+  *waves_per_wg = p.wg_size / 64;
+  *n_waves_out = static_cast<uint32_t>(n_waves);
   // full tiles, as tile_range() counts them on the device
   const uint64_t first_full = p.lead_vecs ? 1 : 0;
   const uint64_t end_full = (p.body_vecs + p.lead_vecs) / (64ull * p.unroll);
@@ -406,7 +374,7 @@ int mi355_blit_copy(mi355_blit_t* h, void* dst, const void* src, size_t bytes, v
   a.n_vec = p.body_vecs;
   a.head = static_cast<uint32_t>(p.head_bytes);
   a.lead = p.lead_vecs;
-  set_tail_waves(p, &a.partial_wave, &a.edge_wave);
+  set_tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
   hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
   hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
   BLIT_HIP(hipGetLastError());
@@ -433,7 +401,7 @@ int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwo
   a.head = static_cast<uint32_t>(p.head_bytes / 4);
   a.lead = p.lead_vecs;
   a.value = value;
-  set_tail_waves(p, &a.partial_wave, &a.edge_wave);
+  set_tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
   hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
   hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
   BLIT_HIP(hipGetLastError());
@@ -491,10 +459,10 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
   }
 
   const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
-  hipLaunchKernelGGL(k_batch_scan_local, dim3(n_blocks), dim3(1024), 0, s, dev_descs,
-                     static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev);
-  hipLaunchKernelGGL(k_batch_scan_top, dim3(1), dim3(1024), 0, s, h->block_sum_dev, n_blocks,
-                     h->chunk_start_dev, static_cast<uint64_t>(n));
+  ScanLocalArgs sl{dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
+  hipLaunchKernelGGL(mi355_batch_scan_local, dim3(n_blocks), dim3(1024), 0, s, sl);
+  ScanTopArgs st{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
+  hipLaunchKernelGGL(mi355_batch_scan_top, dim3(1), dim3(1024), 0, s, st);
   BLIT_HIP(hipGetLastError());
 
   mi355_blit_plan_t p{};
@@ -513,9 +481,10 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
   if (t && t->store_policy >= 1 && t->store_policy <= 4) p.store_policy = t->store_policy - 1;
   if (!descs_on_device) {
     // the host knows the chunk total: one record per chunk
-    hipLaunchKernelGGL(k_batch_make_records, dim3(static_cast<uint32_t>((total_chunks + 255) / 256)),
-                       dim3(256), 0, s, dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev,
-                       h->block_sum_dev, n_blocks, total_chunks, h->records_dev);
+    MakeRecordsArgs mr{dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev,
+                       total_chunks, h->records_dev, n_blocks};
+    hipLaunchKernelGGL(mi355_batch_make_records, dim3(static_cast<uint32_t>((total_chunks + 255) / 256)),
+                       dim3(256), 0, s, mr);
     p.wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size : 256;
     const uint64_t waves_per_wg = p.wg_size / 64;
     unsigned split = kBatchSplit;
@@ -525,12 +494,14 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
     if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
     p.grid = static_cast<uint32_t>(wgs);
     p.unroll = 4 / split;
-    void (*k)(const ChunkRecord*, uint64_t) = select_batch_kernel(split, streaming, p.store_policy);
+    batch_kernel_t k = select_batch_kernel(split, streaming, p.store_policy);
     if (!k) return MI355_BLIT_ERROR;
-    hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, h->records_dev, total_chunks);
+    BatchCopyArgs bc{h->records_dev, total_chunks, static_cast<uint32_t>(waves_per_wg),
+                     static_cast<uint32_t>(wgs * waves_per_wg)};
+    hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, bc);
   } else {
-    hipLaunchKernelGGL(k_batch_finalize, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, s,
-                       static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev);
+    FinalizeArgs fa{static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
+    hipLaunchKernelGGL(mi355_batch_finalize, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, s, fa);
     p.wg_size = 256;
     uint32_t max_grid = h->num_cus * kWgPerCu;
     if (t && t->max_grid) max_grid = t->max_grid;
@@ -539,10 +510,10 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
     // idle waves.
     const uint64_t wgs = static_cast<uint64_t>(n) * 16;
     p.grid = static_cast<uint32_t>(wgs < max_grid ? wgs : max_grid);
-    auto k = streaming ? k_batch_copy_strided<true, kStoreNt> : k_batch_copy_strided<false, kStoreCached>;
     p.store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
-    hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, dev_descs, static_cast<uint64_t>(n),
-                       h->chunk_start_dev);
+    BatchStridedArgs bs{dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, 4u, p.grid * 4u};
+    if (streaming) hipLaunchKernelGGL(mi355_batch_strided_l1_s1, dim3(p.grid), dim3(p.wg_size), 0, s, bs);
+    else hipLaunchKernelGGL(mi355_batch_strided_l0_s0, dim3(p.grid), dim3(p.wg_size), 0, s, bs);
   }
   BLIT_HIP(hipGetLastError());
   BLIT_HIP(hipEventRecord(h->staging_free, s));
@@ -557,8 +528,8 @@ int mi355_blit_signal_complete(mi355_blit_t* h, uint64_t hsa_signal_handle, void
   DeviceScope scope(h->device);
   if (scope.err != hipSuccess) return status_of(scope.err);
   hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
-  hipLaunchKernelGGL(k_signal_complete, dim3(1), dim3(64), 0, s,
-                     reinterpret_cast<HsaSignalAbi*>(hsa_signal_handle));
+  SignalArgs sa{reinterpret_cast<HsaSignalAbi*>(hsa_signal_handle)};
+  hipLaunchKernelGGL(mi355_signal_complete, dim3(1), dim3(64), 0, s, sa);
   BLIT_HIP(hipGetLastError());
   return MI355_BLIT_SUCCESS;
 }

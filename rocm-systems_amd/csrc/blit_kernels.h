@@ -52,6 +52,10 @@ struct CopyArgs {
   // two after the wave of the last full tile, worked out on the host.
   uint32_t partial_wave;
   uint32_t edge_wave;
+  // Launch shape, passed explicitly so that the kernels need no implicit
+  // kernel arguments and can be dispatched from a hand-built AQL packet.
+  uint32_t waves_per_wg;
+  uint32_t n_waves;  // grid * waves_per_wg
 };
 
 struct FillArgs {
@@ -63,6 +67,8 @@ struct FillArgs {
   uint32_t value;
   uint32_t partial_wave;  // as in CopyArgs
   uint32_t edge_wave;
+  uint32_t waves_per_wg;
+  uint32_t n_waves;
 };
 
 template <bool NT>
@@ -223,13 +229,16 @@ __device__ __forceinline__ void copy_edges(uint8_t* dst, const uint8_t* src, uin
   }
 }
 
+// Index of the calling wave among all waves of the launch (wave-uniform).
+__device__ __forceinline__ uint64_t global_wave(unsigned waves_per_wg) {
+  return __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
+}
+
 template <int U, bool NTL, int NTS, bool SHIFT>
-__global__ void __launch_bounds__(1024) k_copy(CopyArgs a) {
+__device__ __forceinline__ void copy_body(const CopyArgs& a) {
   const unsigned lane = threadIdx.x & (kWave - 1);
-  const unsigned waves_per_wg = blockDim.x / kWave;
-  const uint64_t wave =
-      __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
-  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * waves_per_wg;
+  const uint64_t wave = global_wave(a.waves_per_wg);
+  const uint64_t n_waves = a.n_waves;
   const uint8_t* sb = a.src + a.head;
   const unsigned r = SHIFT ? static_cast<unsigned>(reinterpret_cast<uintptr_t>(sb) & 3) : 0;
   copy_vectors<U, NTL, NTS, SHIFT>(reinterpret_cast<v4u*>(a.dst + a.head),
@@ -239,12 +248,10 @@ __global__ void __launch_bounds__(1024) k_copy(CopyArgs a) {
 }
 
 template <int U, int NTS>
-__global__ void __launch_bounds__(1024) k_fill(FillArgs a) {
+__device__ __forceinline__ void fill_body(const FillArgs& a) {
   const unsigned lane = threadIdx.x & (kWave - 1);
-  const unsigned waves_per_wg = blockDim.x / kWave;
-  const uint64_t wave =
-      __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
-  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * waves_per_wg;
+  const uint64_t wave = global_wave(a.waves_per_wg);
+  const uint64_t n_waves = a.n_waves;
   const v4u val = {a.value, a.value, a.value, a.value};
   constexpr uint64_t kTile = kWave * U;
   const TileRange tr = tile_range<U>(a.n_vec, a.lead);
@@ -353,10 +360,18 @@ __device__ __forceinline__ uint32_t block_scan_1024(uint32_t v, uint32_t* lds, u
 //     writes the chunk's record; or k_batch_finalize, one lane per copy:
 //     chunk_start[i] += block_sum[i / 1024], for the kernel that walks
 //     chunk_start itself.
-__global__ void __launch_bounds__(1024) k_batch_scan_local(const BatchDesc* __restrict__ descs,
-                                                           uint64_t n,
-                                                           uint32_t* __restrict__ chunk_start,
-                                                           uint32_t* __restrict__ block_sum) {
+struct ScanLocalArgs {
+  const BatchDesc* descs;
+  uint64_t n;
+  uint32_t* chunk_start;
+  uint32_t* block_sum;
+};
+
+__device__ __forceinline__ void scan_local_body(const ScanLocalArgs& a) {
+  const BatchDesc* __restrict__ descs = a.descs;
+  const uint64_t n = a.n;
+  uint32_t* __restrict__ chunk_start = a.chunk_start;
+  uint32_t* __restrict__ block_sum = a.block_sum;
   __shared__ uint32_t lds[16];
   const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 1024 + threadIdx.x;
   const uint32_t c = i < n ? desc_chunks(descs[i]) : 0;
@@ -366,10 +381,18 @@ __global__ void __launch_bounds__(1024) k_batch_scan_local(const BatchDesc* __re
   if (threadIdx.x == 0) block_sum[blockIdx.x] = total;
 }
 
-__global__ void __launch_bounds__(1024) k_batch_scan_top(uint32_t* __restrict__ block_sum,
-                                                         uint32_t n_blocks,
-                                                         uint32_t* __restrict__ chunk_start,
-                                                         uint64_t n) {
+struct ScanTopArgs {
+  uint32_t* block_sum;
+  uint32_t* chunk_start;
+  uint64_t n;
+  uint32_t n_blocks;
+};
+
+__device__ __forceinline__ void scan_top_body(const ScanTopArgs& a) {
+  uint32_t* __restrict__ block_sum = a.block_sum;
+  uint32_t* __restrict__ chunk_start = a.chunk_start;
+  const uint64_t n = a.n;
+  const uint32_t n_blocks = a.n_blocks;
   __shared__ uint32_t lds[16];
   uint32_t carry = 0;
   for (uint32_t base = 0; base < n_blocks; base += 1024) {
@@ -384,10 +407,16 @@ __global__ void __launch_bounds__(1024) k_batch_scan_top(uint32_t* __restrict__ 
   if (threadIdx.x == 0) chunk_start[n] = carry;
 }
 
-__global__ void __launch_bounds__(256) k_batch_finalize(uint64_t n, uint32_t* __restrict__ chunk_start,
-                                                        const uint32_t* __restrict__ block_sum) {
-  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i < n) chunk_start[i] += block_sum[i / 1024];
+struct FinalizeArgs {
+  uint64_t n;
+  uint32_t* chunk_start;
+  const uint32_t* block_sum;
+};
+
+// launched with workgroups of 256
+__device__ __forceinline__ void finalize_body(const FinalizeArgs& a) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i < a.n) a.chunk_start[i] += a.block_sum[i / 1024];
 }
 
 // Everything a wave needs to move one chunk, so that it reads one record
@@ -423,13 +452,26 @@ __device__ __forceinline__ ChunkRecord make_record(const BatchDesc& d, uint32_t 
   return r;
 }
 
-__global__ void __launch_bounds__(256) k_batch_make_records(const BatchDesc* __restrict__ descs,
-                                                            uint64_t n,
-                                                            const uint32_t* __restrict__ chunk_start,
-                                                            const uint32_t* __restrict__ block_sum,
-                                                            uint32_t n_blocks, uint64_t total_chunks,
-                                                            ChunkRecord* __restrict__ records) {
-  const uint64_t c = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+struct MakeRecordsArgs {
+  const BatchDesc* descs;
+  uint64_t n;
+  const uint32_t* chunk_start;
+  const uint32_t* block_sum;
+  uint64_t total_chunks;
+  ChunkRecord* records;
+  uint32_t n_blocks;
+};
+
+// launched with workgroups of 256, one lane per chunk
+__device__ __forceinline__ void make_records_body(const MakeRecordsArgs& args) {
+  const BatchDesc* __restrict__ descs = args.descs;
+  const uint64_t n = args.n;
+  const uint32_t* __restrict__ chunk_start = args.chunk_start;
+  const uint32_t* __restrict__ block_sum = args.block_sum;
+  const uint32_t n_blocks = args.n_blocks;
+  const uint64_t total_chunks = args.total_chunks;
+  ChunkRecord* __restrict__ records = args.records;
+  const uint64_t c = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
   if (c >= total_chunks) return;
   // last workgroup-of-1024 b with block_sum[b] <= c
   uint32_t lo = 0, hi = n_blocks - 1;
@@ -502,15 +544,21 @@ __device__ __forceinline__ void record_edges(const ChunkRecord& rec, bool do_hea
 // order within a chunk: the dispatcher then walks memory densely, the shape
 // that streams best for a single large copy.  Each wave reads its chunk's
 // record (one 32-byte scalar load) and then moves 256 / SPLIT vectors.
+struct BatchCopyArgs {
+  const ChunkRecord* records;
+  uint64_t total_chunks;
+  uint32_t waves_per_wg;
+  uint32_t n_waves;
+};
+
 template <int SPLIT, bool NTL, int NTS>
-__global__ void __launch_bounds__(1024) k_batch_copy_records(const ChunkRecord* __restrict__ records,
-                                                             uint64_t total_chunks) {
+__device__ __forceinline__ void batch_copy_records_body(const BatchCopyArgs& a) {
   constexpr int U = kChunkVecs / kWave / SPLIT;
+  const ChunkRecord* __restrict__ records = a.records;
+  const uint64_t total_chunks = a.total_chunks;
   const unsigned lane = threadIdx.x & (kWave - 1);
-  const unsigned waves_per_wg = blockDim.x / kWave;
-  const uint64_t wave =
-      __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
-  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * waves_per_wg;
+  const uint64_t wave = global_wave(a.waves_per_wg);
+  const uint64_t n_waves = a.n_waves;
   for (uint64_t w = wave; w < total_chunks * SPLIT; w += n_waves) {
     const ChunkRecord rec = records[w / SPLIT];
     const unsigned q = static_cast<unsigned>(w % SPLIT);
@@ -526,16 +574,23 @@ __global__ void __launch_bounds__(1024) k_batch_copy_records(const ChunkRecord* 
 // Device-filling grid, every wave takes an equal contiguous share of all
 // chunks and finds its first copy by bisection.  Used when the descriptors
 // are device-resident and the host cannot know the chunk total.
+struct BatchStridedArgs {
+  const BatchDesc* descs;
+  uint64_t n;
+  const uint32_t* chunk_start;
+  uint32_t waves_per_wg;
+  uint32_t n_waves;
+};
+
 template <bool NTL, int NTS>
-__global__ void __launch_bounds__(256) k_batch_copy_strided(const BatchDesc* __restrict__ descs,
-                                                            uint64_t n,
-                                                            const uint32_t* __restrict__ chunk_start) {
+__device__ __forceinline__ void batch_copy_strided_body(const BatchStridedArgs& a) {
   constexpr int U = kChunkVecs / kWave;
+  const BatchDesc* __restrict__ descs = a.descs;
+  const uint64_t n = a.n;
+  const uint32_t* __restrict__ chunk_start = a.chunk_start;
   const unsigned lane = threadIdx.x & (kWave - 1);
-  const unsigned waves_per_wg = blockDim.x / kWave;
-  const uint64_t wave =
-      __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
-  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * waves_per_wg;
+  const uint64_t wave = global_wave(a.waves_per_wg);
+  const uint64_t n_waves = a.n_waves;
   const uint64_t total = chunk_start[n];
   const uint64_t c0 = total * wave / n_waves;
   const uint64_t c1 = total * (wave + 1) / n_waves;
@@ -591,7 +646,12 @@ struct HsaSignalAbi {
 };
 static_assert(sizeof(HsaSignalAbi) == 64, "amd_signal_t is 64 bytes");
 
-__global__ void __launch_bounds__(64) k_signal_complete(HsaSignalAbi* sig) {
+struct SignalArgs {
+  HsaSignalAbi* sig;
+};
+
+__device__ __forceinline__ void signal_complete_body(const SignalArgs& a) {
+  HsaSignalAbi* sig = a.sig;
   if (threadIdx.x != 0) return;
   __hip_atomic_fetch_sub(&sig->value, static_cast<int64_t>(1), __ATOMIC_RELEASE,
                          __HIP_MEMORY_SCOPE_SYSTEM);
@@ -606,5 +666,58 @@ __global__ void __launch_bounds__(64) k_signal_complete(HsaSignalAbi* sig) {
 }
 
 }  // namespace mi355
+
+// ---------------------------------------------------------------------------
+// Kernel entry points.  C linkage and systematic names, so that the same
+// kernels can be launched through HIP (by address) and looked up by name in
+// the stand-alone code object that the AQL path loads.  Each takes one
+// plain struct: its bytes are the kernarg segment.
+//   mi355_copy_u<unroll>_l<nt loads>_s<store policy>_r<realign>
+//   mi355_fill_u<unroll>_s<store policy>
+//   mi355_batch_records_p<waves per chunk>_l<nt loads>_s<store policy>
+// ---------------------------------------------------------------------------
+#include "blit_kernel_list.h"
+
+#define MI355_DEFINE_COPY(U, L, S, R)                                                  \
+  extern "C" __global__ void __launch_bounds__(1024)                                   \
+      mi355_copy_u##U##_l##L##_s##S##_r##R(mi355::CopyArgs a) {                        \
+    mi355::copy_body<U, L != 0, S, R != 0>(a);                                         \
+  }
+MI355_FOR_EACH_COPY_KERNEL(MI355_DEFINE_COPY)
+
+#define MI355_DEFINE_FILL(U, S)                                                        \
+  extern "C" __global__ void __launch_bounds__(1024) mi355_fill_u##U##_s##S(mi355::FillArgs a) { \
+    mi355::fill_body<U, S>(a);                                                         \
+  }
+MI355_FOR_EACH_FILL_KERNEL(MI355_DEFINE_FILL)
+
+#define MI355_DEFINE_BATCH_RECORDS(P, L, S)                                            \
+  extern "C" __global__ void __launch_bounds__(1024)                                   \
+      mi355_batch_records_p##P##_l##L##_s##S(mi355::BatchCopyArgs a) {                 \
+    mi355::batch_copy_records_body<P, L != 0, S>(a);                                   \
+  }
+MI355_FOR_EACH_BATCH_RECORDS_KERNEL(MI355_DEFINE_BATCH_RECORDS)
+
+extern "C" __global__ void __launch_bounds__(256) mi355_batch_strided_l0_s0(mi355::BatchStridedArgs a) {
+  mi355::batch_copy_strided_body<false, mi355::kStoreCached>(a);
+}
+extern "C" __global__ void __launch_bounds__(256) mi355_batch_strided_l1_s1(mi355::BatchStridedArgs a) {
+  mi355::batch_copy_strided_body<true, mi355::kStoreNt>(a);
+}
+extern "C" __global__ void __launch_bounds__(1024) mi355_batch_scan_local(mi355::ScanLocalArgs a) {
+  mi355::scan_local_body(a);
+}
+extern "C" __global__ void __launch_bounds__(1024) mi355_batch_scan_top(mi355::ScanTopArgs a) {
+  mi355::scan_top_body(a);
+}
+extern "C" __global__ void __launch_bounds__(256) mi355_batch_finalize(mi355::FinalizeArgs a) {
+  mi355::finalize_body(a);
+}
+extern "C" __global__ void __launch_bounds__(256) mi355_batch_make_records(mi355::MakeRecordsArgs a) {
+  mi355::make_records_body(a);
+}
+extern "C" __global__ void __launch_bounds__(64) mi355_signal_complete(mi355::SignalArgs a) {
+  mi355::signal_complete_body(a);
+}
 
 #endif  // MI355_BLIT_KERNELS_H_

@@ -1,0 +1,91 @@
+/*
+ * mi355_blit_aql -- the gfx950 blit engine submitted the way ROCr's own
+ * BlitKernel submits: AQL packets on an HSA queue, kernels from a stand-alone
+ * code object, dependencies as BARRIER_AND packets and the caller's
+ * hsa_signal_t as the dispatch packet's completion signal.  No HIP: the
+ * library depends on libhsa-runtime64 only.
+ *
+ * Same kernels and the same dispatch sizing as mi355_blit.h; what differs is
+ * the submission half.  Citations are relative to
+ * projects/rocr-runtime/runtime/hsa-runtime/ in ROCm/rocm-systems.
+ *
+ * Signals are passed as hsa_signal_t.handle values (uint64_t), 0 meaning "no
+ * signal".  Status values are hsa_status_t values.  Every entry point may be
+ * called from any thread.
+ */
+#ifndef MI355_BLIT_AQL_H_
+#define MI355_BLIT_AQL_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "mi355_blit.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct mi355_aql mi355_aql_t;
+
+/* Replaces BlitKernel::BlitKernel + Initialize
+ * (core/runtime/amd_blit_kernel.cpp:538-591), GpuAgent::AssembleShader
+ * (core/runtime/amd_gpu_agent.cpp:251-426: here one gfx950 code object is
+ * loaded with hsa_executable_load_agent_code_object instead of wrapping raw
+ * ISA in a hand-filled amd_kernel_code_t) and the creation of the utility
+ * queue (amd_gpu_agent.cpp:692-701).  gpu_ordinal counts GPU agents in
+ * hsa_iterate_agents order.  Calls hsa_init (reference counted). */
+int mi355_aql_create(int gpu_ordinal, mi355_aql_t** out);
+
+/* Replaces BlitKernel::Destroy (amd_blit_kernel.cpp:593-612).  Blocks until
+ * every submitted packet has executed. */
+int mi355_aql_destroy(mi355_aql_t* h);
+
+/* Replaces BlitKernel::SubmitLinearCopyCommand, asynchronous overload
+ * (amd_blit_kernel.cpp:641-785): ceil(num_deps / 5) BARRIER_AND packets, then
+ * one KERNEL_DISPATCH packet whose completion_signal is `completion_signal`
+ * (decremented once by the packet processor when the copy is done).
+ * dst or src NULL -> INVALID_ARGUMENT.  bytes == 0: a barrier packet carries
+ * the dependencies and the completion signal, nothing is copied. */
+int mi355_aql_copy(mi355_aql_t* h, void* dst, const void* src, size_t bytes,
+                   const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal);
+
+/* Replaces the dispatch half of BlitKernel::SubmitLinearFillCommand
+ * (amd_blit_kernel.cpp:787-837), asynchronous like the copy.  ptr NULL or not
+ * 4-byte aligned -> INVALID_ARGUMENT. */
+int mi355_aql_fill32(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dwords,
+                     const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal);
+
+/* Batched small copies (no counterpart in the reference): n host-resident
+ * descriptors, one submission of five packets, the last one carrying the
+ * completion signal. */
+int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t n,
+                         const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal);
+
+/* Blocks until the queue has drained: the wait BlitKernel's blocking calls do
+ * on their completion signal (amd_blit_kernel.cpp:632, 830). */
+int mi355_aql_wait_idle(mi355_aql_t* h);
+
+/* Replaces BlitKernel::PendingBytes (amd_blit_kernel.cpp:943-970), with the
+ * same ledger: bytes queued before each packet index, compared with the
+ * queue's read index.  0 is exact. */
+uint64_t mi355_aql_pending_bytes(mi355_aql_t* h);
+
+/* Replaces BlitKernel::EnableProfiling (amd_blit_kernel.cpp:839-842): sets the
+ * queue's profiling bit, after which the packet processor writes start and end
+ * timestamps into each completion signal. */
+int mi355_aql_enable_profiling(mi355_aql_t* h, int enable);
+
+int mi355_aql_set_tuning(mi355_aql_t* h, const mi355_blit_tuning_t* tuning);
+int mi355_aql_last_launch_info(mi355_aql_t* h, mi355_blit_plan_t* out);
+int mi355_aql_num_cus(mi355_aql_t* h);
+
+/* Fence scope of the dispatch packets' acquire and release: 1 = system (the
+ * reference's choice, amd_blit_kernel.cpp:870-873; the default), 0 = agent,
+ * enough when no other device or the host reads the result without a later
+ * system-scope release. */
+int mi355_aql_set_system_scope_fences(mi355_aql_t* h, int enable);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_BLIT_AQL_H_ */

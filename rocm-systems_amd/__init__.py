@@ -10,4 +10,4 @@ Contents:
   build.py   compile recipe
   capi.py    ctypes binding of include/mi355_blit.h, used by tests and bench
 """
-from . import build, capi  # noqa: F401
+from . import aql, build, capi  # noqa: F401

@@ -1,0 +1,125 @@
+"""ctypes binding of include/mi355_blit_aql.h (the HSA-queue submission path).
+No CPU fallback: if the library is missing, loading raises."""
+import ctypes as C
+import os
+
+from . import build as _build
+from .capi import (Desc, Plan, Tuning, BlitError, SUCCESS, ERROR, ERROR_INVALID_ARGUMENT,  # noqa: F401
+                   ERROR_NOT_INITIALIZED, ERROR_OUT_OF_RESOURCES)
+
+_U64P = C.POINTER(C.c_uint64)
+
+SIGNATURES = {
+    "mi355_aql_create": (C.c_int, [C.c_int, C.POINTER(C.c_void_p)]),
+    "mi355_aql_destroy": (C.c_int, [C.c_void_p]),
+    "mi355_aql_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
+    "mi355_aql_fill32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
+    "mi355_aql_copy_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
+    "mi355_aql_wait_idle": (C.c_int, [C.c_void_p]),
+    "mi355_aql_pending_bytes": (C.c_uint64, [C.c_void_p]),
+    "mi355_aql_enable_profiling": (C.c_int, [C.c_void_p, C.c_int]),
+    "mi355_aql_set_tuning": (C.c_int, [C.c_void_p, C.POINTER(Tuning)]),
+    "mi355_aql_last_launch_info": (C.c_int, [C.c_void_p, C.POINTER(Plan)]),
+    "mi355_aql_num_cus": (C.c_int, [C.c_void_p]),
+    "mi355_aql_set_system_scope_fences": (C.c_int, [C.c_void_p, C.c_int]),
+}
+
+_lib = None
+
+
+def library_path():
+    return _build.AQL_LIB
+
+
+def load():
+    """dlopen lib/libmi355blit_aql.so.  In a process that also uses torch,
+    import torch first so that both share one HSA runtime."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = library_path()
+    if not os.path.exists(path):
+        raise RuntimeError("%s is missing: build it with __graft_entry__.build()" % path)
+    lib = C.CDLL(path, mode=C.RTLD_GLOBAL)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def _deps(deps):
+    if not deps:
+        return None, 0
+    arr = (C.c_uint64 * len(deps))(*deps)
+    return arr, len(deps)
+
+
+class AqlBlit:
+    """Owner of one mi355_aql_t handle; methods map 1:1 to the C ABI."""
+
+    backend = "aql"
+
+    def __init__(self, gpu=0):
+        self.lib = load()
+        h = C.c_void_p()
+        st = self.lib.mi355_aql_create(gpu, C.byref(h))
+        if st != SUCCESS:
+            raise RuntimeError("mi355_aql_create failed: 0x%x" % st)
+        self.handle = h
+
+    def close(self):
+        if self.handle:
+            st = self.lib.mi355_aql_destroy(self.handle)
+            self.handle = None
+            if st != SUCCESS:
+                raise RuntimeError("mi355_aql_destroy failed: 0x%x" % st)
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def copy(self, dst, src, nbytes, *, deps=None, completion=0):
+        arr, n = _deps(deps)
+        return self.lib.mi355_aql_copy(self.handle, dst, src, nbytes, arr, n, completion)
+
+    def fill32(self, ptr, value, num_dwords, *, deps=None, completion=0):
+        arr, n = _deps(deps)
+        return self.lib.mi355_aql_fill32(self.handle, ptr, value, num_dwords, arr, n, completion)
+
+    def copy_batch(self, descs, n, *, deps=None, completion=0):
+        arr, nd = _deps(deps)
+        addr = descs if isinstance(descs, int) or descs is None else C.cast(descs, C.c_void_p)
+        return self.lib.mi355_aql_copy_batch(self.handle, addr, n, arr, nd, completion)
+
+    def synchronize(self):
+        return self.lib.mi355_aql_wait_idle(self.handle)
+
+    def pending_bytes(self):
+        return self.lib.mi355_aql_pending_bytes(self.handle)
+
+    def last_plan(self):
+        p = Plan()
+        self.lib.mi355_aql_last_launch_info(self.handle, C.byref(p))
+        return p
+
+    def set_tuning(self, **kw):
+        if not kw:
+            return self.lib.mi355_aql_set_tuning(self.handle, None)
+        t = Tuning()
+        for k, v in kw.items():
+            setattr(t, k, v)
+        return self.lib.mi355_aql_set_tuning(self.handle, C.byref(t))
+
+    def set_system_scope_fences(self, on):
+        return self.lib.mi355_aql_set_system_scope_fences(self.handle, 1 if on else 0)
+
+    def enable_profiling(self, on):
+        return self.lib.mi355_aql_enable_profiling(self.handle, 1 if on else 0)
+
+    @property
+    def num_cus(self):
+        return self.lib.mi355_aql_num_cus(self.handle)

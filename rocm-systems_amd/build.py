@@ -12,6 +12,8 @@ INCLUDE = os.path.join(ROOT, "include")
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 
 BLIT_LIB = os.path.join(LIB_DIR, "libmi355blit.so")
+AQL_LIB = os.path.join(LIB_DIR, "libmi355blit_aql.so")
+HSACO = os.path.join(LIB_DIR, "mi355_blit_gfx950.hsaco")
 ROCR_LIB = os.path.join(LIB_DIR, "libmi355blit_rocr.so")
 ROCR_TEST = os.path.join(LIB_DIR, "test_rocr_blit")
 ORACLE_LIB = os.path.join(ORACLE_DIR, "libblit_oracle.so")
@@ -48,6 +50,23 @@ def build_blit():
         "-o", BLIT_LIB, os.path.join(CSRC, "blit_capi.hip"),
     ])
     return BLIT_LIB
+
+
+def build_aql():
+    """Stand-alone gfx950 code object + the HSA-only AQL engine ->
+    lib/mi355_blit_gfx950.hsaco, lib/libmi355blit_aql.so"""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    _run([_hipcc()] + HIPCC_FLAGS + [
+        "--cuda-device-only", "--no-gpu-bundle-output", "-I", INCLUDE, "-I", CSRC,
+        "-o", HSACO, os.path.join(CSRC, "blit_code_object.hip"),
+    ])
+    _run(["g++", "-O2", "-std=c++17", "-fPIC", "-Wall", "-shared",
+          "-I", INCLUDE, "-I", CSRC, "-I", os.path.join(ROCM, "include"),
+          "-DHSACO_PATH=\"%s\"" % HSACO,
+          "-o", AQL_LIB, os.path.join(CSRC, "aql_capi.cpp"), os.path.join(CSRC, "hsaco_embed.S"),
+          "-L", os.path.join(ROCM, "lib"), "-lhsa-runtime64", "-lpthread",
+          "-Wl,-rpath," + os.path.join(ROCM, "lib")])
+    return AQL_LIB
 
 
 def build_rocr_adapter():
@@ -88,7 +107,7 @@ def build_oracle():
 
 
 def build_all():
-    out = [build_blit()]
+    out = [build_blit(), build_aql()]
     r = build_rocr_adapter()
     if r:
         out.append(r)

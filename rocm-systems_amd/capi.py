@@ -114,6 +114,8 @@ class Blit:
     """Owner of one mi355_blit_t handle; methods map 1:1 to the C ABI and take
     raw device addresses (ints)."""
 
+    backend = "hip"
+
     def __init__(self, device=0):
         self.lib = load()
         h = C.c_void_p()

@@ -1,0 +1,739 @@
+// The gfx950 blit engine on a raw HSA queue (declarations and the reference
+// interfaces they replace: include/mi355_blit_aql.h).  This is the submission
+// half of ROCr's BlitKernel done with the same means
+// (projects/rocr-runtime/runtime/hsa-runtime/core/runtime/amd_blit_kernel.cpp:
+// 641-924): reserve packet slots with an atomic add on the write index, fill
+// the kernarg slot and the packet body, publish the header with one atomic
+// store, ring the doorbell with the index of the last packet.  Uses the public
+// HSA API only.
+#include <hsa/hsa.h>
+#include <hsa/hsa_ext_amd.h>
+#include <sched.h>
+
+#include <atomic>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "blit_args.h"
+#include "blit_kernel_list.h"
+#include "blit_plan.h"
+#include "mi355_blit_aql.h"
+
+// The gfx950 code object with every kernel variant, linked in as data.
+extern "C" const unsigned char mi355_blit_hsaco[];
+extern "C" const unsigned char mi355_blit_hsaco_end[];
+
+namespace {
+
+using namespace mi355;
+
+// Packets in the queue.  The reference shares the agent's 64-packet utility
+// queue (amd_gpu_agent.h:507-508); a batch here is five packets, so the ring
+// is a little larger.
+constexpr uint32_t kQueuePackets = 256;
+// One kernarg slot per packet slot, as in the reference (amd_blit_kernel.cpp:
+// 565-569): the slot of packet index i is i & mask, so it is free again
+// exactly when the packet slot is.
+constexpr size_t kKernargSlotBytes = 128;
+
+struct Kernel {
+  uint64_t object = 0;
+  uint32_t kernarg_size = 0;
+  uint32_t group_size = 0;
+  uint32_t private_size = 0;
+};
+
+struct CopyKernel { unsigned unroll, nt_load, store, realign; const char* name; Kernel k; };
+struct FillKernel { unsigned unroll, store; const char* name; Kernel k; };
+struct BatchKernel { unsigned split, nt_load, store; const char* name; Kernel k; };
+
+#define MI355_COPY_NAME(U, L, S, R) {U, L, S, R, "mi355_copy_u" #U "_l" #L "_s" #S "_r" #R, {}},
+#define MI355_FILL_NAME(U, S) {U, S, "mi355_fill_u" #U "_s" #S, {}},
+#define MI355_BATCH_NAME(P, L, S) {P, L, S, "mi355_batch_records_p" #P "_l" #L "_s" #S, {}},
+
+struct BytesWritten {
+  uint64_t index;
+  uint64_t bytes;
+};
+
+int to_status(hsa_status_t s) { return static_cast<int>(s); }
+
+#define AQL_HSA(expr)                                   \
+  do {                                                  \
+    hsa_status_t s_ = (expr);                           \
+    if (s_ != HSA_STATUS_SUCCESS) return to_status(s_); \
+  } while (0)
+
+}  // namespace
+
+struct mi355_aql {
+  hsa_agent_t gpu{};
+  hsa_agent_t cpu{};
+  bool have_gpu = false, have_cpu = false;
+  int wanted_ordinal = 0, seen_gpus = 0;
+  uint32_t num_cus = 0;
+
+  hsa_amd_memory_pool_t kernarg_pool{};  // host memory the packet processor reads kernargs from
+  hsa_amd_memory_pool_t host_pool{};     // fine-grained host memory (descriptor staging)
+  hsa_amd_memory_pool_t local_pool{};    // device memory
+  bool have_kernarg = false, have_host = false, have_local = false;
+
+  hsa_queue_t* queue = nullptr;
+  uint32_t queue_mask = 0;
+  uint8_t* kernargs = nullptr;
+
+  hsa_executable_t exe{};
+  hsa_code_object_reader_t reader{};
+  bool have_exe = false, have_reader = false;
+  std::vector<CopyKernel> copy_kernels{MI355_FOR_EACH_COPY_KERNEL(MI355_COPY_NAME)};
+  std::vector<FillKernel> fill_kernels{MI355_FOR_EACH_FILL_KERNEL(MI355_FILL_NAME)};
+  std::vector<BatchKernel> batch_kernels{MI355_FOR_EACH_BATCH_RECORDS_KERNEL(MI355_BATCH_NAME)};
+  Kernel scan_local, scan_top, make_records;
+
+  hsa_signal_t idle_signal{};  // completion signal of wait_idle's barrier packet
+
+  // Orders packet indices and ledger updates (reservation_lock_ of the
+  // reference, amd_blit_kernel.h:209-210).
+  std::mutex reservation_lock;
+  std::vector<BytesWritten> bytes_written;
+  uint64_t bytes_queued = 0;
+  uint64_t last_queued = 0;
+  bool anything_queued = false;
+  // Packets below this index are known to have completed (a wait_idle barrier
+  // behind them was seen to complete).  The queue's read index says the same
+  // but the packet processor publishes it with a delay.
+  std::atomic<uint64_t> known_complete{0};
+
+  std::mutex lock;  // tuning, last plan, batch buffers, wait_idle
+  mi355_blit_tuning_t tuning{};
+  bool has_tuning = false;
+  mi355_blit_plan_t last_plan{};
+  uint16_t fence_scope = HSA_FENCE_SCOPE_SYSTEM;
+  std::atomic<bool> queue_error{false};
+
+  // batched path: two host staging buffers used alternately, device buffers
+  BatchDesc* stage[2] = {nullptr, nullptr};
+  hsa_signal_t stage_free[2] = {{0}, {0}};  // 0 when the upload from stage[i] has finished
+  unsigned next_stage = 0;
+  BatchDesc* descs_dev = nullptr;
+  uint32_t* chunk_start_dev = nullptr;
+  uint32_t* block_sum_dev = nullptr;
+  ChunkRecord* records_dev = nullptr;
+  size_t batch_capacity = 0, records_capacity = 0;
+};
+
+namespace {
+
+hsa_status_t find_pools_cb(hsa_amd_memory_pool_t pool, void* data) {
+  auto* pr = static_cast<std::pair<mi355_aql*, bool>*>(data);
+  mi355_aql* h = pr->first;
+  const bool is_gpu = pr->second;
+  hsa_amd_segment_t seg;
+  if (hsa_amd_memory_pool_get_info(pool, HSA_AMD_MEMORY_POOL_INFO_SEGMENT, &seg) != HSA_STATUS_SUCCESS ||
+      seg != HSA_AMD_SEGMENT_GLOBAL)
+    return HSA_STATUS_SUCCESS;
+  bool can_alloc = false;
+  hsa_amd_memory_pool_get_info(pool, HSA_AMD_MEMORY_POOL_INFO_RUNTIME_ALLOC_ALLOWED, &can_alloc);
+  if (!can_alloc) return HSA_STATUS_SUCCESS;
+  uint32_t flags = 0;
+  hsa_amd_memory_pool_get_info(pool, HSA_AMD_MEMORY_POOL_INFO_GLOBAL_FLAGS, &flags);
+  if (is_gpu) {
+    if (!h->have_local && (flags & HSA_AMD_MEMORY_POOL_GLOBAL_FLAG_COARSE_GRAINED)) {
+      h->local_pool = pool;
+      h->have_local = true;
+    }
+  } else {
+    if (!h->have_kernarg && (flags & HSA_AMD_MEMORY_POOL_GLOBAL_FLAG_KERNARG_INIT)) {
+      h->kernarg_pool = pool;
+      h->have_kernarg = true;
+    }
+    if (!h->have_host && (flags & HSA_AMD_MEMORY_POOL_GLOBAL_FLAG_FINE_GRAINED)) {
+      h->host_pool = pool;
+      h->have_host = true;
+    }
+  }
+  return HSA_STATUS_SUCCESS;
+}
+
+hsa_status_t find_agents_cb(hsa_agent_t agent, void* data) {
+  mi355_aql* h = static_cast<mi355_aql*>(data);
+  hsa_device_type_t type;
+  if (hsa_agent_get_info(agent, HSA_AGENT_INFO_DEVICE, &type) != HSA_STATUS_SUCCESS) return HSA_STATUS_SUCCESS;
+  if (type == HSA_DEVICE_TYPE_GPU) {
+    if (h->seen_gpus++ == h->wanted_ordinal) {
+      h->gpu = agent;
+      h->have_gpu = true;
+    }
+  } else if (type == HSA_DEVICE_TYPE_CPU && !h->have_cpu) {
+    h->cpu = agent;
+    h->have_cpu = true;
+  }
+  return HSA_STATUS_SUCCESS;
+}
+
+void queue_error_cb(hsa_status_t status, hsa_queue_t*, void* data) {
+  mi355_aql* h = static_cast<mi355_aql*>(data);
+  h->queue_error.store(true);
+  const char* msg = nullptr;
+  hsa_status_string(status, &msg);
+  std::fprintf(stderr, "mi355_blit_aql: queue error 0x%x (%s)\n", status, msg ? msg : "?");
+}
+
+int lookup(mi355_aql* h, const char* name, Kernel* out) {
+  const std::string sym = std::string(name) + ".kd";
+  hsa_executable_symbol_t s;
+  AQL_HSA(hsa_executable_get_symbol_by_name(h->exe, sym.c_str(), &h->gpu, &s));
+  AQL_HSA(hsa_executable_symbol_get_info(s, HSA_EXECUTABLE_SYMBOL_INFO_KERNEL_OBJECT, &out->object));
+  AQL_HSA(hsa_executable_symbol_get_info(s, HSA_EXECUTABLE_SYMBOL_INFO_KERNEL_KERNARG_SEGMENT_SIZE,
+                                         &out->kernarg_size));
+  AQL_HSA(hsa_executable_symbol_get_info(s, HSA_EXECUTABLE_SYMBOL_INFO_KERNEL_GROUP_SEGMENT_SIZE,
+                                         &out->group_size));
+  AQL_HSA(hsa_executable_symbol_get_info(s, HSA_EXECUTABLE_SYMBOL_INFO_KERNEL_PRIVATE_SEGMENT_SIZE,
+                                         &out->private_size));
+  if (out->kernarg_size > kKernargSlotBytes || out->private_size != 0) return MI355_BLIT_ERROR;
+  return MI355_BLIT_SUCCESS;
+}
+
+// What AssembleShader does for the reference, with a real code object.
+int load_code_object(mi355_aql* h) {
+  const size_t size = static_cast<size_t>(mi355_blit_hsaco_end - mi355_blit_hsaco);
+  AQL_HSA(hsa_code_object_reader_create_from_memory(mi355_blit_hsaco, size, &h->reader));
+  h->have_reader = true;
+  AQL_HSA(hsa_executable_create_alt(HSA_PROFILE_FULL, HSA_DEFAULT_FLOAT_ROUNDING_MODE_DEFAULT, nullptr, &h->exe));
+  h->have_exe = true;
+  AQL_HSA(hsa_executable_load_agent_code_object(h->exe, h->gpu, h->reader, nullptr, nullptr));
+  AQL_HSA(hsa_executable_freeze(h->exe, nullptr));
+  int rc;
+  for (auto& k : h->copy_kernels)
+    if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
+  for (auto& k : h->fill_kernels)
+    if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
+  for (auto& k : h->batch_kernels)
+    if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
+  if ((rc = lookup(h, "mi355_batch_scan_local", &h->scan_local)) != MI355_BLIT_SUCCESS) return rc;
+  if ((rc = lookup(h, "mi355_batch_scan_top", &h->scan_top)) != MI355_BLIT_SUCCESS) return rc;
+  if ((rc = lookup(h, "mi355_batch_make_records", &h->make_records)) != MI355_BLIT_SUCCESS) return rc;
+  return MI355_BLIT_SUCCESS;
+}
+
+// amd_blit_kernel.cpp:844-854: reserve num_packet slots; yield while the ring
+// is full.
+uint64_t acquire_write_index(mi355_aql* h, uint32_t num_packet) {
+  const uint64_t index = hsa_queue_add_write_index_scacq_screl(h->queue, num_packet);
+  while (index + num_packet - hsa_queue_load_read_index_relaxed(h->queue) > h->queue->size) sched_yield();
+  return index;
+}
+
+// amd_blit_kernel.cpp:935-941
+void record_blit_history(mi355_aql* h, uint64_t size, uint64_t index) {
+  const uint64_t queued = h->bytes_queued;
+  h->bytes_queued += size;
+  h->bytes_written[index & h->queue_mask].bytes = queued;
+  h->bytes_written[index & h->queue_mask].index = index;
+  h->last_queued = index;
+  h->anything_queued = true;
+}
+
+// amd_blit_kernel.cpp:856-861: doorbell = index of the last packet written.
+void release_write_index(mi355_aql* h, uint64_t index, uint32_t num_packet) {
+  hsa_signal_store_screlease(h->queue->doorbell_signal, static_cast<hsa_signal_value_t>(index + num_packet - 1));
+}
+
+void publish(void* slot, uint16_t header, uint16_t setup) {
+  // body first, then the header in one atomic store (amd_blit_kernel.cpp:893-901)
+  std::atomic_thread_fence(std::memory_order_release);
+  __atomic_store_n(static_cast<uint32_t*>(slot), static_cast<uint32_t>(header) | (static_cast<uint32_t>(setup) << 16),
+                   __ATOMIC_RELEASE);
+}
+
+// BARRIER_AND packets for the dependencies, five signals each, fences NONE
+// (amd_blit_kernel.cpp:645-709).  `completion` goes on the last one.
+void write_barriers(mi355_aql* h, uint64_t index, const uint64_t* deps, uint32_t num_deps, uint32_t num_packets,
+                    uint64_t completion, bool barrier_bit) {
+  auto* ring = static_cast<hsa_barrier_and_packet_t*>(h->queue->base_address);
+  uint32_t d = 0;
+  for (uint32_t p = 0; p < num_packets; ++p) {
+    hsa_barrier_and_packet_t pkt;
+    std::memset(&pkt, 0, sizeof(pkt));
+    for (int k = 0; k < 5 && d < num_deps; ++k, ++d) pkt.dep_signal[k].handle = deps[d];
+    if (p + 1 == num_packets) pkt.completion_signal.handle = completion;
+    hsa_barrier_and_packet_t* slot = &ring[(index + p) & h->queue_mask];
+    std::memcpy(reinterpret_cast<uint8_t*>(slot) + 4, reinterpret_cast<uint8_t*>(&pkt) + 4, sizeof(pkt) - 4);
+    uint16_t header = (HSA_PACKET_TYPE_BARRIER_AND << HSA_PACKET_HEADER_TYPE) |
+                      (HSA_FENCE_SCOPE_NONE << HSA_PACKET_HEADER_SCACQUIRE_FENCE_SCOPE) |
+                      (HSA_FENCE_SCOPE_NONE << HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE);
+    if (barrier_bit) header |= 1 << HSA_PACKET_HEADER_BARRIER;
+    publish(slot, header, 0);
+  }
+}
+
+// One KERNEL_DISPATCH packet (amd_blit_kernel.cpp:863-924): 1-D grid, kernarg
+// slot of the same index, acquire and release fences at the configured scope.
+void write_dispatch(mi355_aql* h, uint64_t index, const Kernel& k, const void* args, size_t args_size,
+                    uint32_t grid_wgs, uint32_t wg_size, uint64_t completion, bool barrier_bit) {
+  uint8_t* karg = h->kernargs + (index & h->queue_mask) * kKernargSlotBytes;
+  std::memcpy(karg, args, args_size);
+  hsa_kernel_dispatch_packet_t pkt;
+  std::memset(&pkt, 0, sizeof(pkt));
+  pkt.workgroup_size_x = static_cast<uint16_t>(wg_size);
+  pkt.workgroup_size_y = pkt.workgroup_size_z = 1;
+  pkt.grid_size_x = grid_wgs * wg_size;
+  pkt.grid_size_y = pkt.grid_size_z = 1;
+  pkt.private_segment_size = k.private_size;
+  pkt.group_segment_size = k.group_size;
+  pkt.kernel_object = k.object;
+  pkt.kernarg_address = karg;
+  pkt.completion_signal.handle = completion;
+  auto* ring = static_cast<hsa_kernel_dispatch_packet_t*>(h->queue->base_address);
+  hsa_kernel_dispatch_packet_t* slot = &ring[index & h->queue_mask];
+  std::memcpy(reinterpret_cast<uint8_t*>(slot) + 4, reinterpret_cast<uint8_t*>(&pkt) + 4, sizeof(pkt) - 4);
+  uint16_t header = (HSA_PACKET_TYPE_KERNEL_DISPATCH << HSA_PACKET_HEADER_TYPE) |
+                    (h->fence_scope << HSA_PACKET_HEADER_SCACQUIRE_FENCE_SCOPE) |
+                    (h->fence_scope << HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE);
+  if (barrier_bit) header |= 1 << HSA_PACKET_HEADER_BARRIER;
+  publish(slot, header, 1 << HSA_KERNEL_DISPATCH_PACKET_SETUP_DIMENSIONS);
+}
+
+void tail_waves(const mi355_blit_plan_t& p, uint32_t* partial_wave, uint32_t* edge_wave, uint32_t* waves_per_wg,
+                uint32_t* n_waves_out) {
+  const uint64_t n_waves = static_cast<uint64_t>(p.grid) * (p.wg_size / 64);
+  const uint64_t first_full = p.lead_vecs ? 1 : 0;
+  const uint64_t end_full = (p.body_vecs + p.lead_vecs) / (64ull * p.unroll);
+  const uint64_t n_full = end_full > first_full ? end_full - first_full : 0;
+  *waves_per_wg = p.wg_size / 64;
+  *n_waves_out = static_cast<uint32_t>(n_waves);
+  *partial_wave = static_cast<uint32_t>(n_full % n_waves);
+  *edge_wave = static_cast<uint32_t>((n_full + 1) % n_waves);
+}
+
+uint32_t barrier_packets(uint32_t num_deps) { return (num_deps + 4) / 5; }
+
+void free_device(void* p) {
+  if (p) (void)hsa_amd_memory_pool_free(p);
+}
+
+int alloc(mi355_aql* h, hsa_amd_memory_pool_t pool, size_t bytes, void** out, bool host) {
+  AQL_HSA(hsa_amd_memory_pool_allocate(pool, bytes, 0, out));
+  if (host) {
+    hsa_status_t s = hsa_amd_agents_allow_access(1, &h->gpu, nullptr, *out);
+    if (s != HSA_STATUS_SUCCESS) {
+      (void)hsa_amd_memory_pool_free(*out);
+      *out = nullptr;
+      return to_status(s);
+    }
+  }
+  return MI355_BLIT_SUCCESS;
+}
+
+uint64_t host_desc_chunks(const mi355_blit_desc_t& d) {
+  if (d.bytes == 0) return 0;
+  uint64_t head = (16 - (reinterpret_cast<uintptr_t>(d.dst) & 15)) & 15;
+  if (head > d.bytes) head = d.bytes;
+  const uint64_t n_vec = (d.bytes - head) / 16;
+  const uint64_t lead = ((reinterpret_cast<uintptr_t>(d.dst) + head) & 255) / 16;
+  const uint64_t c = (n_vec + lead + kBatchChunkVecs - 1) / kBatchChunkVecs;
+  return c ? c : 1;
+}
+
+int wait_idle_locked(mi355_aql* h) {
+  hsa_signal_store_relaxed(h->idle_signal, 1);
+  uint64_t index;
+  {
+    std::lock_guard<std::mutex> r(h->reservation_lock);
+    index = acquire_write_index(h, 1);
+    record_blit_history(h, 0, index);
+  }
+  write_barriers(h, index, nullptr, 0, 1, h->idle_signal.handle, true);
+  release_write_index(h, index, 1);
+  while (hsa_signal_wait_scacquire(h->idle_signal, HSA_SIGNAL_CONDITION_LT, 1, UINT64_MAX, HSA_WAIT_STATE_ACTIVE) >= 1) {
+    if (h->queue_error.load()) return MI355_BLIT_ERROR;
+  }
+  // the barrier had its barrier bit set: everything up to it has completed
+  uint64_t seen = h->known_complete.load();
+  while (seen < index + 1 && !h->known_complete.compare_exchange_weak(seen, index + 1)) {
+  }
+  return h->queue_error.load() ? MI355_BLIT_ERROR : MI355_BLIT_SUCCESS;
+}
+
+int ensure_batch_capacity(mi355_aql* h, size_t n, size_t n_records) {
+  if (n <= h->batch_capacity && n_records <= h->records_capacity) return MI355_BLIT_SUCCESS;
+  // buffers may be in use by a batch in flight
+  int rc = wait_idle_locked(h);
+  if (rc != MI355_BLIT_SUCCESS) return rc;
+  if (n > h->batch_capacity) {
+    size_t cap = h->batch_capacity ? h->batch_capacity : 1024;
+    while (cap < n) cap *= 2;
+    for (int i = 0; i < 2; ++i) {
+      free_device(h->stage[i]);
+      h->stage[i] = nullptr;
+    }
+    free_device(h->descs_dev);
+    free_device(h->chunk_start_dev);
+    free_device(h->block_sum_dev);
+    h->descs_dev = nullptr;
+    h->chunk_start_dev = nullptr;
+    h->block_sum_dev = nullptr;
+    h->batch_capacity = 0;
+    for (int i = 0; i < 2; ++i) {
+      if ((rc = alloc(h, h->host_pool, cap * sizeof(BatchDesc), reinterpret_cast<void**>(&h->stage[i]), true)))
+        return rc;
+      hsa_signal_store_relaxed(h->stage_free[i], 0);
+    }
+    if ((rc = alloc(h, h->local_pool, cap * sizeof(BatchDesc), reinterpret_cast<void**>(&h->descs_dev), false))) return rc;
+    if ((rc = alloc(h, h->local_pool, (cap + 1) * sizeof(uint32_t), reinterpret_cast<void**>(&h->chunk_start_dev), false)))
+      return rc;
+    if ((rc = alloc(h, h->local_pool, (cap / 1024 + 1) * sizeof(uint32_t), reinterpret_cast<void**>(&h->block_sum_dev), false)))
+      return rc;
+    h->batch_capacity = cap;
+  }
+  if (n_records > h->records_capacity) {
+    size_t cap = h->records_capacity ? h->records_capacity : 65536;
+    while (cap < n_records) cap *= 2;
+    free_device(h->records_dev);
+    h->records_dev = nullptr;
+    h->records_capacity = 0;
+    if ((rc = alloc(h, h->local_pool, cap * sizeof(ChunkRecord), reinterpret_cast<void**>(&h->records_dev), false))) return rc;
+    h->records_capacity = cap;
+  }
+  return MI355_BLIT_SUCCESS;
+}
+
+const Kernel* find_copy(mi355_aql* h, const mi355_blit_plan_t& p) {
+  for (const auto& v : h->copy_kernels)
+    if (v.unroll == p.unroll && v.nt_load == p.nt_load && v.store == p.store_policy &&
+        v.realign == (p.byte_shift ? 1u : 0u))
+      return &v.k;
+  return nullptr;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi355_aql_create(int gpu_ordinal, mi355_aql_t** out) {
+  if (!out || gpu_ordinal < 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  *out = nullptr;
+  hsa_status_t st = hsa_init();
+  if (st != HSA_STATUS_SUCCESS) return MI355_BLIT_ERROR_NOT_INITIALIZED;
+  mi355_aql* h = new (std::nothrow) mi355_aql;
+  if (!h) {
+    hsa_shut_down();
+    return MI355_BLIT_ERROR_OUT_OF_RESOURCES;
+  }
+  h->wanted_ordinal = gpu_ordinal;
+  int rc = MI355_BLIT_SUCCESS;
+  auto fail = [&](int code) {
+    mi355_aql_destroy(h);
+    return code;
+  };
+  if (hsa_iterate_agents(find_agents_cb, h) != HSA_STATUS_SUCCESS || !h->have_cpu) return fail(MI355_BLIT_ERROR);
+  if (!h->have_gpu) return fail(MI355_BLIT_ERROR_INVALID_ARGUMENT);
+  std::pair<mi355_aql*, bool> ctx{h, false};
+  hsa_amd_agent_iterate_memory_pools(h->cpu, find_pools_cb, &ctx);
+  ctx.second = true;
+  hsa_amd_agent_iterate_memory_pools(h->gpu, find_pools_cb, &ctx);
+  if (!h->have_kernarg || !h->have_host || !h->have_local) return fail(MI355_BLIT_ERROR);
+  if (hsa_agent_get_info(h->gpu, static_cast<hsa_agent_info_t>(HSA_AMD_AGENT_INFO_COMPUTE_UNIT_COUNT), &h->num_cus) !=
+          HSA_STATUS_SUCCESS || h->num_cus == 0)
+    return fail(MI355_BLIT_ERROR);
+  if ((rc = load_code_object(h)) != MI355_BLIT_SUCCESS) return fail(rc);
+  st = hsa_queue_create(h->gpu, kQueuePackets, HSA_QUEUE_TYPE_MULTI, queue_error_cb, h, UINT32_MAX, UINT32_MAX, &h->queue);
+  if (st != HSA_STATUS_SUCCESS) return fail(to_status(st));
+  h->queue_mask = h->queue->size - 1;
+  h->bytes_written.assign(h->queue->size, BytesWritten{~0ull, ~0ull});
+  void* ka = nullptr;
+  if ((rc = alloc(h, h->kernarg_pool, h->queue->size * kKernargSlotBytes, &ka, true)) != MI355_BLIT_SUCCESS) return fail(rc);
+  h->kernargs = static_cast<uint8_t*>(ka);
+  if (hsa_signal_create(1, 0, nullptr, &h->idle_signal) != HSA_STATUS_SUCCESS) return fail(MI355_BLIT_ERROR_OUT_OF_RESOURCES);
+  for (int i = 0; i < 2; ++i)
+    if (hsa_signal_create(0, 0, nullptr, &h->stage_free[i]) != HSA_STATUS_SUCCESS) return fail(MI355_BLIT_ERROR_OUT_OF_RESOURCES);
+  *out = h;
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_aql_destroy(mi355_aql_t* h) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  int rc = MI355_BLIT_SUCCESS;
+  {
+    std::lock_guard<std::mutex> g(h->lock);
+    if (h->queue && h->idle_signal.handle && !h->queue_error.load()) rc = wait_idle_locked(h);
+    if (h->queue) hsa_queue_destroy(h->queue);
+    h->queue = nullptr;
+    free_device(h->kernargs);
+    for (int i = 0; i < 2; ++i) {
+      free_device(h->stage[i]);
+      if (h->stage_free[i].handle) hsa_signal_destroy(h->stage_free[i]);
+    }
+    free_device(h->descs_dev);
+    free_device(h->chunk_start_dev);
+    free_device(h->block_sum_dev);
+    free_device(h->records_dev);
+    if (h->idle_signal.handle) hsa_signal_destroy(h->idle_signal);
+    if (h->have_exe) hsa_executable_destroy(h->exe);
+    if (h->have_reader) hsa_code_object_reader_destroy(h->reader);
+  }
+  delete h;
+  hsa_shut_down();
+  return rc;
+}
+
+int mi355_aql_num_cus(mi355_aql_t* h) { return h ? static_cast<int>(h->num_cus) : 0; }
+
+int mi355_aql_set_tuning(mi355_aql_t* h, const mi355_blit_tuning_t* tuning) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> g(h->lock);
+  h->has_tuning = tuning != nullptr;
+  if (tuning) h->tuning = *tuning;
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_aql_last_launch_info(mi355_aql_t* h, mi355_blit_plan_t* out) {
+  if (!h || !out) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> g(h->lock);
+  *out = h->last_plan;
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_aql_set_system_scope_fences(mi355_aql_t* h, int enable) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> g(h->lock);
+  h->fence_scope = enable ? HSA_FENCE_SCOPE_SYSTEM : HSA_FENCE_SCOPE_AGENT;
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_aql_enable_profiling(mi355_aql_t* h, int enable) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  AQL_HSA(hsa_amd_profiling_set_profiler_enabled(h->queue, enable ? 1 : 0));
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_aql_copy(mi355_aql_t* h, void* dst, const void* src, size_t bytes, const uint64_t* dep_signals,
+                   uint32_t num_deps, uint64_t completion_signal) {
+  if (!h || !dst || !src || (num_deps && !dep_signals)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (h->queue_error.load()) return MI355_BLIT_ERROR;
+  mi355_blit_plan_t p;
+  const Kernel* k = nullptr;
+  CopyArgs a{};
+  {
+    std::lock_guard<std::mutex> g(h->lock);
+    if (bytes) {
+      int rc = plan_copy(reinterpret_cast<uint64_t>(dst), reinterpret_cast<uint64_t>(src), bytes, h->num_cus,
+                         h->has_tuning ? &h->tuning : nullptr, &p);
+      if (rc != MI355_BLIT_SUCCESS) return rc;
+      k = find_copy(h, p);
+      if (!k) return MI355_BLIT_ERROR;
+      h->last_plan = p;
+    }
+  }
+  const uint32_t nb = barrier_packets(num_deps);
+  if (bytes == 0) {
+    // nothing to move: the dependencies and the completion ride on barriers
+    const uint32_t n = nb ? nb : 1;
+    if (!num_deps && !completion_signal) return MI355_BLIT_SUCCESS;
+    uint64_t index;
+    {
+      std::lock_guard<std::mutex> r(h->reservation_lock);
+      index = acquire_write_index(h, n);
+      record_blit_history(h, 0, index + n - 1);
+    }
+    write_barriers(h, index, dep_signals, num_deps, n, completion_signal, false);
+    release_write_index(h, index, n);
+    return MI355_BLIT_SUCCESS;
+  }
+  a.dst = static_cast<uint8_t*>(dst);
+  a.src = static_cast<const uint8_t*>(src);
+  a.bytes = bytes;
+  a.n_vec = p.body_vecs;
+  a.head = static_cast<uint32_t>(p.head_bytes);
+  a.lead = p.lead_vecs;
+  tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
+  const uint32_t total = nb + 1;
+  uint64_t index;
+  {
+    std::lock_guard<std::mutex> r(h->reservation_lock);
+    index = acquire_write_index(h, total);
+    record_blit_history(h, bytes, index + total - 1);
+  }
+  write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
+  // Barrier bit clear, as in the reference: consecutive blits may overlap
+  // unless linked by signals.  After dependency barriers the bit is set so
+  // that the copy cannot start before them.
+  write_dispatch(h, index + nb, *k, &a, sizeof(a), p.grid, p.wg_size, completion_signal, nb != 0);
+  release_write_index(h, index, total);
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_aql_fill32(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dwords, const uint64_t* dep_signals,
+                     uint32_t num_deps, uint64_t completion_signal) {
+  if (!h || !ptr || (reinterpret_cast<uintptr_t>(ptr) & 3) || (num_deps && !dep_signals))
+    return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (h->queue_error.load()) return MI355_BLIT_ERROR;
+  if (num_dwords == 0) {
+    // same as a zero-size copy: only the signals matter
+    return mi355_aql_copy(h, ptr, ptr, 0, dep_signals, num_deps, completion_signal);
+  }
+  mi355_blit_plan_t p;
+  const Kernel* k = nullptr;
+  {
+    std::lock_guard<std::mutex> g(h->lock);
+    int rc = plan_fill(reinterpret_cast<uint64_t>(ptr), num_dwords, h->num_cus, h->has_tuning ? &h->tuning : nullptr, &p);
+    if (rc != MI355_BLIT_SUCCESS) return rc;
+    for (const auto& v : h->fill_kernels)
+      if (v.unroll == p.unroll && v.store == p.store_policy) k = &v.k;
+    if (!k) return MI355_BLIT_ERROR;
+    h->last_plan = p;
+  }
+  FillArgs a{};
+  a.dst = static_cast<uint32_t*>(ptr);
+  a.n_dwords = num_dwords;
+  a.n_vec = p.body_vecs;
+  a.head = static_cast<uint32_t>(p.head_bytes / 4);
+  a.lead = p.lead_vecs;
+  a.value = value;
+  tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
+  const uint32_t nb = barrier_packets(num_deps);
+  const uint32_t total = nb + 1;
+  uint64_t index;
+  {
+    std::lock_guard<std::mutex> r(h->reservation_lock);
+    index = acquire_write_index(h, total);
+    record_blit_history(h, num_dwords * 4, index + total - 1);
+  }
+  write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
+  write_dispatch(h, index + nb, *k, &a, sizeof(a), p.grid, p.wg_size, completion_signal, nb != 0);
+  release_write_index(h, index, total);
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t n, const uint64_t* dep_signals,
+                         uint32_t num_deps, uint64_t completion_signal) {
+  if (!h || (!descs && n) || (num_deps && !dep_signals)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (n > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (h->queue_error.load()) return MI355_BLIT_ERROR;
+  uint64_t total_bytes = 0, total_chunks = 0;
+  for (size_t i = 0; i < n; ++i) {
+    if (descs[i].bytes && (!descs[i].dst || !descs[i].src)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+    total_bytes += descs[i].bytes;
+    total_chunks += host_desc_chunks(descs[i]);
+  }
+  if (total_chunks > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (total_chunks == 0) return mi355_aql_copy(h, h, h, 0, dep_signals, num_deps, completion_signal);
+
+  std::lock_guard<std::mutex> g(h->lock);
+  int rc = ensure_batch_capacity(h, n, total_chunks);
+  if (rc != MI355_BLIT_SUCCESS) return rc;
+  const mi355_blit_tuning_t* t = h->has_tuning ? &h->tuning : nullptr;
+
+  // stage the descriptors in host memory the GPU can read; the buffer is
+  // free again when the upload that read it last has finished
+  const unsigned b = h->next_stage;
+  h->next_stage ^= 1;
+  while (hsa_signal_wait_scacquire(h->stage_free[b], HSA_SIGNAL_CONDITION_LT, 1, UINT64_MAX, HSA_WAIT_STATE_ACTIVE) >= 1) {
+    if (h->queue_error.load()) return MI355_BLIT_ERROR;
+  }
+  std::memcpy(h->stage[b], descs, n * sizeof(BatchDesc));
+  hsa_signal_store_relaxed(h->stage_free[b], 1);
+
+  // 1. upload: our own copy kernel pulls the descriptors into device memory
+  mi355_blit_plan_t up;
+  rc = plan_copy(reinterpret_cast<uint64_t>(h->descs_dev), reinterpret_cast<uint64_t>(h->stage[b]), n * sizeof(BatchDesc),
+                 h->num_cus, nullptr, &up);
+  if (rc != MI355_BLIT_SUCCESS) return rc;
+  const Kernel* up_k = find_copy(h, up);
+  if (!up_k) return MI355_BLIT_ERROR;
+  CopyArgs ua{};
+  ua.dst = reinterpret_cast<uint8_t*>(h->descs_dev);
+  ua.src = reinterpret_cast<const uint8_t*>(h->stage[b]);
+  ua.bytes = n * sizeof(BatchDesc);
+  ua.n_vec = up.body_vecs;
+  ua.head = static_cast<uint32_t>(up.head_bytes);
+  ua.lead = up.lead_vecs;
+  tail_waves(up, &ua.partial_wave, &ua.edge_wave, &ua.waves_per_wg, &ua.n_waves);
+
+  // 2..4. prefix sum and records
+  const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
+  ScanLocalArgs sl{h->descs_dev, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
+  ScanTopArgs stp{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
+  MakeRecordsArgs mr{h->descs_dev, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev, total_chunks,
+                     h->records_dev, n_blocks};
+
+  // 5. the copy
+  mi355_blit_plan_t p{};
+  p.kernel = MI355_BLIT_KERNEL_COPY_BATCH;
+  p.body_vecs = total_chunks;
+  bool streaming = total_bytes >= (4ull << 20);
+  if (t && t->nt_load) streaming = (t->nt_load == 2);
+  p.nt_load = streaming;
+  p.store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
+  if (t && t->store_policy >= 1 && t->store_policy <= 4) p.store_policy = t->store_policy - 1;
+  p.wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size : 256;
+  unsigned split = 4;
+  if (t && (t->unroll == 1 || t->unroll == 2 || t->unroll == 4)) split = 4 / t->unroll;
+  p.unroll = 4 / split;
+  const uint64_t waves_per_wg = p.wg_size / 64;
+  uint64_t wgs = (total_chunks * split + waves_per_wg - 1) / waves_per_wg;
+  if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
+  if (wgs * p.wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / p.wg_size;
+  p.grid = static_cast<uint32_t>(wgs);
+  const Kernel* bk = nullptr;
+  for (const auto& v : h->batch_kernels)
+    if (v.split == split && v.nt_load == (streaming ? 1u : 0u) && v.store == p.store_policy) bk = &v.k;
+  if (!bk) return MI355_BLIT_ERROR;
+  BatchCopyArgs bc{h->records_dev, total_chunks, static_cast<uint32_t>(waves_per_wg),
+                   static_cast<uint32_t>(wgs * waves_per_wg)};
+  h->last_plan = p;
+
+  const uint32_t nb = barrier_packets(num_deps);
+  const uint32_t total = nb + 5;
+  uint64_t index;
+  {
+    std::lock_guard<std::mutex> r(h->reservation_lock);
+    index = acquire_write_index(h, total);
+    record_blit_history(h, total_bytes, index + total - 1);
+  }
+  write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
+  uint64_t i = index + nb;
+  // every packet of the sequence waits for the one before (barrier bit); the
+  // first also waits for whatever still uses the shared device buffers
+  write_dispatch(h, i++, *up_k, &ua, sizeof(ua), up.grid, up.wg_size, h->stage_free[b].handle, true);
+  write_dispatch(h, i++, h->scan_local, &sl, sizeof(sl), n_blocks, 1024, 0, true);
+  write_dispatch(h, i++, h->scan_top, &stp, sizeof(stp), 1, 1024, 0, true);
+  write_dispatch(h, i++, h->make_records, &mr, sizeof(mr), static_cast<uint32_t>((total_chunks + 255) / 256), 256, 0, true);
+  write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true);
+  release_write_index(h, index, total);
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_aql_wait_idle(mi355_aql_t* h) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> g(h->lock);
+  return wait_idle_locked(h);
+}
+
+// amd_blit_kernel.cpp:943-970
+uint64_t mi355_aql_pending_bytes(mi355_aql_t* h) {
+  if (!h) return 0;
+  std::lock_guard<std::mutex> r(h->reservation_lock);
+  if (!h->anything_queued) return 0;
+  uint64_t read = hsa_queue_load_read_index_relaxed(h->queue);
+  const uint64_t known = h->known_complete.load();
+  if (known > read) read = known;
+  const uint64_t last = h->last_queued;
+  // If the last blit command has been run then the blit is empty.
+  if (read > last) return 0;
+  for (uint64_t index = read; index <= last; ++index) {
+    const BytesWritten& rec = h->bytes_written[index & h->queue_mask];
+    // a record that was not overwritten by a later lap of the ring
+    if (rec.index == index) {
+      const uint64_t pending = h->bytes_queued - rec.bytes;
+      return pending ? pending : 1;  // commands without bytes still count as work
+    }
+  }
+  return 1;
+}
+
+}  // extern "C"

@@ -32,6 +32,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "blit_args.h"
+
 namespace mi355 {
 
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
@@ -39,37 +41,6 @@ typedef unsigned v4u __attribute__((ext_vector_type(4)));
 // global_load_dwordx4, which the memory pipeline accepts at any dword address.
 typedef v4u v4u_a4 __attribute__((aligned(4)));
 
-constexpr unsigned kWave = 64;
-
-struct CopyArgs {
-  uint8_t* dst;
-  const uint8_t* src;
-  uint64_t bytes;
-  uint64_t n_vec;  // 16-byte vectors in the body
-  uint32_t head;   // bytes in front of the body, <= 15
-  uint32_t lead;   // ((dst + head) & 255) / 16: vector slots below the body in its first tile
-  // Waves that take the cut tiles at both ends and the head/tail bytes: the
-  // two after the wave of the last full tile, worked out on the host.
-  uint32_t partial_wave;
-  uint32_t edge_wave;
-  // Launch shape, passed explicitly so that the kernels need no implicit
-  // kernel arguments and can be dispatched from a hand-built AQL packet.
-  uint32_t waves_per_wg;
-  uint32_t n_waves;  // grid * waves_per_wg
-};
-
-struct FillArgs {
-  uint32_t* dst;
-  uint64_t n_dwords;
-  uint64_t n_vec;  // 16-byte vectors in the body
-  uint32_t head;   // dwords in front of the body, <= 3
-  uint32_t lead;   // as in CopyArgs
-  uint32_t value;
-  uint32_t partial_wave;  // as in CopyArgs
-  uint32_t edge_wave;
-  uint32_t waves_per_wg;
-  uint32_t n_waves;
-};
 
 template <bool NT>
 __device__ __forceinline__ v4u ld_v4(const v4u_a4* p) {
@@ -289,13 +260,6 @@ __device__ __forceinline__ void fill_body(const FillArgs& a) {
 // work, so a 64-byte copy and a 256 KiB copy load the device evenly.
 // ---------------------------------------------------------------------------
 
-struct BatchDesc {
-  uint8_t* dst;
-  const uint8_t* src;
-  uint64_t bytes;
-};
-
-constexpr unsigned kChunkVecs = 256;  // 4 KiB
 
 // The head / body split of one descriptor.
 struct DescShape {
@@ -360,13 +324,6 @@ __device__ __forceinline__ uint32_t block_scan_1024(uint32_t v, uint32_t* lds, u
 //     writes the chunk's record; or k_batch_finalize, one lane per copy:
 //     chunk_start[i] += block_sum[i / 1024], for the kernel that walks
 //     chunk_start itself.
-struct ScanLocalArgs {
-  const BatchDesc* descs;
-  uint64_t n;
-  uint32_t* chunk_start;
-  uint32_t* block_sum;
-};
-
 __device__ __forceinline__ void scan_local_body(const ScanLocalArgs& a) {
   const BatchDesc* __restrict__ descs = a.descs;
   const uint64_t n = a.n;
@@ -380,13 +337,6 @@ __device__ __forceinline__ void scan_local_body(const ScanLocalArgs& a) {
   if (i < n) chunk_start[i] = excl;
   if (threadIdx.x == 0) block_sum[blockIdx.x] = total;
 }
-
-struct ScanTopArgs {
-  uint32_t* block_sum;
-  uint32_t* chunk_start;
-  uint64_t n;
-  uint32_t n_blocks;
-};
 
 __device__ __forceinline__ void scan_top_body(const ScanTopArgs& a) {
   uint32_t* __restrict__ block_sum = a.block_sum;
@@ -407,30 +357,11 @@ __device__ __forceinline__ void scan_top_body(const ScanTopArgs& a) {
   if (threadIdx.x == 0) chunk_start[n] = carry;
 }
 
-struct FinalizeArgs {
-  uint64_t n;
-  uint32_t* chunk_start;
-  const uint32_t* block_sum;
-};
-
 // launched with workgroups of 256
 __device__ __forceinline__ void finalize_body(const FinalizeArgs& a) {
   const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
   if (i < a.n) a.chunk_start[i] += a.block_sum[i / 1024];
 }
-
-// Everything a wave needs to move one chunk, so that it reads one record
-// instead of a map entry, a descriptor and two prefix sums in sequence.
-struct __attribute__((aligned(32))) ChunkRecord {
-  uint8_t* dst;        // first 16-byte vector of the chunk (16-byte aligned)
-  const uint8_t* src;  // source byte that lands on dst[0]
-  uint32_t n_vec;      // vectors in the chunk, <= kChunkVecs - lead
-  uint16_t head;       // bytes in front of dst, first chunk of a copy only
-  uint16_t tail;       // bytes behind the last vector, last chunk only
-  uint32_t lead;       // (dst & 255) / 16: non-zero on a copy's first chunk only
-  uint32_t pad;
-};
-static_assert(sizeof(ChunkRecord) == 32, "one s_load_dwordx8");
 
 // Chunk k of a copy.
 __device__ __forceinline__ ChunkRecord make_record(const BatchDesc& d, uint32_t k) {
@@ -451,16 +382,6 @@ __device__ __forceinline__ ChunkRecord make_record(const BatchDesc& d, uint32_t 
   r.pad = 0;
   return r;
 }
-
-struct MakeRecordsArgs {
-  const BatchDesc* descs;
-  uint64_t n;
-  const uint32_t* chunk_start;
-  const uint32_t* block_sum;
-  uint64_t total_chunks;
-  ChunkRecord* records;
-  uint32_t n_blocks;
-};
 
 // launched with workgroups of 256, one lane per chunk
 __device__ __forceinline__ void make_records_body(const MakeRecordsArgs& args) {
@@ -544,13 +465,6 @@ __device__ __forceinline__ void record_edges(const ChunkRecord& rec, bool do_hea
 // order within a chunk: the dispatcher then walks memory densely, the shape
 // that streams best for a single large copy.  Each wave reads its chunk's
 // record (one 32-byte scalar load) and then moves 256 / SPLIT vectors.
-struct BatchCopyArgs {
-  const ChunkRecord* records;
-  uint64_t total_chunks;
-  uint32_t waves_per_wg;
-  uint32_t n_waves;
-};
-
 template <int SPLIT, bool NTL, int NTS>
 __device__ __forceinline__ void batch_copy_records_body(const BatchCopyArgs& a) {
   constexpr int U = kChunkVecs / kWave / SPLIT;
@@ -574,14 +488,6 @@ __device__ __forceinline__ void batch_copy_records_body(const BatchCopyArgs& a) 
 // Device-filling grid, every wave takes an equal contiguous share of all
 // chunks and finds its first copy by bisection.  Used when the descriptors
 // are device-resident and the host cannot know the chunk total.
-struct BatchStridedArgs {
-  const BatchDesc* descs;
-  uint64_t n;
-  const uint32_t* chunk_start;
-  uint32_t waves_per_wg;
-  uint32_t n_waves;
-};
-
 template <bool NTL, int NTS>
 __device__ __forceinline__ void batch_copy_strided_body(const BatchStridedArgs& a) {
   constexpr int U = kChunkVecs / kWave;
@@ -631,24 +537,6 @@ __device__ __forceinline__ void batch_copy_strided_body(const BatchStridedArgs& 
 // value and, when the signal has an event mailbox, post the event id there
 // and raise the interrupt that wakes waiters sleeping in the kernel driver.
 // ---------------------------------------------------------------------------
-
-// Layout of amd_signal_t (inc/amd_hsa_signal.h, struct amd_signal_s).
-struct HsaSignalAbi {
-  int64_t kind;
-  int64_t value;
-  uint64_t event_mailbox_ptr;
-  uint32_t event_id;
-  uint32_t reserved1;
-  uint64_t start_ts;
-  uint64_t end_ts;
-  uint64_t queue_ptr;
-  uint32_t reserved3[2];
-};
-static_assert(sizeof(HsaSignalAbi) == 64, "amd_signal_t is 64 bytes");
-
-struct SignalArgs {
-  HsaSignalAbi* sig;
-};
 
 __device__ __forceinline__ void signal_complete_body(const SignalArgs& a) {
   HsaSignalAbi* sig = a.sig;

@@ -112,9 +112,16 @@ def capi(pkg, torch_cuda):
     return pkg.capi
 
 
-@pytest.fixture(scope="session")
-def blit(capi):
-    b = capi.Blit(0)
+@pytest.fixture(scope="session", params=["hip", "aql"])
+def blit(request, capi, pkg):
+    """The engine under test, once per submission path: HIP stream launches
+    (mi355_blit.h) and hand-built AQL packets on an HSA queue (mi355_blit_aql.h).
+    Both run the same kernels."""
+    if request.param == "hip":
+        b = capi.Blit(0)
+    else:
+        assert os.path.exists(pkg.aql.library_path()), "AQL library missing: no fallback"
+        b = pkg.aql.AqlBlit(0)
     yield b
     b.close()
 

@@ -148,3 +148,45 @@ def test_kernel_choice_matches_reference_predicate(capi_host, oracle):
             st, p = capi_host.plan_copy(0x10000 + d, 0x90000 + s, 4096)
             ref = oracle.oracle_ref_plan_copy(0x10000 + d, 0x90000 + s, 4096, 256, C.byref(ka))
             assert p.kernel == ref
+
+
+def test_aql_library_exports_every_declared_symbol(pkg):
+    import torch  # noqa: F401
+    header = open(os.path.join(ROOT, "include", "mi355_blit_aql.h")).read()
+    declared = set(re.findall(r"\b(mi355_aql_[a-z0-9_]+)\s*\(", header))
+    assert declared
+    lib = C.CDLL(pkg.aql.library_path())
+    for name in sorted(declared):
+        assert hasattr(lib, name), "library does not export %s" % name
+    assert declared == set(pkg.aql.SIGNATURES)
+
+
+def test_aql_code_object_holds_every_kernel_variant(pkg):
+    """The stand-alone gfx950 code object names its kernels systematically; the
+    AQL engine resolves them by those names."""
+    import subprocess
+    out = subprocess.run(["/opt/rocm/llvm/bin/llvm-readelf", "-s", pkg.build.HSACO],
+                         stdout=subprocess.PIPE, text=True, check=True).stdout
+    names = set(re.findall(r"\b(mi355_[a-z0-9_]+)\.kd\b", out))
+    for u in (1, 2, 4):
+        for l in (0, 1):
+            for s in range(4):
+                for r in (0, 1):
+                    assert "mi355_copy_u%d_l%d_s%d_r%d" % (u, l, s, r) in names
+        for s in range(4):
+            assert "mi355_fill_u%d_s%d" % (u, s) in names
+    for p in (1, 2, 4):
+        for l in (0, 1):
+            for s in range(4):
+                assert "mi355_batch_records_p%d_l%d_s%d" % (p, l, s) in names
+    for n in ("mi355_batch_scan_local", "mi355_batch_scan_top", "mi355_batch_make_records",
+              "mi355_batch_finalize", "mi355_signal_complete"):
+        assert n in names
+
+
+def test_aql_create_without_gpu_fails_loudly(pkg):
+    if _has_gpu():
+        pytest.skip("a GPU is present")
+    h = C.c_void_p()
+    st = pkg.aql.load().mi355_aql_create(0, C.byref(h))
+    assert st != 0 and not h.value

@@ -394,6 +394,8 @@ def test_batch_edge_lengths(capi, blit, oracle, arenas):
 
 
 def test_batch_device_resident_descriptors(capi, blit, oracle, arenas, torch_cuda):
+    if blit.backend != "hip":
+        pytest.skip("device-resident descriptors are a feature of the HIP-stream path")
     torch = torch_cuda
     src, src_host, dst = arenas
     n = 777
@@ -473,7 +475,10 @@ def test_argument_validation(capi, blit, arenas):
     assert blit.copy(dst.base, src.base, 0) == capi.SUCCESS
     assert blit.fill32(dst.base, 1, 0) == capi.SUCCESS
     assert blit.copy_batch(None, 0) == capi.SUCCESS
-    assert blit.lib.mi355_blit_copy_batch(blit.handle, None, 3, 0, None) == inv
+    if blit.backend == "hip":
+        assert blit.lib.mi355_blit_copy_batch(blit.handle, None, 3, 0, None) == inv
+    else:
+        assert blit.lib.mi355_aql_copy_batch(blit.handle, None, 3, None, 0, 0) == inv
     bad = (capi.Desc * 1)()
     bad[0].dst, bad[0].src, bad[0].bytes = None, src.base, 8
     assert blit.copy_batch(bad, 1) == inv
@@ -492,10 +497,20 @@ def test_pending_bytes_zero_is_exact(capi, blit, arenas):
     assert pending % n == 0 and pending <= 100 * n
     check_ok(capi, blit.synchronize(), "synchronize")
     assert blit.pending_bytes() == 0
+    # without a synchronize the count reaches zero by itself once the work is done
+    for _ in range(10):
+        check_ok(capi, blit.copy(dst.base, src.base, n), "copy")
+    import time
+    deadline = time.time() + 5.0
+    while blit.pending_bytes() != 0 and time.time() < deadline:
+        time.sleep(0.001)
+    assert blit.pending_bytes() == 0
 
 
 def test_external_stream_and_ordering(capi, blit, oracle, arenas, torch_cuda):
     """Commands on a caller's stream run in order with that stream's other work."""
+    if blit.backend != "hip":
+        pytest.skip("streams belong to the HIP-stream path")
     torch = torch_cuda
     src, src_host, dst = arenas
     s = torch.cuda.Stream()
@@ -543,10 +558,16 @@ def test_concurrent_submitters(capi, blit, oracle, arenas):
     assert np.array_equal(got, want)
 
 
-def test_create_destroy_many(capi):
+def test_create_destroy_many(capi, pkg):
     for _ in range(5):
         b = capi.Blit(0)
         assert b.num_cus > 0 and b.stream
         b.close()
+    for _ in range(3):
+        a = pkg.aql.AqlBlit(0)
+        assert a.num_cus > 0
+        a.close()
+    with pytest.raises(RuntimeError):
+        pkg.aql.AqlBlit(1000)
     h = C.c_void_p()
     assert capi.load().mi355_blit_create(10_000, C.byref(h)) == capi.ERROR_INVALID_ARGUMENT

@@ -212,6 +212,81 @@ def small_copy_latency(r, sizes=(4096, 65536, MIB)):
     return out
 
 
+def aql_path(r, pkg):
+    """The same workloads submitted as hand-built AQL packets on an HSA queue
+    (include/mi355_blit_aql.h).  Device time per command from the packet
+    processor's own timestamps in the completion signal; small copies as
+    host-observed microseconds, submit -> completion signal seen."""
+    import numpy as np
+    aql = pkg.aql
+    eng = aql.AqlBlit(0)
+    sig = aql.HsaSignals()
+    out = {}
+    try:
+        eng.enable_profiling(True)
+        src = r.device_bytes(GIB + 64, seed=0xB1170003)
+        dst = r.device_bytes(GIB + 64)
+        S, D = aligned_ptr(src), aligned_ptr(dst)
+        cases = (("copy_1GiB", lambda c: eng.copy(D, S, GIB, completion=c), 2 * GIB),
+                 ("fill_1GiB", lambda c: eng.fill32(D, FILL_VALUE, GIB // 4, completion=c), GIB),
+                 ("misaligned_1GiB", lambda c: eng.copy(D + 9, S + 3, GIB - 64, completion=c), 2 * (GIB - 64)))
+        for key, submit, algo in cases:
+            # one command at a time: with the barrier bit clear, commands
+            # queued together would overlap and stretch each other's time
+            sigs = [sig.create(1) for _ in range(23)]
+            for c in sigs:
+                r.check(submit(c), key)
+                sig.wait_below_one(c)
+            us = [eng.command_time_us(c) for c in sigs[3:]]
+            for c in sigs:
+                sig.destroy(c)
+            avg = sum(us) / len(us)
+            out[key] = {"gbs": round(algo / avg / 1e3, 1), "frac_of_peak": round(algo / avg / 1e3 / HBM_PEAK_GBS, 4),
+                        "us_per_launch": round(avg, 2)}
+        so = (-src.data_ptr()) % 256 + 3
+        do = (-dst.data_ptr()) % 256 + 9
+        assert r.torch.equal(dst[do:do + GIB - 64], src[so:so + GIB - 64]), "AQL copy result differs"
+        eng.enable_profiling(False)
+        lat = {}
+        c = sig.create(1)
+        for n in (4096, 65536, MIB):
+            ts = []
+            for i in range(220):
+                sig.store(c, 1)
+                t0 = time.perf_counter()
+                r.check(eng.copy(D, S, n, completion=c), "copy")
+                sig.wait_below_one(c)
+                ts.append(time.perf_counter() - t0)
+            ts = sorted(ts[20:])
+            lat[str(n)] = round(ts[len(ts) // 2] * 1e6, 2)
+        sig.destroy(c)
+        out["small_copy_us"] = lat
+        del src, dst
+        r.torch.cuda.empty_cache()
+        # the batch, whole submission by the host clock
+        hip_blit = r.blit
+        fn, verify, algo, keep = make_batch(r)
+        descs = keep[2]
+        n = len(descs)
+        for _ in range(3):
+            r.check(eng.copy_batch(descs, n), "copy_batch")
+        r.check(eng.synchronize(), "wait_idle")
+        t0 = time.perf_counter()
+        for _ in range(20):
+            r.check(eng.copy_batch(descs, n), "copy_batch")
+        r.check(eng.synchronize(), "wait_idle")
+        us = (time.perf_counter() - t0) / 20 * 1e6
+        verify()
+        out["batch_65536"] = {"gbs": round(algo / us / 1e3, 1), "frac_of_peak": round(algo / us / 1e3 / HBM_PEAK_GBS, 4),
+                              "us_per_launch": round(us, 2)}
+        out["how"] = ("AQL packets on an HSA queue; 1 GiB cases: packet-processor timestamps of 20 commands; "
+                      "batch: host clock over 20 submissions; small copies: host clock, median of 200")
+        del keep, hip_blit
+    finally:
+        eng.close()
+    return out
+
+
 def reference_gpu_path(r):
     """The reference's own blit kernels on this GPU, for orientation: the ROCr
     this process already runs on (libhsa-runtime64, the binary build of the same
@@ -368,6 +443,7 @@ def main():
             del f2, v2, k2
             torch.cuda.empty_cache()
         also["small_copy_us"] = small_copy_latency(r)
+        also["aql_submission"] = aql_path(r, pkg)
         also["reference_gpu_path"] = reference_gpu_path(r)
 
     line = {

@@ -75,6 +75,14 @@ uint64_t mi355_aql_pending_bytes(mi355_aql_t* h);
  * timestamps into each completion signal. */
 int mi355_aql_enable_profiling(mi355_aql_t* h, int enable);
 
+/* Start and end of the command whose completion signal is given, as stamped
+ * by the packet processor while profiling is enabled, in ticks of the system
+ * timestamp (ticks_per_second of them in a second): what
+ * hsa_amd_profiling_get_async_copy_time reports for a copy
+ * (core/runtime/hsa_ext_amd.cpp:474-502). */
+int mi355_aql_get_command_time(mi355_aql_t* h, uint64_t completion_signal, uint64_t* start_ticks,
+                               uint64_t* end_ticks, uint64_t* ticks_per_second);
+
 int mi355_aql_set_tuning(mi355_aql_t* h, const mi355_blit_tuning_t* tuning);
 int mi355_aql_last_launch_info(mi355_aql_t* h, mi355_blit_plan_t* out);
 int mi355_aql_num_cus(mi355_aql_t* h);

@@ -18,6 +18,7 @@ SIGNATURES = {
     "mi355_aql_wait_idle": (C.c_int, [C.c_void_p]),
     "mi355_aql_pending_bytes": (C.c_uint64, [C.c_void_p]),
     "mi355_aql_enable_profiling": (C.c_int, [C.c_void_p, C.c_int]),
+    "mi355_aql_get_command_time": (C.c_int, [C.c_void_p, C.c_uint64, _U64P, _U64P, _U64P]),
     "mi355_aql_set_tuning": (C.c_int, [C.c_void_p, C.POINTER(Tuning)]),
     "mi355_aql_last_launch_info": (C.c_int, [C.c_void_p, C.POINTER(Plan)]),
     "mi355_aql_num_cus": (C.c_int, [C.c_void_p]),
@@ -120,6 +121,52 @@ class AqlBlit:
     def enable_profiling(self, on):
         return self.lib.mi355_aql_enable_profiling(self.handle, 1 if on else 0)
 
+    def command_time_us(self, completion):
+        """Device time of the command that completed `completion`, in microseconds
+        (needs enable_profiling(True) before the command was submitted)."""
+        a, b, f = C.c_uint64(), C.c_uint64(), C.c_uint64()
+        st = self.lib.mi355_aql_get_command_time(self.handle, completion, C.byref(a), C.byref(b), C.byref(f))
+        if st != SUCCESS:
+            raise RuntimeError("mi355_aql_get_command_time failed: 0x%x" % st)
+        return (b.value - a.value) * 1e6 / f.value
+
     @property
     def num_cus(self):
         return self.lib.mi355_aql_num_cus(self.handle)
+
+
+class HsaSignals:
+    """hsa_signal_create / wait / destroy through ctypes, for callers of the
+    AQL path that want completion signals from Python (tests, benchmark)."""
+
+    def __init__(self):
+        self.hsa = C.CDLL("libhsa-runtime64.so.1")
+        self.hsa.hsa_signal_create.argtypes = [C.c_int64, C.c_uint32, C.c_void_p, _U64P]
+        self.hsa.hsa_signal_destroy.argtypes = [C.c_uint64]
+        self.hsa.hsa_signal_store_relaxed.argtypes = [C.c_uint64, C.c_int64]
+        self.hsa.hsa_signal_store_screlease.argtypes = [C.c_uint64, C.c_int64]
+        self.hsa.hsa_signal_load_scacquire.argtypes = [C.c_uint64]
+        self.hsa.hsa_signal_load_scacquire.restype = C.c_int64
+        self.hsa.hsa_signal_wait_scacquire.argtypes = [C.c_uint64, C.c_int, C.c_int64, C.c_uint64, C.c_int]
+        self.hsa.hsa_signal_wait_scacquire.restype = C.c_int64
+
+    def create(self, value=1):
+        h = C.c_uint64()
+        st = self.hsa.hsa_signal_create(value, 0, None, C.byref(h))
+        if st != 0:
+            raise RuntimeError("hsa_signal_create failed: 0x%x" % st)
+        return h.value
+
+    def destroy(self, s):
+        self.hsa.hsa_signal_destroy(s)
+
+    def store(self, s, value):
+        self.hsa.hsa_signal_store_screlease(s, value)
+
+    def load(self, s):
+        return self.hsa.hsa_signal_load_scacquire(s)
+
+    def wait_below_one(self, s, active=True):
+        """Blocks until the signal is < 1 (HSA_SIGNAL_CONDITION_LT = 2)."""
+        while self.hsa.hsa_signal_wait_scacquire(s, 2, 1, 0xFFFFFFFFFFFFFFFF, 1 if active else 0) >= 1:
+            pass

@@ -78,9 +78,9 @@ def build_rocr_adapter():
     os.makedirs(LIB_DIR, exist_ok=True)
     common = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-I", INCLUDE, "-I", CSRC,
               "-I", os.path.join(ROCM, "include")]
-    link = ["-L", LIB_DIR, "-lmi355blit", "-L", os.path.join(ROCM, "lib"), "-lhsa-runtime64",
+    link = ["-L", LIB_DIR, "-lmi355blit", "-lmi355blit_aql", "-L", os.path.join(ROCM, "lib"), "-lhsa-runtime64",
             "-lpthread", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(ROCM, "lib")]
-    _run(["g++"] + common + ["-shared", "-o", ROCR_LIB, src] + link)
+    _run(["g++"] + common + ["-shared", "-o", ROCR_LIB, src, os.path.join(CSRC, "rocr_blit_aql.cpp")] + link)
     return ROCR_LIB
 
 
@@ -92,7 +92,7 @@ def build_rocr_test():
     _run(["g++", "-O2", "-std=c++17", "-Wall", "-D__HIP_PLATFORM_AMD__",
           "-I", INCLUDE, "-I", CSRC, "-I", os.path.join(ROCM, "include"),
           "-o", ROCR_TEST, test_src,
-          "-L", LIB_DIR, "-lmi355blit_rocr", "-lmi355blit",
+          "-L", LIB_DIR, "-lmi355blit_rocr", "-lmi355blit", "-lmi355blit_aql",
           "-L", ORACLE_DIR, "-lblit_oracle",
           "-L", os.path.join(ROCM, "lib"), "-lhsa-runtime64", "-lamdhip64", "-lpthread",
           "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,$ORIGIN/../../oracle",

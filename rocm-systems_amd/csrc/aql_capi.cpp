@@ -9,9 +9,11 @@
 #include <hsa/hsa.h>
 #include <hsa/hsa_ext_amd.h>
 #include <sched.h>
+#include <xmmintrin.h>
 
 #include <atomic>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <new>
@@ -85,6 +87,12 @@ struct mi355_aql {
   hsa_queue_t* queue = nullptr;
   uint32_t queue_mask = 0;
   uint8_t* kernargs = nullptr;
+  // The kernarg ring lives in device memory when the host can write there
+  // (large BAR): a wave then reads its arguments from HBM instead of from
+  // host memory across the bus, which on MI355X takes ~11 us off a dispatch
+  // of a few hundred workgroups.  Host memory otherwise, as in the reference
+  // (amd_blit_kernel.cpp:565-569).
+  bool kernargs_in_device_memory = false;
 
   hsa_executable_t exe{};
   hsa_code_object_reader_t reader{};
@@ -183,6 +191,13 @@ void queue_error_cb(hsa_status_t status, hsa_queue_t*, void* data) {
   std::fprintf(stderr, "mi355_blit_aql: queue error 0x%x (%s)\n", status, msg ? msg : "?");
 }
 
+// MI355_BLIT_HOST_KERNARGS=1 keeps the kernarg ring in host memory (for
+// measurements and for systems whose BAR writes misbehave).
+bool force_host_kernargs() {
+  const char* v = std::getenv("MI355_BLIT_HOST_KERNARGS");
+  return v && v[0] == '1';
+}
+
 int lookup(mi355_aql* h, const char* name, Kernel* out) {
   const std::string sym = std::string(name) + ".kd";
   hsa_executable_symbol_t s;
@@ -277,6 +292,14 @@ void write_dispatch(mi355_aql* h, uint64_t index, const Kernel& k, const void* a
                     uint32_t grid_wgs, uint32_t wg_size, uint64_t completion, bool barrier_bit) {
   uint8_t* karg = h->kernargs + (index & h->queue_mask) * kKernargSlotBytes;
   std::memcpy(karg, args, args_size);
+  if (h->kernargs_in_device_memory) {
+    // Writes across the bus are posted: order them, then read one back so
+    // that they have landed before the doorbell lets a wave read them (the
+    // reference fences its packet writes the same way when the ring is in
+    // device memory, amd_blit_kernel.cpp:896-899).
+    _mm_sfence();
+    (void)*reinterpret_cast<volatile uint32_t*>(karg + ((args_size - 1) & ~size_t(3)));
+  }
   hsa_kernel_dispatch_packet_t pkt;
   std::memset(&pkt, 0, sizeof(pkt));
   pkt.workgroup_size_x = static_cast<uint16_t>(wg_size);
@@ -446,7 +469,19 @@ int mi355_aql_create(int gpu_ordinal, mi355_aql_t** out) {
   h->queue_mask = h->queue->size - 1;
   h->bytes_written.assign(h->queue->size, BytesWritten{~0ull, ~0ull});
   void* ka = nullptr;
-  if ((rc = alloc(h, h->kernarg_pool, h->queue->size * kKernargSlotBytes, &ka, true)) != MI355_BLIT_SUCCESS) return fail(rc);
+  hsa_amd_memory_pool_access_t host_access = HSA_AMD_MEMORY_POOL_ACCESS_NEVER_ALLOWED;
+  hsa_amd_agent_memory_pool_get_info(h->cpu, h->local_pool, HSA_AMD_AGENT_MEMORY_POOL_INFO_ACCESS, &host_access);
+  if (host_access != HSA_AMD_MEMORY_POOL_ACCESS_NEVER_ALLOWED && !force_host_kernargs() &&
+      hsa_amd_memory_pool_allocate(h->local_pool, h->queue->size * kKernargSlotBytes, 0, &ka) == HSA_STATUS_SUCCESS) {
+    if (hsa_amd_agents_allow_access(1, &h->cpu, nullptr, ka) == HSA_STATUS_SUCCESS) {
+      h->kernargs_in_device_memory = true;
+    } else {
+      (void)hsa_amd_memory_pool_free(ka);
+      ka = nullptr;
+    }
+  }
+  if (!ka && (rc = alloc(h, h->kernarg_pool, h->queue->size * kKernargSlotBytes, &ka, true)) != MI355_BLIT_SUCCESS)
+    return fail(rc);
   h->kernargs = static_cast<uint8_t*>(ka);
   if (hsa_signal_create(1, 0, nullptr, &h->idle_signal) != HSA_STATUS_SUCCESS) return fail(MI355_BLIT_ERROR_OUT_OF_RESOURCES);
   for (int i = 0; i < 2; ++i)
@@ -508,6 +543,19 @@ int mi355_aql_set_system_scope_fences(mi355_aql_t* h, int enable) {
 int mi355_aql_enable_profiling(mi355_aql_t* h, int enable) {
   if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   AQL_HSA(hsa_amd_profiling_set_profiler_enabled(h->queue, enable ? 1 : 0));
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_aql_get_command_time(mi355_aql_t* h, uint64_t completion_signal, uint64_t* start_ticks,
+                               uint64_t* end_ticks, uint64_t* ticks_per_second) {
+  if (!h || !completion_signal || !start_ticks || !end_ticks) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  hsa_signal_t s;
+  s.handle = completion_signal;
+  hsa_amd_profiling_dispatch_time_t t{0, 0};
+  AQL_HSA(hsa_amd_profiling_get_dispatch_time(h->gpu, s, &t));
+  *start_ticks = t.start;
+  *end_ticks = t.end;
+  if (ticks_per_second) AQL_HSA(hsa_system_get_info(HSA_SYSTEM_INFO_TIMESTAMP_FREQUENCY, ticks_per_second));
   return MI355_BLIT_SUCCESS;
 }
 

@@ -28,6 +28,7 @@
 #include <vector>
 
 struct mi355_blit;
+struct mi355_aql;
 
 namespace rocr {
 namespace core {
@@ -177,6 +178,41 @@ class BlitKernelGfx950 : public core::Blit {
   uint64_t waiting_bytes_;
 
   std::atomic<bool> profiling_;
+};
+
+// The same interface over hand-built AQL packets (include/mi355_blit_aql.h):
+// dependencies become BARRIER_AND packets, out_signal is the dispatch packet's
+// completion signal and the packet processor decrements it, exactly as in
+// AMD::BlitKernel (core/runtime/amd_blit_kernel.cpp:641-785).  No submission
+// thread, no HIP.  This is the class that replaces AMD::BlitKernel in tree.
+class BlitKernelGfx950Aql : public core::Blit {
+ public:
+  explicit BlitKernelGfx950Aql(core::Queue* queue);
+  ~BlitKernelGfx950Aql() override;
+
+  hsa_status_t Initialize(const core::Agent& agent);
+  hsa_status_t Destroy(const core::Agent& agent) override;
+  hsa_status_t SubmitLinearCopyCommand(void* dst, const void* src, size_t size) override;
+  hsa_status_t SubmitLinearCopyCommand(void* dst, const void* src, size_t size,
+                                       std::vector<core::Signal*>& dep_signals,
+                                       core::Signal& out_signal,
+                                       std::vector<core::Signal*>& gang_signals) override;
+  hsa_status_t SubmitLinearFillCommand(void* ptr, uint32_t value, size_t count) override;
+  /// Batched small copies (host-resident descriptors); no counterpart in core::Blit.
+  hsa_status_t SubmitBatchCopyCommand(const void* descs, size_t n, bool descs_on_device,
+                                      std::vector<core::Signal*>& dep_signals,
+                                      core::Signal& out_signal);
+  hsa_status_t EnableProfiling(bool enable) override;
+  uint64_t PendingBytes() override;
+  void GangLeader(bool) override {}
+  bool GangLeader() const override { return false; }
+
+ private:
+  core::Queue* queue_;
+  mi355_aql* blit_;
+  /// Completion signal of the blocking calls; guarded by lock_.
+  hsa_signal_t completion_signal_;
+  std::mutex lock_;
 };
 
 }  // namespace AMD

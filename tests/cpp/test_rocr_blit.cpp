@@ -7,12 +7,14 @@
 // (rocrtst/samples/async_mem_copy/async_mem_copy.cc:269-357).
 #include <hip/hip_runtime_api.h>
 #include <hsa/hsa.h>
+#include <hsa/hsa_ext_amd.h>
 
 #include <algorithm>
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <functional>
 #include <string>
 #include <thread>
 #include <vector>
@@ -22,18 +24,24 @@
 #include "rocr_blit.h"
 
 using rocr::AMD::BlitKernelGfx950;
+using rocr::AMD::BlitKernelGfx950Aql;
+using rocr::core::Blit;
 using rocr::core::Signal;
+
+// SubmitBatchCopyCommand is not part of core::Blit; each engine supplies it.
+typedef std::function<hsa_status_t(const void*, size_t, std::vector<Signal*>&, Signal&)> BatchFn;
 
 namespace {
 
 int g_failures = 0;
+std::string g_suffix;  // "_hip" or "_aql": which engine the cases run on
 constexpr size_t kGuard = 256;
 constexpr uint8_t kGuardByte = 0xEE;
 
 #define REQUIRE(cond, ...)                         \
   do {                                             \
     if (!(cond)) {                                 \
-      std::printf("FAIL %s: ", name);              \
+      std::printf("FAIL %s%s: ", name, g_suffix.c_str()); \
       std::printf(__VA_ARGS__);                    \
       std::printf(" (line %d)\n", __LINE__);       \
       std::fflush(stdout);                         \
@@ -86,7 +94,7 @@ std::vector<uint8_t> seeded(size_t n, uint64_t seed) {
 
 // ---------------------------------------------------------------------------
 
-void test_blocking_copy(BlitKernelGfx950& blit) {
+void test_blocking_copy(Blit& blit) {
   const char* name = "blocking_copy_offsets_and_sizes";
   const size_t max_n = (3u << 20) + 77;
   std::vector<uint8_t> src_h = seeded(max_n + 64, 0xB1170003);
@@ -106,10 +114,10 @@ void test_blocking_copy(BlitKernelGfx950& blit) {
       REQUIRE(got == want, "bytes differ n=%zu so=%zu do=%zu", n, so, dof);
     }
   }
-  std::printf("PASS %s\n", name);
+  std::printf("PASS %s%s\n", name, g_suffix.c_str());
 }
 
-void test_blocking_fill(BlitKernelGfx950& blit) {
+void test_blocking_fill(Blit& blit) {
   const char* name = "blocking_fill_reference_patterns";
   // rocrtst/samples/async_mem_copy/async_mem_copy.cc:62-65
   const uint32_t values[] = {0xabcdef12, 0xba5eba11, 0xfeed5a1e, 0xbaadf00d, 0xA5C30F1E};
@@ -140,10 +148,10 @@ void test_blocking_fill(BlitKernelGfx950& blit) {
   }
   REQUIRE(dst.download(got), "download");
   REQUIRE(got == want, "rejected fill wrote memory");
-  std::printf("PASS %s\n", name);
+  std::printf("PASS %s%s\n", name, g_suffix.c_str());
 }
 
-void test_async_copy_signal(BlitKernelGfx950& blit, hsa_wait_state_t state, const char* name) {
+void test_async_copy_signal(Blit& blit, hsa_wait_state_t state, const char* name) {
   const size_t n = (8u << 20) + 5;
   std::vector<uint8_t> src_h = seeded(n + 16, 0xB1170002);
   DeviceBuf src(src_h.size()), dst(n + 2 * kGuard + 16);
@@ -170,10 +178,10 @@ void test_async_copy_signal(BlitKernelGfx950& blit, hsa_wait_state_t state, cons
   }
   REQUIRE(pending == 0, "PendingBytes stuck at %llu", (unsigned long long)pending);
   hsa_signal_destroy(done);
-  std::printf("PASS %s\n", name);
+  std::printf("PASS %s%s\n", name, g_suffix.c_str());
 }
 
-void test_dependencies(BlitKernelGfx950& blit, size_t n_deps, const char* name) {
+void test_dependencies(Blit& blit, size_t n_deps, const char* name) {
   const size_t n = (1u << 20) + 9;
   std::vector<uint8_t> src_h = seeded(n, 0xB1170004);
   DeviceBuf src(n), dst(n + 2 * kGuard);
@@ -219,10 +227,10 @@ void test_dependencies(BlitKernelGfx950& blit, size_t n_deps, const char* name) 
   for (hsa_signal_t h : dep_handles) hsa_signal_destroy(h);
   hsa_signal_destroy(done);
   hsa_signal_destroy(done2);
-  std::printf("PASS %s\n", name);
+  std::printf("PASS %s%s\n", name, g_suffix.c_str());
 }
 
-void test_chain(BlitKernelGfx950& blit) {
+void test_chain(Blit& blit) {
   const char* name = "chain_a_to_b_to_c";
   const size_t n = (2u << 20) + 11;
   std::vector<uint8_t> a_h = seeded(n, 0xB1170005);
@@ -245,10 +253,10 @@ void test_chain(BlitKernelGfx950& blit) {
   REQUIRE(got == want, "bytes differ");
   hsa_signal_destroy(s1);
   hsa_signal_destroy(s2);
-  std::printf("PASS %s\n", name);
+  std::printf("PASS %s%s\n", name, g_suffix.c_str());
 }
 
-void test_zero_size_and_bad_args(BlitKernelGfx950& blit) {
+void test_zero_size_and_bad_args(Blit& blit) {
   const char* name = "zero_size_and_bad_arguments";
   DeviceBuf d(4096);
   REQUIRE(d.p, "hipMalloc");
@@ -267,10 +275,10 @@ void test_zero_size_and_bad_args(BlitKernelGfx950& blit) {
   REQUIRE(blit.EnableProfiling(true) == HSA_STATUS_SUCCESS && blit.EnableProfiling(false) == HSA_STATUS_SUCCESS,
           "EnableProfiling");
   hsa_signal_destroy(s);
-  std::printf("PASS %s\n", name);
+  std::printf("PASS %s%s\n", name, g_suffix.c_str());
 }
 
-void test_batch(BlitKernelGfx950& blit) {
+void test_batch(Blit& blit, const BatchFn& submit_batch) {
   const char* name = "batched_copies_with_signal";
   const size_t ncopy = 500;
   std::vector<size_t> len(ncopy), off(ncopy), so(ncopy), dof(ncopy);
@@ -299,15 +307,15 @@ void test_batch(BlitKernelGfx950& blit) {
   hsa_signal_t s = make_signal(1);
   Signal sig(s);
   std::vector<Signal*> none;
-  REQUIRE(blit.SubmitBatchCopyCommand(descs.data(), ncopy, false, none, sig) == HSA_STATUS_SUCCESS, "submit");
+  REQUIRE(submit_batch(descs.data(), ncopy, none, sig) == HSA_STATUS_SUCCESS, "submit");
   REQUIRE(wait_zero(s, HSA_WAIT_STATE_BLOCKED), "batch never completed");
   REQUIRE(dst.download(got), "download");
   REQUIRE(got == want, "bytes differ");
   hsa_signal_destroy(s);
-  std::printf("PASS %s\n", name);
+  std::printf("PASS %s%s\n", name, g_suffix.c_str());
 }
 
-void test_threads(BlitKernelGfx950& blit) {
+void test_threads(Blit& blit) {
   const char* name = "concurrent_submitters";
   const int kThreads = 4, kPer = 6;
   const size_t n = (1u << 18) + 13, region = ((n + 2 * kGuard + 255) / 256) * 256;
@@ -337,10 +345,50 @@ void test_threads(BlitKernelGfx950& blit) {
   }
   REQUIRE(dst.download(got), "download");
   REQUIRE(got == want, "bytes differ");
-  std::printf("PASS %s\n", name);
+  std::printf("PASS %s%s\n", name, g_suffix.c_str());
 }
 
-void latency_report(BlitKernelGfx950& blit, const char* mode) {
+hsa_status_t first_gpu_cb(hsa_agent_t agent, void* data) {
+  hsa_device_type_t type;
+  if (hsa_agent_get_info(agent, HSA_AGENT_INFO_DEVICE, &type) == HSA_STATUS_SUCCESS && type == HSA_DEVICE_TYPE_GPU) {
+    *static_cast<hsa_agent_t*>(data) = agent;
+    return HSA_STATUS_INFO_BREAK;
+  }
+  return HSA_STATUS_SUCCESS;
+}
+
+// With profiling on, the packet processor stamps the completion signal
+// (amd_blit_kernel.cpp:839-842; read back like hsa_ext_amd.cpp:474-502 does).
+void test_profiling_timestamps(Blit& blit) {
+  const char* name = "profiling_timestamps";
+  hsa_agent_t gpu{0};
+  hsa_iterate_agents(first_gpu_cb, &gpu);
+  REQUIRE(gpu.handle, "no GPU agent");
+  const size_t n = 64u << 20;
+  DeviceBuf a(n), b(n);
+  REQUIRE(a.p && b.p, "hipMalloc");
+  REQUIRE(blit.EnableProfiling(true) == HSA_STATUS_SUCCESS, "EnableProfiling(true)");
+  hsa_signal_t s = make_signal(1);
+  Signal sig(s);
+  std::vector<Signal*> none, gang;
+  REQUIRE(blit.SubmitLinearCopyCommand(b.p, a.p, n, none, sig, gang) == HSA_STATUS_SUCCESS, "submit");
+  REQUIRE(wait_zero(s, HSA_WAIT_STATE_BLOCKED), "copy never completed");
+  hsa_amd_profiling_dispatch_time_t t{0, 0};
+  hsa_status_t st = hsa_amd_profiling_get_dispatch_time(gpu, s, &t);
+  REQUIRE(st == HSA_STATUS_SUCCESS, "get_dispatch_time 0x%x", st);
+  REQUIRE(t.end > t.start, "timestamps not written: start %llu end %llu", (unsigned long long)t.start,
+          (unsigned long long)t.end);
+  uint64_t freq = 0;
+  hsa_system_get_info(HSA_SYSTEM_INFO_TIMESTAMP_FREQUENCY, &freq);
+  const double us = freq ? double(t.end - t.start) * 1e6 / double(freq) : 0.0;
+  std::printf("INFO profiling_copy_64MiB_us %.1f\n", us);
+  REQUIRE(us > 5.0 && us < 5000.0, "implausible copy time %.1f us", us);
+  REQUIRE(blit.EnableProfiling(false) == HSA_STATUS_SUCCESS, "EnableProfiling(false)");
+  hsa_signal_destroy(s);
+  std::printf("PASS %s%s\n", name, g_suffix.c_str());
+}
+
+void latency_report(Blit& blit, const char* mode) {
   // host-observed time per blocking call, submit -> completion seen
   // (the way memory_async_copy.cc:396-405 times a copy)
   DeviceBuf a(1 << 20), b(1 << 20);
@@ -362,10 +410,14 @@ void latency_report(BlitKernelGfx950& blit, const char* mode) {
 
 int main(int argc, char** argv) {
   if (argc > 1 && std::string(argv[1]) == "--list") {
-    std::printf("blocking_copy_offsets_and_sizes\nblocking_fill_reference_patterns\nasync_copy_active_wait\n"
-                "async_copy_blocked_wait\ndependencies_1\ndependencies_6\nchain_a_to_b_to_c\n"
-                "zero_size_and_bad_arguments\nbatched_copies_with_signal\nconcurrent_submitters\n"
-                "host_callback_async_copy\n");
+    const char* cases[] = {"blocking_copy_offsets_and_sizes", "blocking_fill_reference_patterns",
+                           "async_copy_active_wait", "async_copy_blocked_wait", "dependencies_1", "dependencies_6",
+                           "chain_a_to_b_to_c", "zero_size_and_bad_arguments", "batched_copies_with_signal",
+                           "concurrent_submitters", "destroy"};
+    for (const char* engine : {"_hip", "_aql"})
+      for (const char* c : cases) std::printf("%s%s\n", c, engine);
+    std::printf("async_copy_blocked_wait_hip_callback\nchain_a_to_b_to_c_hip_callback\n"
+                "profiling_timestamps_aql\n");
     return 0;
   }
   if (hsa_init() != HSA_STATUS_SUCCESS) {
@@ -379,44 +431,67 @@ int main(int argc, char** argv) {
   }
   rocr::core::Agent agent(0);
   {
-    // the host-callback completion mode: one asynchronous and one blocking case
+    // the host-callback completion mode of the HIP-stream engine
+    g_suffix = "_hip_callback";
     BlitKernelGfx950 cb(nullptr, BlitKernelGfx950::Completion::kHostCallback);
     if (cb.Initialize(agent) != HSA_STATUS_SUCCESS) {
       std::printf("FAIL setup: Initialize (host callback)\n");
       return 2;
     }
-    test_async_copy_signal(cb, HSA_WAIT_STATE_BLOCKED, "host_callback_async_copy");
+    test_async_copy_signal(cb, HSA_WAIT_STATE_BLOCKED, "async_copy_blocked_wait");
     test_chain(cb);
-    latency_report(cb, "host_callback");
+    latency_report(cb, "hip_host_callback");
     if (cb.Destroy(agent) != HSA_STATUS_SUCCESS) {
       std::printf("FAIL destroy (host callback)\n");
       ++g_failures;
     }
   }
-  BlitKernelGfx950* blit = new BlitKernelGfx950(nullptr);
-  if (blit->Initialize(agent) != HSA_STATUS_SUCCESS) {
-    std::printf("FAIL setup: Initialize\n");
-    return 2;
+  for (int engine = 0; engine < 2; ++engine) {
+    Blit* blit = nullptr;
+    BatchFn batch;
+    hsa_status_t init;
+    if (engine == 0) {
+      g_suffix = "_hip";
+      auto* b = new BlitKernelGfx950(nullptr);
+      init = b->Initialize(agent);
+      batch = [b](const void* d, size_t n, std::vector<Signal*>& deps, Signal& out) {
+        return b->SubmitBatchCopyCommand(d, n, false, deps, out);
+      };
+      blit = b;
+    } else {
+      g_suffix = "_aql";
+      auto* b = new BlitKernelGfx950Aql(nullptr);
+      init = b->Initialize(agent);
+      batch = [b](const void* d, size_t n, std::vector<Signal*>& deps, Signal& out) {
+        return b->SubmitBatchCopyCommand(d, n, false, deps, out);
+      };
+      blit = b;
+    }
+    if (init != HSA_STATUS_SUCCESS) {
+      std::printf("FAIL setup%s: Initialize returned 0x%x\n", g_suffix.c_str(), init);
+      return 2;
+    }
+    test_blocking_copy(*blit);
+    test_blocking_fill(*blit);
+    test_async_copy_signal(*blit, HSA_WAIT_STATE_ACTIVE, "async_copy_active_wait");
+    test_async_copy_signal(*blit, HSA_WAIT_STATE_BLOCKED, "async_copy_blocked_wait");
+    test_dependencies(*blit, 1, "dependencies_1");
+    test_dependencies(*blit, 6, "dependencies_6");  // more than one barrier packet's worth
+    test_chain(*blit);
+    test_zero_size_and_bad_args(*blit);
+    test_batch(*blit, batch);
+    test_threads(*blit);
+    if (engine == 1) test_profiling_timestamps(*blit);
+    latency_report(*blit, engine == 0 ? "hip_device_signal" : "aql");
+    hsa_status_t st = blit->Destroy(agent);
+    if (st != HSA_STATUS_SUCCESS) {
+      std::printf("FAIL destroy%s: status 0x%x\n", g_suffix.c_str(), st);
+      ++g_failures;
+    } else {
+      std::printf("PASS destroy%s\n", g_suffix.c_str());
+    }
+    delete blit;
   }
-  test_blocking_copy(*blit);
-  test_blocking_fill(*blit);
-  test_async_copy_signal(*blit, HSA_WAIT_STATE_ACTIVE, "async_copy_active_wait");
-  test_async_copy_signal(*blit, HSA_WAIT_STATE_BLOCKED, "async_copy_blocked_wait");
-  test_dependencies(*blit, 1, "dependencies_1");
-  test_dependencies(*blit, 6, "dependencies_6");  // more than one barrier packet's worth in the reference
-  test_chain(*blit);
-  test_zero_size_and_bad_args(*blit);
-  test_batch(*blit);
-  test_threads(*blit);
-  latency_report(*blit, "device_signal");
-  hsa_status_t st = blit->Destroy(agent);
-  if (st != HSA_STATUS_SUCCESS) {
-    std::printf("FAIL destroy: status 0x%x\n", st);
-    ++g_failures;
-  } else {
-    std::printf("PASS destroy\n");
-  }
-  delete blit;
   hsa_shut_down();
   std::printf("%s (%d failures)\n", g_failures ? "FAILED" : "OK", g_failures);
   return g_failures ? 1 : 0;

@@ -21,11 +21,12 @@ def test_adapter_is_built_and_exports_the_interface(pkg):
     lib, exe = _paths(pkg)
     assert os.path.exists(lib) and os.path.exists(exe), "run __graft_entry__.build() first"
     syms = subprocess.run(["nm", "-DC", lib], stdout=subprocess.PIPE, text=True, check=True).stdout
-    for member in ("Initialize(rocr::core::Agent const&)", "Destroy(rocr::core::Agent const&)",
-                   "SubmitLinearCopyCommand(void*, void const*, unsigned long)",
-                   "SubmitLinearFillCommand(void*, unsigned int, unsigned long)",
-                   "SubmitBatchCopyCommand", "EnableProfiling(bool)", "PendingBytes()"):
-        assert "rocr::AMD::BlitKernelGfx950::" + member in syms, member
+    for cls in ("BlitKernelGfx950", "BlitKernelGfx950Aql"):
+        for member in ("Initialize(rocr::core::Agent const&)", "Destroy(rocr::core::Agent const&)",
+                       "SubmitLinearCopyCommand(void*, void const*, unsigned long)",
+                       "SubmitLinearFillCommand(void*, unsigned int, unsigned long)",
+                       "SubmitBatchCopyCommand", "EnableProfiling(bool)", "PendingBytes()"):
+            assert "rocr::AMD::%s::%s" % (cls, member) in syms, (cls, member)
     # the asynchronous overload with dependency, completion and gang signals
     assert re.search(r"BlitKernelGfx950::SubmitLinearCopyCommand\(void\*, void const\*, unsigned long, "
                      r"std::vector<rocr::core::Signal\*.*rocr::core::Signal&, std::vector<rocr::core::Signal\*", syms)
@@ -56,7 +57,9 @@ def test_adapter_interface_mirrors_reference_blit_h():
 def test_native_driver_lists_its_cases(pkg):
     _, exe = _paths(pkg)
     out = subprocess.run([exe, "--list"], stdout=subprocess.PIPE, text=True, check=True).stdout.split()
-    assert "dependencies_6" in out and "async_copy_blocked_wait" in out and len(out) >= 10
+    for engine in ("_hip", "_aql"):
+        assert "dependencies_6" + engine in out and "async_copy_blocked_wait" + engine in out
+    assert "profiling_timestamps_aql" in out and len(out) >= 24
 
 
 @pytest.mark.gpu
@@ -66,6 +69,6 @@ def test_native_driver_passes_on_gpu(pkg, torch_cuda):
     proc = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=240)
     print(proc.stdout)
     assert proc.returncode == 0, proc.stdout[-4000:]
-    for case in cases + ["destroy"]:
-        assert "PASS " + case in proc.stdout, "case %s did not pass" % case
+    for case in cases:
+        assert "PASS " + case + "\n" in proc.stdout, "case %s did not pass" % case
     assert "FAIL" not in proc.stdout

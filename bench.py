@@ -190,6 +190,31 @@ def make_batch(r, n=65536, arena=8 * GIB):
     return fn, verify, int(2 * lens.sum()), (src, dst, descs)
 
 
+def size_sweep(r):
+    """Aligned copy and fill at 4 KiB -> 4 GiB in powers of 4: microseconds per
+    launch (HIP events around back-to-back launches) and algorithmic GB/s.
+    Sizes up to a few hundred MiB are helped by the 256 MiB last-level cache."""
+    out = {"copy": {}, "fill": {}}
+    top = 4 * GIB
+    src = r.device_bytes(top + 64, seed=None)
+    dst = r.device_bytes(top + 64)
+    src.random_(0, 256)
+    r.torch.cuda.synchronize()
+    S, D = aligned_ptr(src), aligned_ptr(dst)
+    for k in range(11):
+        n = 4096 * 4 ** k
+        iters = 100 if n <= MIB else (30 if n <= 256 * MIB else 8)
+        _, us = r.time_launches(lambda: r.check(r.blit.copy(D, S, n, r.stream), "copy"), iters, 3)
+        out["copy"][str(n)] = {"us": round(us, 2), "gbs": round(2 * n / us / 1e3, 1)}
+        _, us = r.time_launches(lambda: r.check(r.blit.fill32(D, FILL_VALUE, n // 4, r.stream), "fill32"), iters, 3)
+        out["fill"][str(n)] = {"us": round(us, 2), "gbs": round(n / us / 1e3, 1)}
+    so, do = (-src.data_ptr()) % 256, (-dst.data_ptr()) % 256
+    r.check(r.blit.copy(D, S, top, r.stream), "copy")
+    r.tstream.synchronize()
+    assert r.torch.equal(dst[do:do + top], src[so:so + top]), "4 GiB copy differs"
+    return out
+
+
 def small_copy_latency(r, sizes=(4096, 65536, MIB)):
     """Host-observed microseconds per blocking copy (submit -> completion seen),
     the way rocrtst times hsa_amd_memory_async_copy (memory_async_copy.cc:396-405)."""
@@ -443,6 +468,8 @@ def main():
             del f2, v2, k2
             torch.cuda.empty_cache()
         also["small_copy_us"] = small_copy_latency(r)
+        also["size_sweep"] = size_sweep(r)
+        r.torch.cuda.empty_cache()
         also["aql_submission"] = aql_path(r, pkg)
         also["reference_gpu_path"] = reference_gpu_path(r)
 

@@ -93,6 +93,49 @@ int mi355_aql_num_cus(mi355_aql_t* h);
  * system-scope release. */
 int mi355_aql_set_system_scope_fences(mi355_aql_t* h, int enable);
 
+/* hsa_agent_t.handle of the engine's GPU. */
+uint64_t mi355_aql_gpu_agent(mi355_aql_t* h);
+
+/* Two host buffers of `half_bytes` each that the GPU can access, owned by the
+ * engine (allocated on first use from the fine-grained host pool, kept until
+ * destroy): the bounce buffers of host<->device copies whose host side cannot
+ * be locked.  The caller serialises their use. */
+int mi355_aql_staging(mi355_aql_t* h, size_t* half_bytes, void** half0, void** half1);
+
+/* ---- caller policy: what sits between the HSA API and the blit ------------
+ * The three entry points below restate, over this engine, the decisions ROCr
+ * takes before it reaches core::Blit, so that they can stand in for
+ * hsa_memory_copy, hsa_amd_memory_fill and hsa_amd_memory_async_copy on one
+ * GPU.  Pointers are classified with hsa_amd_pointer_info, as
+ * Runtime::CopyMemory does (core/runtime/runtime.cpp:469-552). */
+
+/* hsa_memory_copy (core/runtime/hsa.cpp:1170-1184 + Runtime::CopyMemory,
+ * runtime.cpp:469-552).  Blocking.  NULL -> INVALID_ARGUMENT; size 0 ->
+ * SUCCESS; host<->host is one memcpy on the calling thread (:507-510); when
+ * one side is host memory unknown to the runtime it is locked for the GPU for
+ * the duration of the copy (:521-537), or, where the system refuses to lock
+ * existing memory, bounced through the engine's staging buffers in 4 MiB
+ * pieces; everything else goes to the blit. */
+int mi355_hsa_memory_copy(mi355_aql_t* h, void* dst, const void* src, size_t size);
+
+/* hsa_amd_memory_fill (core/runtime/hsa_ext_amd.cpp:237-251 + Runtime::FillMemory,
+ * runtime.cpp:627-664).  Blocking.  NULL or ptr % 4 -> INVALID_ARGUMENT;
+ * count 0 -> SUCCESS; memory the GPU can reach is filled by the blit; plain
+ * host memory is filled on the host with the full 32-bit pattern (the
+ * reference's memset(ptr, value, count*4) there keeps only the low byte,
+ * runtime.cpp:657-661: a defect, not reproduced). */
+int mi355_hsa_amd_memory_fill(mi355_aql_t* h, void* ptr, uint32_t value, size_t count);
+
+/* hsa_amd_memory_async_copy for copies this GPU executes
+ * (core/runtime/hsa_ext_amd.cpp:253-294).  NULL pointers, or a dependency count
+ * that disagrees with the array pointer, or a zero completion signal ->
+ * INVALID_ARGUMENT; size 0 -> SUCCESS without touching the signal (:285-291);
+ * both ranges must already be accessible to the GPU (device memory, or host
+ * memory allocated or locked through the runtime), as the API demands. */
+int mi355_hsa_amd_memory_async_copy(mi355_aql_t* h, void* dst, const void* src, size_t size,
+                                    uint32_t num_dep_signals, const uint64_t* dep_signals,
+                                    uint64_t completion_signal);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,6 +23,12 @@ SIGNATURES = {
     "mi355_aql_last_launch_info": (C.c_int, [C.c_void_p, C.POINTER(Plan)]),
     "mi355_aql_num_cus": (C.c_int, [C.c_void_p]),
     "mi355_aql_set_system_scope_fences": (C.c_int, [C.c_void_p, C.c_int]),
+    "mi355_aql_gpu_agent": (C.c_uint64, [C.c_void_p]),
+    "mi355_aql_staging": (C.c_int, [C.c_void_p, C.POINTER(C.c_size_t), C.POINTER(C.c_void_p), C.POINTER(C.c_void_p)]),
+    "mi355_hsa_memory_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
+    "mi355_hsa_amd_memory_fill": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t]),
+    "mi355_hsa_amd_memory_async_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint32,
+                                                  _U64P, C.c_uint64]),
 }
 
 _lib = None
@@ -120,6 +126,17 @@ class AqlBlit:
 
     def enable_profiling(self, on):
         return self.lib.mi355_aql_enable_profiling(self.handle, 1 if on else 0)
+
+    # caller policy (hsa_memory_copy / hsa_amd_memory_fill / hsa_amd_memory_async_copy stand-ins)
+    def hsa_memory_copy(self, dst, src, nbytes):
+        return self.lib.mi355_hsa_memory_copy(self.handle, dst, src, nbytes)
+
+    def hsa_amd_memory_fill(self, ptr, value, count):
+        return self.lib.mi355_hsa_amd_memory_fill(self.handle, ptr, value, count)
+
+    def hsa_amd_memory_async_copy(self, dst, src, nbytes, deps=None, completion=0):
+        arr, n = _deps(deps)
+        return self.lib.mi355_hsa_amd_memory_async_copy(self.handle, dst, src, nbytes, n, arr, completion)
 
     def command_time_us(self, completion):
         """Device time of the command that completed `completion`, in microseconds

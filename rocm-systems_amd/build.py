@@ -63,7 +63,8 @@ def build_aql():
     _run(["g++", "-O2", "-std=c++17", "-fPIC", "-Wall", "-shared",
           "-I", INCLUDE, "-I", CSRC, "-I", os.path.join(ROCM, "include"),
           "-DHSACO_PATH=\"%s\"" % HSACO,
-          "-o", AQL_LIB, os.path.join(CSRC, "aql_capi.cpp"), os.path.join(CSRC, "hsaco_embed.S"),
+          "-o", AQL_LIB, os.path.join(CSRC, "aql_capi.cpp"), os.path.join(CSRC, "aql_runtime.cpp"),
+          os.path.join(CSRC, "hsaco_embed.S"),
           "-L", os.path.join(ROCM, "lib"), "-lhsa-runtime64", "-lpthread",
           "-Wl,-rpath," + os.path.join(ROCM, "lib")])
     return AQL_LIB

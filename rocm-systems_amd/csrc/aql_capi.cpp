@@ -132,6 +132,9 @@ struct mi355_aql {
   uint32_t* block_sum_dev = nullptr;
   ChunkRecord* records_dev = nullptr;
   size_t batch_capacity = 0, records_capacity = 0;
+
+  // bounce buffers of host<->device copies (mi355_aql_staging)
+  void* bounce[2] = {nullptr, nullptr};
 };
 
 namespace {
@@ -507,6 +510,8 @@ int mi355_aql_destroy(mi355_aql_t* h) {
     free_device(h->chunk_start_dev);
     free_device(h->block_sum_dev);
     free_device(h->records_dev);
+    free_device(h->bounce[0]);
+    free_device(h->bounce[1]);
     if (h->idle_signal.handle) hsa_signal_destroy(h->idle_signal);
     if (h->have_exe) hsa_executable_destroy(h->exe);
     if (h->have_reader) hsa_code_object_reader_destroy(h->reader);
@@ -517,6 +522,24 @@ int mi355_aql_destroy(mi355_aql_t* h) {
 }
 
 int mi355_aql_num_cus(mi355_aql_t* h) { return h ? static_cast<int>(h->num_cus) : 0; }
+
+uint64_t mi355_aql_gpu_agent(mi355_aql_t* h) { return h ? h->gpu.handle : 0; }
+
+int mi355_aql_staging(mi355_aql_t* h, size_t* half_bytes, void** half0, void** half1) {
+  if (!h || !half_bytes || !half0 || !half1) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  constexpr size_t kHalf = 4u << 20;
+  std::lock_guard<std::mutex> g(h->lock);
+  for (int i = 0; i < 2; ++i) {
+    if (!h->bounce[i]) {
+      int rc = alloc(h, h->host_pool, kHalf, &h->bounce[i], true);
+      if (rc != MI355_BLIT_SUCCESS) return rc;
+    }
+  }
+  *half_bytes = kHalf;
+  *half0 = h->bounce[0];
+  *half1 = h->bounce[1];
+  return MI355_BLIT_SUCCESS;
+}
 
 int mi355_aql_set_tuning(mi355_aql_t* h, const mi355_blit_tuning_t* tuning) {
   if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;

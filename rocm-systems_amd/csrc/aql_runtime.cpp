@@ -1,0 +1,213 @@
+// Caller policy over the AQL blit engine: the decisions ROCr takes between the
+// HSA API and core::Blit, restated with the public HSA API
+// (projects/rocr-runtime/runtime/hsa-runtime/core/runtime/runtime.cpp:469-664,
+// hsa.cpp:1170-1184, hsa_ext_amd.cpp:237-294).  Declarations:
+// include/mi355_blit_aql.h.
+#include <hsa/hsa.h>
+#include <hsa/hsa_ext_amd.h>
+
+#include <atomic>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+
+#include "mi355_blit_aql.h"
+
+namespace {
+
+enum class Where { kHost, kHostUnknown, kGpu };
+
+// runtime.cpp:483-500: a pointer inside an allocation the runtime knows belongs
+// to that allocation's owner; anything else is system memory that must be
+// locked before a GPU can touch it.
+struct Placement {
+  Where where = Where::kHostUnknown;
+  bool gpu_can_access = false;  // without locking
+};
+
+int classify(mi355_aql_t* h, const void* ptr, size_t size, Placement* out) {
+  hsa_amd_pointer_info_t info;
+  std::memset(&info, 0, sizeof(info));
+  info.size = sizeof(info);
+  uint32_t n_access = 0;
+  hsa_agent_t* access = nullptr;
+  hsa_status_t st = hsa_amd_pointer_info(ptr, &info, std::malloc, &n_access, &access);
+  if (st != HSA_STATUS_SUCCESS) return static_cast<int>(st);
+  const uint64_t gpu = mi355_aql_gpu_agent(h);
+  Placement p;
+  const char* base = static_cast<const char*>(info.agentBaseAddress);
+  const char* cp = static_cast<const char*>(ptr);
+  const bool known = info.type != HSA_EXT_POINTER_TYPE_UNKNOWN && base != nullptr && base <= cp &&
+                     cp + size <= base + info.sizeInBytes;
+  if (known) {
+    hsa_agent_t owner = info.agentOwner;
+    if (owner.handle == 0 && n_access) owner = access[0];
+    hsa_device_type_t type = HSA_DEVICE_TYPE_CPU;
+    if (owner.handle) hsa_agent_get_info(owner, HSA_AGENT_INFO_DEVICE, &type);
+    p.where = type == HSA_DEVICE_TYPE_GPU ? Where::kGpu : Where::kHost;
+    for (uint32_t i = 0; i < n_access; ++i)
+      if (access[i].handle == gpu) p.gpu_can_access = true;
+    if (owner.handle == gpu) p.gpu_can_access = true;
+  }
+  std::free(access);
+  *out = p;
+  return MI355_BLIT_SUCCESS;
+}
+
+// Locks [ptr, ptr+size) for the GPU when it is host memory the runtime does
+// not know (runtime.cpp:521-535); unlocks on destruction.
+class ScopedLock {
+ public:
+  ScopedLock() = default;
+  ~ScopedLock() {
+    if (host_) hsa_amd_memory_unlock(host_);
+  }
+  int Lock(mi355_aql_t* h, const void* ptr, size_t size, void** agent_ptr) {
+    // a system that refuses to lock existing memory refuses every time
+    static std::atomic<bool> refused{false};
+    if (refused.load()) return MI355_BLIT_ERROR;
+    hsa_agent_t gpu;
+    gpu.handle = mi355_aql_gpu_agent(h);
+    void* mapped = nullptr;
+    hsa_status_t st = hsa_amd_memory_lock(const_cast<void*>(ptr), size, &gpu, 1, &mapped);
+    if (st != HSA_STATUS_SUCCESS) {
+      refused.store(true);
+      return static_cast<int>(st);
+    }
+    host_ = const_cast<void*>(ptr);
+    *agent_ptr = mapped;
+    return MI355_BLIT_SUCCESS;
+  }
+
+ private:
+  void* host_ = nullptr;
+};
+
+// Host<->device copy through the engine's two GPU-visible bounce buffers, for
+// host memory that can neither be reached by the GPU nor locked: while the
+// blit moves one half the host fills (or drains) the other.  to_device says
+// which side is the host's.
+std::mutex g_bounce_lock;  // one bounced copy at a time per process
+
+int bounced_copy(mi355_aql_t* h, void* dst, const void* src, size_t size, bool to_device) {
+  std::lock_guard<std::mutex> g(g_bounce_lock);
+  size_t half = 0;
+  void* buf[2] = {nullptr, nullptr};
+  int rc = mi355_aql_staging(h, &half, &buf[0], &buf[1]);
+  if (rc != MI355_BLIT_SUCCESS) return rc;
+  hsa_signal_t done[2];
+  for (int i = 0; i < 2; ++i)
+    if (hsa_signal_create(0, 0, nullptr, &done[i]) != HSA_STATUS_SUCCESS) {
+      if (i) hsa_signal_destroy(done[0]);
+      return MI355_BLIT_ERROR_OUT_OF_RESOURCES;
+    }
+  auto wait = [&](int i) {
+    while (hsa_signal_wait_scacquire(done[i], HSA_SIGNAL_CONDITION_LT, 1, UINT64_MAX, HSA_WAIT_STATE_ACTIVE) >= 1) {
+    }
+  };
+  const char* s = static_cast<const char*>(src);
+  char* d = static_cast<char*>(dst);
+  size_t prev_off = 0, prev_len = 0;
+  int piece = 0;
+  for (size_t off = 0; off < size && rc == MI355_BLIT_SUCCESS; off += half, ++piece) {
+    const int b = piece & 1;
+    const size_t len = size - off < half ? size - off : half;
+    wait(b);  // the blit that used this half two pieces ago
+    if (to_device) {
+      std::memcpy(buf[b], s + off, len);
+      hsa_signal_store_relaxed(done[b], 1);
+      rc = mi355_aql_copy(h, d + off, buf[b], len, nullptr, 0, done[b].handle);
+    } else {
+      hsa_signal_store_relaxed(done[b], 1);
+      rc = mi355_aql_copy(h, buf[b], s + off, len, nullptr, 0, done[b].handle);
+      // drain the previous piece while this one is in flight
+      if (piece > 0) {
+        wait(b ^ 1);
+        std::memcpy(d + prev_off, buf[b ^ 1], prev_len);
+      }
+      prev_off = off;
+      prev_len = len;
+    }
+  }
+  wait(0);
+  wait(1);
+  if (!to_device && rc == MI355_BLIT_SUCCESS && piece > 0) std::memcpy(d + prev_off, buf[(piece - 1) & 1], prev_len);
+  hsa_signal_destroy(done[0]);
+  hsa_signal_destroy(done[1]);
+  return rc;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi355_hsa_memory_copy(mi355_aql_t* h, void* dst, const void* src, size_t size) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  // hsa.cpp:1174-1180
+  if (dst == nullptr || src == nullptr) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (size == 0) return MI355_BLIT_SUCCESS;
+  Placement ps, pd;
+  int rc = classify(h, src, size, &ps);
+  if (rc == MI355_BLIT_SUCCESS) rc = classify(h, dst, size, &pd);
+  if (rc != MI355_BLIT_SUCCESS) return rc;
+  const bool src_sys = ps.where != Where::kGpu, dst_sys = pd.where != Where::kGpu;
+  // CPU-CPU (runtime.cpp:507-510)
+  if (src_sys && dst_sys) {
+    std::memcpy(dst, src, size);
+    return MI355_BLIT_SUCCESS;
+  }
+  // Same GPU, or GPU-CPU with the host side made visible to the GPU first.
+  // Where existing host memory cannot be locked the copy is bounced instead.
+  ScopedLock lock_src, lock_dst;
+  void* d = dst;
+  const void* s = src;
+  if (src_sys && !ps.gpu_can_access) {
+    void* mapped = nullptr;
+    if (lock_src.Lock(h, src, size, &mapped) != MI355_BLIT_SUCCESS) return bounced_copy(h, dst, src, size, true);
+    s = mapped;
+  }
+  if (dst_sys && !pd.gpu_can_access) {
+    void* mapped = nullptr;
+    if (lock_dst.Lock(h, dst, size, &mapped) != MI355_BLIT_SUCCESS) return bounced_copy(h, dst, src, size, false);
+    d = mapped;
+  }
+  if ((rc = mi355_aql_copy(h, d, s, size, nullptr, 0, 0)) != MI355_BLIT_SUCCESS) return rc;
+  return mi355_aql_wait_idle(h);
+}
+
+int mi355_hsa_amd_memory_fill(mi355_aql_t* h, void* ptr, uint32_t value, size_t count) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  // hsa_ext_amd.cpp:241-247
+  if (ptr == nullptr || (reinterpret_cast<uintptr_t>(ptr) % 4) != 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (count == 0) return MI355_BLIT_SUCCESS;
+  Placement p;
+  int rc = classify(h, ptr, count * sizeof(uint32_t), &p);
+  if (rc != MI355_BLIT_SUCCESS) return rc;
+  // runtime.cpp:640-655: any GPU that can reach the memory fills it
+  if (p.where == Where::kGpu || p.gpu_can_access) {
+    if ((rc = mi355_aql_fill32(h, ptr, value, count, nullptr, 0, 0)) != MI355_BLIT_SUCCESS) return rc;
+    return mi355_aql_wait_idle(h);
+  }
+  // host memory: the full pattern, dword by dword
+  uint32_t* out = static_cast<uint32_t*>(ptr);
+  for (size_t i = 0; i < count; ++i) out[i] = value;
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_hsa_amd_memory_async_copy(mi355_aql_t* h, void* dst, const void* src, size_t size,
+                                    uint32_t num_dep_signals, const uint64_t* dep_signals,
+                                    uint64_t completion_signal) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  // hsa_ext_amd.cpp:258-283
+  if (dst == nullptr || src == nullptr) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if ((num_dep_signals == 0 && dep_signals != nullptr) || (num_dep_signals > 0 && dep_signals == nullptr))
+    return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  for (uint32_t i = 0; i < num_dep_signals; ++i)
+    if (dep_signals[i] == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (completion_signal == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  // hsa_ext_amd.cpp:285-293: size 0 succeeds and leaves the signal alone
+  if (size == 0) return MI355_BLIT_SUCCESS;
+  return mi355_aql_copy(h, dst, src, size, dep_signals, num_dep_signals, completion_signal);
+}
+
+}  // extern "C"

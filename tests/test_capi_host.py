@@ -153,8 +153,8 @@ def test_kernel_choice_matches_reference_predicate(capi_host, oracle):
 def test_aql_library_exports_every_declared_symbol(pkg):
     import torch  # noqa: F401
     header = open(os.path.join(ROOT, "include", "mi355_blit_aql.h")).read()
-    declared = set(re.findall(r"\b(mi355_aql_[a-z0-9_]+)\s*\(", header))
-    assert declared
+    declared = set(re.findall(r"\b(mi355_(?:aql|hsa)_[a-z0-9_]+)\s*\(", header))
+    assert declared and "mi355_hsa_memory_copy" in declared
     lib = C.CDLL(pkg.aql.library_path())
     for name in sorted(declared):
         assert hasattr(lib, name), "library does not export %s" % name

@@ -1,0 +1,170 @@
+"""The stand-ins for hsa_memory_copy, hsa_amd_memory_fill and
+hsa_amd_memory_async_copy (include/mi355_blit_aql.h, csrc/aql_runtime.cpp):
+same answers at the API edge as the reference (hsa.cpp:1170-1184,
+hsa_ext_amd.cpp:237-294) and the same routing by pointer ownership as
+Runtime::CopyMemory / FillMemory (runtime.cpp:469-664), bytes checked against
+the CPU oracle."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+GUARD = 256
+MIB = 1 << 20
+
+
+@pytest.fixture(scope="module")
+def eng(pkg, torch_cuda):
+    e = pkg.aql.AqlBlit(0)
+    yield e
+    e.close()
+
+
+@pytest.fixture(scope="module")
+def signals(pkg, torch_cuda):
+    return pkg.aql.HsaSignals()
+
+
+def _host(n, fill=0xEE):
+    return np.full(n, fill, dtype=np.uint8)
+
+
+@pytest.mark.parametrize("n", [1, 17, 4099, MIB + 3, 9 * MIB + 1])
+def test_memory_copy_all_directions(eng, oracle, rand, torch_cuda, n):
+    """host->device (unregistered host memory is locked for the GPU), device->device,
+    device->host, host->host: one seeded payload goes round and must come back intact."""
+    torch = torch_cuda
+    payload = rand(n + 16, 0xB1170001)
+    dev_a = torch.full((n + 2 * GUARD + 16,), 0xEE, dtype=torch.uint8, device="cuda:0")
+    dev_b = torch.full((n + 2 * GUARD + 16,), 0xEE, dtype=torch.uint8, device="cuda:0")
+    back = _host(n + 2 * GUARD + 16)
+    final = _host(n + 2 * GUARD + 16)
+    torch.cuda.synchronize()
+    ok = eng.lib.mi355_hsa_memory_copy
+    # host (numpy, unknown to the runtime) -> device, odd offsets
+    assert ok(eng.handle, dev_a.data_ptr() + GUARD + 3, payload.ctypes.data + 5, n) == 0
+    # device -> device
+    assert ok(eng.handle, dev_b.data_ptr() + GUARD + 9, dev_a.data_ptr() + GUARD + 3, n) == 0
+    # device -> host
+    assert ok(eng.handle, back.ctypes.data + GUARD + 1, dev_b.data_ptr() + GUARD + 9, n) == 0
+    # host -> host (plain memcpy on the calling thread)
+    assert ok(eng.handle, final.ctypes.data + GUARD + 2, back.ctypes.data + GUARD + 1, n) == 0
+    want_a = _host(n + 2 * GUARD + 16)
+    oracle.oracle_copy(want_a.ctypes.data + GUARD + 3, payload.ctypes.data + 5, n)
+    assert np.array_equal(dev_a.cpu().numpy(), want_a)
+    want_b = _host(n + 2 * GUARD + 16)
+    oracle.oracle_copy(want_b.ctypes.data + GUARD + 9, payload.ctypes.data + 5, n)
+    assert np.array_equal(dev_b.cpu().numpy(), want_b)
+    want_back = _host(n + 2 * GUARD + 16)
+    oracle.oracle_copy(want_back.ctypes.data + GUARD + 1, payload.ctypes.data + 5, n)
+    assert np.array_equal(back, want_back)
+    want_final = _host(n + 2 * GUARD + 16)
+    oracle.oracle_copy(want_final.ctypes.data + GUARD + 2, payload.ctypes.data + 5, n)
+    assert np.array_equal(final, want_final)
+
+
+def test_memory_copy_pinned_host(eng, oracle, rand, torch_cuda):
+    """Host memory allocated through the runtime (pinned) needs no locking."""
+    torch = torch_cuda
+    n = 3 * MIB + 7
+    pinned = torch.empty(n + 64, dtype=torch.uint8, pin_memory=True)
+    payload = rand(n + 64, 0xB1170002)
+    pinned.numpy()[:] = payload
+    dev = torch.full((n + 2 * GUARD,), 0xEE, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    assert eng.hsa_memory_copy(dev.data_ptr() + GUARD, pinned.data_ptr() + 1, n) == 0
+    want = _host(n + 2 * GUARD)
+    oracle.oracle_copy(want.ctypes.data + GUARD, payload.ctypes.data + 1, n)
+    assert np.array_equal(dev.cpu().numpy(), want)
+    out = torch.full((n + 64,), 0xEE, dtype=torch.uint8).pin_memory()
+    assert eng.hsa_memory_copy(out.data_ptr() + 2, dev.data_ptr() + GUARD, n) == 0
+    assert np.array_equal(out.numpy()[2:2 + n], payload[1:1 + n]) and out.numpy()[0] == 0xEE
+
+
+def test_memory_copy_api_edge(eng, torch_cuda):
+    """hsa.cpp:1174-1180"""
+    torch = torch_cuda
+    dev = torch.zeros(64, dtype=torch.uint8, device="cuda:0")
+    inv = 0x1001
+    assert eng.hsa_memory_copy(None, dev.data_ptr(), 8) == inv
+    assert eng.hsa_memory_copy(dev.data_ptr(), None, 8) == inv
+    assert eng.hsa_memory_copy(dev.data_ptr(), dev.data_ptr() + 32, 0) == 0
+
+
+@pytest.mark.parametrize("value", [0xabcdef12, 0xA5C30F1E])
+def test_memory_fill_device_and_host(eng, oracle, torch_cuda, value):
+    """Device memory goes to the blit; plain host memory is filled on the host
+    with the whole 32-bit pattern (the reference's memset there truncates it)."""
+    torch = torch_cuda
+    count = MIB // 4 + 3
+    dev = torch.full((4 * count + 2 * GUARD,), 0xEE, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    off = GUARD + (-(dev.data_ptr() + GUARD)) % 4
+    assert eng.hsa_amd_memory_fill(dev.data_ptr() + off, value, count) == 0
+    want = _host(4 * count + 2 * GUARD)
+    oracle.oracle_fill32(want.ctypes.data + off, value, count)
+    assert np.array_equal(dev.cpu().numpy(), want)
+    host = _host(4 * count + 2 * GUARD)
+    hoff = GUARD + (-(host.ctypes.data + GUARD)) % 4
+    assert eng.hsa_amd_memory_fill(host.ctypes.data + hoff, value, count) == 0
+    want = _host(4 * count + 2 * GUARD)
+    oracle.oracle_fill32(want.ctypes.data + hoff, value, count)
+    assert np.array_equal(host, want)
+    # what the reference's host fallback would have left instead
+    quirk = _host(4 * count + 2 * GUARD)
+    oracle.oracle_ref_host_fill(quirk.ctypes.data + hoff, value, count)
+    assert not np.array_equal(host, quirk)
+
+
+def test_memory_fill_api_edge(eng, torch_cuda):
+    """hsa_ext_amd.cpp:241-247"""
+    torch = torch_cuda
+    dev = torch.zeros(64, dtype=torch.uint8, device="cuda:0")
+    base = dev.data_ptr() + (-dev.data_ptr()) % 4
+    inv = 0x1001
+    assert eng.hsa_amd_memory_fill(None, 1, 4) == inv
+    for off in (1, 2, 3):
+        assert eng.hsa_amd_memory_fill(base + off, 1, 4) == inv
+    assert eng.hsa_amd_memory_fill(base, 1, 0) == 0
+    torch.cuda.synchronize()
+    assert not dev.cpu().numpy().any()
+
+
+def test_async_copy_api_edge_and_completion(eng, signals, oracle, rand, torch_cuda):
+    """hsa_ext_amd.cpp:253-294: argument checks, size 0 leaves the signal alone,
+    a real copy decrements it once; dependencies hold the copy back."""
+    torch = torch_cuda
+    n = 2 * MIB + 5
+    payload = rand(n, 0xB1170003)
+    src = torch.from_numpy(payload).to("cuda:0")
+    dst = torch.full((n + 2 * GUARD,), 0xEE, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    inv = 0x1001
+    done = signals.create(1)
+    dep = signals.create(1)
+    f = eng.lib.mi355_hsa_amd_memory_async_copy
+    assert f(eng.handle, None, src.data_ptr(), n, 0, None, done) == inv
+    assert f(eng.handle, dst.data_ptr(), None, n, 0, None, done) == inv
+    assert f(eng.handle, dst.data_ptr(), src.data_ptr(), n, 1, None, done) == inv      # count without array
+    one = (C.c_uint64 * 1)(dep)
+    assert f(eng.handle, dst.data_ptr(), src.data_ptr(), n, 0, one, done) == inv       # array without count
+    assert f(eng.handle, dst.data_ptr(), src.data_ptr(), n, 0, None, 0) == inv         # no completion signal
+    assert f(eng.handle, dst.data_ptr(), src.data_ptr(), 0, 0, None, done) == 0
+    assert signals.load(done) == 1                                                     # untouched
+    # a copy behind an unsatisfied dependency
+    assert f(eng.handle, dst.data_ptr() + GUARD, src.data_ptr(), n, 1, one, done) == 0
+    import time
+    time.sleep(0.05)
+    assert signals.load(done) == 1
+    torch.cuda.synchronize()
+    assert bool((dst == 0xEE).all())
+    signals.store(dep, 0)
+    signals.wait_below_one(done, active=False)
+    assert signals.load(done) == 0
+    want = _host(n + 2 * GUARD)
+    oracle.oracle_copy(want.ctypes.data + GUARD, payload.ctypes.data, n)
+    assert np.array_equal(dst.cpu().numpy(), want)
+    signals.destroy(done)
+    signals.destroy(dep)

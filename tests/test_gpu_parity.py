@@ -233,6 +233,47 @@ def test_misaligned_1gib_headline(capi, blit, oracle, rand, torch_cuda, so, do):
     assert np.array_equal(got, want)
 
 
+def test_random_copies_and_shapes(capi, fresh_tuning, oracle, arenas):
+    """Seeded random walk over offsets, lengths and launch shapes (the seed and
+    case are in the failure message)."""
+    blit = fresh_tuning
+    src, src_host, dst = arenas
+    rng = np.random.default_rng(0xF00D)
+    for case in range(600):
+        so = int(rng.integers(0, 4096))
+        do = GUARD + int(rng.integers(0, 4096))
+        n = int(max(1, np.floor(2.0 ** (24 * rng.random()))))  # 1 B .. 16 MiB
+        if case % 3 == 0:
+            blit.set_tuning()
+        else:
+            blit.set_tuning(wg_size=int(rng.choice([64, 128, 256, 512, 1024])), unroll=int(rng.choice([1, 2, 4])),
+                            nt_load=int(rng.integers(1, 3)), store_policy=int(rng.integers(1, 5)),
+                            max_grid=int(rng.choice([0, 0, 3, 64])))
+        try:
+            run_copy_case(capi, blit, oracle, src, src_host, dst, so, do, n)
+        except AssertionError as e:
+            raise AssertionError("fuzz case %d (so=%d do=%d n=%d): %s" % (case, so, do, n, e))
+
+
+def test_copy_8gib_grid_limits(capi, blit, torch_cuda):
+    """Twice the largest sweep size: 64-bit indexing and the grid's work-item
+    limit (the plan caps the grid, waves then stride over the tiles)."""
+    torch = torch_cuda
+    n = 8 << 30
+    src = Arena(torch, n)
+    dst = Arena(torch, n + 2 * GUARD, fill=GUARD_BYTE)
+    # a cheap varied pattern: 32-bit counter
+    src.view.view(torch.int32).copy_(torch.arange(n // 4, dtype=torch.int32, device="cuda:0"))
+    torch.cuda.synchronize()
+    check_ok(capi, blit.copy(dst.base + GUARD + 5, src.base + 2, n - 16), "copy")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert torch.equal(dst.view[GUARD + 5:GUARD + 5 + n - 16], src.view[2:2 + n - 16])
+    assert bool((dst.view[:GUARD + 5] == GUARD_BYTE).all())
+    assert bool((dst.view[GUARD + 5 + n - 16:] == GUARD_BYTE).all())
+    p = blit.last_plan()
+    assert p.grid * p.wg_size < 2 ** 31
+
+
 # ------------------------------------------------------------------------- fill
 
 def run_fill_case(capi, blit, oracle, dst, d_off, count, value):

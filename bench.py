@@ -10,7 +10,7 @@ HBM3E peak.  Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
-Workloads: copy (default, the headline), fill, misaligned, batch, and calib (a
+Workloads: copy (default, the headline), fill, misaligned, batch, rect, and calib (a
 plain torch copy_ of the same size: not this library, only the known-size
 kernel that scales the profiler's HBM counters).  Whatever the
 workload, the line also carries the other configurations' figures under
@@ -39,7 +39,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="copy", choices=["copy", "fill", "misaligned", "batch", "calib"])
+    ap.add_argument("--workload", default="copy", choices=["copy", "fill", "misaligned", "batch", "rect", "calib"])
     ap.add_argument("--bytes", type=int, default=GIB, help="transfer size of the copy/fill workloads")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-also", action="store_true", help="skip the secondary configurations")
@@ -52,11 +52,15 @@ def aligned_ptr(t, a=256):
     return p + (-p) % a
 
 
+def seeded_bytes(n, seed):
+    import numpy as np
+    return np.random.default_rng(seed).integers(0, 256, n, dtype=np.uint8)
+
+
 class Runner:
-    def __init__(self, torch, pkg, ora):
+    def __init__(self, torch, pkg):
         self.torch = torch
         self.capi = pkg.capi
-        self.ora = ora
         self.blit = pkg.capi.Blit(0)
         # a stream torch can time: events are recorded on the stream the
         # kernels are launched on
@@ -68,14 +72,13 @@ class Runner:
         import numpy as np
         t = self.torch.empty(n + 512, dtype=self.torch.uint8, device="cuda:0")
         if seed is not None:
-            # seeded on the host by the shared generator, in 64 MiB pieces
+            # seeded on the host, in 64 MiB pieces
             step = 64 * MIB
-            host = np.empty(min(step, n), dtype=np.uint8)
             off = (-t.data_ptr()) % 256
             for lo in range(0, n, step):
                 m = min(step, n - lo)
-                self.ora.oracle_fill_random(host.ctypes.data, m, seed + lo // step)
-                t[off + lo:off + lo + m].copy_(self.torch.from_numpy(host[:m]))
+                host = seeded_bytes(m, seed + lo // step)
+                t[off + lo:off + lo + m].copy_(self.torch.from_numpy(host))
         self.torch.cuda.synchronize()
         return t
 
@@ -111,16 +114,10 @@ def make_copy(r, nbytes, s_off=0, d_off=0):
     fn = lambda: r.check(r.blit.copy(D, S, nbytes, r.stream), "copy")
 
     def verify():
-        # device compare of the whole range, oracle compare of a 64 MiB sample
-        import numpy as np
+        # device compare of the whole range (the parity tests hold the oracle comparison)
         so = (-src.data_ptr()) % 256 + s_off
         do = (-dst.data_ptr()) % 256 + d_off
         assert r.torch.equal(dst[do:do + nbytes], src[so:so + nbytes]), "copy result differs"
-        m = min(nbytes, 64 * MIB)
-        hs = src[so:so + m].cpu().numpy()
-        want = np.empty(m, dtype=np.uint8)
-        r.ora.oracle_copy(want.ctypes.data, hs.ctypes.data, m)
-        assert np.array_equal(dst[do:do + m].cpu().numpy(), want), "copy differs from oracle"
     return fn, verify, 2 * nbytes, (src, dst)
 
 
@@ -165,8 +162,7 @@ def make_batch(r, n=65536, arena=8 * GIB):
     src = r.torch.empty(arena + 512, dtype=r.torch.uint8, device="cuda:0")
     dst = r.torch.empty(arena + 512, dtype=r.torch.uint8, device="cuda:0")
     # seeded 64 MiB block repeated: cheap to make, every region still has varied bytes
-    blk = np.empty(64 * MIB, dtype=np.uint8)
-    r.ora.oracle_fill_random(blk.ctypes.data, blk.size, 0xB1170005)
+    blk = seeded_bytes(64 * MIB, 0xB1170005)
     blk_d = r.torch.from_numpy(blk).to("cuda:0")
     for lo in range(0, arena, blk.size):
         src[lo:lo + blk.size].copy_(blk_d[:min(blk.size, arena - lo)])
@@ -188,6 +184,61 @@ def make_batch(r, n=65536, arena=8 * GIB):
             b = src[sh + int(offs[i] + so[i]):sh + int(offs[i] + so[i] + lens[i])]
             assert r.torch.equal(a, b), "batched copy %d differs" % i
     return fn, verify, int(2 * lens.sum()), (src, dst, descs)
+
+
+def make_rect(r, rows=8192, width=128 * 1024, pitch=256 * 1024, s_x=0, d_x=0):
+    """rows x width bytes out of two pitched 2-D surfaces (rows x pitch each),
+    the region starting s_x / d_x bytes into each row."""
+    import numpy as np
+    total = rows * pitch
+    src = r.torch.empty(total + 512, dtype=r.torch.uint8, device="cuda:0")
+    dst = r.torch.empty(total + 512, dtype=r.torch.uint8, device="cuda:0")
+    blk = seeded_bytes(min(64 * MIB, total), 0xB1170006)
+    blk_d = r.torch.from_numpy(blk).to("cuda:0")
+    for lo in range(0, total, blk.size):
+        m = min(blk.size, total - lo)
+        src[lo:lo + m].copy_(blk_d[:m])
+    dst.zero_()
+    r.torch.cuda.synchronize()
+    S, D = aligned_ptr(src), aligned_ptr(dst)
+    sp, dp = (S, pitch, 0), (D, pitch, 0)
+    fn = lambda: r.check(r.blit.copy_rect(dp, (d_x, 0, 0), sp, (s_x, 0, 0), (width, rows, 1), r.stream), "copy_rect")
+
+    def verify():
+        sh = (-src.data_ptr()) % 256
+        dh = (-dst.data_ptr()) % 256
+        s2 = src[sh:sh + total].view(rows, pitch)
+        d2 = dst[dh:dh + total].view(rows, pitch)
+        assert r.torch.equal(d2[:, d_x:d_x + width], s2[:, s_x:s_x + width]), "rect copy differs"
+        assert int(d2[:, :d_x].max().item() if d_x else 0) == 0, "rect copy wrote in front of the region"
+        if d_x + width < pitch:
+            assert int(d2[:, d_x + width:].max().item()) == 0, "rect copy wrote behind the region"
+    return fn, verify, 2 * rows * width, (src, dst)
+
+
+RECT_SHAPES = (
+    # rows, width, pitch, src x, dst x: 1 GiB moved each (the last two 256 MiB)
+    (8192, 128 * 1024, 256 * 1024, 0, 0),
+    (8192, 128 * 1024 - 7, 256 * 1024 + 4, 3, 9),
+    (262144, 4096, 8192, 0, 0),
+    (1048576, 1024, 2048, 0, 0),
+    (1048576, 256, 512, 0, 0),
+    (1048576, 64, 256, 0, 0),
+)
+
+
+def rect_shapes(r):
+    out = {}
+    for rows, width, pitch, sx, dx in RECT_SHAPES:
+        fn, verify, algo, keep = make_rect(r, rows, width, pitch, sx, dx)
+        _, us = r.time_launches(fn, 10, 2)
+        verify()
+        out["%dx%d/%d+%d,%d" % (rows, width, pitch, sx, dx)] = {
+            "gbs": round(algo / us / 1e3, 1), "us_per_launch": round(us, 2),
+            "unroll": r.blit.last_plan().unroll}
+        del fn, verify, keep
+        r.torch.cuda.empty_cache()
+    return out
 
 
 def size_sweep(r):
@@ -421,8 +472,7 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     pkg = entry.load_package()
-    ora = entry.load_oracle()
-    r = Runner(torch, pkg, ora)
+    r = Runner(torch, pkg)
     nbytes = args.bytes
 
     if args.workload == "copy":
@@ -437,6 +487,10 @@ def main():
         fn, verify, algo, keep = make_copy(r, nbytes - 64, s_off=3, d_off=9)
         name = "misaligned D2D copy, %d MiB - 64 B, src&15=3 dst&15=9" % (nbytes // MIB)
         traffic_key = "misaligned_1GiB" if nbytes == GIB else None
+    elif args.workload == "rect":
+        fn, verify, algo, keep = make_rect(r)
+        name = "pitched 2-D region copy, 8192 rows x 128 KiB out of 256 KiB-pitch surfaces (1 GiB moved)"
+        traffic_key = "rect_8192x128KiB"
     elif args.workload == "calib":
         fn, verify, algo, keep = make_calib(r, nbytes)
         name = "calibration: torch copy_ of %d MiB (not this library)" % (nbytes // MIB)
@@ -459,7 +513,8 @@ def main():
         for key, maker in (("copy_1GiB", lambda: make_copy(r, GIB)),
                            ("fill_1GiB", lambda: make_fill(r, GIB)),
                            ("misaligned_1GiB", lambda: make_copy(r, GIB - 64, s_off=3, d_off=9)),
-                           ("batch_65536", lambda: make_batch(r))):
+                           ("batch_65536", lambda: make_batch(r)),
+                           ("rect_8192x128KiB", lambda: make_rect(r))):
             f2, v2, a2, k2 = maker()
             w2, us2 = r.time_launches(f2, 20, 3)
             v2()
@@ -469,6 +524,7 @@ def main():
             torch.cuda.empty_cache()
         also["small_copy_us"] = small_copy_latency(r)
         also["size_sweep"] = size_sweep(r)
+        also["rect_shapes"] = rect_shapes(r)
         r.torch.cuda.empty_cache()
         also["aql_submission"] = aql_path(r, pkg)
         also["reference_gpu_path"] = reference_gpu_path(r)
@@ -488,7 +544,7 @@ def main():
         "also": also,
     }
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(ora, args.cpu_seconds)
+        line["cpu_baseline"] = cpu_baseline(entry.load_oracle(), args.cpu_seconds)
     r.blit.close()
     print(json.dumps(line))
 

@@ -43,7 +43,8 @@ enum {
   MI355_BLIT_KERNEL_COPY = 0,         /* (src - dst) % 4 == 0 */
   MI355_BLIT_KERNEL_COPY_REALIGN = 1, /* (src - dst) % 4 != 0 */
   MI355_BLIT_KERNEL_FILL = 2,
-  MI355_BLIT_KERNEL_COPY_BATCH = 3
+  MI355_BLIT_KERNEL_COPY_BATCH = 3,
+  MI355_BLIT_KERNEL_COPY_RECT = 4
 };
 
 typedef struct mi355_blit mi355_blit_t;
@@ -98,6 +99,22 @@ typedef struct {
   uint64_t bytes;
 } mi355_blit_desc_t;
 
+/* A pitched pointer and a 3-D extent, laid out as hsa_pitched_ptr_t and
+ * hsa_dim3_t (inc/hsa_ext_amd.h:1842-1846, inc/hsa.h hsa_dim3_s): pitch is the
+ * byte distance between rows, slice between layers; x counts bytes, y rows
+ * and z layers. */
+typedef struct {
+  void* base;
+  size_t pitch;
+  size_t slice;
+} mi355_pitched_ptr_t;
+
+typedef struct {
+  uint32_t x;
+  uint32_t y;
+  uint32_t z;
+} mi355_dim3_t;
+
 /* Replaces BlitKernel::BlitKernel + Initialize (core/runtime/amd_blit_kernel.cpp:
  * 538-591): binds to a GPU, reads its CU count, loads the kernels' code object
  * (what GpuAgent::AssembleShader does for the reference,
@@ -130,6 +147,57 @@ int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwo
  * valid until completion).  Regions must not overlap one another. */
 int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n,
                           int descs_on_device, void* stream);
+
+/* Pitched 3-D region copy as a shader: range->z layers of range->y rows of
+ * range->x bytes, from src at src_offset to dst at dst_offset.  The reference
+ * has this on its SDMA engines only: GpuAgent::DmaCopyRect answers
+ * OUT_OF_RESOURCES when the agent's blits are shader blits
+ * (core/runtime/amd_gpu_agent.cpp:1255-1283), and BlitSdma's
+ * SubmitCopyRectCommand needs 4-byte aligned elements
+ * (inc/hsa_ext_amd.h:1840).  Here any byte alignment of bases, offsets,
+ * pitches and widths is accepted.  One launch, no staging memory.
+ * NULL argument or base -> INVALID_ARGUMENT; a zero in range -> SUCCESS
+ * without a launch (core/runtime/hsa_ext_amd.cpp:367-410); a region that is
+ * not a box inside both surfaces (offset.x + range.x > pitch, offset.y +
+ * range.y > slice / pitch when slice != 0, range.z > 1 with slice == 0:
+ * core/runtime/amd_blit_sdma.cpp:577-585) or more than 2^32-1 rows in all ->
+ * INVALID_ARGUMENT.  Source and destination regions must not
+ * overlap. */
+int mi355_blit_copy_rect(mi355_blit_t* h, const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
+                         const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
+                         const mi355_dim3_t* range, void* stream);
+
+/* How mi355_blit_copy_rect launches a region: pure host arithmetic, for
+ * harnesses.  Rows (and layers) that are contiguous on both sides are merged
+ * first; a region that merges into one run is a linear copy (linear = 1,
+ * width = its bytes).  Otherwise a row is cut into units of 64 * unroll
+ * 16-byte vectors anchored at 256-byte boundaries of its destination, the
+ * last unit of a row taking up to 15 vectors more; `slots` is the largest unit
+ * count of any row and the grid has one wave for each of rows * layers *
+ * slots unit slots.  Rows that touch at most 64 16-byte slots of the
+ * destination are packed instead: lanes_per_row lanes per row (one per slot),
+ * rows * layers * lanes_per_row lanes in all, 64 to a wave; slots and unroll
+ * are 0 then. */
+typedef struct {
+  uint32_t empty;
+  uint32_t linear;
+  uint64_t dst;   /* first byte of the region on each side */
+  uint64_t src;
+  uint64_t width; /* bytes per merged row */
+  uint64_t dst_pitch, dst_slice, src_pitch, src_slice;
+  uint32_t rows, layers;
+  uint32_t slots;
+  uint32_t unroll;
+  uint32_t lanes_per_row;
+  uint32_t reserved;
+  uint32_t wg_size, grid, nt_load, store_policy;
+  uint64_t total_bytes;
+} mi355_blit_rect_plan_t;
+
+int mi355_blit_plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
+                         const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
+                         const mi355_dim3_t* range, const mi355_blit_tuning_t* tuning,
+                         mi355_blit_rect_plan_t* out);
 
 /* Decrements an HSA signal by 1 from the GPU once every command submitted
  * before it on the stream has completed, and wakes its waiters: replaces the

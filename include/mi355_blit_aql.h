@@ -61,6 +61,19 @@ int mi355_aql_fill32(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dword
 int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t n,
                          const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal);
 
+/* Pitched 3-D region copy, asynchronous like mi355_aql_copy: the shader
+ * counterpart of BlitSdmaBase::SubmitCopyRectCommand
+ * (core/inc/amd_blit_sdma.h:68-73), which the reference reaches through
+ * hsa_amd_memory_async_copy_rect -> GpuAgent::DmaCopyRect
+ * (core/runtime/hsa_ext_amd.cpp:367-410, amd_gpu_agent.cpp:1255-1283) on SDMA
+ * engines only.  One dispatch packet behind the dependency barriers.
+ * Argument rules as for mi355_blit_copy_rect; with a zero in range the
+ * dependencies and the completion signal ride on a barrier packet. */
+int mi355_aql_copy_rect(mi355_aql_t* h, const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
+                        const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
+                        const mi355_dim3_t* range, const uint64_t* dep_signals, uint32_t num_deps,
+                        uint64_t completion_signal);
+
 /* Blocks until the queue has drained: the wait BlitKernel's blocking calls do
  * on their completion signal (amd_blit_kernel.cpp:632, 830). */
 int mi355_aql_wait_idle(mi355_aql_t* h);
@@ -135,6 +148,18 @@ int mi355_hsa_amd_memory_fill(mi355_aql_t* h, void* ptr, uint32_t value, size_t 
 int mi355_hsa_amd_memory_async_copy(mi355_aql_t* h, void* dst, const void* src, size_t size,
                                     uint32_t num_dep_signals, const uint64_t* dep_signals,
                                     uint64_t completion_signal);
+
+/* hsa_amd_memory_async_copy_rect for copies this GPU executes
+ * (core/runtime/hsa_ext_amd.cpp:367-410): NULL pointers, a dependency count
+ * that disagrees with the array pointer, a zero completion signal or
+ * dir == 0 (hsaHostToHost) -> INVALID_ARGUMENT; a zero in range -> SUCCESS
+ * without touching the signal (:400-402).  Where the reference then fails with
+ * OUT_OF_RESOURCES unless an SDMA engine is available, this runs the shader. */
+int mi355_hsa_amd_memory_async_copy_rect(mi355_aql_t* h, const mi355_pitched_ptr_t* dst,
+                                         const mi355_dim3_t* dst_offset, const mi355_pitched_ptr_t* src,
+                                         const mi355_dim3_t* src_offset, const mi355_dim3_t* range, int dir,
+                                         uint32_t num_dep_signals, const uint64_t* dep_signals,
+                                         uint64_t completion_signal);
 
 #ifdef __cplusplus
 }

@@ -22,6 +22,43 @@ void oracle_fill32(void* ptr, uint32_t value, size_t count) {
   for (size_t i = 0; i < count; ++i) p[i] = value;
 }
 
+/* inc/hsa_ext_amd.h:1859-1872 */
+void oracle_copy_rect(const oracle_pitched_ptr_t* dst, const oracle_dim3_t* dst_offset,
+                      const oracle_pitched_ptr_t* src, const oracle_dim3_t* src_offset,
+                      const oracle_dim3_t* range) {
+  for (uint32_t z = 0; z < range->z; ++z) {
+    for (uint32_t y = 0; y < range->y; ++y) {
+      uint8_t* d = (uint8_t*)dst->base + (size_t)(dst_offset->z + z) * dst->slice +
+                   (size_t)(dst_offset->y + y) * dst->pitch + dst_offset->x;
+      const uint8_t* s = (const uint8_t*)src->base + (size_t)(src_offset->z + z) * src->slice +
+                         (size_t)(src_offset->y + y) * src->pitch + src_offset->x;
+      memcpy(d, s, range->x);
+    }
+  }
+}
+
+/* core/runtime/hsa_ext_amd.cpp:372-405, core/runtime/amd_blit_sdma.cpp:570-585 */
+int oracle_ref_validate_rect(const oracle_pitched_ptr_t* dst, const oracle_dim3_t* dst_offset,
+                             const oracle_pitched_ptr_t* src, const oracle_dim3_t* src_offset,
+                             const oracle_dim3_t* range, int dir, int* does_work, int* sdma_alignment_ok) {
+  enum { kSuccess = 0, kInvalidArgument = 0x1001 };
+  if (does_work) *does_work = 0;
+  if (sdma_alignment_ok) *sdma_alignment_ok = 1;
+  if (!dst || !src || !dst_offset || !src_offset || !range) return kInvalidArgument;
+  if (dir == 0) return kInvalidArgument; /* hsaHostToHost */
+  if (range->x == 0 || range->y == 0 || range->z == 0) return kSuccess;
+  if (sdma_alignment_ok)
+    *sdma_alignment_ok = ((uintptr_t)dst->base % 4 == 0 && (uintptr_t)src->base % 4 == 0 && dst->pitch % 4 == 0 &&
+                          src->pitch % 4 == 0 && dst->slice % 4 == 0 && src->slice % 4 == 0);
+  if ((uint64_t)src_offset->x + range->x > src->pitch || (uint64_t)dst_offset->x + range->x > dst->pitch)
+    return kInvalidArgument;
+  if (src->slice != 0 && (uint64_t)src_offset->y + range->y > src->slice / src->pitch) return kInvalidArgument;
+  if (dst->slice != 0 && (uint64_t)dst_offset->y + range->y > dst->slice / dst->pitch) return kInvalidArgument;
+  if (range->z > 1 && (src->slice == 0 || dst->slice == 0)) return kInvalidArgument;
+  if (does_work) *does_work = 1;
+  return kSuccess;
+}
+
 /* core/runtime/runtime.cpp:657-661: memset(ptr, value, count * sizeof(uint32_t)). */
 void oracle_ref_host_fill(void* ptr, uint32_t value, size_t count) {
   memset(ptr, (int)value, count * sizeof(uint32_t));

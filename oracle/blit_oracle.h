@@ -27,6 +27,16 @@
  *                         each kernel.  Misaligned offsets and odd lengths are
  *                         not covered by any test the reference holds, so for
  *                         those the memcpy closed form is the only pin.
+ *   oracle_copy_rect      row-by-row memcpy of a pitched 3-D region, the
+ *                         meaning inc/hsa_ext_amd.h:1859-1872 gives the SDMA
+ *                         rect copy ("offsets and range carry x in bytes, y
+ *                         and z in rows and layers").  The reference holds no
+ *                         golden vector for it; pinned against numpy slice
+ *                         assignment on 3-D byte arrays and against guard
+ *                         bytes around the region.
+ *   oracle_ref_validate_rect  the argument checks of
+ *                         hsa_amd_memory_async_copy_rect and
+ *                         BlitSdma::SubmitCopyRectCommand, case by case.
  *   oracle_ref_host_fill  restates the reference's host fallback
  *                         memset(ptr, value, count*4) (runtime.cpp:657-661),
  *                         which keeps only the low byte of the pattern.  It is
@@ -78,6 +88,32 @@ void oracle_copy(void* dst, const void* src, size_t size);
 
 /* count dwords set to value, inc/hsa_ext_amd.h:2261-2281. */
 void oracle_fill32(void* ptr, uint32_t value, size_t count);
+
+/* hsa_pitched_ptr_t / hsa_dim3_t (inc/hsa_ext_amd.h:1842-1846). */
+typedef struct {
+  void* base;
+  size_t pitch;
+  size_t slice;
+} oracle_pitched_ptr_t;
+typedef struct {
+  uint32_t x, y, z;
+} oracle_dim3_t;
+
+/* Pitched 3-D region copy: range.z layers of range.y rows of range.x bytes
+ * (inc/hsa_ext_amd.h:1859-1872). */
+void oracle_copy_rect(const oracle_pitched_ptr_t* dst, const oracle_dim3_t* dst_offset,
+                      const oracle_pitched_ptr_t* src, const oracle_dim3_t* src_offset,
+                      const oracle_dim3_t* range);
+
+/* Status of hsa_amd_memory_async_copy_rect's and SubmitCopyRectCommand's
+ * argument checks (core/runtime/hsa_ext_amd.cpp:372-405,
+ * core/runtime/amd_blit_sdma.cpp:577-585; the SDMA packet's dword-alignment
+ * checks, :570-575, are reported separately in *sdma_alignment_ok).
+ * Returns hsa_status_t values; *does_work is 0 when the call returns SUCCESS
+ * without submitting anything. */
+int oracle_ref_validate_rect(const oracle_pitched_ptr_t* dst, const oracle_dim3_t* dst_offset,
+                             const oracle_pitched_ptr_t* src, const oracle_dim3_t* src_offset,
+                             const oracle_dim3_t* range, int dir, int* does_work, int* sdma_alignment_ok);
 
 /* The reference's host fill fallback, runtime.cpp:657-661 (low byte only). */
 void oracle_ref_host_fill(void* ptr, uint32_t value, size_t count);

@@ -4,7 +4,7 @@ import ctypes as C
 import os
 
 from . import build as _build
-from .capi import (Desc, Plan, Tuning, BlitError, SUCCESS, ERROR, ERROR_INVALID_ARGUMENT,  # noqa: F401
+from .capi import (Desc, Plan, Tuning, PitchedPtr, Dim3, rect_args, BlitError, SUCCESS, ERROR, ERROR_INVALID_ARGUMENT,  # noqa: F401
                    ERROR_NOT_INITIALIZED, ERROR_OUT_OF_RESOURCES)
 
 _U64P = C.POINTER(C.c_uint64)
@@ -15,6 +15,8 @@ SIGNATURES = {
     "mi355_aql_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
     "mi355_aql_fill32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
     "mi355_aql_copy_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
+    "mi355_aql_copy_rect": (C.c_int, [C.c_void_p, C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
+                                      C.POINTER(Dim3), C.POINTER(Dim3), _U64P, C.c_uint32, C.c_uint64]),
     "mi355_aql_wait_idle": (C.c_int, [C.c_void_p]),
     "mi355_aql_pending_bytes": (C.c_uint64, [C.c_void_p]),
     "mi355_aql_enable_profiling": (C.c_int, [C.c_void_p, C.c_int]),
@@ -29,6 +31,9 @@ SIGNATURES = {
     "mi355_hsa_amd_memory_fill": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t]),
     "mi355_hsa_amd_memory_async_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint32,
                                                   _U64P, C.c_uint64]),
+    "mi355_hsa_amd_memory_async_copy_rect": (C.c_int, [C.c_void_p, C.POINTER(PitchedPtr), C.POINTER(Dim3),
+                                                       C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(Dim3),
+                                                       C.c_int, C.c_uint32, _U64P, C.c_uint64]),
 }
 
 _lib = None
@@ -102,6 +107,12 @@ class AqlBlit:
         addr = descs if isinstance(descs, int) or descs is None else C.cast(descs, C.c_void_p)
         return self.lib.mi355_aql_copy_batch(self.handle, addr, n, arr, nd, completion)
 
+    def copy_rect(self, dst, dst_offset, src, src_offset, extent, *, deps=None, completion=0):
+        """dst, src: (base, pitch, slice); offsets and extent: (x bytes, y rows, z layers)."""
+        arr, n = _deps(deps)
+        a = rect_args(dst, dst_offset, src, src_offset, extent)
+        return self.lib.mi355_aql_copy_rect(self.handle, *a, arr, n, completion)
+
     def synchronize(self):
         return self.lib.mi355_aql_wait_idle(self.handle)
 
@@ -137,6 +148,12 @@ class AqlBlit:
     def hsa_amd_memory_async_copy(self, dst, src, nbytes, deps=None, completion=0):
         arr, n = _deps(deps)
         return self.lib.mi355_hsa_amd_memory_async_copy(self.handle, dst, src, nbytes, n, arr, completion)
+
+    def hsa_amd_memory_async_copy_rect(self, dst, dst_offset, src, src_offset, extent, direction=3, deps=None,
+                                       completion=0):
+        arr, n = _deps(deps)
+        a = rect_args(dst, dst_offset, src, src_offset, extent)
+        return self.lib.mi355_hsa_amd_memory_async_copy_rect(self.handle, *a, direction, n, arr, completion)
 
     def command_time_us(self, completion):
         """Device time of the command that completed `completion`, in microseconds

@@ -17,6 +17,7 @@ KERNEL_COPY = 0
 KERNEL_COPY_REALIGN = 1
 KERNEL_FILL = 2
 KERNEL_COPY_BATCH = 3
+KERNEL_COPY_RECT = 4
 
 STORE_CACHED = 0
 STORE_NT = 1
@@ -47,6 +48,35 @@ class Desc(C.Structure):
     _fields_ = [("dst", C.c_void_p), ("src", C.c_void_p), ("bytes", C.c_uint64)]
 
 
+class PitchedPtr(C.Structure):
+    _fields_ = [("base", C.c_void_p), ("pitch", C.c_size_t), ("slice", C.c_size_t)]
+
+
+class Dim3(C.Structure):
+    _fields_ = [("x", C.c_uint32), ("y", C.c_uint32), ("z", C.c_uint32)]
+
+
+class RectPlan(C.Structure):
+    _fields_ = [
+        ("empty", C.c_uint32), ("linear", C.c_uint32), ("dst", C.c_uint64), ("src", C.c_uint64),
+        ("width", C.c_uint64), ("dst_pitch", C.c_uint64), ("dst_slice", C.c_uint64),
+        ("src_pitch", C.c_uint64), ("src_slice", C.c_uint64), ("rows", C.c_uint32), ("layers", C.c_uint32),
+        ("slots", C.c_uint32), ("unroll", C.c_uint32), ("lanes_per_row", C.c_uint32),
+        ("reserved", C.c_uint32), ("wg_size", C.c_uint32), ("grid", C.c_uint32),
+        ("nt_load", C.c_uint32), ("store_policy", C.c_uint32), ("total_bytes", C.c_uint64),
+    ]
+
+
+def rect_args(dst, dst_offset, src, src_offset, extent):
+    """(base, pitch, slice) and (x, y, z) tuples -> ctypes structures; None stays None."""
+    def ptr(t):
+        return None if t is None else PitchedPtr(*t)
+
+    def dim(t):
+        return None if t is None else Dim3(*t)
+    return ptr(dst), dim(dst_offset), ptr(src), dim(src_offset), dim(extent)
+
+
 # every symbol include/mi355_blit.h declares: name -> (restype, argtypes)
 SIGNATURES = {
     "mi355_blit_create": (C.c_int, [C.c_int, C.POINTER(C.c_void_p)]),
@@ -54,6 +84,10 @@ SIGNATURES = {
     "mi355_blit_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "mi355_blit_fill32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t, C.c_void_p]),
     "mi355_blit_copy_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]),
+    "mi355_blit_copy_rect": (C.c_int, [C.c_void_p, C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
+                                       C.POINTER(Dim3), C.POINTER(Dim3), C.c_void_p]),
+    "mi355_blit_plan_rect": (C.c_int, [C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
+                                       C.POINTER(Dim3), C.POINTER(Dim3), C.POINTER(Tuning), C.POINTER(RectPlan)]),
     "mi355_blit_signal_complete": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p]),
     "mi355_blit_add_callback": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "mi355_blit_synchronize": (C.c_int, [C.c_void_p]),
@@ -144,6 +178,11 @@ class Blit:
         addr = descs if isinstance(descs, int) else C.cast(descs, C.c_void_p)
         return self.lib.mi355_blit_copy_batch(self.handle, addr, n, 1 if on_device else 0, stream)
 
+    def copy_rect(self, dst, dst_offset, src, src_offset, extent, stream=None):
+        """dst, src: (base, pitch, slice); offsets and extent: (x bytes, y rows, z layers)."""
+        a = rect_args(dst, dst_offset, src, src_offset, extent)
+        return self.lib.mi355_blit_copy_rect(self.handle, *a, stream)
+
     def synchronize(self):
         return self.lib.mi355_blit_synchronize(self.handle)
 
@@ -177,6 +216,14 @@ def plan_copy(dst, src, nbytes, num_cus=256, tuning=None):
     st = load().mi355_blit_plan_copy(dst, src, nbytes, num_cus,
                                      C.byref(tuning) if tuning is not None else None, C.byref(p))
     return st, p
+
+
+def plan_rect(dst, dst_offset, src, src_offset, extent, tuning=None):
+    """(status, RectPlan) for a region given as in Blit.copy_rect."""
+    out = RectPlan()
+    a = rect_args(dst, dst_offset, src, src_offset, extent)
+    st = load().mi355_blit_plan_rect(*a, tuning, C.byref(out))
+    return st, out
 
 
 def plan_fill(ptr, num_dwords, num_cus=256, tuning=None):

@@ -23,6 +23,7 @@
 #include "blit_args.h"
 #include "blit_kernel_list.h"
 #include "blit_plan.h"
+#include "blit_rect.h"
 #include "mi355_blit_aql.h"
 
 // The gfx950 code object with every kernel variant, linked in as data.
@@ -56,6 +57,8 @@ struct BatchKernel { unsigned split, nt_load, store; const char* name; Kernel k;
 #define MI355_COPY_NAME(U, L, S, R) {U, L, S, R, "mi355_copy_u" #U "_l" #L "_s" #S "_r" #R, {}},
 #define MI355_FILL_NAME(U, S) {U, S, "mi355_fill_u" #U "_s" #S, {}},
 #define MI355_BATCH_NAME(P, L, S) {P, L, S, "mi355_batch_records_p" #P "_l" #L "_s" #S, {}},
+#define MI355_RECT_NAME(U, L, S) {U, L, S, "mi355_rect_u" #U "_l" #L "_s" #S, {}},
+#define MI355_RECT_NARROW_NAME(L, S) {0, L, S, "mi355_rect_narrow_l" #L "_s" #S, {}},
 
 struct BytesWritten {
   uint64_t index;
@@ -100,6 +103,8 @@ struct mi355_aql {
   std::vector<CopyKernel> copy_kernels{MI355_FOR_EACH_COPY_KERNEL(MI355_COPY_NAME)};
   std::vector<FillKernel> fill_kernels{MI355_FOR_EACH_FILL_KERNEL(MI355_FILL_NAME)};
   std::vector<BatchKernel> batch_kernels{MI355_FOR_EACH_BATCH_RECORDS_KERNEL(MI355_BATCH_NAME)};
+  std::vector<BatchKernel> rect_kernels{MI355_FOR_EACH_RECT_KERNEL(MI355_RECT_NAME)};
+  std::vector<BatchKernel> rect_narrow_kernels{MI355_FOR_EACH_RECT_NARROW_KERNEL(MI355_RECT_NARROW_NAME)};
   Kernel scan_local, scan_top, make_records;
 
   hsa_signal_t idle_signal{};  // completion signal of wait_idle's barrier packet
@@ -231,6 +236,10 @@ int load_code_object(mi355_aql* h) {
   for (auto& k : h->fill_kernels)
     if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
   for (auto& k : h->batch_kernels)
+    if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
+  for (auto& k : h->rect_kernels)
+    if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
+  for (auto& k : h->rect_narrow_kernels)
     if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_scan_local", &h->scan_local)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_scan_top", &h->scan_top)) != MI355_BLIT_SUCCESS) return rc;
@@ -775,6 +784,49 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   write_dispatch(h, i++, h->scan_top, &stp, sizeof(stp), 1, 1024, 0, true);
   write_dispatch(h, i++, h->make_records, &mr, sizeof(mr), static_cast<uint32_t>((total_chunks + 255) / 256), 256, 0, true);
   write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true);
+  release_write_index(h, index, total);
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_aql_copy_rect(mi355_aql_t* h, const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
+                        const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
+                        const mi355_dim3_t* range, const uint64_t* dep_signals, uint32_t num_deps,
+                        uint64_t completion_signal) {
+  if (!h || (num_deps && !dep_signals)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (h->queue_error.load()) return MI355_BLIT_ERROR;
+  RectPlan rp;
+  const Kernel* k = nullptr;
+  {
+    std::lock_guard<std::mutex> g(h->lock);
+    int rc = plan_rect(dst, dst_offset, src, src_offset, range, h->has_tuning ? &h->tuning : nullptr, &rp);
+    if (rc != MI355_BLIT_SUCCESS) return rc;
+    if (!rp.empty && !rp.linear) {
+      if (rp.narrow) {
+        for (const auto& v : h->rect_narrow_kernels)
+          if (v.nt_load == rp.streaming && v.store == rp.store_policy) k = &v.k;
+      } else {
+        for (const auto& v : h->rect_kernels)
+          if (v.split == rp.unroll && v.nt_load == rp.streaming && v.store == rp.store_policy) k = &v.k;
+      }
+      if (!k) return MI355_BLIT_ERROR;
+      rect_launch_info(rp, &h->last_plan);
+    }
+  }
+  if (rp.empty) return mi355_aql_copy(h, h, h, 0, dep_signals, num_deps, completion_signal);
+  if (rp.linear) return mi355_aql_copy(h, rp.args.dst, rp.args.src, rp.args.width, dep_signals, num_deps, completion_signal);
+  const uint32_t nb = barrier_packets(num_deps);
+  const uint32_t total = nb + 1;
+  uint64_t index;
+  {
+    std::lock_guard<std::mutex> r(h->reservation_lock);
+    index = acquire_write_index(h, total);
+    record_blit_history(h, rp.total_bytes, index + total - 1);
+  }
+  write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
+  if (rp.narrow)
+    write_dispatch(h, index + nb, *k, &rp.nargs, sizeof(rp.nargs), rp.grid, rp.wg_size, completion_signal, nb != 0);
+  else
+    write_dispatch(h, index + nb, *k, &rp.args, sizeof(rp.args), rp.grid, rp.wg_size, completion_signal, nb != 0);
   release_write_index(h, index, total);
   return MI355_BLIT_SUCCESS;
 }

@@ -210,4 +210,25 @@ int mi355_hsa_amd_memory_async_copy(mi355_aql_t* h, void* dst, const void* src, 
   return mi355_aql_copy(h, dst, src, size, dep_signals, num_dep_signals, completion_signal);
 }
 
+int mi355_hsa_amd_memory_async_copy_rect(mi355_aql_t* h, const mi355_pitched_ptr_t* dst,
+                                         const mi355_dim3_t* dst_offset, const mi355_pitched_ptr_t* src,
+                                         const mi355_dim3_t* src_offset, const mi355_dim3_t* range, int dir,
+                                         uint32_t num_dep_signals, const uint64_t* dep_signals,
+                                         uint64_t completion_signal) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  // hsa_ext_amd.cpp:372-381
+  if (dst == nullptr || src == nullptr || dst_offset == nullptr || src_offset == nullptr || range == nullptr)
+    return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if ((num_dep_signals == 0 && dep_signals != nullptr) || (num_dep_signals > 0 && dep_signals == nullptr))
+    return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (dir == 0 /* hsaHostToHost */) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  for (uint32_t i = 0; i < num_dep_signals; ++i)
+    if (dep_signals[i] == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (completion_signal == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  // hsa_ext_amd.cpp:400-405: an empty range succeeds and leaves the signal alone
+  if (range->x == 0 || range->y == 0 || range->z == 0) return MI355_BLIT_SUCCESS;
+  return mi355_aql_copy_rect(h, dst, dst_offset, src, src_offset, range, dep_signals, num_dep_signals,
+                             completion_signal);
+}
+
 }  // extern "C"

@@ -108,6 +108,48 @@ struct BatchStridedArgs {
   uint32_t n_waves;
 };
 
+// A pitched 3-D region copy: `layers` slices of `rows` rows of `width` bytes.
+// dst and src address the first byte of row 0 in layer 0 (offsets folded in by
+// the host).  Each row is cut into units of 64 * unroll vectors, one per wave;
+// `slots` is the largest unit count any row has, so that unit slot s belongs
+// to row s / slots: no prefix sum and no memory beyond the two regions.
+struct RectArgs {
+  uint8_t* dst;
+  const uint8_t* src;
+  uint64_t dst_pitch;
+  uint64_t dst_slice;
+  uint64_t src_pitch;
+  uint64_t src_slice;
+  uint64_t width;
+  uint32_t rows;
+  uint32_t slots;
+  uint32_t total_slots;  // rows * layers * slots
+  uint32_t waves_per_wg;
+  uint32_t n_waves;
+  uint32_t pad;
+};
+
+// The same region copy for rows of up to about 1 KiB: every 16-byte slot of a
+// row's destination takes a lane, lanes_per_row of them per row, and the
+// (row, slot) pairs of the whole region are dealt out to waves 64 at a time.
+struct RectNarrowArgs {
+  uint8_t* dst;
+  const uint8_t* src;
+  uint64_t dst_pitch;
+  uint64_t dst_slice;
+  uint64_t src_pitch;
+  uint64_t src_slice;
+  uint64_t magic64;  // ceil(2^64 / lanes_per_row): n / lanes_per_row == mulhi(n, magic64), n < 2^38
+  uint32_t width;
+  uint32_t rows;     // rows per layer
+  uint32_t lines;    // rows * layers
+  uint32_t lanes_per_row;
+  uint32_t magic;    // ceil(2^16 / lanes_per_row): n / lanes_per_row == (n * magic) >> 16, n < 128
+  uint32_t waves_per_wg;
+  uint32_t n_waves;
+  uint32_t pad;
+};
+
 // Layout of amd_signal_t (inc/amd_hsa_signal.h, struct amd_signal_s).
 struct HsaSignalAbi {
   int64_t kind;

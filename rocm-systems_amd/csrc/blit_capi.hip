@@ -14,6 +14,7 @@
 
 #include "blit_kernels.h"
 #include "blit_plan.h"
+#include "blit_rect.h"
 #include "mi355_blit.h"
 
 namespace {
@@ -107,11 +108,15 @@ struct DeviceScope {
 typedef void (*copy_kernel_t)(CopyArgs);
 typedef void (*fill_kernel_t)(FillArgs);
 typedef void (*batch_kernel_t)(BatchCopyArgs);
+typedef void (*rect_kernel_t)(RectArgs);
+typedef void (*rect_narrow_kernel_t)(RectNarrowArgs);
 
 // One row per kernel variant, generated from the same list as the kernels.
 struct CopyVariant { unsigned unroll, nt_load, store, realign; copy_kernel_t fn; };
 struct FillVariant { unsigned unroll, store; fill_kernel_t fn; };
 struct BatchVariant { unsigned split, nt_load, store; batch_kernel_t fn; };
+struct RectVariant { unsigned unroll, nt_load, store; rect_kernel_t fn; };
+struct RectNarrowVariant { unsigned nt_load, store; rect_narrow_kernel_t fn; };
 
 #define MI355_COPY_ROW(U, L, S, R) {U, L, S, R, mi355_copy_u##U##_l##L##_s##S##_r##R},
 const CopyVariant kCopyVariants[] = {MI355_FOR_EACH_COPY_KERNEL(MI355_COPY_ROW)};
@@ -119,6 +124,10 @@ const CopyVariant kCopyVariants[] = {MI355_FOR_EACH_COPY_KERNEL(MI355_COPY_ROW)}
 const FillVariant kFillVariants[] = {MI355_FOR_EACH_FILL_KERNEL(MI355_FILL_ROW)};
 #define MI355_BATCH_ROW(P, L, S) {P, L, S, mi355_batch_records_p##P##_l##L##_s##S},
 const BatchVariant kBatchVariants[] = {MI355_FOR_EACH_BATCH_RECORDS_KERNEL(MI355_BATCH_ROW)};
+#define MI355_RECT_ROW(U, L, S) {U, L, S, mi355_rect_u##U##_l##L##_s##S},
+const RectVariant kRectVariants[] = {MI355_FOR_EACH_RECT_KERNEL(MI355_RECT_ROW)};
+#define MI355_RECT_NARROW_ROW(L, S) {L, S, mi355_rect_narrow_l##L##_s##S},
+const RectNarrowVariant kRectNarrowVariants[] = {MI355_FOR_EACH_RECT_NARROW_KERNEL(MI355_RECT_NARROW_ROW)};
 
 copy_kernel_t select_copy_kernel(const mi355_blit_plan_t& p) {
   for (const CopyVariant& v : kCopyVariants)
@@ -137,6 +146,12 @@ fill_kernel_t select_fill_kernel(const mi355_blit_plan_t& p) {
 batch_kernel_t select_batch_kernel(unsigned split, bool ntl, unsigned policy) {
   for (const BatchVariant& v : kBatchVariants)
     if (v.split == split && v.nt_load == (ntl ? 1u : 0u) && v.store == policy) return v.fn;
+  return nullptr;
+}
+
+rect_kernel_t select_rect_kernel(unsigned unroll, bool ntl, unsigned policy) {
+  for (const RectVariant& v : kRectVariants)
+    if (v.unroll == unroll && v.nt_load == (ntl ? 1u : 0u) && v.store == policy) return v.fn;
   return nullptr;
 }
 
@@ -520,6 +535,74 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
   h->staging_busy = true;
   h->last_plan = p;
   return ledger_record(h, s, total_bytes);
+}
+
+int mi355_blit_copy_rect(mi355_blit_t* h, const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
+                         const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
+                         const mi355_dim3_t* range, void* stream) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  RectPlan rp;
+  {
+    std::lock_guard<std::mutex> g(h->lock);
+    int rc = plan_rect(dst, dst_offset, src, src_offset, range, h->has_tuning ? &h->tuning : nullptr, &rp);
+    if (rc != MI355_BLIT_SUCCESS) return rc;
+  }
+  if (rp.empty) return MI355_BLIT_SUCCESS;
+  if (rp.linear) return mi355_blit_copy(h, rp.args.dst, rp.args.src, rp.args.width, stream);
+  std::lock_guard<std::mutex> g(h->lock);
+  DeviceScope scope(h->device);
+  if (scope.err != hipSuccess) return status_of(scope.err);
+  hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
+  if (rp.narrow) {
+    rect_narrow_kernel_t k = nullptr;
+    for (const RectNarrowVariant& v : kRectNarrowVariants)
+      if (v.nt_load == rp.streaming && v.store == rp.store_policy) k = v.fn;
+    if (!k) return MI355_BLIT_ERROR;
+    hipLaunchKernelGGL(k, dim3(rp.grid), dim3(rp.wg_size), 0, s, rp.nargs);
+  } else {
+    rect_kernel_t k = select_rect_kernel(rp.unroll, rp.streaming != 0, rp.store_policy);
+    if (!k) return MI355_BLIT_ERROR;
+    hipLaunchKernelGGL(k, dim3(rp.grid), dim3(rp.wg_size), 0, s, rp.args);
+  }
+  BLIT_HIP(hipGetLastError());
+  rect_launch_info(rp, &h->last_plan);
+  return ledger_record(h, s, rp.total_bytes);
+}
+
+int mi355_blit_plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
+                         const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
+                         const mi355_dim3_t* range, const mi355_blit_tuning_t* tuning,
+                         mi355_blit_rect_plan_t* out) {
+  if (!out) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  RectPlan rp;
+  int rc = plan_rect(dst, dst_offset, src, src_offset, range, tuning, &rp);
+  if (rc != MI355_BLIT_SUCCESS) return rc;
+  *out = mi355_blit_rect_plan_t{};
+  out->empty = rp.empty;
+  out->linear = rp.linear;
+  out->dst = reinterpret_cast<uint64_t>(rp.args.dst);
+  out->src = reinterpret_cast<uint64_t>(rp.args.src);
+  out->width = rp.args.width;
+  out->total_bytes = rp.total_bytes;
+  if (rp.empty || rp.linear) return MI355_BLIT_SUCCESS;
+  out->dst_pitch = rp.args.dst_pitch;
+  out->dst_slice = rp.args.dst_slice;
+  out->src_pitch = rp.args.src_pitch;
+  out->src_slice = rp.args.src_slice;
+  out->rows = rp.args.rows;
+  if (rp.narrow) {
+    out->layers = rp.nargs.lines / rp.nargs.rows;
+    out->lanes_per_row = rp.nargs.lanes_per_row;
+  } else {
+    out->slots = rp.args.slots;
+    out->layers = rp.args.total_slots / (rp.args.slots * rp.args.rows);
+    out->unroll = rp.unroll;
+  }
+  out->wg_size = rp.wg_size;
+  out->grid = rp.grid;
+  out->nt_load = rp.streaming;
+  out->store_policy = rp.store_policy;
+  return MI355_BLIT_SUCCESS;
 }
 
 int mi355_blit_signal_complete(mi355_blit_t* h, uint64_t hsa_signal_handle, void* stream) {

@@ -19,4 +19,11 @@
 #define MI355_BATCH_L_(X, P) MI355_BATCH_S_(X, P, 0) MI355_BATCH_S_(X, P, 1)
 #define MI355_FOR_EACH_BATCH_RECORDS_KERNEL(X) MI355_BATCH_L_(X, 1) MI355_BATCH_L_(X, 2) MI355_BATCH_L_(X, 4)
 
+// X(unroll, nt_load, store_policy): the pitched-region copy
+#define MI355_FOR_EACH_RECT_KERNEL(X) MI355_BATCH_L_(X, 1) MI355_BATCH_L_(X, 2) MI355_BATCH_L_(X, 4)
+
+// X(nt_load, store_policy): the region copy of narrow rows
+#define MI355_RECT_NARROW_S_(X, L) X(L, 0) X(L, 1) X(L, 2) X(L, 3)
+#define MI355_FOR_EACH_RECT_NARROW_KERNEL(X) MI355_RECT_NARROW_S_(X, 0) MI355_RECT_NARROW_S_(X, 1)
+
 #endif  // MI355_BLIT_KERNEL_LIST_H_

@@ -528,6 +528,187 @@ __device__ __forceinline__ void batch_copy_strided_body(const BatchStridedArgs& 
   }
 }
 
+// Pitched 3-D region copy.  Every row is a copy of `width` bytes, cut into
+// units of 64 * U vectors anchored at 256-byte boundaries of its destination
+// like the tiles of a linear copy; one wave moves one unit.  A row's last unit
+// also takes up to kRowOverflowVecs vectors beyond its end (one more vector
+// for a few lanes), so that a row whose destination sits a little above a
+// 256-byte boundary does not need a wave for the spill alone.  Everything
+// follows from the unit's index by arithmetic: unit s is unit s % slots of row
+// s / slots, `slots` being the largest unit count any row has; rows that need
+// fewer skip the rest.  No memory beyond the two regions, one launch.
+constexpr unsigned kRowOverflowVecs = 15;
+
+__device__ __forceinline__ unsigned row_units(unsigned n_virtual, unsigned unit) {
+  return n_virtual > kRowOverflowVecs + unit ? (n_virtual - kRowOverflowVecs + unit - 1) / unit : 1;
+}
+
+template <int U, bool NTL, int NTS>
+__device__ __forceinline__ void rect_copy_body(const RectArgs& a) {
+  constexpr unsigned kUnit = kWave * U;
+  const unsigned lane = threadIdx.x & (kWave - 1);
+  const uint64_t wave = global_wave(a.waves_per_wg);
+  const uint64_t n_waves = a.n_waves;
+  for (uint64_t w = wave; w < a.total_slots; w += n_waves) {
+    const uint32_t slot = static_cast<uint32_t>(w);
+    const uint32_t line = slot / a.slots;  // row index through all layers
+    const uint32_t kq = slot - line * a.slots;
+    const uint32_t layer = line / a.rows;
+    const uint32_t y = line - layer * a.rows;
+    BatchDesc row;
+    row.dst = a.dst + layer * a.dst_slice + y * a.dst_pitch;
+    row.src = a.src + layer * a.src_slice + y * a.src_pitch;
+    row.bytes = a.width;
+    const DescShape sh = desc_shape(row);
+    const unsigned n_virtual = static_cast<unsigned>(sh.n_vec) + sh.lead;
+    const unsigned units = row_units(n_virtual, kUnit);
+    if (kq >= units) continue;
+    const bool last = kq + 1 == units;
+    const unsigned v0 = kq * kUnit;
+    const unsigned lo = v0 > sh.lead ? v0 : sh.lead;
+    const unsigned end = last ? n_virtual : v0 + kUnit;
+    const uint8_t* sb = row.src + sh.head;
+    const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(sb)) & 3;
+    const v4u_a4* sv = reinterpret_cast<const v4u_a4*>(sb - r) - sh.lead;
+    v4u* dv = reinterpret_cast<v4u*>(row.dst + sh.head) - sh.lead;
+    // U vectors per lane, and one more for the overflow of a row's last unit
+    v4u x[U + 1];
+#pragma unroll
+    for (int u = 0; u <= U; ++u) {
+      const unsigned idx = v0 + lane + u * kWave;
+      if (idx >= lo && idx < end) x[u] = ld_v4<NTL>(sv + idx);
+    }
+    // the dword behind the unit's last vector: with r != 0 it holds that
+    // vector's last r bytes
+    unsigned e = 0;
+    if (r && end > lo) e = ld_u32<NTL>(reinterpret_cast<const unsigned*>(sv + end));
+#pragma unroll
+    for (int u = 0; u <= U; ++u) {
+      const unsigned idx = v0 + lane + u * kWave;
+      const unsigned nxt = x[u < U ? u + 1 : u].x;  // lane 0's copy is what lane 63 needs
+      unsigned w4 = wave_rotate_down1(lane == 0 ? nxt : x[u].x);
+      if (idx + 1 == end) w4 = e;
+      if (idx >= lo && idx < end) st_v4<NTS>(dv + idx, realign(x[u], w4, r));
+    }
+    // bytes in front of the first vector and behind the last
+    const unsigned tail = static_cast<unsigned>(row.bytes - sh.head - 16 * sh.n_vec);
+    if (kq == 0 && lane < sh.head) {
+      row.dst[lane] = row.src[lane];
+    } else if (last && lane >= 16 && lane - 16 < tail) {
+      const uint64_t off = sh.head + 16 * sh.n_vec + lane - 16;
+      row.dst[off] = row.src[off];
+    }
+  }
+}
+
+// Moves bytes [off, end) of the 16-byte aligned destination slot `slot`, not
+// all 16 of them; sa is the source of byte off.  Whole dwords where the range
+// has them, single bytes at its ragged ends; the source is read in the aligned
+// dwords that hold at least one wanted byte, all loads before the first store.
+template <bool NTL>
+__device__ __forceinline__ void copy_partial_slot(uintptr_t slot, unsigned off, unsigned end,
+                                                  const uint8_t* sa) {
+  const uintptr_t ss = reinterpret_cast<uintptr_t>(sa) - off;  // source of the slot's byte 0
+  const unsigned r = static_cast<unsigned>(ss) & 3;
+  const unsigned* base = reinterpret_cast<const unsigned*>(ss - r);
+  unsigned wd[5];
+#pragma unroll
+  for (int k = 0; k < 5; ++k) {
+    const int b0 = 4 * k - static_cast<int>(r);  // slot byte the dword starts at
+    const bool wanted = b0 < static_cast<int>(end) && b0 + 4 > static_cast<int>(off);
+    wd[k] = wanted ? ld_u32<NTL>(base + k) : 0u;
+  }
+  const v4u x = {wd[0], wd[1], wd[2], wd[3]};
+  const v4u img = realign(x, wd[4], r);
+  const unsigned o[4] = {img.x, img.y, img.z, img.w};
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const unsigned b_lo = 4u * q > off ? 4u * q : off;
+    const unsigned b_hi = 4u * q + 4 < end ? 4u * q + 4 : end;
+    if (b_hi <= b_lo) continue;
+    if (b_hi - b_lo == 4) {
+      *reinterpret_cast<unsigned*>(slot + 4 * q) = o[q];
+    } else {
+#pragma unroll
+      for (unsigned b = 0; b < 4; ++b)
+        if (4u * q + b >= b_lo && 4u * q + b < b_hi)
+          *reinterpret_cast<uint8_t*>(slot + 4 * q + b) = static_cast<uint8_t>(o[q] >> (8 * b));
+    }
+  }
+}
+
+// 16-byte accesses at any byte address: gfx950 under HSA runs with unaligned
+// global access enabled, and the compiler emits one dwordx4 for these too.
+typedef v4u v4u_a1 __attribute__((aligned(1)));
+
+template <bool NT>
+__device__ __forceinline__ v4u ld_v4_any(const uint8_t* p) {
+  if constexpr (NT) return __builtin_nontemporal_load(reinterpret_cast<const v4u_a1*>(p));
+  else return *reinterpret_cast<const v4u_a1*>(p);
+}
+
+template <int POLICY>
+__device__ __forceinline__ void st_v4_any(uintptr_t p, v4u v) {
+  if constexpr (POLICY == kStoreNt) {
+    __builtin_nontemporal_store(v, reinterpret_cast<v4u_a1*>(p));
+  } else if constexpr (POLICY == kStoreAgentWt || POLICY == kStoreSystemWt) {
+    st_v4<POLICY>(reinterpret_cast<v4u*>(p), v);  // the asm forms take any address
+  } else {
+    *reinterpret_cast<v4u_a1*>(p) = v;
+  }
+}
+
+// Region copy of narrow rows.  With one wave per row a 256-byte row would use
+// a quarter of the wave and the launch would be bound by the rate at which
+// waves start.  Here every 16-byte slot of a row's destination gets a lane:
+// the (row, slot) pairs of the whole region are numbered row by row and wave w
+// takes numbers [64 w, 64 w + 64), whatever rows they belong to, so all lanes
+// work and a wave's loads and stores cover several whole rows.  A slot the row
+// covers completely is one aligned 16-byte store.  A slot cut by the row's
+// first or last byte is moved as the 16 bytes at the row's start or end
+// instead, an unaligned vector that overlaps its neighbour's slot with the
+// same values: no byte loop and no divergence.  Only rows under 16 bytes go
+// through copy_partial_slot.
+template <bool NTL, int NTS>
+__device__ __forceinline__ void rect_narrow_body(const RectNarrowArgs& a) {
+  const unsigned lane = threadIdx.x & (kWave - 1);
+  const uint64_t wave = global_wave(a.waves_per_wg);
+  const uint32_t lpr = a.lanes_per_row;
+  const uint64_t total = static_cast<uint64_t>(a.lines) * lpr;
+  const uint64_t n_groups = (total + kWave - 1) / kWave;
+  for (uint64_t w = wave; w < n_groups; w += a.n_waves) {
+    // row and slot of this lane's number 64 w + lane
+    const uint64_t first = w * kWave;
+    const uint64_t line0 = lpr == 1 ? first : __umul64hi(first, a.magic64);  // first / lpr
+    const unsigned t = static_cast<unsigned>(first - line0 * lpr) + lane;    // < 128
+    const unsigned g = (t * a.magic) >> 16;                                  // t / lpr
+    const unsigned j = t - g * lpr;
+    const uint64_t line = line0 + g;
+    if (line >= a.lines) continue;
+    uint32_t layer = 0, y = static_cast<uint32_t>(line);
+    if (a.lines > a.rows) {
+      layer = static_cast<uint32_t>(line) / a.rows;
+      y = static_cast<uint32_t>(line) - layer * a.rows;
+    }
+    uint8_t* d = a.dst + layer * a.dst_slice + y * a.dst_pitch;
+    const uint8_t* s = a.src + layer * a.src_slice + y * a.src_pitch;
+    const uintptr_t row_lo = reinterpret_cast<uintptr_t>(d);
+    const uintptr_t row_hi = row_lo + a.width;
+    const uintptr_t slot = (row_lo & ~static_cast<uintptr_t>(15)) + 16 * j;
+    if (slot >= row_hi) continue;  // rows that start higher in their first slot need one slot less
+    if (a.width >= 16) {
+      uintptr_t p = slot > row_lo ? slot : row_lo;
+      if (p + 16 > row_hi) p = row_hi - 16;
+      st_v4_any<NTS>(p, ld_v4_any<NTL>(s + (p - row_lo)));
+    } else {
+      const uintptr_t lo = slot > row_lo ? slot : row_lo;
+      const uintptr_t hi = slot + 16 < row_hi ? slot + 16 : row_hi;
+      copy_partial_slot<NTL>(slot, static_cast<unsigned>(lo - slot), static_cast<unsigned>(hi - slot),
+                             s + (lo - row_lo));
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Completion of an HSA signal from the device, queued behind a command.  In
 // the reference the packet processor does this with the dispatch packet's
@@ -563,6 +744,8 @@ __device__ __forceinline__ void signal_complete_body(const SignalArgs& a) {
 //   mi355_copy_u<unroll>_l<nt loads>_s<store policy>_r<realign>
 //   mi355_fill_u<unroll>_s<store policy>
 //   mi355_batch_records_p<waves per chunk>_l<nt loads>_s<store policy>
+//   mi355_rect_u<unroll>_l<nt loads>_s<store policy>
+//   mi355_rect_narrow_l<nt loads>_s<store policy>
 // ---------------------------------------------------------------------------
 #include "blit_kernel_list.h"
 
@@ -585,6 +768,20 @@ MI355_FOR_EACH_FILL_KERNEL(MI355_DEFINE_FILL)
     mi355::batch_copy_records_body<P, L != 0, S>(a);                                   \
   }
 MI355_FOR_EACH_BATCH_RECORDS_KERNEL(MI355_DEFINE_BATCH_RECORDS)
+
+#define MI355_DEFINE_RECT(U, L, S)                                                     \
+  extern "C" __global__ void __launch_bounds__(1024)                                   \
+      mi355_rect_u##U##_l##L##_s##S(mi355::RectArgs a) {                               \
+    mi355::rect_copy_body<U, L != 0, S>(a);                                            \
+  }
+MI355_FOR_EACH_RECT_KERNEL(MI355_DEFINE_RECT)
+
+#define MI355_DEFINE_RECT_NARROW(L, S)                                                 \
+  extern "C" __global__ void __launch_bounds__(1024)                                   \
+      mi355_rect_narrow_l##L##_s##S(mi355::RectNarrowArgs a) {                         \
+    mi355::rect_narrow_body<L != 0, S>(a);                                             \
+  }
+MI355_FOR_EACH_RECT_NARROW_KERNEL(MI355_DEFINE_RECT_NARROW)
 
 extern "C" __global__ void __launch_bounds__(256) mi355_batch_strided_l0_s0(mi355::BatchStridedArgs a) {
   mi355::batch_copy_strided_body<false, mi355::kStoreCached>(a);

@@ -1,0 +1,196 @@
+// Host arithmetic of the pitched 3-D region copy: folds the offsets into the
+// base addresses, merges rows and layers that are contiguous on both sides,
+// and sizes the launch of the rect kernel.  Pure host code, shared by the HIP
+// and the AQL submission paths.
+//
+// The reference hands such copies to its SDMA engines
+// (projects/rocr-runtime/runtime/hsa-runtime/core/runtime/amd_gpu_agent.cpp:
+// 1255-1283) and has no shader for them.
+#ifndef MI355_BLIT_RECT_H_
+#define MI355_BLIT_RECT_H_
+
+#include <stdint.h>
+
+#include "blit_args.h"
+#include "blit_plan.h"
+#include "mi355_blit.h"
+
+namespace mi355 {
+
+// Rows that touch at most this many 16-byte destination slots go to the
+// kernel that packs several rows into a wave.
+constexpr uint32_t kRectNarrowSlots = 64;
+
+struct RectPlan {
+  bool empty;    // a zero in the range: nothing to move
+  bool linear;   // the region is one contiguous run on both sides
+  bool narrow;   // rows of a few hundred bytes: several rows per wave (nargs)
+  RectArgs args; // linear: dst, src and width describe the run
+  RectNarrowArgs nargs;
+  uint64_t total_bytes;
+  uint32_t unroll;     // vectors per lane: a wave moves a unit of 64 * unroll vectors
+  uint32_t streaming;  // non-temporal loads and stores
+  uint32_t store_policy;
+  uint32_t wg_size;
+  uint32_t grid;
+};
+
+// Units of `unit` vectors that a row of `width` bytes is cut into when its
+// destination address is `residue` modulo 256 (row_units in the kernels): the
+// last unit also takes up to 15 vectors of overflow.
+inline uint64_t rect_row_units(uint64_t residue, uint64_t width, uint64_t unit) {
+  uint64_t head = (16 - (residue & 15)) & 15;
+  if (head > width) head = width;
+  const uint64_t n_virtual = (width - head) / 16 + ((residue + head) & 255) / 16;
+  return n_virtual > 15 + unit ? (n_virtual - 15 + unit - 1) / unit : 1;
+}
+
+inline uint64_t rect_gcd(uint64_t a, uint64_t b) {
+  while (b) {
+    const uint64_t t = a % b;
+    a = b;
+    b = t;
+  }
+  return a;
+}
+
+inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset, const mi355_pitched_ptr_t* src,
+                     const mi355_dim3_t* src_offset, const mi355_dim3_t* range, const mi355_blit_tuning_t* t,
+                     RectPlan* out) {
+  if (!dst || !dst_offset || !src || !src_offset || !range || !out) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  *out = RectPlan{};
+  if (range->x == 0 || range->y == 0 || range->z == 0) {
+    out->empty = true;
+    return MI355_BLIT_SUCCESS;
+  }
+  if (!dst->base || !src->base) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  // The region must be a geometric box inside both surfaces
+  // (core/runtime/amd_blit_sdma.cpp:577-585); the dword alignment that file
+  // also demands (:570-575) is a limit of the SDMA packet and not kept.
+  if (uint64_t(src_offset->x) + range->x > src->pitch || uint64_t(dst_offset->x) + range->x > dst->pitch)
+    return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (src->slice != 0 && uint64_t(src_offset->y) + range->y > src->slice / src->pitch)
+    return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (dst->slice != 0 && uint64_t(dst_offset->y) + range->y > dst->slice / dst->pitch)
+    return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (range->z > 1 && (src->slice == 0 || dst->slice == 0)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  uint64_t width = range->x, rows = range->y, layers = range->z;
+  uint64_t dp = dst->pitch, ds = dst->slice, sp = src->pitch, ss = src->slice;
+  uint8_t* d0 = static_cast<uint8_t*>(dst->base) + dst_offset->z * ds + dst_offset->y * dp + dst_offset->x;
+  const uint8_t* s0 = static_cast<const uint8_t*>(src->base) + src_offset->z * ss + src_offset->y * sp + src_offset->x;
+  out->total_bytes = width * rows * layers;
+  // one row per layer: the layers are the rows
+  if (rows == 1) {
+    rows = layers;
+    layers = 1;
+    dp = ds;
+    sp = ss;
+  }
+  // rows that follow one another without a gap on both sides are one row
+  while (rows > 1 && width == dp && width == sp) {
+    width *= rows;
+    rows = layers;
+    layers = 1;
+    dp = ds;
+    sp = ss;
+  }
+  RectArgs& a = out->args;
+  a.dst = d0;
+  a.src = s0;
+  a.width = width;
+  if (rows == 1) {
+    out->linear = true;
+    return MI355_BLIT_SUCCESS;
+  }
+  if (rows * layers > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  a.dst_pitch = dp;
+  a.dst_slice = layers > 1 ? ds : 0;
+  a.src_pitch = sp;
+  a.src_slice = layers > 1 ? ss : 0;
+  a.rows = static_cast<uint32_t>(rows);
+  bool streaming = out->total_bytes >= (4ull << 20);
+  if (t && t->nt_load) streaming = (t->nt_load == 2);
+  out->streaming = streaming;
+  out->store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
+  if (t && t->store_policy >= 1 && t->store_policy <= 4) out->store_policy = t->store_policy - 1;
+
+  // 16-byte destination slots a row touches, at the worst alignment its rows
+  // can have (they differ by multiples of g16 modulo 16)
+  uint64_t g16 = rect_gcd(dp % 16, 16);
+  if (layers > 1) g16 = rect_gcd(ds % 16, g16);
+  uint64_t row_slots = 0;
+  for (uint64_t r = reinterpret_cast<uintptr_t>(d0) % g16; r < 16; r += g16) {
+    const uint64_t c = (r + width + 15) / 16;
+    if (c > row_slots) row_slots = c;
+  }
+  if (row_slots <= kRectNarrowSlots) {
+    out->narrow = true;
+    RectNarrowArgs& n = out->nargs;
+    n.dst = d0;
+    n.src = s0;
+    n.dst_pitch = a.dst_pitch;
+    n.dst_slice = a.dst_slice;
+    n.src_pitch = a.src_pitch;
+    n.src_slice = a.src_slice;
+    n.width = static_cast<uint32_t>(width);
+    n.rows = a.rows;
+    n.lines = static_cast<uint32_t>(rows * layers);
+    n.lanes_per_row = static_cast<uint32_t>(row_slots);
+    n.magic = (65536 + n.lanes_per_row - 1) / n.lanes_per_row;
+    n.magic64 = n.lanes_per_row > 1 ? ~0ull / n.lanes_per_row + 1 : 0;  // unused for 1
+    out->unroll = 1;
+    out->wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size : 256;
+    const uint64_t waves_per_wg = out->wg_size / 64;
+    const uint64_t groups = (rows * layers * n.lanes_per_row + 63) / 64;
+    uint64_t wgs = (groups + waves_per_wg - 1) / waves_per_wg;
+    if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
+    if (wgs * out->wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / out->wg_size;
+    out->grid = static_cast<uint32_t>(wgs);
+    n.waves_per_wg = static_cast<uint32_t>(waves_per_wg);
+    n.n_waves = static_cast<uint32_t>(wgs * waves_per_wg);
+    return MI355_BLIT_SUCCESS;
+  }
+
+  // Measured on MI355X, 1 GiB moved in rows of 1 KiB .. 128 KiB: two vectors
+  // per lane (units of 2 KiB) are best throughout.
+  uint32_t unroll = 2;
+  if (t && (t->unroll == 1 || t->unroll == 2 || t->unroll == 4)) unroll = t->unroll;
+  out->unroll = unroll;
+  // Row destinations differ by multiples of g modulo 256: the largest unit
+  // count over those residues is the number of slots every row gets.
+  uint64_t g = rect_gcd(dp % 256, 256);
+  if (layers > 1) g = rect_gcd(ds % 256, g);
+  uint64_t slots = 0;
+  for (uint64_t r = reinterpret_cast<uintptr_t>(d0) % g; r < 256; r += g) {
+    const uint64_t c = rect_row_units(r, width, 64 * unroll);
+    if (c > slots) slots = c;
+  }
+  const uint64_t total_slots = rows * layers * slots;
+  if (total_slots > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  a.slots = static_cast<uint32_t>(slots);
+  a.total_slots = static_cast<uint32_t>(total_slots);
+  out->wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size : 128;
+  const uint64_t waves_per_wg = out->wg_size / 64;
+  uint64_t wgs = (total_slots + waves_per_wg - 1) / waves_per_wg;
+  if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
+  if (wgs * out->wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / out->wg_size;
+  out->grid = static_cast<uint32_t>(wgs);
+  a.waves_per_wg = static_cast<uint32_t>(waves_per_wg);
+  a.n_waves = static_cast<uint32_t>(wgs * waves_per_wg);
+  return MI355_BLIT_SUCCESS;
+}
+
+inline void rect_launch_info(const RectPlan& rp, mi355_blit_plan_t* p) {
+  *p = mi355_blit_plan_t{};
+  p->kernel = MI355_BLIT_KERNEL_COPY_RECT;
+  p->wg_size = rp.wg_size;
+  p->grid = rp.grid;
+  p->unroll = rp.unroll;
+  p->nt_load = rp.streaming;
+  p->store_policy = rp.store_policy;
+  p->body_vecs = rp.narrow ? rp.nargs.lines : rp.args.total_slots;  // rows, or chunk slots
+}
+
+}  // namespace mi355
+
+#endif  // MI355_BLIT_RECT_H_

@@ -37,6 +37,14 @@ class KernArgs(C.Union):
                 ("raw", C.c_uint8 * 96)]
 
 
+class PitchedPtr(C.Structure):
+    _fields_ = [("base", C.c_void_p), ("pitch", C.c_size_t), ("slice", C.c_size_t)]
+
+
+class Dim3(C.Structure):
+    _fields_ = [("x", C.c_uint32), ("y", C.c_uint32), ("z", C.c_uint32)]
+
+
 class Bounds(C.Structure):
     _fields_ = [("dst_lo", C.c_uint64), ("dst_hi", C.c_uint64),
                 ("src_lo", C.c_uint64), ("src_hi", C.c_uint64)]
@@ -58,12 +66,34 @@ def _declare_oracle(lib):
         "oracle_ref_blit_copy": (i, [vp, vp, sz, i, C.POINTER(Bounds)]),
         "oracle_ref_blit_fill": (i, [vp, u32, sz, i, C.POINTER(Bounds)]),
         "oracle_ref_same_gpu_uses_blit_kernel": (i, [u64, u64]),
+        "oracle_copy_rect": (None, [C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
+                                    C.POINTER(Dim3), C.POINTER(Dim3)]),
+        "oracle_ref_validate_rect": (i, [C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
+                                         C.POINTER(Dim3), C.POINTER(Dim3), i, C.POINTER(i), C.POINTER(i)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
     return lib
+
+
+def oracle_rect(oracle, dst, dst_offset, src, src_offset, extent):
+    """oracle_copy_rect over (base, pitch, slice) and (x, y, z) tuples."""
+    oracle.oracle_copy_rect(PitchedPtr(*dst), Dim3(*dst_offset), PitchedPtr(*src), Dim3(*src_offset), Dim3(*extent))
+
+
+def oracle_validate_rect(oracle, dst, dst_offset, src, src_offset, extent, direction=3):
+    """(status, does_work, sdma_alignment_ok) of the reference's argument checks; None = NULL."""
+    def ptr(t):
+        return None if t is None else PitchedPtr(*t)
+
+    def dim(t):
+        return None if t is None else Dim3(*t)
+    work, aligned = C.c_int(-1), C.c_int(-1)
+    st = oracle.oracle_ref_validate_rect(ptr(dst), dim(dst_offset), ptr(src), dim(src_offset), dim(extent),
+                                         direction, C.byref(work), C.byref(aligned))
+    return st, work.value, aligned.value
 
 
 @pytest.fixture(scope="session")

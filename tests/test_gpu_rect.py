@@ -1,0 +1,243 @@
+"""Parity of the pitched 3-D region copy (mi355_blit_copy_rect,
+mi355_aql_copy_rect, mi355_hsa_amd_memory_async_copy_rect) with the CPU
+oracle, through the C ABI and over both submission paths.  Bit-exact: the
+whole destination surface, everything outside the region included, must equal
+what oracle_copy_rect leaves on the same seeded inputs."""
+import numpy as np
+import pytest
+
+from conftest import oracle_rect
+
+pytestmark = pytest.mark.gpu
+
+GUARD_BYTE = 0xEE
+MIB = 1 << 20
+
+
+class Surface:
+    """A pitched device surface of [layers, rows, pitch] bytes at a chosen
+    address residue modulo 256, with its host image."""
+
+    def __init__(self, torch, shape, residue=0, host=None):
+        self.torch = torch
+        self.shape = shape
+        self.nbytes = int(np.prod(shape))
+        self.t = torch.empty(self.nbytes + 512, dtype=torch.uint8, device="cuda:0")
+        shift = (residue - self.t.data_ptr()) % 256
+        self.base = self.t.data_ptr() + shift
+        self.view = self.t[shift:shift + self.nbytes]
+        self.t.fill_(GUARD_BYTE)
+        if host is not None:
+            self.view.copy_(torch.from_numpy(host.reshape(-1)))
+        torch.cuda.synchronize()
+        self.shift = shift
+
+    def pitched(self, base=None):
+        z, y, x = self.shape
+        return (self.base if base is None else base, x, y * x)
+
+    def whole(self):
+        return self.t.cpu().numpy()
+
+
+def run_rect_case(capi, blit, oracle, rand, sshape, dshape, ext, so, do, s_res=0, d_res=0, seed=1,
+                  flat=False, submit=None):
+    """ext, so, do are (x, y, z).  Returns the launch plan."""
+    import torch
+    src_host = rand(int(np.prod(sshape)), seed)
+    src = Surface(torch, sshape, s_res, host=src_host)
+    dst = Surface(torch, dshape, d_res)
+    sp, dp = src.pitched(), dst.pitched()
+    if flat:  # 2-D surfaces may leave the slice pitch at 0
+        sp, dp = (sp[0], sp[1], 0), (dp[0], dp[1], 0)
+    if submit is None:
+        st = blit.copy_rect(dp, do, sp, so, ext)
+    else:
+        st = submit(dp, do, sp, so, ext)
+    assert st == capi.SUCCESS, "copy_rect returned 0x%x" % st
+    assert blit.synchronize() == capi.SUCCESS
+    got = dst.whole()
+    want = np.full(got.size, GUARD_BYTE, dtype=np.uint8)
+    oracle_rect(oracle, (want.ctypes.data + dst.shift,) + dp[1:], do, (src_host.ctypes.data,) + sp[1:], so, ext)
+    bad = np.flatnonzero(got != want)
+    assert bad.size == 0, "first mismatch at surface byte %d of %d (%d wrong)" % (
+        bad[0] - dst.shift, dst.nbytes, bad.size)
+    return blit.last_plan()
+
+
+CASES = [
+    # sshape (z, y, pitch), dshape, extent (x, y, z), src offset, dst offset, src residue, dst residue
+    ((1, 16, 300), (1, 12, 517), (100, 7, 1), (13, 2, 0), (5, 3, 0), 0, 0),
+    ((1, 16, 300), (1, 12, 517), (100, 7, 1), (13, 2, 0), (5, 3, 0), 7, 201),
+    ((4, 9, 1031), (5, 11, 1500), (1000, 5, 3), (31, 4, 1), (499, 6, 2), 3, 9),
+    ((1, 64, 131072), (1, 64, 131072), (65536, 64, 1), (0, 0, 0), (65536, 0, 0), 0, 0),
+    ((1, 64, 131072), (1, 70, 131072 + 256), (65536, 64, 1), (1, 0, 0), (48, 3, 0), 0, 0),
+    ((1, 4096, 256), (1, 4096, 256), (64, 4096, 1), (64, 0, 0), (128, 0, 0), 0, 0),
+    ((1, 4096, 256), (1, 4096, 260), (64, 4096, 1), (63, 0, 0), (130, 0, 0), 0, 0),
+    ((3, 300, 37), (3, 301, 41), (1, 300, 3), (36, 0, 0), (0, 1, 0), 1, 255),
+    ((2, 50, 4096), (2, 50, 4096), (4096, 50, 2), (0, 0, 0), (0, 0, 0), 0, 0),       # merges into one run
+    ((2, 64, 4096), (2, 50, 4096), (4096, 50, 2), (0, 14, 0), (0, 0, 0), 0, 16),     # merges into two rows
+    ((8, 1, 5000), (8, 3, 6000), (4999, 1, 8), (1, 0, 0), (2, 2, 0), 5, 6),          # one row per layer
+    ((1, 1, 70000), (1, 1, 90000), (66000, 1, 1), (1234, 0, 0), (4321, 0, 0), 2, 3),  # a single row
+    ((1, 33, 9001), (1, 35, 9473), (8999, 33, 1), (1, 0, 0), (471, 2, 0), 0, 0),
+    ((2, 17, 20000), (3, 19, 21000), (16385, 17, 2), (3000, 0, 0), (17, 1, 1), 11, 13),
+    ((1, 2048, 4096), (1, 2048, 8192), (2048, 2048, 1), (2048, 0, 0), (4096, 0, 0), 0, 0),  # 4 MiB: streaming
+]
+
+
+@pytest.mark.parametrize("case", range(len(CASES)))
+def test_rect_cases_are_exact(capi, blit, oracle, rand, case):
+    sshape, dshape, ext, so, do, s_res, d_res = CASES[case]
+    run_rect_case(capi, blit, oracle, rand, sshape, dshape, ext, so, do, s_res, d_res, seed=0x2EC70000 + case)
+
+
+def test_rect_flat_surfaces_need_no_slice(capi, blit, oracle, rand):
+    run_rect_case(capi, blit, oracle, rand, (1, 40, 3000), (1, 50, 3100), (2999, 40, 1), (1, 0, 0), (99, 10, 0),
+                  flat=True, seed=77)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_rect_random_regions(capi, fresh_tuning, oracle, rand, seed):
+    """Seeded regions with every alignment of bases, pitches, offsets and
+    widths, under random launch shapes."""
+    blit = fresh_tuning
+    rng = np.random.default_rng(0x5EC7 + seed)
+    sshape = tuple(int(v) for v in rng.integers(1, [5, 40, 12000]))
+    dshape = tuple(int(v) for v in rng.integers(1, [5, 40, 12000]))
+    ext = [int(rng.integers(1, min(sshape[k], dshape[k]) + 1)) for k in range(3)]
+    so = [int(rng.integers(0, sshape[k] - ext[k] + 1)) for k in range(3)]
+    do = [int(rng.integers(0, dshape[k] - ext[k] + 1)) for k in range(3)]
+    if seed % 2:
+        blit.set_tuning(wg_size=int(rng.choice([64, 128, 256, 512, 1024])), unroll=int(rng.choice([1, 2, 4])),
+                        max_grid=int(rng.choice([0, 1, 7, 300])), nt_load=int(rng.integers(0, 3)),
+                        store_policy=int(rng.integers(0, 5)))
+    run_rect_case(capi, blit, oracle, rand, sshape, dshape, tuple(ext[::-1]), tuple(so[::-1]), tuple(do[::-1]),
+                  int(rng.integers(0, 256)), int(rng.integers(0, 256)), seed=0x7EC70000 + seed)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_rect_random_narrow_rows(capi, fresh_tuning, oracle, rand, seed):
+    """Rows of 1..1100 bytes, the widths that are packed several rows to a wave
+    (and the first ones beyond), many rows, every alignment."""
+    blit = fresh_tuning
+    rng = np.random.default_rng(0xA220 + seed)
+    widest = 700 if seed < 16 else 1400
+    sshape = tuple(int(v) for v in rng.integers(1, [5, 700, widest]))
+    dshape = tuple(int(v) for v in rng.integers(1, [5, 700, widest]))
+    ext = [int(rng.integers(1, min(sshape[k], dshape[k]) + 1)) for k in range(3)]
+    ext[2] = min(ext[2], 1100)
+    if seed % 3 == 0:  # pitches that keep every row at one alignment
+        sshape = (sshape[0], sshape[1], (sshape[2] + 15) // 16 * 16)
+        dshape = (dshape[0], dshape[1], (dshape[2] + 15) // 16 * 16)
+    so = [int(rng.integers(0, sshape[k] - ext[k] + 1)) for k in range(3)]
+    do = [int(rng.integers(0, dshape[k] - ext[k] + 1)) for k in range(3)]
+    if seed % 2:
+        blit.set_tuning(wg_size=int(rng.choice([64, 256, 1024])), max_grid=int(rng.choice([0, 1, 5])),
+                        nt_load=int(rng.integers(0, 3)), store_policy=int(rng.integers(0, 5)))
+    run_rect_case(capi, blit, oracle, rand, sshape, dshape, tuple(ext[::-1]), tuple(so[::-1]), tuple(do[::-1]),
+                  int(rng.integers(0, 256)), int(rng.integers(0, 256)), seed=0x7A220000 + seed)
+
+
+def test_rect_plan_shapes(capi, blit, oracle, rand):
+    """What the launch record says: a rect kernel with one wave per 2 KiB of
+    row for aligned rows, a linear copy when the region is one run."""
+    p = run_rect_case(capi, blit, oracle, rand, (1, 64, 16384), (1, 64, 16384), (8192, 64, 1), (0, 0, 0), (8192, 0, 0))
+    assert p.kernel == capi.KERNEL_COPY_RECT and p.body_vecs == 64 * 4 and p.unroll == 2
+    assert p.grid * (p.wg_size // 64) == 64 * 4
+    p = run_rect_case(capi, blit, oracle, rand, (1, 64, 8192), (1, 64, 8192), (8192, 64, 1), (0, 0, 0), (0, 0, 0))
+    assert p.kernel == capi.KERNEL_COPY
+
+
+def test_rect_argument_checks(capi, blit, torch_cuda):
+    torch = torch_cuda
+    buf = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    d = (buf.data_ptr(), 256, 256 * 16)
+    s = (buf.data_ptr() + (1 << 15), 256, 256 * 16)
+    z = (0, 0, 0)
+    ok = [d, z, s, z, (64, 4, 2)]
+    for missing in range(5):
+        args = list(ok)
+        args[missing] = None
+        assert blit.copy_rect(*args) == capi.ERROR_INVALID_ARGUMENT
+    assert blit.copy_rect((0, 256, 0), z, s, z, (64, 4, 1)) == capi.ERROR_INVALID_ARGUMENT
+    assert blit.copy_rect(d, (200, 0, 0), s, z, (64, 4, 2)) == capi.ERROR_INVALID_ARGUMENT      # width out of range
+    assert blit.copy_rect(d, z, s, (0, 13, 0), (64, 4, 2)) == capi.ERROR_INVALID_ARGUMENT       # height out of range
+    assert blit.copy_rect((d[0], 256, 0), z, s, z, (64, 4, 2)) == capi.ERROR_INVALID_ARGUMENT   # slice needed
+    for ext in ((0, 4, 2), (64, 0, 2), (64, 4, 0)):
+        assert blit.copy_rect(d, z, s, z, ext) == capi.SUCCESS
+    assert blit.synchronize() == capi.SUCCESS
+    assert int(buf.sum().item()) == 0
+
+
+def test_rect_one_gib_region(capi, blit, oracle, rand, torch_cuda):
+    """8192 rows of 128 KiB out of 256 KiB-pitch surfaces: 1 GiB moved.  The
+    whole destination is checked on the device against torch's own strided
+    view assignment, and sampled rows against the oracle on the host."""
+    torch = torch_cuda
+    rows, pitch, width = 8192, 256 * 1024, 128 * 1024
+    seedrow = torch.from_numpy(rand(pitch + 4096, 0x16187EC7)).to("cuda:0")
+    src = torch.empty(rows * pitch, dtype=torch.uint8, device="cuda:0")
+    s2 = src.view(rows, pitch)
+    for blk in range(0, rows, 1024):  # every row differs: rotate the seed row
+        idx = (torch.arange(blk, blk + 1024, device="cuda:0") * 37 % 4096)[:, None] + \
+            torch.arange(pitch, device="cuda:0")[None, :]
+        s2[blk:blk + 1024] = seedrow[idx]
+        del idx
+    dst = torch.full((rows * pitch,), GUARD_BYTE, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    so, do = (4096 + 3, 0, 0), (65536 + 16, 0, 0)
+    st = blit.copy_rect((dst.data_ptr(), pitch, 0), do, (src.data_ptr(), pitch, 0), so, (width, rows, 1))
+    assert st == capi.SUCCESS and blit.synchronize() == capi.SUCCESS
+    p = blit.last_plan()
+    assert p.kernel == capi.KERNEL_COPY_RECT and p.nt_load == 1
+    d2 = dst.view(rows, pitch)
+    assert torch.equal(d2[:, do[0]:do[0] + width], s2[:, so[0]:so[0] + width])
+    assert bool((d2[:, :do[0]] == GUARD_BYTE).all()) and bool((d2[:, do[0] + width:] == GUARD_BYTE).all())
+    for y in (0, 1, 63, 4095, 8190, 8191):
+        src_row = s2[y].cpu().numpy()
+        want = np.full(pitch, GUARD_BYTE, dtype=np.uint8)
+        oracle_rect(oracle, (want.ctypes.data, pitch, 0), (do[0], 0, 0), (src_row.ctypes.data, pitch, 0),
+                    (so[0], 0, 0), (width, 1, 1))
+        assert np.array_equal(d2[y].cpu().numpy(), want)
+
+
+def test_async_copy_rect_stand_in(capi, pkg, oracle, rand, torch_cuda):
+    """mi355_hsa_amd_memory_async_copy_rect: the reference's answers at the API
+    edge (hsa_ext_amd.cpp:367-410), dependencies honoured, the completion signal
+    decremented once, bytes as the oracle's."""
+    eng = pkg.aql.AqlBlit(0)
+    sig = pkg.aql.HsaSignals()
+    try:
+        dep, done = sig.create(1), sig.create(1)
+
+        def submit(dp, do, sp, so, ext):
+            st = eng.hsa_amd_memory_async_copy_rect(dp, do, sp, so, ext, 3, [dep], done)
+            assert sig.load(done) == 1          # blocked behind the dependency
+            sig.store(dep, 0)
+            sig.wait_below_one(done)
+            assert sig.load(done) == 0
+            return st
+        run_rect_case(capi, eng, oracle, rand, (2, 30, 5000), (2, 31, 5100), (4097, 29, 2), (3, 1, 0), (1, 0, 0),
+                      5, 250, seed=99, submit=submit)
+        d, s, z, ext = (0x1000, 64, 0), (0x2000, 64, 0), (0, 0, 0), (8, 2, 1)
+        f = eng.hsa_amd_memory_async_copy_rect
+        assert f(d, z, s, z, ext, 0, None, done) == capi.ERROR_INVALID_ARGUMENT           # hsaHostToHost
+        assert f(d, z, s, z, ext, 3, None, 0) == capi.ERROR_INVALID_ARGUMENT              # no completion signal
+        for missing in range(5):
+            args = [d, z, s, z, ext]
+            args[missing] = None
+            assert f(*args, 3, None, done) == capi.ERROR_INVALID_ARGUMENT
+        arr = (pkg.aql.C.c_uint64 * 1)(dep)
+        lib = eng.lib.mi355_hsa_amd_memory_async_copy_rect
+        a = pkg.capi.rect_args(d, z, s, z, ext)
+        assert lib(eng.handle, *a, 3, 0, arr, done) == capi.ERROR_INVALID_ARGUMENT        # array without a count
+        assert lib(eng.handle, *a, 3, 1, None, done) == capi.ERROR_INVALID_ARGUMENT       # count without an array
+        sig.store(done, 1)
+        assert f(d, z, s, z, (8, 0, 1), 3, None, done) == capi.SUCCESS                    # empty: signal untouched
+        assert eng.synchronize() == capi.SUCCESS
+        assert sig.load(done) == 1
+        sig.destroy(dep)
+        sig.destroy(done)
+    finally:
+        eng.close()

@@ -18,6 +18,7 @@
 #define MI355_ROCR_BLIT_H_
 
 #include <hsa/hsa.h>
+#include <hsa/hsa_ext_amd.h>
 #include <stdint.h>
 
 #include <atomic>
@@ -202,6 +203,15 @@ class BlitKernelGfx950Aql : public core::Blit {
   hsa_status_t SubmitBatchCopyCommand(const void* descs, size_t n, bool descs_on_device,
                                       std::vector<core::Signal*>& dep_signals,
                                       core::Signal& out_signal);
+  /// Pitched 3-D region copy with the signature of BlitSdmaBase::SubmitCopyRectCommand
+  /// (core/inc/amd_blit_sdma.h:68-73), so that GpuAgent::DmaCopyRect
+  /// (core/runtime/amd_gpu_agent.cpp:1255-1283) can call a shader blit where it
+  /// now answers OUT_OF_RESOURCES.  Any byte alignment; the region must be a
+  /// box inside both surfaces (amd_blit_sdma.cpp:577-585).
+  hsa_status_t SubmitCopyRectCommand(const hsa_pitched_ptr_t* dst, const hsa_dim3_t* dst_offset,
+                                     const hsa_pitched_ptr_t* src, const hsa_dim3_t* src_offset,
+                                     const hsa_dim3_t* range, std::vector<core::Signal*>& dep_signals,
+                                     core::Signal& out_signal);
   hsa_status_t EnableProfiling(bool enable) override;
   uint64_t PendingBytes() override;
   void GangLeader(bool) override {}

@@ -101,6 +101,24 @@ hsa_status_t BlitKernelGfx950Aql::SubmitBatchCopyCommand(const void* descs, size
                                      core::Signal::Convert(&out_signal).handle));
 }
 
+static_assert(sizeof(hsa_pitched_ptr_t) == sizeof(mi355_pitched_ptr_t) && sizeof(hsa_dim3_t) == sizeof(mi355_dim3_t),
+              "the C ABI's pitched pointer and extent are laid out as HSA's");
+
+hsa_status_t BlitKernelGfx950Aql::SubmitCopyRectCommand(const hsa_pitched_ptr_t* dst, const hsa_dim3_t* dst_offset,
+                                                        const hsa_pitched_ptr_t* src, const hsa_dim3_t* src_offset,
+                                                        const hsa_dim3_t* range,
+                                                        std::vector<core::Signal*>& dep_signals,
+                                                        core::Signal& out_signal) {
+  if (blit_ == nullptr) return HSA_STATUS_ERROR_NOT_INITIALIZED;
+  const std::vector<uint64_t> deps = handles(dep_signals);
+  return to_hsa(mi355_aql_copy_rect(blit_, reinterpret_cast<const mi355_pitched_ptr_t*>(dst),
+                                    reinterpret_cast<const mi355_dim3_t*>(dst_offset),
+                                    reinterpret_cast<const mi355_pitched_ptr_t*>(src),
+                                    reinterpret_cast<const mi355_dim3_t*>(src_offset),
+                                    reinterpret_cast<const mi355_dim3_t*>(range), deps.empty() ? nullptr : deps.data(),
+                                    static_cast<uint32_t>(deps.size()), core::Signal::Convert(&out_signal).handle));
+}
+
 hsa_status_t BlitKernelGfx950Aql::EnableProfiling(bool enable) {
   // amd_blit_kernel.cpp:839-842: the queue's profiling bit
   if (blit_ == nullptr) return HSA_STATUS_ERROR_NOT_INITIALIZED;

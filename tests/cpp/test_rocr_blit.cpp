@@ -315,6 +315,41 @@ void test_batch(Blit& blit, const BatchFn& submit_batch) {
   std::printf("PASS %s%s\n", name, g_suffix.c_str());
 }
 
+// A 3-D box out of one pitched surface into another, behind a dependency:
+// what GpuAgent::DmaCopyRect would submit.
+void test_copy_rect(BlitKernelGfx950Aql& blit) {
+  const char* name = "copy_rect_with_signal";
+  const size_t s_pitch = 5011, s_rows = 40, d_pitch = 6001, d_rows = 37, layers = 3;
+  std::vector<uint8_t> src_h = seeded(s_pitch * s_rows * layers, 0xB1170061);
+  DeviceBuf src(src_h.size()), dst(d_pitch * d_rows * layers);
+  REQUIRE(src.p && dst.p, "hipMalloc");
+  REQUIRE(src.upload(src_h), "upload");
+  std::vector<uint8_t> want(dst.n, kGuardByte), got;
+  REQUIRE(dst.upload(want), "upload");
+  hsa_pitched_ptr_t sp{src.p, s_pitch, s_pitch * s_rows}, dp{dst.p, d_pitch, d_pitch * d_rows};
+  hsa_dim3_t so{7, 3, 1}, dof{1001, 2, 0}, range{4999, 33, 2};
+  oracle_pitched_ptr_t osp{src_h.data(), s_pitch, s_pitch * s_rows}, odp{want.data(), d_pitch, d_pitch * d_rows};
+  oracle_dim3_t oso{so.x, so.y, so.z}, odo{dof.x, dof.y, dof.z}, orange{range.x, range.y, range.z};
+  oracle_copy_rect(&odp, &odo, &osp, &oso, &orange);
+  hsa_signal_t dep = make_signal(1), done = make_signal(1);
+  Signal dep_sig(dep), done_sig(done);
+  std::vector<Signal*> deps{&dep_sig};
+  REQUIRE(blit.SubmitCopyRectCommand(&dp, &dof, &sp, &so, &range, deps, done_sig) == HSA_STATUS_SUCCESS, "submit");
+  REQUIRE(hsa_signal_load_relaxed(done) == 1, "ran before its dependency");
+  hsa_signal_store_screlease(dep, 0);
+  REQUIRE(wait_zero(done, HSA_WAIT_STATE_BLOCKED), "rect copy never completed");
+  REQUIRE(dst.download(got), "download");
+  REQUIRE(got == want, "bytes differ");
+  // not a box inside the surface: refused like amd_blit_sdma.cpp:577-579
+  hsa_dim3_t wide{static_cast<uint32_t>(d_pitch), 1, 1};
+  std::vector<Signal*> none;
+  REQUIRE(blit.SubmitCopyRectCommand(&dp, &dof, &sp, &so, &wide, none, done_sig) == HSA_STATUS_ERROR_INVALID_ARGUMENT,
+          "width out of range accepted");
+  hsa_signal_destroy(dep);
+  hsa_signal_destroy(done);
+  std::printf("PASS %s%s\n", name, g_suffix.c_str());
+}
+
 void test_threads(Blit& blit) {
   const char* name = "concurrent_submitters";
   const int kThreads = 4, kPer = 6;
@@ -417,7 +452,7 @@ int main(int argc, char** argv) {
     for (const char* engine : {"_hip", "_aql"})
       for (const char* c : cases) std::printf("%s%s\n", c, engine);
     std::printf("async_copy_blocked_wait_hip_callback\nchain_a_to_b_to_c_hip_callback\n"
-                "profiling_timestamps_aql\n");
+                "profiling_timestamps_aql\ncopy_rect_with_signal_aql\n");
     return 0;
   }
   if (hsa_init() != HSA_STATUS_SUCCESS) {
@@ -481,7 +516,10 @@ int main(int argc, char** argv) {
     test_zero_size_and_bad_args(*blit);
     test_batch(*blit, batch);
     test_threads(*blit);
-    if (engine == 1) test_profiling_timestamps(*blit);
+    if (engine == 1) {
+      test_profiling_timestamps(*blit);
+      test_copy_rect(*static_cast<BlitKernelGfx950Aql*>(blit));
+    }
     latency_report(*blit, engine == 0 ? "hip_device_signal" : "aql");
     hsa_status_t st = blit->Destroy(agent);
     if (st != HSA_STATUS_SUCCESS) {

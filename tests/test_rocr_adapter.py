@@ -59,7 +59,7 @@ def test_native_driver_lists_its_cases(pkg):
     out = subprocess.run([exe, "--list"], stdout=subprocess.PIPE, text=True, check=True).stdout.split()
     for engine in ("_hip", "_aql"):
         assert "dependencies_6" + engine in out and "async_copy_blocked_wait" + engine in out
-    assert "profiling_timestamps_aql" in out and len(out) >= 24
+    assert "profiling_timestamps_aql" in out and "copy_rect_with_signal_aql" in out and len(out) >= 25
 
 
 @pytest.mark.gpu

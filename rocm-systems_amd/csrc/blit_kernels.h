@@ -78,6 +78,27 @@ __device__ __forceinline__ void st_v4(v4u* p, v4u v) {
   }
 }
 
+// 16-byte accesses at any byte address: gfx950 under HSA runs with unaligned
+// global access enabled, and the compiler emits one dwordx4 for these too.
+typedef v4u v4u_a1 __attribute__((aligned(1)));
+
+template <bool NT>
+__device__ __forceinline__ v4u ld_v4_any(const uint8_t* p) {
+  if constexpr (NT) return __builtin_nontemporal_load(reinterpret_cast<const v4u_a1*>(p));
+  else return *reinterpret_cast<const v4u_a1*>(p);
+}
+
+template <int POLICY>
+__device__ __forceinline__ void st_v4_any(uintptr_t p, v4u v) {
+  if constexpr (POLICY == kStoreNt) {
+    __builtin_nontemporal_store(v, reinterpret_cast<v4u_a1*>(p));
+  } else if constexpr (POLICY == kStoreAgentWt || POLICY == kStoreSystemWt) {
+    st_v4<POLICY>(reinterpret_cast<v4u*>(p), v);  // the asm forms take any address
+  } else {
+    *reinterpret_cast<v4u_a1*>(p) = v;
+  }
+}
+
 // Lane i receives the value lane (i + 1) % 64 passed in (DPP wave_rol:1).
 __device__ __forceinline__ unsigned wave_rotate_down1(unsigned v) {
   return __builtin_amdgcn_update_dpp(0u, v, 0x134, 0xf, 0xf, false);
@@ -634,27 +655,6 @@ __device__ __forceinline__ void copy_partial_slot(uintptr_t slot, unsigned off, 
         if (4u * q + b >= b_lo && 4u * q + b < b_hi)
           *reinterpret_cast<uint8_t*>(slot + 4 * q + b) = static_cast<uint8_t>(o[q] >> (8 * b));
     }
-  }
-}
-
-// 16-byte accesses at any byte address: gfx950 under HSA runs with unaligned
-// global access enabled, and the compiler emits one dwordx4 for these too.
-typedef v4u v4u_a1 __attribute__((aligned(1)));
-
-template <bool NT>
-__device__ __forceinline__ v4u ld_v4_any(const uint8_t* p) {
-  if constexpr (NT) return __builtin_nontemporal_load(reinterpret_cast<const v4u_a1*>(p));
-  else return *reinterpret_cast<const v4u_a1*>(p);
-}
-
-template <int POLICY>
-__device__ __forceinline__ void st_v4_any(uintptr_t p, v4u v) {
-  if constexpr (POLICY == kStoreNt) {
-    __builtin_nontemporal_store(v, reinterpret_cast<v4u_a1*>(p));
-  } else if constexpr (POLICY == kStoreAgentWt || POLICY == kStoreSystemWt) {
-    st_v4<POLICY>(reinterpret_cast<v4u*>(p), v);  // the asm forms take any address
-  } else {
-    *reinterpret_cast<v4u_a1*>(p) = v;
   }
 }
 

@@ -130,7 +130,11 @@ int mi355_blit_destroy(mi355_blit_t* h);
  * (core/runtime/blit_shaders/blit_copyAligned.s, blit_copyMisaligned.s).
  * Non-blocking.  stream is a hipStream_t, or NULL for the handle's own stream.
  * dst or src NULL -> INVALID_ARGUMENT; bytes == 0 -> SUCCESS without a launch
- * (core/runtime/hsa.cpp:1170-1184). */
+ * (core/runtime/hsa.cpp:1170-1184).
+ * Copy, fill and region copy are one kernel launch each and allocate nothing,
+ * so they may be issued on a stream under HIP graph capture; such commands
+ * are not counted by mi355_blit_pending_bytes.  The batched copy stages its
+ * descriptors and may not. */
 int mi355_blit_copy(mi355_blit_t* h, void* dst, const void* src, size_t bytes, void* stream);
 
 /* Replaces the dispatch half of BlitKernel::SubmitLinearFillCommand

@@ -190,6 +190,14 @@ int ledger_mark(mi355_blit* h) {
 
 // Notes `bytes` as queued on `s`.  Caller holds h->lock.
 int ledger_record(mi355_blit* h, hipStream_t s, uint64_t bytes) {
+  if (s != h->stream) {
+    // A command recorded into a graph under stream capture is not queued
+    // anywhere: nothing is pending because of it, and no marker event may be
+    // recorded on the capturing stream.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capture) == hipSuccess && capture == hipStreamCaptureStatusActive)
+      return MI355_BLIT_SUCCESS;
+  }
   if (h->unmarked && h->last_stream != s) {
     // a marker only orders against its own stream
     int rc = ledger_mark(h);

@@ -1,0 +1,64 @@
+"""Copy, fill and region copy of the HIP-stream path recorded into a HIP graph:
+each is one kernel launch with its arguments by value and no allocation, so a
+captured sequence must replay exactly.  The graph is replayed several times
+with the program's own eager work and synchronisations in between, new source
+bytes before every replay, and every replay is checked against the CPU oracle."""
+import numpy as np
+import pytest
+
+from conftest import oracle_rect
+
+pytestmark = pytest.mark.gpu
+
+GUARD_BYTE = 0xEE
+FILL_VALUE = 0x0BADC0DE
+
+
+def test_captured_commands_replay_exactly(capi, oracle, rand, torch_cuda):
+    torch = torch_cuda
+    n, s_off, d_off = 3 * (1 << 20) + 77, 3, 9
+    rows, width, s_pitch, d_pitch = 300, 1501, 1777, 2049
+    fill_dwords = 100_003
+    src = torch.empty(n + 64, dtype=torch.uint8, device="cuda:0")
+    dst = torch.empty(n + 600, dtype=torch.uint8, device="cuda:0")
+    rsrc = torch.empty(rows * s_pitch, dtype=torch.uint8, device="cuda:0")
+    rdst = torch.empty(rows * d_pitch, dtype=torch.uint8, device="cuda:0")
+    fbuf = torch.empty(4 * fill_dwords + 512, dtype=torch.uint8, device="cuda:0")
+    f_at = (-fbuf.data_ptr()) % 4 + 256
+    with capi.Blit(0) as blit:
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            s = torch.cuda.current_stream().cuda_stream
+            assert blit.copy(dst.data_ptr() + 256 + d_off, src.data_ptr() + s_off, n, s) == capi.SUCCESS
+            assert blit.fill32(fbuf.data_ptr() + f_at, FILL_VALUE, fill_dwords, s) == capi.SUCCESS
+            assert blit.copy_rect((rdst.data_ptr(), d_pitch, 0), (5, 0, 0), (rsrc.data_ptr(), s_pitch, 0), (7, 0, 0),
+                                  (width, rows, 1), s) == capi.SUCCESS
+        # nothing ran and nothing is pending because of the capture
+        assert blit.pending_bytes() == 0
+        for replay in range(4):
+            src_h = rand(n + 64, 0x6EA90000 + replay)
+            rsrc_h = rand(rows * s_pitch, 0x6EA91000 + replay)
+            src.copy_(torch.from_numpy(src_h))
+            rsrc.copy_(torch.from_numpy(rsrc_h))
+            dst.fill_(GUARD_BYTE)
+            rdst.fill_(GUARD_BYTE)
+            fbuf.fill_(GUARD_BYTE)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            want = np.full(n + 600, GUARD_BYTE, dtype=np.uint8)
+            oracle.oracle_copy(want.ctypes.data + 256 + d_off, src_h.ctypes.data + s_off, n)
+            assert np.array_equal(dst.cpu().numpy(), want), "copy, replay %d" % replay
+            want = np.full(4 * fill_dwords + 512, GUARD_BYTE, dtype=np.uint8)
+            oracle.oracle_fill32(want.ctypes.data + f_at, FILL_VALUE, fill_dwords)
+            assert np.array_equal(fbuf.cpu().numpy(), want), "fill, replay %d" % replay
+            want = np.full(rows * d_pitch, GUARD_BYTE, dtype=np.uint8)
+            oracle_rect(oracle, (want.ctypes.data, d_pitch, 0), (5, 0, 0), (rsrc_h.ctypes.data, s_pitch, 0), (7, 0, 0),
+                        (width, rows, 1))
+            assert np.array_equal(rdst.cpu().numpy(), want), "region copy, replay %d" % replay
+            # an eager command between replays, on the engine's own stream
+            assert blit.copy(dst.data_ptr(), src.data_ptr(), 4096) == capi.SUCCESS
+            assert blit.synchronize() == capi.SUCCESS
+        del graph

@@ -1,5 +1,5 @@
 // Device kernels of the gfx950 blit engine: linear copy, dword fill, batched
-// small copies.  They take the place of ROCr's CopyAligned, CopyMisaligned and
+// small copies, pitched 3-D region copies.  They take the place of ROCr's CopyAligned, CopyMisaligned and
 // Fill shaders (projects/rocr-runtime/runtime/hsa-runtime/core/runtime/
 // blit_shaders/blit_copyAligned.s:76-259, blit_copyMisaligned.s:90-182,
 // blit_fill.s:91-185) but share none of their structure:
@@ -22,7 +22,9 @@
 //    each lane loads the dword-aligned 16 bytes that contain its source bytes,
 //    takes the 17th..20th byte from the next lane with a DPP wave rotate, and
 //    rebuilds its vector with four v_alignbyte_b32.  No sub-dword access is
-//    made outside the <=15-byte head and tail of a copy.
+//    made outside the <=15-byte head and tail of a copy.  (The region copy
+//    of narrow rows is the exception: it moves a row's cut first and last
+//    slot as unaligned 16-byte vectors.)
 //  * The source is never read outside the aligned dwords that contain at
 //    least one requested byte, so no access can touch a page the copy does
 //    not own.
@@ -335,14 +337,14 @@ __device__ __forceinline__ uint32_t block_scan_1024(uint32_t v, uint32_t* lds, u
 
 // Prefix sum of the chunk counts in three small launches (no workgroup ever
 // waits for another):
-//  1. k_batch_scan_local, one workgroup per 1024 copies: chunk_start[i] =
+//  1. mi355_batch_scan_local, one workgroup per 1024 copies: chunk_start[i] =
 //     chunks of the copies before i in the same workgroup, block_sum[b] = all
 //     chunks of workgroup b;
-//  2. k_batch_scan_top, one workgroup: block_sum becomes its own exclusive
+//  2. mi355_batch_scan_top, one workgroup: block_sum becomes its own exclusive
 //     prefix, chunk_start[n] = all chunks;
-//  3. either k_batch_make_records, one lane per chunk: finds the chunk's copy
+//  3. either mi355_batch_make_records, one lane per chunk: finds the chunk's copy
 //     by bisecting block_sum and then that workgroup's chunk_start, and
-//     writes the chunk's record; or k_batch_finalize, one lane per copy:
+//     writes the chunk's record; or mi355_batch_finalize, one lane per copy:
 //     chunk_start[i] += block_sum[i / 1024], for the kernel that walks
 //     chunk_start itself.
 __device__ __forceinline__ void scan_local_body(const ScanLocalArgs& a) {

@@ -41,6 +41,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="copy", choices=["copy", "fill", "misaligned", "batch", "rect", "calib"])
     ap.add_argument("--bytes", type=int, default=GIB, help="transfer size of the copy/fill workloads")
+    ap.add_argument("--rect", default="8192,131072,262144,0,0",
+                    help="shape of the rect workload: rows,width,pitch[,source x,destination x] in bytes")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-also", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget")
@@ -488,9 +490,12 @@ def main():
         name = "misaligned D2D copy, %d MiB - 64 B, src&15=3 dst&15=9" % (nbytes // MIB)
         traffic_key = "misaligned_1GiB" if nbytes == GIB else None
     elif args.workload == "rect":
-        fn, verify, algo, keep = make_rect(r)
-        name = "pitched 2-D region copy, 8192 rows x 128 KiB out of 256 KiB-pitch surfaces (1 GiB moved)"
-        traffic_key = "rect_8192x128KiB"
+        shape = tuple(int(v) for v in args.rect.split(","))
+        shape = shape + (0,) * (5 - len(shape))
+        fn, verify, algo, keep = make_rect(r, *shape)
+        name = "pitched 2-D region copy, %d rows x %d B out of %d B-pitch surfaces, x offsets %d / %d (%d MiB moved)" % (
+            shape[0], shape[1], shape[2], shape[3], shape[4], shape[0] * shape[1] // MIB)
+        traffic_key = "rect_%dx%d_%d" % shape[:3]
     elif args.workload == "calib":
         fn, verify, algo, keep = make_calib(r, nbytes)
         name = "calibration: torch copy_ of %d MiB (not this library)" % (nbytes // MIB)
@@ -514,7 +519,7 @@ def main():
                            ("fill_1GiB", lambda: make_fill(r, GIB)),
                            ("misaligned_1GiB", lambda: make_copy(r, GIB - 64, s_off=3, d_off=9)),
                            ("batch_65536", lambda: make_batch(r)),
-                           ("rect_8192x128KiB", lambda: make_rect(r))):
+                           ("rect_8192x131072_262144", lambda: make_rect(r))):
             f2, v2, a2, k2 = maker()
             w2, us2 = r.time_launches(f2, 20, 3)
             v2()

@@ -562,7 +562,7 @@ __device__ __forceinline__ void batch_copy_strided_body(const BatchStridedArgs& 
 // fewer skip the rest.  No memory beyond the two regions, one launch.
 constexpr unsigned kRowOverflowVecs = 15;
 
-__device__ __forceinline__ unsigned row_units(unsigned n_virtual, unsigned unit) {
+__device__ __forceinline__ uint64_t row_units(uint64_t n_virtual, unsigned unit) {
   return n_virtual > kRowOverflowVecs + unit ? (n_virtual - kRowOverflowVecs + unit - 1) / unit : 1;
 }
 
@@ -583,13 +583,14 @@ __device__ __forceinline__ void rect_copy_body(const RectArgs& a) {
     row.src = a.src + layer * a.src_slice + y * a.src_pitch;
     row.bytes = a.width;
     const DescShape sh = desc_shape(row);
-    const unsigned n_virtual = static_cast<unsigned>(sh.n_vec) + sh.lead;
-    const unsigned units = row_units(n_virtual, kUnit);
+    // merged rows can be longer than 2^32 vectors: 64-bit indices
+    const uint64_t n_virtual = sh.n_vec + sh.lead;
+    const uint64_t units = row_units(n_virtual, kUnit);
     if (kq >= units) continue;
     const bool last = kq + 1 == units;
-    const unsigned v0 = kq * kUnit;
-    const unsigned lo = v0 > sh.lead ? v0 : sh.lead;
-    const unsigned end = last ? n_virtual : v0 + kUnit;
+    const uint64_t v0 = static_cast<uint64_t>(kq) * kUnit;
+    const uint64_t lo = v0 > sh.lead ? v0 : sh.lead;
+    const uint64_t end = last ? n_virtual : v0 + kUnit;
     const uint8_t* sb = row.src + sh.head;
     const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(sb)) & 3;
     const v4u_a4* sv = reinterpret_cast<const v4u_a4*>(sb - r) - sh.lead;
@@ -598,7 +599,7 @@ __device__ __forceinline__ void rect_copy_body(const RectArgs& a) {
     v4u x[U + 1];
 #pragma unroll
     for (int u = 0; u <= U; ++u) {
-      const unsigned idx = v0 + lane + u * kWave;
+      const uint64_t idx = v0 + lane + u * kWave;
       if (idx >= lo && idx < end) x[u] = ld_v4<NTL>(sv + idx);
     }
     // the dword behind the unit's last vector: with r != 0 it holds that
@@ -607,7 +608,7 @@ __device__ __forceinline__ void rect_copy_body(const RectArgs& a) {
     if (r && end > lo) e = ld_u32<NTL>(reinterpret_cast<const unsigned*>(sv + end));
 #pragma unroll
     for (int u = 0; u <= U; ++u) {
-      const unsigned idx = v0 + lane + u * kWave;
+      const uint64_t idx = v0 + lane + u * kWave;
       const unsigned nxt = x[u < U ? u + 1 : u].x;  // lane 0's copy is what lane 63 needs
       unsigned w4 = wave_rotate_down1(lane == 0 ? nxt : x[u].x);
       if (idx + 1 == end) w4 = e;

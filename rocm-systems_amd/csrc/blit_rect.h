@@ -75,6 +75,8 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
     return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   if (range->z > 1 && (src->slice == 0 || dst->slice == 0)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   uint64_t width = range->x, rows = range->y, layers = range->z;
+  // x, y and z are 32-bit: rows * layers fits 64 bits, the byte total may not
+  if (width > (1ull << 62) / (rows * layers)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   uint64_t dp = dst->pitch, ds = dst->slice, sp = src->pitch, ss = src->slice;
   uint8_t* d0 = static_cast<uint8_t*>(dst->base) + dst_offset->z * ds + dst_offset->y * dp + dst_offset->x;
   const uint8_t* s0 = static_cast<const uint8_t*>(src->base) + src_offset->z * ss + src_offset->y * sp + src_offset->x;

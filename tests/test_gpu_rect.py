@@ -202,6 +202,35 @@ def test_rect_one_gib_region(capi, blit, oracle, rand, torch_cuda):
         assert np.array_equal(d2[y].cpu().numpy(), want)
 
 
+def test_rect_merged_rows_beyond_4gib(capi, blit, torch_cuda):
+    """Two layers of 4608 contiguous 1 MiB rows: each layer merges into one row
+    of 4.5 GiB, more than a 32-bit byte count, 256 bytes off the 256-byte grid."""
+    torch = torch_cuda
+    row, rows, layers = MIB, 4608, 2
+    layer_bytes = row * rows
+    s_slice, d_slice = layer_bytes + 4096, layer_bytes + 8192
+    src = torch.empty(layers * s_slice + 512, dtype=torch.uint8, device="cuda:0")
+    pattern = torch.arange(0, 64 * MIB, dtype=torch.int32, device="cuda:0")
+    pattern = (pattern * 2654435761 >> 7).to(torch.uint8)
+    for lo in range(0, src.numel(), pattern.numel()):
+        m = min(pattern.numel(), src.numel() - lo)
+        src[lo:lo + m] = pattern[:m] + (lo >> 26)
+    del pattern
+    dst = torch.full((layers * d_slice + 512,), GUARD_BYTE, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    s_at, d_at = 48, 112
+    st = blit.copy_rect((dst.data_ptr() + d_at, row, d_slice), (0, 0, 0), (src.data_ptr() + s_at, row, s_slice),
+                        (0, 0, 0), (row, rows, layers))
+    assert st == capi.SUCCESS and blit.synchronize() == capi.SUCCESS
+    p = blit.last_plan()
+    assert p.kernel == capi.KERNEL_COPY_RECT
+    for z in range(layers):
+        d0, s0 = d_at + z * d_slice, s_at + z * s_slice
+        assert torch.equal(dst[d0:d0 + layer_bytes], src[s0:s0 + layer_bytes]), "layer %d" % z
+        assert bool((dst[d0 + layer_bytes:d0 + d_slice] == GUARD_BYTE).all()), "gap behind layer %d" % z
+    assert bool((dst[:d_at] == GUARD_BYTE).all())
+
+
 def test_async_copy_rect_stand_in(capi, pkg, oracle, rand, torch_cuda):
     """mi355_hsa_amd_memory_async_copy_rect: the reference's answers at the API
     edge (hsa_ext_amd.cpp:367-410), dependencies honoured, the completion signal

@@ -484,6 +484,23 @@ __device__ __forceinline__ void record_edges(const ChunkRecord& rec, bool do_hea
   }
 }
 
+// One record, fetched with a scalar load.  The records were written by an
+// earlier launch and are only read here; reading them through the constant
+// address space tells the compiler so (a pointer taken out of the argument
+// struct carries no such promise, and the record would otherwise be fetched by
+// all 64 lanes with vector loads).
+__device__ __forceinline__ ChunkRecord load_record(const ChunkRecord* p) {
+  typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+  typedef const u32x8 __attribute__((address_space(4))) * ConstPtr;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wold-style-cast"
+  const u32x8 v = *(ConstPtr)(p);
+#pragma clang diagnostic pop
+  ChunkRecord r;
+  __builtin_memcpy(&r, &v, sizeof(r));
+  return r;
+}
+
 // SPLIT waves per 4 KiB chunk, chunks in global order and waves in address
 // order within a chunk: the dispatcher then walks memory densely, the shape
 // that streams best for a single large copy.  Each wave reads its chunk's
@@ -497,7 +514,7 @@ __device__ __forceinline__ void batch_copy_records_body(const BatchCopyArgs& a) 
   const uint64_t wave = global_wave(a.waves_per_wg);
   const uint64_t n_waves = a.n_waves;
   for (uint64_t w = wave; w < total_chunks * SPLIT; w += n_waves) {
-    const ChunkRecord rec = records[w / SPLIT];
+    const ChunkRecord rec = load_record(records + w / SPLIT);
     const unsigned q = static_cast<unsigned>(w % SPLIT);
     const unsigned v0 = q * (kChunkVecs / SPLIT);
     v4u x[U];

@@ -35,7 +35,7 @@ namespace {
 using namespace mi355;
 
 // Packets in the queue.  The reference shares the agent's 64-packet utility
-// queue (amd_gpu_agent.h:507-508); a batch here is five packets, so the ring
+// queue (amd_gpu_agent.h:507-508); a batch here is four packets, so the ring
 // is a little larger.
 constexpr uint32_t kQueuePackets = 256;
 // One kernarg slot per packet slot, as in the reference (amd_blit_kernel.cpp:
@@ -718,30 +718,16 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   std::memcpy(h->stage[b], descs, n * sizeof(BatchDesc));
   hsa_signal_store_relaxed(h->stage_free[b], 1);
 
-  // 1. upload: our own copy kernel pulls the descriptors into device memory
-  mi355_blit_plan_t up;
-  rc = plan_copy(reinterpret_cast<uint64_t>(h->descs_dev), reinterpret_cast<uint64_t>(h->stage[b]), n * sizeof(BatchDesc),
-                 h->num_cus, nullptr, &up);
-  if (rc != MI355_BLIT_SUCCESS) return rc;
-  const Kernel* up_k = find_copy(h, up);
-  if (!up_k) return MI355_BLIT_ERROR;
-  CopyArgs ua{};
-  ua.dst = reinterpret_cast<uint8_t*>(h->descs_dev);
-  ua.src = reinterpret_cast<const uint8_t*>(h->stage[b]);
-  ua.bytes = n * sizeof(BatchDesc);
-  ua.n_vec = up.body_vecs;
-  ua.head = static_cast<uint32_t>(up.head_bytes);
-  ua.lead = up.lead_vecs;
-  tail_waves(up, &ua.partial_wave, &ua.edge_wave, &ua.waves_per_wg, &ua.n_waves);
-
-  // 2..4. prefix sum and records
+  // 1..3. prefix sum and records.  The first kernel reads the descriptors
+  // straight from the staging buffer in host memory and leaves a copy in
+  // device memory for the ones that follow.
   const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
-  ScanLocalArgs sl{h->descs_dev, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
+  ScanLocalArgs sl{h->stage[b], static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev, h->descs_dev};
   ScanTopArgs stp{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
   MakeRecordsArgs mr{h->descs_dev, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev, total_chunks,
                      h->records_dev, n_blocks};
 
-  // 5. the copy
+  // 4. the copy
   mi355_blit_plan_t p{};
   p.kernel = MI355_BLIT_KERNEL_COPY_BATCH;
   p.body_vecs = total_chunks;
@@ -768,7 +754,7 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   h->last_plan = p;
 
   const uint32_t nb = barrier_packets(num_deps);
-  const uint32_t total = nb + 5;
+  const uint32_t total = nb + 4;
   uint64_t index;
   {
     std::lock_guard<std::mutex> r(h->reservation_lock);
@@ -778,9 +764,9 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
   uint64_t i = index + nb;
   // every packet of the sequence waits for the one before (barrier bit); the
-  // first also waits for whatever still uses the shared device buffers
-  write_dispatch(h, i++, *up_k, &ua, sizeof(ua), up.grid, up.wg_size, h->stage_free[b].handle, true);
-  write_dispatch(h, i++, h->scan_local, &sl, sizeof(sl), n_blocks, 1024, 0, true);
+  // first also waits for whatever still uses the shared device buffers, and
+  // frees the staging buffer when it is done with it
+  write_dispatch(h, i++, h->scan_local, &sl, sizeof(sl), n_blocks, 1024, h->stage_free[b].handle, true);
   write_dispatch(h, i++, h->scan_top, &stp, sizeof(stp), 1, 1024, 0, true);
   write_dispatch(h, i++, h->make_records, &mr, sizeof(mr), static_cast<uint32_t>((total_chunks + 255) / 256), 256, 0, true);
   write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true);

@@ -68,6 +68,10 @@ struct ScanLocalArgs {
   uint64_t n;
   uint32_t* chunk_start;
   uint32_t* block_sum;
+  // When not null, descs is host memory the GPU reads across the bus and each
+  // lane leaves a copy of its descriptor here, in device memory, for the
+  // kernels that follow.
+  BatchDesc* device_copy;
 };
 
 struct ScanTopArgs {

@@ -465,6 +465,8 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
   // own upload, two batches ago, has finished.
   if (h->staging_busy) BLIT_HIP(hipStreamWaitEvent(s, h->staging_free, 0));
   const BatchDesc* dev_descs;
+  const BatchDesc* host_descs = nullptr;
+  int host_buffer = -1;
   if (descs_on_device) {
     dev_descs = reinterpret_cast<const BatchDesc*>(descs);
   } else {
@@ -475,15 +477,23 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
       h->upload_busy[b] = false;
     }
     std::memcpy(h->descs_host[b], descs, n * sizeof(BatchDesc));
-    BLIT_HIP(hipMemcpyAsync(h->descs_dev, h->descs_host[b], n * sizeof(BatchDesc), hipMemcpyHostToDevice, s));
-    BLIT_HIP(hipEventRecord(h->upload_done[b], s));
-    h->upload_busy[b] = true;
+    host_descs = h->descs_host[b];
+    host_buffer = static_cast<int>(b);
     dev_descs = h->descs_dev;
   }
 
+  // The first kernel reads host-resident descriptors straight from the pinned
+  // buffer and leaves the device copy behind: a separate upload would cost a
+  // copy-engine transfer and two engine switches (measured: 33 us + 26 us of
+  // gaps for 65,536 descriptors, against 30 us of reading across the bus).
   const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
-  ScanLocalArgs sl{dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
+  ScanLocalArgs sl{host_descs ? host_descs : dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev,
+                   h->block_sum_dev, host_descs ? h->descs_dev : nullptr};
   hipLaunchKernelGGL(mi355_batch_scan_local, dim3(n_blocks), dim3(1024), 0, s, sl);
+  if (host_buffer >= 0) {
+    BLIT_HIP(hipEventRecord(h->upload_done[host_buffer], s));
+    h->upload_busy[host_buffer] = true;
+  }
   ScanTopArgs st{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
   hipLaunchKernelGGL(mi355_batch_scan_top, dim3(1), dim3(1024), 0, s, st);
   BLIT_HIP(hipGetLastError());

@@ -354,7 +354,12 @@ __device__ __forceinline__ void scan_local_body(const ScanLocalArgs& a) {
   uint32_t* __restrict__ block_sum = a.block_sum;
   __shared__ uint32_t lds[16];
   const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 1024 + threadIdx.x;
-  const uint32_t c = i < n ? desc_chunks(descs[i]) : 0;
+  uint32_t c = 0;
+  if (i < n) {
+    const BatchDesc d = descs[i];
+    if (a.device_copy) a.device_copy[i] = d;
+    c = desc_chunks(d);
+  }
   uint32_t total;
   const uint32_t excl = block_scan_1024(c, lds, &total);
   if (i < n) chunk_start[i] = excl;

@@ -53,6 +53,7 @@ struct Kernel {
 struct CopyKernel { unsigned unroll, nt_load, store, realign; const char* name; Kernel k; };
 struct FillKernel { unsigned unroll, store; const char* name; Kernel k; };
 struct BatchKernel { unsigned split, nt_load, store; const char* name; Kernel k; };
+struct RectKernel { unsigned unroll, nt_load, store; const char* name; Kernel k; };  // unroll 0: the narrow-row kernel
 
 #define MI355_COPY_NAME(U, L, S, R) {U, L, S, R, "mi355_copy_u" #U "_l" #L "_s" #S "_r" #R, {}},
 #define MI355_FILL_NAME(U, S) {U, S, "mi355_fill_u" #U "_s" #S, {}},
@@ -103,8 +104,8 @@ struct mi355_aql {
   std::vector<CopyKernel> copy_kernels{MI355_FOR_EACH_COPY_KERNEL(MI355_COPY_NAME)};
   std::vector<FillKernel> fill_kernels{MI355_FOR_EACH_FILL_KERNEL(MI355_FILL_NAME)};
   std::vector<BatchKernel> batch_kernels{MI355_FOR_EACH_BATCH_RECORDS_KERNEL(MI355_BATCH_NAME)};
-  std::vector<BatchKernel> rect_kernels{MI355_FOR_EACH_RECT_KERNEL(MI355_RECT_NAME)};
-  std::vector<BatchKernel> rect_narrow_kernels{MI355_FOR_EACH_RECT_NARROW_KERNEL(MI355_RECT_NARROW_NAME)};
+  std::vector<RectKernel> rect_kernels{MI355_FOR_EACH_RECT_KERNEL(MI355_RECT_NAME)};
+  std::vector<RectKernel> rect_narrow_kernels{MI355_FOR_EACH_RECT_NARROW_KERNEL(MI355_RECT_NARROW_NAME)};
   Kernel scan_local, scan_top, make_records;
 
   hsa_signal_t idle_signal{};  // completion signal of wait_idle's barrier packet
@@ -130,7 +131,7 @@ struct mi355_aql {
 
   // batched path: two host staging buffers used alternately, device buffers
   BatchDesc* stage[2] = {nullptr, nullptr};
-  hsa_signal_t stage_free[2] = {{0}, {0}};  // 0 when the upload from stage[i] has finished
+  hsa_signal_t stage_free[2] = {{0}, {0}};  // 0 when the kernel that reads stage[i] has finished
   unsigned next_stage = 0;
   BatchDesc* descs_dev = nullptr;
   uint32_t* chunk_start_dev = nullptr;
@@ -792,7 +793,7 @@ int mi355_aql_copy_rect(mi355_aql_t* h, const mi355_pitched_ptr_t* dst, const mi
           if (v.nt_load == rp.streaming && v.store == rp.store_policy) k = &v.k;
       } else {
         for (const auto& v : h->rect_kernels)
-          if (v.split == rp.unroll && v.nt_load == rp.streaming && v.store == rp.store_policy) k = &v.k;
+          if (v.unroll == rp.unroll && v.nt_load == rp.streaming && v.store == rp.store_policy) k = &v.k;
       }
       if (!k) return MI355_BLIT_ERROR;
       rect_launch_info(rp, &h->last_plan);

@@ -17,6 +17,7 @@ HSACO = os.path.join(LIB_DIR, "mi355_blit_gfx950.hsaco")
 ROCR_LIB = os.path.join(LIB_DIR, "libmi355blit_rocr.so")
 ROCR_TEST = os.path.join(LIB_DIR, "test_rocr_blit")
 ORACLE_LIB = os.path.join(ORACLE_DIR, "libblit_oracle.so")
+HOST_LOGIC_TEST = os.path.join(LIB_DIR, "test_host_logic")
 
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
@@ -101,6 +102,21 @@ def build_rocr_test():
     return ROCR_TEST
 
 
+def build_host_logic_test():
+    """Native test of the host arithmetic (plans of copies, fills and region
+    copies) under AddressSanitizer and UBSan; host code only, the CPU oracle
+    compiled in as its checker."""
+    test_src = os.path.join(ROOT, "tests", "cpp", "test_host_logic.cpp")
+    if not os.path.exists(test_src):
+        return None
+    os.makedirs(LIB_DIR, exist_ok=True)
+    _run(["g++", "-O1", "-g", "-Wall", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+          "-static-libasan", "-static-libubsan", "-I", INCLUDE, "-I", CSRC,
+          "-o", HOST_LOGIC_TEST, "-x", "c", os.path.join(ORACLE_DIR, "blit_oracle.c"),
+          "-x", "c++", "-std=c++17", test_src, "-lpthread"])
+    return HOST_LOGIC_TEST
+
+
 def build_oracle():
     """CPU oracle (test infrastructure) -> oracle/libblit_oracle.so"""
     _run(["make", "-C", ORACLE_DIR, "-B", "libblit_oracle.so"])
@@ -113,9 +129,9 @@ def build_all():
     if r:
         out.append(r)
     out.append(build_oracle())
-    t = build_rocr_test()
-    if t:
-        out.append(t)
+    for t in (build_rocr_test(), build_host_logic_test()):
+        if t:
+            out.append(t)
     return out
 
 

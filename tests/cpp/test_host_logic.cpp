@@ -1,0 +1,252 @@
+// Host arithmetic of the blit engine under AddressSanitizer and UBSan, at a
+// volume the Python tests cannot reach: the copy / fill plans
+// (csrc/blit_plan.h) and the region-copy plans (csrc/blit_rect.h) over
+// hundreds of thousands of seeded cases.  Every plan is checked against
+// invariants that do not restate its formulas: a plan must tile its byte range
+// exactly, a region plan's units (or packed slots) must cover every row's bytes
+// once, in order and inside the row, and the region validation must give the
+// reference's verdict (oracle_ref_validate_rect).  No GPU, no device code.
+//
+//   test_host_logic [cases]      exit status 0 = all checks passed
+#include <cinttypes>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "../../oracle/blit_oracle.h"
+#include "blit_plan.h"
+#include "blit_rect.h"
+
+namespace {
+
+using namespace mi355;
+
+uint64_t g_state = 0x9E3779B97F4A7C15ull;
+uint64_t rnd() {  // splitmix64
+  uint64_t z = (g_state += 0x9E3779B97F4A7C15ull);
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+uint64_t below(uint64_t n) { return n ? rnd() % n : 0; }
+
+int g_failures = 0;
+#define CHECK(cond, ...)                          \
+  do {                                            \
+    if (!(cond)) {                                \
+      if (g_failures < 20) {                      \
+        std::printf("FAIL %s:%d: ", __FILE__, __LINE__); \
+        std::printf(__VA_ARGS__);                 \
+        std::printf("\n");                        \
+      }                                           \
+      ++g_failures;                               \
+      return;                                     \
+    }                                             \
+  } while (0)
+
+mi355_blit_tuning_t random_tuning() {
+  mi355_blit_tuning_t t{};
+  const uint32_t wgs[] = {0, 64, 128, 256, 512, 1024, 100, 2048};
+  const uint32_t unrolls[] = {0, 1, 2, 4, 3};
+  t.wg_size = wgs[below(8)];
+  t.unroll = unrolls[below(5)];
+  t.max_grid = below(3) ? 0 : static_cast<uint32_t>(below(5000));
+  t.nt_load = static_cast<uint32_t>(below(3));
+  t.store_policy = static_cast<uint32_t>(below(6));
+  return t;
+}
+
+uint64_t random_size() {
+  switch (below(4)) {
+    case 0: return below(600);
+    case 1: return below(1u << 20);
+    case 2: return (1ull << (20 + below(16))) + below(4096) - below(64);
+    default: return rnd() >> (16 + below(40));
+  }
+}
+
+void check_linear_plan(const mi355_blit_plan_t& p, uint64_t dst, uint64_t bytes, uint32_t kernel) {
+  CHECK(p.kernel == kernel, "kernel %u", p.kernel);
+  CHECK(p.head_bytes + 16 * p.body_vecs + p.tail_bytes == bytes, "plan does not tile %" PRIu64 " bytes", bytes);
+  CHECK(p.head_bytes <= 15 && p.tail_bytes <= 15, "head %" PRIu64 " tail %" PRIu64, p.head_bytes, p.tail_bytes);
+  CHECK(p.body_vecs == 0 || (dst + p.head_bytes) % 16 == 0, "body not 16-byte aligned");
+  CHECK(p.lead_vecs == ((dst + p.head_bytes) & 255) / 16, "lead %u", p.lead_vecs);
+  CHECK(p.wg_size >= 64 && p.wg_size <= 1024 && p.wg_size % 64 == 0, "wg %u", p.wg_size);
+  CHECK(p.unroll == 1 || p.unroll == 2 || p.unroll == 4, "unroll %u", p.unroll);
+  CHECK(p.grid >= 1 && static_cast<uint64_t>(p.grid) * p.wg_size <= 0x7fffffc0ull, "grid %u x %u", p.grid, p.wg_size);
+  CHECK(p.store_policy <= 3 && p.nt_load <= 1, "policy");
+}
+
+void one_copy_plan() {
+  const uint64_t dst = (1ull << 40) + below(1 << 20), src = (2ull << 40) + below(1 << 20);
+  const uint64_t bytes = random_size();
+  const bool tuned = below(2);
+  mi355_blit_tuning_t t = random_tuning();
+  mi355_blit_plan_t p;
+  CHECK(plan_copy(dst, src, bytes, 256, tuned ? &t : nullptr, &p) == MI355_BLIT_SUCCESS, "plan_copy failed");
+  // the reference's predicate for its two copy shaders (amd_blit_kernel.cpp:716)
+  const bool same_dword_phase = (src & 3) == (dst & 3);
+  check_linear_plan(p, dst, bytes, same_dword_phase ? MI355_BLIT_KERNEL_COPY : MI355_BLIT_KERNEL_COPY_REALIGN);
+  CHECK(p.byte_shift == ((src - dst) & 3), "byte shift");
+  if (!tuned || t.max_grid == 0) {
+    // uncapped: one wave per tile and one for the edges
+    const uint64_t tile = 64ull * p.unroll;
+    const uint64_t tiles = (p.body_vecs + p.lead_vecs + tile - 1) / tile;
+    const uint64_t waves = static_cast<uint64_t>(p.grid) * (p.wg_size / 64);
+    CHECK(waves >= tiles + 1 || waves * 64 + p.wg_size > 0x7fffffc0ull, "grid %u too small for %" PRIu64 " tiles", p.grid, tiles);
+  }
+}
+
+void one_fill_plan() {
+  const uint64_t ptr = (1ull << 40) + 4 * below(1 << 18);
+  const uint64_t dwords = random_size() / 4;
+  mi355_blit_tuning_t t = random_tuning();
+  mi355_blit_plan_t p;
+  CHECK(plan_fill(ptr, dwords, 256, below(2) ? &t : nullptr, &p) == MI355_BLIT_SUCCESS, "plan_fill failed");
+  check_linear_plan(p, ptr, dwords * 4, MI355_BLIT_KERNEL_FILL);
+  CHECK(p.head_bytes % 4 == 0 && p.tail_bytes % 4 == 0, "fill edges are whole dwords");
+  CHECK(plan_fill(ptr + 1 + below(3), dwords, 256, nullptr, &p) == MI355_BLIT_ERROR_INVALID_ARGUMENT, "misaligned fill accepted");
+}
+
+// Bytes [*lo, *hi) of a row that unit kq of the wide-row kernel moves.
+void unit_range(uint64_t d, uint64_t width, uint64_t unit, uint64_t kq, uint64_t units, uint64_t* lo, uint64_t* hi,
+                uint64_t* vectors) {
+  uint64_t head = (16 - (d & 15)) & 15;
+  if (head > width) head = width;
+  const uint64_t n_vec = (width - head) / 16, lead = ((d + head) & 255) / 16, n_virtual = n_vec + lead;
+  const bool last = kq + 1 == units;
+  const uint64_t v_lo = kq * unit > lead ? kq * unit : lead;
+  const uint64_t v_hi = last ? n_virtual : kq * unit + unit;
+  *lo = kq == 0 ? 0 : head + 16 * (v_lo - lead);
+  *hi = last ? width : head + 16 * (v_hi - lead);
+  *vectors = v_hi - kq * unit;
+}
+
+void one_rect_plan() {
+  mi355_pitched_ptr_t dst{}, src{};
+  dst.base = reinterpret_cast<void*>((1ull << 40) + below(512));
+  src.base = reinterpret_cast<void*>((2ull << 40) + below(512));
+  const bool narrow = below(2);
+  mi355_dim3_t range{static_cast<uint32_t>(1 + below(narrow ? 1200 : 40000)), static_cast<uint32_t>(1 + below(40)),
+                     static_cast<uint32_t>(1 + below(4))};
+  mi355_dim3_t doff{static_cast<uint32_t>(below(300)), static_cast<uint32_t>(below(8)), static_cast<uint32_t>(below(3))};
+  mi355_dim3_t soff{static_cast<uint32_t>(below(300)), static_cast<uint32_t>(below(8)), static_cast<uint32_t>(below(3))};
+  dst.pitch = below(8) ? doff.x + range.x + below(300) : range.x;
+  src.pitch = below(8) ? soff.x + range.x + below(300) : range.x;
+  if (below(16) == 0) dst.pitch = below(dst.pitch + 1);  // sometimes too small
+  dst.slice = below(5) ? dst.pitch * (doff.y + range.y + below(5)) : (below(2) ? 0 : dst.pitch * below(range.y + 2));
+  src.slice = below(5) ? src.pitch * (soff.y + range.y + below(5)) : (below(2) ? 0 : src.pitch * below(range.y + 2));
+  if (below(50) == 0) range.x = 0;
+  mi355_blit_tuning_t t = random_tuning();
+  const bool tuned = below(3) == 0;
+  RectPlan rp;
+  const int st = plan_rect(&dst, &doff, &src, &soff, &range, tuned ? &t : nullptr, &rp);
+
+  oracle_pitched_ptr_t od{dst.base, dst.pitch, dst.slice}, os{src.base, src.pitch, src.slice};
+  oracle_dim3_t odo{doff.x, doff.y, doff.z}, oso{soff.x, soff.y, soff.z}, orange{range.x, range.y, range.z};
+  int does_work = -1, aligned = -1;
+  const int want = oracle_ref_validate_rect(&od, &odo, &os, &oso, &orange, 3, &does_work, &aligned);
+  CHECK(st == want, "status 0x%x, the reference's checks say 0x%x", st, want);
+  if (st != MI355_BLIT_SUCCESS) return;
+  CHECK(rp.empty == (does_work == 0), "empty flag");
+  if (rp.empty) return;
+
+  const uint64_t d0 = reinterpret_cast<uint64_t>(dst.base) + doff.z * dst.slice + doff.y * dst.pitch + doff.x;
+  const uint64_t s0 = reinterpret_cast<uint64_t>(src.base) + soff.z * src.slice + soff.y * src.pitch + soff.x;
+  const uint64_t total = static_cast<uint64_t>(range.x) * range.y * range.z;
+  CHECK(rp.total_bytes == total, "total bytes");
+  CHECK(reinterpret_cast<uint64_t>(rp.args.dst) == d0 && reinterpret_cast<uint64_t>(rp.args.src) == s0, "region origin");
+  if (rp.linear) {
+    CHECK(rp.args.width == total, "a linear region is all of its bytes");
+    // contiguous on both sides: the last byte of the box sits total - 1 bytes after the first
+    const uint64_t last_d = d0 + (range.z - 1) * dst.slice + (range.y - 1) * dst.pitch + range.x - 1;
+    const uint64_t last_s = s0 + (range.z - 1) * src.slice + (range.y - 1) * src.pitch + range.x - 1;
+    CHECK(last_d - d0 == total - 1 && last_s - s0 == total - 1, "region merged into one run is not contiguous");
+    return;
+  }
+  // merged rows: every merged row is a run of whole original rows
+  const uint64_t width = rp.narrow ? rp.nargs.width : rp.args.width;
+  const uint64_t rows = rp.args.rows;
+  const uint64_t lines = rp.narrow ? rp.nargs.lines : rp.args.total_slots / rp.args.slots;
+  CHECK(rows >= 1 && lines % rows == 0 && width * lines == total, "merged geometry");
+  CHECK(width % range.x == 0, "merged width is not a multiple of the row width");
+  const uint64_t per = width / range.x;  // original rows per merged row
+  const uint64_t dp = rp.narrow ? rp.nargs.dst_pitch : rp.args.dst_pitch, ds = rp.narrow ? rp.nargs.dst_slice : rp.args.dst_slice;
+  const uint64_t sp = rp.narrow ? rp.nargs.src_pitch : rp.args.src_pitch, ss = rp.narrow ? rp.nargs.src_slice : rp.args.src_slice;
+  for (uint64_t line = 0; line < lines; ++line) {
+    const uint64_t layer = line / rows, y = line % rows;
+    const uint64_t d = d0 + layer * ds + y * dp, s = s0 + layer * ss + y * sp;
+    // where the original geometry puts the first row of this merged row
+    const uint64_t first = line * per;  // index among all original rows, layer-major
+    const uint64_t oz = first / range.y, oy = first % range.y;
+    CHECK(d == d0 + oz * dst.slice + oy * dst.pitch && s == s0 + oz * src.slice + oy * src.pitch, "row origin");
+    if (per > 1) CHECK(dst.pitch == range.x && src.pitch == range.x, "rows merged across a gap");
+    if (rp.narrow) {
+      const uint64_t lpr = rp.nargs.lanes_per_row;
+      CHECK(lpr >= 1 && lpr <= 64, "lanes per row %" PRIu64, lpr);
+      uint64_t covered = d;  // bytes of the row below this address have been written
+      for (uint64_t j = 0; j < lpr; ++j) {
+        const uint64_t slot = (d & ~15ull) + 16 * j;
+        if (slot >= d + width) continue;
+        uint64_t lo, hi;
+        if (width >= 16) {
+          lo = slot > d ? slot : d;
+          if (lo + 16 > d + width) lo = d + width - 16;
+          hi = lo + 16;
+        } else {
+          lo = slot > d ? slot : d;
+          hi = slot + 16 < d + width ? slot + 16 : d + width;
+        }
+        CHECK(lo >= d && hi <= d + width && lo <= covered, "slot %" PRIu64 " leaves a hole or the row", j);
+        if (hi > covered) covered = hi;
+      }
+      CHECK(covered == d + width, "row not covered by its %" PRIu64 " slots", lpr);
+      // the host's magic numbers divide as the kernel needs them to
+      for (uint64_t n = 0; n < 128; ++n) CHECK(((n * rp.nargs.magic) >> 16) == n / lpr, "16-bit magic");
+      if (lpr > 1) {
+        const uint64_t probe = below(1ull << 38);
+        CHECK(static_cast<uint64_t>((static_cast<unsigned __int128>(probe) * rp.nargs.magic64) >> 64) == probe / lpr,
+              "64-bit magic");
+      }
+    } else {
+      const uint64_t unit = 64ull * rp.unroll;
+      uint64_t head = (16 - (d & 15)) & 15;
+      if (head > width) head = width;
+      const uint64_t n_virtual = (width - head) / 16 + ((d + head) & 255) / 16;
+      const uint64_t units = n_virtual > 15 + unit ? (n_virtual - 15 + unit - 1) / unit : 1;
+      CHECK(units <= rp.args.slots, "row needs %" PRIu64 " units, plan has %u slots", units, rp.args.slots);
+      uint64_t at = 0;
+      for (uint64_t kq = 0; kq < units; ++kq) {
+        uint64_t lo, hi, vectors;
+        unit_range(d, width, unit, kq, units, &lo, &hi, &vectors);
+        CHECK(lo == at && hi >= lo && hi <= width, "unit %" PRIu64 " does not continue the row", kq);
+        CHECK(vectors <= unit + 64, "a lane would need more than one extra vector");
+        at = hi;
+      }
+      CHECK(at == width, "units stop short of the row's end");
+    }
+  }
+  if (!rp.narrow) {
+    CHECK(rp.args.n_waves == rp.grid * rp.args.waves_per_wg && rp.args.waves_per_wg == rp.wg_size / 64, "launch shape");
+    if (!tuned || t.max_grid == 0) CHECK(rp.args.n_waves >= rp.args.total_slots, "grid smaller than the unit slots");
+  } else {
+    CHECK(rp.nargs.n_waves == rp.grid * rp.nargs.waves_per_wg, "launch shape");
+    if (!tuned || t.max_grid == 0)
+      CHECK(64ull * rp.nargs.n_waves >= static_cast<uint64_t>(rp.nargs.lines) * rp.nargs.lanes_per_row, "grid smaller than the slots");
+  }
+}
+
+}  // namespace
+
+int main(int argc, char** argv) {
+  const long cases = argc > 1 ? std::atol(argv[1]) : 200000;
+  for (long i = 0; i < cases; ++i) {
+    one_copy_plan();
+    one_fill_plan();
+    one_rect_plan();
+  }
+  std::printf("%s: %ld cases each of copy, fill and region plans, %d failures\n", g_failures ? "FAILED" : "OK", cases,
+              g_failures);
+  return g_failures ? 1 : 0;
+}

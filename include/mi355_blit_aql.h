@@ -61,6 +61,13 @@ int mi355_aql_fill32(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dword
 int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t n,
                          const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal);
 
+/* The same with device-resident descriptors (read in place; they must stay
+ * valid until completion and be ready when the dependencies are).  The host
+ * cannot know the work's size, so the copy runs on a device-filling grid
+ * whose waves share the chunks out evenly.  Four packets. */
+int mi355_aql_copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, size_t n,
+                                const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal);
+
 /* Pitched 3-D region copy, asynchronous like mi355_aql_copy: the shader
  * counterpart of BlitSdmaBase::SubmitCopyRectCommand
  * (core/inc/amd_blit_sdma.h:68-73), which the reference reaches through

@@ -15,6 +15,7 @@ SIGNATURES = {
     "mi355_aql_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
     "mi355_aql_fill32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
     "mi355_aql_copy_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
+    "mi355_aql_copy_batch_device": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
     "mi355_aql_copy_rect": (C.c_int, [C.c_void_p, C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
                                       C.POINTER(Dim3), C.POINTER(Dim3), _U64P, C.c_uint32, C.c_uint64]),
     "mi355_aql_wait_idle": (C.c_int, [C.c_void_p]),
@@ -102,9 +103,11 @@ class AqlBlit:
         arr, n = _deps(deps)
         return self.lib.mi355_aql_fill32(self.handle, ptr, value, num_dwords, arr, n, completion)
 
-    def copy_batch(self, descs, n, *, deps=None, completion=0):
+    def copy_batch(self, descs, n, on_device=False, *, deps=None, completion=0):
         arr, nd = _deps(deps)
         addr = descs if isinstance(descs, int) or descs is None else C.cast(descs, C.c_void_p)
+        if on_device:
+            return self.lib.mi355_aql_copy_batch_device(self.handle, addr, n, arr, nd, completion)
         return self.lib.mi355_aql_copy_batch(self.handle, addr, n, arr, nd, completion)
 
     def copy_rect(self, dst, dst_offset, src, src_offset, extent, *, deps=None, completion=0):

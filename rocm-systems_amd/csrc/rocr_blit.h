@@ -199,7 +199,7 @@ class BlitKernelGfx950Aql : public core::Blit {
                                        core::Signal& out_signal,
                                        std::vector<core::Signal*>& gang_signals) override;
   hsa_status_t SubmitLinearFillCommand(void* ptr, uint32_t value, size_t count) override;
-  /// Batched small copies (host-resident descriptors); no counterpart in core::Blit.
+  /// Batched small copies, descriptors in host or device memory; no counterpart in core::Blit.
   hsa_status_t SubmitBatchCopyCommand(const void* descs, size_t n, bool descs_on_device,
                                       std::vector<core::Signal*>& dep_signals,
                                       core::Signal& out_signal);

@@ -435,8 +435,6 @@ def test_batch_edge_lengths(capi, blit, oracle, arenas):
 
 
 def test_batch_device_resident_descriptors(capi, blit, oracle, arenas, torch_cuda):
-    if blit.backend != "hip":
-        pytest.skip("device-resident descriptors are a feature of the HIP-stream path")
     torch = torch_cuda
     src, src_host, dst = arenas
     n = 777

@@ -129,7 +129,12 @@ struct mi355_aql {
   uint16_t fence_scope = HSA_FENCE_SCOPE_SYSTEM;
   std::atomic<bool> queue_error{false};
 
-  // batched path: two host staging buffers used alternately, device buffers
+  // batched path: two staging buffers used alternately, device buffers.  The
+  // staging buffers sit in device memory when the host can write there (as
+  // the kernarg ring does): the host's copy of the descriptors then lands in
+  // HBM while the batch before still runs, and the GPU does not fetch 24 bytes
+  // per copy across the bus at the head of the batch.
+  bool stage_in_device_memory[2] = {false, false};
   BatchDesc* stage[2] = {nullptr, nullptr};
   hsa_signal_t stage_free[2] = {{0}, {0}};  // 0 when the kernel that reads stage[i] has finished
   unsigned next_stage = 0;
@@ -368,6 +373,26 @@ int alloc(mi355_aql* h, hsa_amd_memory_pool_t pool, size_t bytes, void** out, bo
   return MI355_BLIT_SUCCESS;
 }
 
+// One staging buffer of the batched path: device memory the host can write
+// when the kernarg ring found that to work, host memory the GPU can read
+// otherwise.
+int alloc_stage(mi355_aql* h, size_t bytes, int i) {
+  h->stage[i] = nullptr;
+  h->stage_in_device_memory[i] = false;
+  if (h->kernargs_in_device_memory) {
+    void* p = nullptr;
+    if (hsa_amd_memory_pool_allocate(h->local_pool, bytes, 0, &p) == HSA_STATUS_SUCCESS) {
+      if (hsa_amd_agents_allow_access(1, &h->cpu, nullptr, p) == HSA_STATUS_SUCCESS) {
+        h->stage[i] = static_cast<BatchDesc*>(p);
+        h->stage_in_device_memory[i] = true;
+        return MI355_BLIT_SUCCESS;
+      }
+      (void)hsa_amd_memory_pool_free(p);
+    }
+  }
+  return alloc(h, h->host_pool, bytes, reinterpret_cast<void**>(&h->stage[i]), true);
+}
+
 uint64_t host_desc_chunks(const mi355_blit_desc_t& d) {
   if (d.bytes == 0) return 0;
   uint64_t head = (16 - (reinterpret_cast<uintptr_t>(d.dst) & 15)) & 15;
@@ -418,8 +443,7 @@ int ensure_batch_capacity(mi355_aql* h, size_t n, size_t n_records) {
     h->block_sum_dev = nullptr;
     h->batch_capacity = 0;
     for (int i = 0; i < 2; ++i) {
-      if ((rc = alloc(h, h->host_pool, cap * sizeof(BatchDesc), reinterpret_cast<void**>(&h->stage[i]), true)))
-        return rc;
+      if ((rc = alloc_stage(h, cap * sizeof(BatchDesc), i)) != MI355_BLIT_SUCCESS) return rc;
       hsa_signal_store_relaxed(h->stage_free[i], 0);
     }
     if ((rc = alloc(h, h->local_pool, cap * sizeof(BatchDesc), reinterpret_cast<void**>(&h->descs_dev), false))) return rc;
@@ -720,11 +744,17 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
     if (h->queue_error.load()) return MI355_BLIT_ERROR;
   }
   std::memcpy(h->stage[b], descs, n * sizeof(BatchDesc));
+  if (h->stage_in_device_memory[b]) {
+    // posted writes across the bus: order them and read one back, as for kernargs
+    _mm_sfence();
+    (void)*reinterpret_cast<volatile uint64_t*>(&h->stage[b][n - 1].bytes);
+  }
   hsa_signal_store_relaxed(h->stage_free[b], 1);
 
   // 1..3. prefix sum and records.  The first kernel reads the descriptors
-  // straight from the staging buffer in host memory and leaves a copy in
-  // device memory for the ones that follow.
+  // straight from the staging buffer (with system-scope loads: the host wrote
+  // it, across the bus or into host memory) and leaves a copy in device memory
+  // for the ones that follow.
   const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
   ScanLocalArgs sl{h->stage[b], static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev, h->descs_dev};
   ScanTopArgs stp{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};

@@ -6,8 +6,11 @@
 // 641-785).
 #include <hip/hip_runtime.h>
 
+#include <xmmintrin.h>
+
 #include <atomic>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <new>
@@ -58,8 +61,15 @@ struct mi355_blit {
   hipStream_t last_stream = nullptr;
 
   // batched path staging (grown on demand, never shrunk)
-  BatchDesc* descs_host[2] = {nullptr, nullptr};  // pinned, used alternately
-  hipEvent_t upload_done[2] = {nullptr, nullptr};  // the upload from descs_host[i] has finished
+  // Two staging buffers for host-resident descriptors, used alternately.  On a
+  // device whose memory the host can write (large BAR) they are device memory:
+  // the host's copy lands in HBM while the batch before still runs (measured:
+  // 1.5 MiB in 35 us of host time) and the first kernel reads it at HBM speed
+  // instead of fetching it across the bus (32 us at the head of every batch).
+  // Pinned host memory otherwise.
+  bool stage_in_device_memory = false;
+  BatchDesc* descs_host[2] = {nullptr, nullptr};
+  hipEvent_t upload_done[2] = {nullptr, nullptr};  // the kernel that reads descs_host[i] has finished
   bool upload_busy[2] = {false, false};
   unsigned next_host = 0;
   BatchDesc* descs_dev = nullptr;
@@ -211,7 +221,10 @@ int ledger_record(mi355_blit* h, hipStream_t s, uint64_t bytes) {
 
 void free_batch_buffers(mi355_blit* h) {
   for (int i = 0; i < 2; ++i) {
-    if (h->descs_host[i]) (void)hipHostFree(h->descs_host[i]);
+    if (h->descs_host[i]) {
+      if (h->stage_in_device_memory) (void)hipFree(h->descs_host[i]);
+      else (void)hipHostFree(h->descs_host[i]);
+    }
     h->descs_host[i] = nullptr;
   }
   if (h->descs_dev) (void)hipFree(h->descs_dev);
@@ -239,7 +252,10 @@ int ensure_batch_capacity(mi355_blit* h, size_t n, size_t n_records) {
     for (int i = 0; i < 2; ++i) {
       // uploads from the old pinned buffers are over: staging_free was waited for above
       h->upload_busy[i] = false;
-      BLIT_HIP(hipHostMalloc(reinterpret_cast<void**>(&h->descs_host[i]), cap * sizeof(BatchDesc), hipHostMallocDefault));
+      if (h->stage_in_device_memory)
+        BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->descs_host[i]), cap * sizeof(BatchDesc)));
+      else
+        BLIT_HIP(hipHostMalloc(reinterpret_cast<void**>(&h->descs_host[i]), cap * sizeof(BatchDesc), hipHostMallocDefault));
     }
     BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->descs_dev), cap * sizeof(BatchDesc)));
     BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->chunk_start_dev), (cap + 1) * sizeof(uint32_t)));
@@ -326,6 +342,10 @@ int mi355_blit_create(int device_ordinal, mi355_blit_t** out) {
     return e == hipSuccess ? MI355_BLIT_ERROR : status_of(e);
   }
   h->num_cus = cus;
+  int large_bar = 0;
+  if (hipDeviceGetAttribute(&large_bar, hipDeviceAttributeIsLargeBar, device_ordinal) == hipSuccess && large_bar &&
+      !std::getenv("MI355_BLIT_HOST_STAGING"))
+    h->stage_in_device_memory = true;
   *out = h;
   return MI355_BLIT_SUCCESS;
 }
@@ -477,15 +497,21 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
       h->upload_busy[b] = false;
     }
     std::memcpy(h->descs_host[b], descs, n * sizeof(BatchDesc));
+    if (h->stage_in_device_memory) {
+      // posted writes across the bus: order them, then read one back so that
+      // they have landed before the launch below can reach the GPU
+      _mm_sfence();
+      (void)*reinterpret_cast<volatile uint64_t*>(&h->descs_host[b][n - 1].bytes);
+    }
     host_descs = h->descs_host[b];
     host_buffer = static_cast<int>(b);
     dev_descs = h->descs_dev;
   }
 
-  // The first kernel reads host-resident descriptors straight from the pinned
+  // The first kernel reads host-resident descriptors straight from the staging
   // buffer and leaves the device copy behind: a separate upload would cost a
   // copy-engine transfer and two engine switches (measured: 33 us + 26 us of
-  // gaps for 65,536 descriptors, against 30 us of reading across the bus).
+  // gaps for 65,536 descriptors).
   const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
   ScanLocalArgs sl{host_descs ? host_descs : dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev,
                    h->block_sum_dev, host_descs ? h->descs_dev : nullptr};

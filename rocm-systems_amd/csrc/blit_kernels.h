@@ -356,8 +356,18 @@ __device__ __forceinline__ void scan_local_body(const ScanLocalArgs& a) {
   const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 1024 + threadIdx.x;
   uint32_t c = 0;
   if (i < n) {
-    const BatchDesc d = descs[i];
-    if (a.device_copy) a.device_copy[i] = d;
+    BatchDesc d;
+    if (a.device_copy) {
+      // Written by the host, into host memory or across the bus into device
+      // memory, behind the GPU's caches: read at system scope.
+      const uint64_t* w = reinterpret_cast<const uint64_t*>(descs + i);
+      d.dst = reinterpret_cast<uint8_t*>(__hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM));
+      d.src = reinterpret_cast<const uint8_t*>(__hip_atomic_load(w + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM));
+      d.bytes = __hip_atomic_load(w + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      a.device_copy[i] = d;
+    } else {
+      d = descs[i];
+    }
     c = desc_chunks(d);
   }
   uint32_t total;

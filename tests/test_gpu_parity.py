@@ -434,6 +434,42 @@ def test_batch_edge_lengths(capi, blit, oracle, arenas):
     assert np.array_equal(dst.host(0, total), _expect_batch(oracle, src_host, total, lens, offs, so, do))
 
 
+def test_batches_in_a_row_with_different_descriptors(capi, blit, oracle, arenas):
+    """Eight batches back to back on one engine, each with its own descriptors,
+    submitted without waiting in between: the two staging buffers are rewritten
+    by the host while earlier batches run, and every batch must still read its
+    own descriptors (not a cached image of the buffer's previous content)."""
+    src, src_host, dst = arenas
+    # disjoint destination windows of 8 MiB, one per batch
+    window = 8 * MIB
+    batches = []
+    for k in range(8):
+        rng = np.random.default_rng(9000 + k)
+        n = int(rng.integers(200, 1500))
+        lens = np.floor(64 * 2.0 ** (10 * rng.random(n))).astype(np.int64)      # 64 B .. 64 KiB
+        stride = ((lens + 255) // 256) * 256 + 512
+        keep = np.cumsum(stride) + 512 < window
+        lens, stride, n = lens[keep], stride[keep], int(keep.sum())
+        offs = np.concatenate([[0], np.cumsum(stride)[:-1]]) + 256 + k * window
+        so, do = rng.integers(0, 16, n), rng.integers(0, 256, n)
+        descs = (capi.Desc * n)()
+        for i in range(n):
+            descs[i].dst = dst.base + int(offs[i] + do[i])
+            descs[i].src = src.base + int(offs[i] + so[i])
+            descs[i].bytes = int(lens[i])
+        batches.append((descs, n, lens, offs, so, do))
+    dst.fill(0, 8 * window, GUARD_BYTE)
+    for descs, n, *_ in batches:
+        check_ok(capi, blit.copy_batch(descs, n), "copy_batch")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    want = np.full(8 * window, GUARD_BYTE, dtype=np.uint8)
+    for _, n, lens, offs, so, do in batches:
+        for i in range(n):
+            oracle.oracle_copy(want.ctypes.data + int(offs[i] + do[i]), src_host.ctypes.data + int(offs[i] + so[i]),
+                               int(lens[i]))
+    assert np.array_equal(dst.host(0, 8 * window), want)
+
+
 def test_batch_device_resident_descriptors(capi, blit, oracle, arenas, torch_cuda):
     torch = torch_cuda
     src, src_host, dst = arenas

@@ -56,7 +56,7 @@ int mi355_aql_fill32(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dword
                      const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal);
 
 /* Batched small copies (no counterpart in the reference): n host-resident
- * descriptors, one submission of four packets, the last one carrying the
+ * descriptors, one submission of two packets, the last one carrying the
  * completion signal. */
 int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t n,
                          const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal);

@@ -22,6 +22,7 @@
 
 #include "blit_args.h"
 #include "blit_kernel_list.h"
+#include "blit_batch_host.h"
 #include "blit_plan.h"
 #include "blit_rect.h"
 #include "mi355_blit_aql.h"
@@ -35,7 +36,7 @@ namespace {
 using namespace mi355;
 
 // Packets in the queue.  The reference shares the agent's 64-packet utility
-// queue (amd_gpu_agent.h:507-508); a batch here is four packets, so the ring
+// queue (amd_gpu_agent.h:507-508); a batch here is two packets, so the ring
 // is a little larger.
 constexpr uint32_t kQueuePackets = 256;
 // One kernarg slot per packet slot, as in the reference (amd_blit_kernel.cpp:
@@ -106,7 +107,7 @@ struct mi355_aql {
   std::vector<BatchKernel> batch_kernels{MI355_FOR_EACH_BATCH_RECORDS_KERNEL(MI355_BATCH_NAME)};
   std::vector<RectKernel> rect_kernels{MI355_FOR_EACH_RECT_KERNEL(MI355_RECT_NAME)};
   std::vector<RectKernel> rect_narrow_kernels{MI355_FOR_EACH_RECT_NARROW_KERNEL(MI355_RECT_NARROW_NAME)};
-  Kernel scan_local, scan_top, make_records, finalize, strided_cached, strided_streaming;
+  Kernel scan_local, scan_top, emit_records, finalize, strided_cached, strided_streaming;
 
   hsa_signal_t idle_signal{};  // completion signal of wait_idle's barrier packet
 
@@ -136,9 +137,9 @@ struct mi355_aql {
   // per copy across the bus at the head of the batch.
   bool stage_in_device_memory[2] = {false, false};
   BatchDesc* stage[2] = {nullptr, nullptr};
+  BatchImage stage_image;  // built in ordinary memory, then copied to a staging buffer
   hsa_signal_t stage_free[2] = {{0}, {0}};  // 0 when the kernel that reads stage[i] has finished
   unsigned next_stage = 0;
-  BatchDesc* descs_dev = nullptr;
   uint32_t* chunk_start_dev = nullptr;
   uint32_t* block_sum_dev = nullptr;
   ChunkRecord* records_dev = nullptr;
@@ -249,7 +250,7 @@ int load_code_object(mi355_aql* h) {
     if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_scan_local", &h->scan_local)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_scan_top", &h->scan_top)) != MI355_BLIT_SUCCESS) return rc;
-  if ((rc = lookup(h, "mi355_batch_make_records", &h->make_records)) != MI355_BLIT_SUCCESS) return rc;
+  if ((rc = lookup(h, "mi355_batch_emit_records", &h->emit_records)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_finalize", &h->finalize)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_strided_l0_s0", &h->strided_cached)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_strided_l1_s1", &h->strided_streaming)) != MI355_BLIT_SUCCESS) return rc;
@@ -393,16 +394,6 @@ int alloc_stage(mi355_aql* h, size_t bytes, int i) {
   return alloc(h, h->host_pool, bytes, reinterpret_cast<void**>(&h->stage[i]), true);
 }
 
-uint64_t host_desc_chunks(const mi355_blit_desc_t& d) {
-  if (d.bytes == 0) return 0;
-  uint64_t head = (16 - (reinterpret_cast<uintptr_t>(d.dst) & 15)) & 15;
-  if (head > d.bytes) head = d.bytes;
-  const uint64_t n_vec = (d.bytes - head) / 16;
-  const uint64_t lead = ((reinterpret_cast<uintptr_t>(d.dst) + head) & 255) / 16;
-  const uint64_t c = (n_vec + lead + kBatchChunkVecs - 1) / kBatchChunkVecs;
-  return c ? c : 1;
-}
-
 int wait_idle_locked(mi355_aql* h) {
   hsa_signal_store_relaxed(h->idle_signal, 1);
   uint64_t index;
@@ -435,18 +426,15 @@ int ensure_batch_capacity(mi355_aql* h, size_t n, size_t n_records) {
       free_device(h->stage[i]);
       h->stage[i] = nullptr;
     }
-    free_device(h->descs_dev);
     free_device(h->chunk_start_dev);
     free_device(h->block_sum_dev);
-    h->descs_dev = nullptr;
     h->chunk_start_dev = nullptr;
     h->block_sum_dev = nullptr;
     h->batch_capacity = 0;
     for (int i = 0; i < 2; ++i) {
-      if ((rc = alloc_stage(h, cap * sizeof(BatchDesc), i)) != MI355_BLIT_SUCCESS) return rc;
+      if ((rc = alloc_stage(h, batch_stage_bytes(cap), i)) != MI355_BLIT_SUCCESS) return rc;
       hsa_signal_store_relaxed(h->stage_free[i], 0);
     }
-    if ((rc = alloc(h, h->local_pool, cap * sizeof(BatchDesc), reinterpret_cast<void**>(&h->descs_dev), false))) return rc;
     if ((rc = alloc(h, h->local_pool, (cap + 1) * sizeof(uint32_t), reinterpret_cast<void**>(&h->chunk_start_dev), false)))
       return rc;
     if ((rc = alloc(h, h->local_pool, (cap / 1024 + 1) * sizeof(uint32_t), reinterpret_cast<void**>(&h->block_sum_dev), false)))
@@ -543,7 +531,6 @@ int mi355_aql_destroy(mi355_aql_t* h) {
       free_device(h->stage[i]);
       if (h->stage_free[i].handle) hsa_signal_destroy(h->stage_free[i]);
     }
-    free_device(h->descs_dev);
     free_device(h->chunk_start_dev);
     free_device(h->block_sum_dev);
     free_device(h->records_dev);
@@ -722,46 +709,42 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   if (!h || (!descs && n) || (num_deps && !dep_signals)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   if (n > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   if (h->queue_error.load()) return MI355_BLIT_ERROR;
-  uint64_t total_bytes = 0, total_chunks = 0;
-  for (size_t i = 0; i < n; ++i) {
-    if (descs[i].bytes && (!descs[i].dst || !descs[i].src)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
-    total_bytes += descs[i].bytes;
-    total_chunks += host_desc_chunks(descs[i]);
+  std::unique_lock<std::mutex> g(h->lock);
+  BatchShape shape;
+  int rc = batch_build(descs, n, &h->stage_image, &shape);
+  if (rc != MI355_BLIT_SUCCESS) return rc;
+  const uint64_t total_bytes = shape.total_bytes, total_chunks = shape.total_chunks;
+  if (total_chunks == 0) {
+    g.unlock();
+    return mi355_aql_copy(h, h, h, 0, dep_signals, num_deps, completion_signal);
   }
-  if (total_chunks > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
-  if (total_chunks == 0) return mi355_aql_copy(h, h, h, 0, dep_signals, num_deps, completion_signal);
-
-  std::lock_guard<std::mutex> g(h->lock);
-  int rc = ensure_batch_capacity(h, n, total_chunks);
+  rc = ensure_batch_capacity(h, shape.pieces, total_chunks);
   if (rc != MI355_BLIT_SUCCESS) return rc;
   const mi355_blit_tuning_t* t = h->has_tuning ? &h->tuning : nullptr;
 
-  // stage the descriptors in host memory the GPU can read; the buffer is
-  // free again when the upload that read it last has finished
+  // Stage what the GPU needs: the descriptors, cut into pieces of at most
+  // 1 MiB, and each piece's first record index (the host, which walks the
+  // descriptors anyway, does the prefix sum).  The buffer is free again when
+  // the kernel that read it last has finished.
   const unsigned b = h->next_stage;
   h->next_stage ^= 1;
   while (hsa_signal_wait_scacquire(h->stage_free[b], HSA_SIGNAL_CONDITION_LT, 1, UINT64_MAX, HSA_WAIT_STATE_ACTIVE) >= 1) {
     if (h->queue_error.load()) return MI355_BLIT_ERROR;
   }
-  std::memcpy(h->stage[b], descs, n * sizeof(BatchDesc));
+  const size_t image_bytes = batch_stage_bytes(shape.pieces);
+  batch_stage(h->stage_image, h->stage[b]);
   if (h->stage_in_device_memory[b]) {
     // posted writes across the bus: order them and read one back, as for kernargs
     _mm_sfence();
-    (void)*reinterpret_cast<volatile uint64_t*>(&h->stage[b][n - 1].bytes);
+    (void)*(reinterpret_cast<volatile uint32_t*>(reinterpret_cast<uint8_t*>(h->stage[b]) + image_bytes) - 1);
   }
   hsa_signal_store_relaxed(h->stage_free[b], 1);
 
-  // 1..3. prefix sum and records.  The first kernel reads the descriptors
-  // straight from the staging buffer (with system-scope loads: the host wrote
-  // it, across the bus or into host memory) and leaves a copy in device memory
-  // for the ones that follow.
-  const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
-  ScanLocalArgs sl{h->stage[b], static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev, h->descs_dev};
-  ScanTopArgs stp{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
-  MakeRecordsArgs mr{h->descs_dev, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev, total_chunks,
-                     h->records_dev, n_blocks};
+  // 1. one lane per piece writes the piece's chunk records
+  EmitRecordsArgs er{h->stage[b], reinterpret_cast<const uint32_t*>(h->stage[b] + shape.pieces), shape.pieces,
+                     h->records_dev};
 
-  // 4. the copy
+  // 2. the copy
   mi355_blit_plan_t p{};
   p.kernel = MI355_BLIT_KERNEL_COPY_BATCH;
   p.body_vecs = total_chunks;
@@ -788,7 +771,7 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   h->last_plan = p;
 
   const uint32_t nb = barrier_packets(num_deps);
-  const uint32_t total = nb + 4;
+  const uint32_t total = nb + 2;
   uint64_t index;
   {
     std::lock_guard<std::mutex> r(h->reservation_lock);
@@ -797,12 +780,11 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   }
   write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
   uint64_t i = index + nb;
-  // every packet of the sequence waits for the one before (barrier bit); the
-  // first also waits for whatever still uses the shared device buffers, and
-  // frees the staging buffer when it is done with it
-  write_dispatch(h, i++, h->scan_local, &sl, sizeof(sl), n_blocks, 1024, h->stage_free[b].handle, true);
-  write_dispatch(h, i++, h->scan_top, &stp, sizeof(stp), 1, 1024, 0, true);
-  write_dispatch(h, i++, h->make_records, &mr, sizeof(mr), static_cast<uint32_t>((total_chunks + 255) / 256), 256, 0, true);
+  // Both packets wait for everything before them (barrier bit): the first for
+  // whatever still reads the shared record buffer; it frees the staging buffer
+  // when it is done with it.
+  write_dispatch(h, i++, h->emit_records, &er, sizeof(er), static_cast<uint32_t>((shape.pieces + 255) / 256), 256,
+                 h->stage_free[b].handle, true);
   write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true);
   release_write_index(h, index, total);
   return MI355_BLIT_SUCCESS;
@@ -821,7 +803,7 @@ int mi355_aql_copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_
   const mi355_blit_tuning_t* t = h->has_tuning ? &h->tuning : nullptr;
   const BatchDesc* descs = reinterpret_cast<const BatchDesc*>(device_descs);
   const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
-  ScanLocalArgs sl{descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev, nullptr};
+  ScanLocalArgs sl{descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
   ScanTopArgs stp{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
   FinalizeArgs fa{static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
 

@@ -68,10 +68,6 @@ struct ScanLocalArgs {
   uint64_t n;
   uint32_t* chunk_start;
   uint32_t* block_sum;
-  // When not null, descs is host memory the GPU reads across the bus and each
-  // lane leaves a copy of its descriptor here, in device memory, for the
-  // kernels that follow.
-  BatchDesc* device_copy;
 };
 
 struct ScanTopArgs {
@@ -87,14 +83,13 @@ struct FinalizeArgs {
   const uint32_t* block_sum;
 };
 
-struct MakeRecordsArgs {
-  const BatchDesc* descs;
+// Host-resident descriptors: the host has cut them into pieces and summed
+// their chunk counts; one lane per piece writes the piece's records.
+struct EmitRecordsArgs {
+  const BatchDesc* descs;       // staged by the host
+  const uint32_t* first_record; // index of each piece's first record
   uint64_t n;
-  const uint32_t* chunk_start;
-  const uint32_t* block_sum;
-  uint64_t total_chunks;
   ChunkRecord* records;
-  uint32_t n_blocks;
 };
 
 struct BatchCopyArgs {

@@ -1,0 +1,112 @@
+// Host half of the batched copy with host-resident descriptors, shared by the
+// HIP and the AQL submission paths: validation, the chunk count of every
+// copy, and the staging image the GPU reads.  Pure host code.
+//
+// The host walks the descriptors anyway to validate them, so it also does the
+// prefix sum over their chunk counts: the GPU then needs one small kernel (one
+// lane per copy writes that copy's chunk records) before the copy kernel.
+// Copies longer than 1 MiB are cut at 1 MiB boundaries of the destination into
+// pieces that are copies in their own right, so that no lane has more than
+// 257 records to write.  No counterpart in the reference.
+#ifndef MI355_BLIT_BATCH_HOST_H_
+#define MI355_BLIT_BATCH_HOST_H_
+
+#include <stdint.h>
+#include <string.h>
+
+#include <vector>
+
+#include "blit_args.h"
+#include "blit_plan.h"
+#include "mi355_blit.h"
+
+namespace mi355 {
+
+constexpr uint64_t kBatchPieceBytes = 1ull << 20;
+
+struct BatchShape {
+  uint64_t pieces = 0;        // descriptors after cutting
+  uint64_t total_chunks = 0;  // 4 KiB chunks of all pieces
+  uint64_t total_bytes = 0;
+};
+
+// Chunks of one copy (desc_chunks in the kernels).
+inline uint64_t batch_desc_chunks(uint64_t dst, uint64_t bytes) {
+  if (bytes == 0) return 0;
+  uint64_t head = (16 - (dst & 15)) & 15;
+  if (head > bytes) head = bytes;
+  const uint64_t n_vec = (bytes - head) / 16;
+  const uint64_t lead = ((dst + head) & 255) / 16;
+  const uint64_t c = (n_vec + lead + kBatchChunkVecs - 1) / kBatchChunkVecs;
+  return c ? c : 1;
+}
+
+// Calls f(dst, src, bytes) for every piece of one copy.
+template <typename F>
+inline void batch_for_each_piece(const mi355_blit_desc_t& d, F f) {
+  const uint64_t dst = reinterpret_cast<uintptr_t>(d.dst), src = reinterpret_cast<uintptr_t>(d.src);
+  uint64_t at = 0;
+  while (at < d.bytes) {
+    uint64_t end = ((dst + at) / kBatchPieceBytes + 1) * kBatchPieceBytes - dst;
+    if (end > d.bytes) end = d.bytes;
+    f(dst + at, src + at, end - at);
+    at = end;
+  }
+}
+
+// The staging image of a batch, built in ordinary host memory: the pieces and,
+// for each, the index of its first chunk record.
+struct BatchImage {
+  std::vector<BatchDesc> pieces;
+  std::vector<uint32_t> first_record;
+};
+
+// Validates the descriptors, cuts them into pieces, sums the chunk counts: one
+// pass.  image is reused between calls (its vectors keep their capacity).
+inline int batch_build(const mi355_blit_desc_t* descs, size_t n, BatchImage* image, BatchShape* out) {
+  BatchShape s;
+  image->pieces.clear();
+  image->first_record.clear();
+  if (image->pieces.capacity() < n) {
+    image->pieces.reserve(n + n / 8 + 16);
+    image->first_record.reserve(n + n / 8 + 16);
+  }
+  auto add = [&](uint64_t dst, uint64_t src, uint64_t bytes) {
+    BatchDesc p;
+    p.dst = reinterpret_cast<uint8_t*>(dst);
+    p.src = reinterpret_cast<const uint8_t*>(src);
+    p.bytes = bytes;
+    image->pieces.push_back(p);
+    image->first_record.push_back(static_cast<uint32_t>(s.total_chunks));
+    s.total_chunks += batch_desc_chunks(dst, bytes);
+  };
+  for (size_t i = 0; i < n; ++i) {
+    const mi355_blit_desc_t& d = descs[i];
+    if (d.bytes == 0) continue;
+    if (!d.dst || !d.src) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+    s.total_bytes += d.bytes;
+    batch_for_each_piece(d, add);
+    if (s.total_chunks > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  }
+  s.pieces = image->pieces.size();
+  if (s.pieces > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  *out = s;
+  return MI355_BLIT_SUCCESS;
+}
+
+// Bytes of the staging buffer for `pieces` descriptors: the descriptors, then,
+// right behind them, each one's first record index.
+inline size_t batch_stage_bytes(uint64_t pieces) {
+  return static_cast<size_t>(pieces) * (sizeof(BatchDesc) + sizeof(uint32_t));
+}
+
+// Copies the image to where the GPU reads it.
+inline void batch_stage(const BatchImage& image, void* stage) {
+  const size_t n = image.pieces.size();
+  memcpy(stage, image.pieces.data(), n * sizeof(BatchDesc));
+  memcpy(static_cast<uint8_t*>(stage) + n * sizeof(BatchDesc), image.first_record.data(), n * sizeof(uint32_t));
+}
+
+}  // namespace mi355
+
+#endif  // MI355_BLIT_BATCH_HOST_H_

@@ -14,8 +14,10 @@
 #include <cstring>
 #include <mutex>
 #include <new>
+#include <vector>
 
 #include "blit_kernels.h"
+#include "blit_batch_host.h"
 #include "blit_plan.h"
 #include "blit_rect.h"
 #include "mi355_blit.h"
@@ -69,10 +71,10 @@ struct mi355_blit {
   // Pinned host memory otherwise.
   bool stage_in_device_memory = false;
   BatchDesc* descs_host[2] = {nullptr, nullptr};
+  BatchImage stage_image;  // built in ordinary memory, then copied to a staging buffer
   hipEvent_t upload_done[2] = {nullptr, nullptr};  // the kernel that reads descs_host[i] has finished
   bool upload_busy[2] = {false, false};
   unsigned next_host = 0;
-  BatchDesc* descs_dev = nullptr;
   uint32_t* chunk_start_dev = nullptr;
   uint32_t* block_sum_dev = nullptr;
   ChunkRecord* records_dev = nullptr;  // one per chunk
@@ -227,10 +229,8 @@ void free_batch_buffers(mi355_blit* h) {
     }
     h->descs_host[i] = nullptr;
   }
-  if (h->descs_dev) (void)hipFree(h->descs_dev);
   if (h->chunk_start_dev) (void)hipFree(h->chunk_start_dev);
   if (h->block_sum_dev) (void)hipFree(h->block_sum_dev);
-  h->descs_dev = nullptr;
   h->chunk_start_dev = nullptr;
   h->block_sum_dev = nullptr;
   h->batch_capacity = 0;
@@ -253,11 +253,10 @@ int ensure_batch_capacity(mi355_blit* h, size_t n, size_t n_records) {
       // uploads from the old pinned buffers are over: staging_free was waited for above
       h->upload_busy[i] = false;
       if (h->stage_in_device_memory)
-        BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->descs_host[i]), cap * sizeof(BatchDesc)));
+        BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->descs_host[i]), batch_stage_bytes(cap)));
       else
-        BLIT_HIP(hipHostMalloc(reinterpret_cast<void**>(&h->descs_host[i]), cap * sizeof(BatchDesc), hipHostMallocDefault));
+        BLIT_HIP(hipHostMalloc(reinterpret_cast<void**>(&h->descs_host[i]), batch_stage_bytes(cap), hipHostMallocDefault));
     }
-    BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->descs_dev), cap * sizeof(BatchDesc)));
     BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->chunk_start_dev), (cap + 1) * sizeof(uint32_t)));
     BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->block_sum_dev), (cap / 1024 + 1) * sizeof(uint32_t)));
     h->batch_capacity = cap;
@@ -272,17 +271,6 @@ int ensure_batch_capacity(mi355_blit* h, size_t n, size_t n_records) {
     h->records_capacity = cap;
   }
   return MI355_BLIT_SUCCESS;
-}
-
-// Same split as desc_head / desc_chunks on the device.
-inline uint64_t host_desc_chunks(const mi355_blit_desc_t& d) {
-  if (d.bytes == 0) return 0;
-  uint64_t head = (16 - (reinterpret_cast<uintptr_t>(d.dst) & 15)) & 15;
-  if (head > d.bytes) head = d.bytes;
-  const uint64_t n_vec = (d.bytes - head) / 16;
-  const uint64_t lead = ((reinterpret_cast<uintptr_t>(d.dst) + head) & 255) / 16;
-  const uint64_t c = (n_vec + lead + kBatchChunkVecs - 1) / kBatchChunkVecs;
-  return c ? c : 1;
 }
 
 }  // namespace
@@ -462,103 +450,92 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
   if (scope.err != hipSuccess) return status_of(scope.err);
   hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
 
-  uint64_t total_bytes = 0;
-  uint64_t total_chunks = 0;
+  BatchShape shape;
   if (!descs_on_device) {
-    for (size_t i = 0; i < n; ++i) {
-      if (descs[i].bytes && (!descs[i].dst || !descs[i].src)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
-      total_bytes += descs[i].bytes;
-      total_chunks += host_desc_chunks(descs[i]);
-    }
-    if (total_chunks == 0) return MI355_BLIT_SUCCESS;
-    if (total_chunks > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+    int rc = batch_build(descs, n, &h->stage_image, &shape);
+    if (rc != MI355_BLIT_SUCCESS) return rc;
+    if (shape.total_chunks == 0) return MI355_BLIT_SUCCESS;
   } else {
-    total_bytes = n;  // lengths are only known on the device; keep the record non-zero
+    shape.pieces = n;
+    shape.total_bytes = n;  // lengths are only known on the device; keep the record non-zero
   }
-  int rc = ensure_batch_capacity(h, n, descs_on_device ? 0 : total_chunks);
+  int rc = ensure_batch_capacity(h, shape.pieces, shape.total_chunks);
   if (rc != MI355_BLIT_SUCCESS) return rc;
 
-  // The device-side staging buffers are shared by consecutive batches: the
-  // next batch waits for the previous one on the stream.  The host writes the
-  // pinned descriptor copies alternately, so preparing one batch overlaps the
-  // execution of the one before; a pinned buffer is only waited for until its
-  // own upload, two batches ago, has finished.
+  // The device-side buffers (records, prefix sums) are shared by consecutive
+  // batches: the next batch waits for the previous one on the stream.
   if (h->staging_busy) BLIT_HIP(hipStreamWaitEvent(s, h->staging_free, 0));
-  const BatchDesc* dev_descs;
-  const BatchDesc* host_descs = nullptr;
-  int host_buffer = -1;
-  if (descs_on_device) {
-    dev_descs = reinterpret_cast<const BatchDesc*>(descs);
-  } else {
+
+  mi355_blit_plan_t p{};
+  p.kernel = MI355_BLIT_KERNEL_COPY_BATCH;
+  p.unroll = kBatchChunkVecs / 64;
+  p.body_vecs = shape.total_chunks;  // chunks, when known
+  const mi355_blit_tuning_t* t = h->has_tuning ? &h->tuning : nullptr;
+  // Measured on MI355X with 65,536 copies of 64 B..256 KiB: non-temporal loads
+  // and stores are best (739 us against 824 us cached); written-through
+  // stores are worst (958 us), because a chunk's first and last cache line
+  // are shared with its neighbours and written through in halves.
+  bool streaming = descs_on_device || shape.total_bytes >= (4ull << 20);
+  if (t && t->nt_load) streaming = (t->nt_load == 2);
+  p.nt_load = streaming;
+  p.store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
+  if (t && t->store_policy >= 1 && t->store_policy <= 4) p.store_policy = t->store_policy - 1;
+
+  if (!descs_on_device) {
+    // Host-resident descriptors.  The host has walked them to validate them
+    // and does the prefix sum over their chunk counts on the way; the image it
+    // stages (the descriptors, cut into pieces of at most 1 MiB, and each
+    // piece's first record index) is all the GPU needs to write the records
+    // with one lane per piece.  The two staging buffers alternate, so staging
+    // one batch overlaps the execution of the one before; a buffer is only
+    // waited for until the kernel that read it, two batches ago, has finished.
     const unsigned b = h->next_host;
     h->next_host ^= 1;
     if (h->upload_busy[b]) {
       BLIT_HIP(hipEventSynchronize(h->upload_done[b]));
       h->upload_busy[b] = false;
     }
-    std::memcpy(h->descs_host[b], descs, n * sizeof(BatchDesc));
+    const size_t image_bytes = batch_stage_bytes(shape.pieces);
+    batch_stage(h->stage_image, h->descs_host[b]);
     if (h->stage_in_device_memory) {
       // posted writes across the bus: order them, then read one back so that
       // they have landed before the launch below can reach the GPU
       _mm_sfence();
-      (void)*reinterpret_cast<volatile uint64_t*>(&h->descs_host[b][n - 1].bytes);
+      (void)*(reinterpret_cast<volatile uint32_t*>(reinterpret_cast<uint8_t*>(h->descs_host[b]) + image_bytes) - 1);
     }
-    host_descs = h->descs_host[b];
-    host_buffer = static_cast<int>(b);
-    dev_descs = h->descs_dev;
-  }
+    const BatchDesc* staged = h->descs_host[b];
+    EmitRecordsArgs er{staged, reinterpret_cast<const uint32_t*>(staged + shape.pieces), shape.pieces, h->records_dev};
+    hipLaunchKernelGGL(mi355_batch_emit_records, dim3(static_cast<uint32_t>((shape.pieces + 255) / 256)), dim3(256),
+                       0, s, er);
+    BLIT_HIP(hipGetLastError());
+    BLIT_HIP(hipEventRecord(h->upload_done[b], s));
+    h->upload_busy[b] = true;
 
-  // The first kernel reads host-resident descriptors straight from the staging
-  // buffer and leaves the device copy behind: a separate upload would cost a
-  // copy-engine transfer and two engine switches (measured: 33 us + 26 us of
-  // gaps for 65,536 descriptors).
-  const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
-  ScanLocalArgs sl{host_descs ? host_descs : dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev,
-                   h->block_sum_dev, host_descs ? h->descs_dev : nullptr};
-  hipLaunchKernelGGL(mi355_batch_scan_local, dim3(n_blocks), dim3(1024), 0, s, sl);
-  if (host_buffer >= 0) {
-    BLIT_HIP(hipEventRecord(h->upload_done[host_buffer], s));
-    h->upload_busy[host_buffer] = true;
-  }
-  ScanTopArgs st{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
-  hipLaunchKernelGGL(mi355_batch_scan_top, dim3(1), dim3(1024), 0, s, st);
-  BLIT_HIP(hipGetLastError());
-
-  mi355_blit_plan_t p{};
-  p.kernel = MI355_BLIT_KERNEL_COPY_BATCH;
-  p.unroll = kBatchChunkVecs / 64;
-  p.body_vecs = total_chunks;  // chunks, when known
-  const mi355_blit_tuning_t* t = h->has_tuning ? &h->tuning : nullptr;
-  // Measured on MI355X with 65,536 copies of 64 B..256 KiB: non-temporal loads
-  // and stores are best (739 us against 824 us cached); written-through
-  // stores are worst (958 us), because a chunk's first and last cache line
-  // are shared with its neighbours and written through in halves.
-  bool streaming = descs_on_device || total_bytes >= (4ull << 20);
-  if (t && t->nt_load) streaming = (t->nt_load == 2);
-  p.nt_load = streaming;
-  p.store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
-  if (t && t->store_policy >= 1 && t->store_policy <= 4) p.store_policy = t->store_policy - 1;
-  if (!descs_on_device) {
-    // the host knows the chunk total: one record per chunk
-    MakeRecordsArgs mr{dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev,
-                       total_chunks, h->records_dev, n_blocks};
-    hipLaunchKernelGGL(mi355_batch_make_records, dim3(static_cast<uint32_t>((total_chunks + 255) / 256)),
-                       dim3(256), 0, s, mr);
     p.wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size : 256;
     const uint64_t waves_per_wg = p.wg_size / 64;
     unsigned split = kBatchSplit;
     if (t && (t->unroll == 1 || t->unroll == 2 || t->unroll == 4)) split = 4 / t->unroll;
-    const uint64_t waves = total_chunks * split;
+    const uint64_t waves = shape.total_chunks * split;
     uint64_t wgs = (waves + waves_per_wg - 1) / waves_per_wg;
     if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
+    if (wgs * p.wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / p.wg_size;
     p.grid = static_cast<uint32_t>(wgs);
     p.unroll = 4 / split;
     batch_kernel_t k = select_batch_kernel(split, streaming, p.store_policy);
     if (!k) return MI355_BLIT_ERROR;
-    BatchCopyArgs bc{h->records_dev, total_chunks, static_cast<uint32_t>(waves_per_wg),
+    BatchCopyArgs bc{h->records_dev, shape.total_chunks, static_cast<uint32_t>(waves_per_wg),
                      static_cast<uint32_t>(wgs * waves_per_wg)};
     hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, bc);
   } else {
+    // Device-resident descriptors: the prefix sum runs on the device and, as
+    // the host cannot size a per-chunk grid without a read-back, the copy runs
+    // on a device-filling grid whose waves share the chunks out evenly.
+    const BatchDesc* dev_descs = reinterpret_cast<const BatchDesc*>(descs);
+    const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
+    ScanLocalArgs sl{dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
+    hipLaunchKernelGGL(mi355_batch_scan_local, dim3(n_blocks), dim3(1024), 0, s, sl);
+    ScanTopArgs st{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
+    hipLaunchKernelGGL(mi355_batch_scan_top, dim3(1), dim3(1024), 0, s, st);
     FinalizeArgs fa{static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
     hipLaunchKernelGGL(mi355_batch_finalize, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, s, fa);
     p.wg_size = 256;
@@ -578,7 +555,7 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
   BLIT_HIP(hipEventRecord(h->staging_free, s));
   h->staging_busy = true;
   h->last_plan = p;
-  return ledger_record(h, s, total_bytes);
+  return ledger_record(h, s, shape.total_bytes);
 }
 
 int mi355_blit_copy_rect(mi355_blit_t* h, const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,

@@ -5,7 +5,9 @@
 // invariants that do not restate its formulas: a plan must tile its byte range
 // exactly, a region plan's units (or packed slots) must cover every row's bytes
 // once, in order and inside the row, and the region validation must give the
-// reference's verdict (oracle_ref_validate_rect).  No GPU, no device code.
+// reference's verdict (oracle_ref_validate_rect), and the staging image of a
+// batch must tile every copy into pieces with the right record indices.  No
+// GPU, no device code.
 //
 //   test_host_logic [cases]      exit status 0 = all checks passed
 #include <cinttypes>
@@ -13,8 +15,10 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <vector>
 
 #include "../../oracle/blit_oracle.h"
+#include "blit_batch_host.h"
 #include "blit_plan.h"
 #include "blit_rect.h"
 
@@ -237,6 +241,62 @@ void one_rect_plan() {
   }
 }
 
+// The staging image of a batch: the pieces must tile every copy in order, no
+// piece may be longer than 1 MiB or cross a 1 MiB boundary of the destination,
+// and the record indices must be the running sum of the pieces' chunk counts.
+void one_batch_stage() {
+  const size_t n = 1 + below(40);
+  std::vector<mi355_blit_desc_t> descs(n);
+  for (auto& d : descs) {
+    d.dst = reinterpret_cast<void*>((1ull << 40) + below(1ull << 34));
+    d.src = reinterpret_cast<const void*>((2ull << 40) + below(1ull << 34));
+    switch (below(5)) {
+      case 0: d.bytes = 0; break;
+      case 1: d.bytes = 1 + below(5000); break;
+      case 2: d.bytes = 1 + below(3u << 20); break;
+      case 3: d.bytes = (1ull << 20) * below(5) + below(3) ; break;
+      default: d.bytes = 1 + below(1ull << 28); break;
+    }
+  }
+  BatchShape shape;
+  static BatchImage image;  // reused, as the engine does
+  CHECK(batch_build(descs.data(), n, &image, &shape) == MI355_BLIT_SUCCESS, "batch_build failed");
+  const std::vector<BatchDesc>& pieces = image.pieces;
+  const std::vector<uint32_t>& starts = image.first_record;
+  CHECK(pieces.size() == shape.pieces && starts.size() == shape.pieces, "image size");
+  uint64_t p = 0, chunks = 0, bytes = 0;
+  for (const auto& d : descs) {
+    uint64_t at = 0;
+    while (at < d.bytes) {
+      CHECK(p < shape.pieces, "more pieces than counted");
+      const BatchDesc& q = pieces[p];
+      const uint64_t qd = reinterpret_cast<uint64_t>(q.dst), qs = reinterpret_cast<uint64_t>(q.src);
+      CHECK(qd == reinterpret_cast<uint64_t>(d.dst) + at && qs == reinterpret_cast<uint64_t>(d.src) + at,
+            "piece %" PRIu64 " does not continue its copy", p);
+      CHECK(q.bytes >= 1 && q.bytes <= kBatchPieceBytes && at + q.bytes <= d.bytes, "piece length %" PRIu64, q.bytes);
+      CHECK(qd / kBatchPieceBytes == (qd + q.bytes - 1) / kBatchPieceBytes, "piece crosses a 1 MiB boundary");
+      CHECK(at + q.bytes == d.bytes || (qd + q.bytes) % kBatchPieceBytes == 0, "piece stops short of the boundary");
+      CHECK(starts[p] == chunks, "record index of piece %" PRIu64, p);
+      // the chunk count, from the geometry of 256-byte anchored 4 KiB chunks
+      const uint64_t head = q.bytes < ((16 - (qd & 15)) & 15) ? q.bytes : ((16 - (qd & 15)) & 15);
+      const uint64_t body_lo = qd + head, body_hi = body_lo + (q.bytes - head) / 16 * 16;
+      // 4 KiB steps from the 256-byte boundary below the body's first vector
+      const uint64_t anchor = body_lo & ~255ull;
+      const uint64_t c = body_hi > body_lo ? (body_hi - anchor + 4095) / 4096 : 1;
+      CHECK(c <= 257, "a piece with %" PRIu64 " chunks", c);
+      chunks += c;
+      bytes += q.bytes;
+      at += q.bytes;
+      ++p;
+    }
+  }
+  CHECK(p == shape.pieces && chunks == shape.total_chunks && bytes == shape.total_bytes, "shape totals");
+  mi355_blit_desc_t bad = descs[0];
+  bad.bytes = 8;
+  bad.dst = nullptr;
+  CHECK(batch_build(&bad, 1, &image, &shape) == MI355_BLIT_ERROR_INVALID_ARGUMENT, "NULL destination accepted");
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
@@ -245,6 +305,7 @@ int main(int argc, char** argv) {
     one_copy_plan();
     one_fill_plan();
     one_rect_plan();
+    if (i % 8 == 0) one_batch_stage();
   }
   std::printf("%s: %ld cases each of copy, fill and region plans, %d failures\n", g_failures ? "FAILED" : "OK", cases,
               g_failures);

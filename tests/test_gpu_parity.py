@@ -434,6 +434,31 @@ def test_batch_edge_lengths(capi, blit, oracle, arenas):
     assert np.array_equal(dst.host(0, total), _expect_batch(oracle, src_host, total, lens, offs, so, do))
 
 
+def test_batch_with_copies_beyond_one_mib(capi, blit, oracle, arenas):
+    """Copies longer than 1 MiB are cut into pieces at 1 MiB boundaries of the
+    destination on the host; mixed here with short ones, at odd offsets."""
+    src, src_host, dst = arenas
+    lens = [5 * MIB + 3, 77, MIB, MIB + 1, 3 * MIB - 17, 4096, 2 * MIB, 1, 9 * MIB + 12345, 300000]
+    so = [3, 0, 1, 15, 7, 2, 0, 9, 5, 11]
+    do = [9, 1, 0, 255, 130, 16, 0, 3, 77, 200]
+    offs, at = [], 256
+    for n in lens:
+        offs.append(at)
+        at += (n + 255) // 256 * 256 + 512
+    total = at + 256
+    assert total <= dst.nbytes
+    descs = (capi.Desc * len(lens))()
+    for i, n in enumerate(lens):
+        descs[i].dst = dst.base + offs[i] + do[i]
+        descs[i].src = src.base + offs[i] + so[i]
+        descs[i].bytes = n
+    dst.fill(0, total, GUARD_BYTE)
+    check_ok(capi, blit.copy_batch(descs, len(lens)), "copy_batch")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    want = _expect_batch(oracle, src_host, total, np.array(lens), np.array(offs), np.array(so), np.array(do))
+    assert np.array_equal(dst.host(0, total), want)
+
+
 def test_batches_in_a_row_with_different_descriptors(capi, blit, oracle, arenas):
     """Eight batches back to back on one engine, each with its own descriptors,
     submitted without waiting in between: the two staging buffers are rewritten

@@ -72,16 +72,19 @@ struct mi355_blit {
   bool stage_in_device_memory = false;
   BatchDesc* descs_host[2] = {nullptr, nullptr};
   BatchImage stage_image;  // built in ordinary memory, then copied to a staging buffer
-  hipEvent_t upload_done[2] = {nullptr, nullptr};  // the kernel that reads descs_host[i] has finished
-  bool upload_busy[2] = {false, false};
+  // One event per batch, recorded behind its copy kernel, alternating like the
+  // staging buffers: it frees the batch's staging buffer for the host, and it
+  // is what a batch on another stream, or a reallocation, waits for.  (An
+  // event between the two kernels of a batch costs ~5 us of queue time.)
+  hipEvent_t batch_done[2] = {nullptr, nullptr};
+  bool batch_busy[2] = {false, false};
   unsigned next_host = 0;
+  hipStream_t last_batch_stream = nullptr;
   uint32_t* chunk_start_dev = nullptr;
   uint32_t* block_sum_dev = nullptr;
   ChunkRecord* records_dev = nullptr;  // one per chunk
   size_t records_capacity = 0;
   size_t batch_capacity = 0;
-  hipEvent_t staging_free = nullptr;  // previous batch has consumed the staging buffers
-  bool staging_busy = false;
 };
 
 namespace {
@@ -241,17 +244,17 @@ void free_batch_buffers(mi355_blit* h) {
 int ensure_batch_capacity(mi355_blit* h, size_t n, size_t n_records) {
   if (n <= h->batch_capacity && n_records <= h->records_capacity) return MI355_BLIT_SUCCESS;
   // the old buffers may still be read by a batch in flight
-  if (h->staging_busy) {
-    BLIT_HIP(hipEventSynchronize(h->staging_free));
-    h->staging_busy = false;
+  for (int i = 0; i < 2; ++i) {
+    if (h->batch_busy[i]) {
+      BLIT_HIP(hipEventSynchronize(h->batch_done[i]));
+      h->batch_busy[i] = false;
+    }
   }
   if (n > h->batch_capacity) {
     size_t cap = h->batch_capacity ? h->batch_capacity : 1024;
     while (cap < n) cap *= 2;
     free_batch_buffers(h);
     for (int i = 0; i < 2; ++i) {
-      // uploads from the old pinned buffers are over: staging_free was waited for above
-      h->upload_busy[i] = false;
       if (h->stage_in_device_memory)
         BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->descs_host[i]), batch_stage_bytes(cap)));
       else
@@ -322,9 +325,8 @@ int mi355_blit_create(int device_ordinal, mi355_blit_t** out) {
   if (e == hipSuccess && cus > 0) e = hipStreamCreateWithFlags(&h->stream, hipStreamNonBlocking);
   for (unsigned i = 0; e == hipSuccess && i < kLedgerSlots; ++i)
     e = hipEventCreateWithFlags(&h->ledger[i].done, hipEventDisableTiming);
-  if (e == hipSuccess) e = hipEventCreateWithFlags(&h->staging_free, hipEventDisableTiming);
   for (int i = 0; e == hipSuccess && i < 2; ++i)
-    e = hipEventCreateWithFlags(&h->upload_done[i], hipEventDisableTiming);
+    e = hipEventCreateWithFlags(&h->batch_done[i], hipEventDisableTiming);
   if (e != hipSuccess || cus <= 0) {
     mi355_blit_destroy(h);
     return e == hipSuccess ? MI355_BLIT_ERROR : status_of(e);
@@ -357,9 +359,8 @@ int mi355_blit_destroy(mi355_blit_t* h) {
       if (hipStreamSynchronize(h->stream) != hipSuccess) rc = MI355_BLIT_ERROR;
       (void)hipStreamDestroy(h->stream);
     }
-    if (h->staging_free) (void)hipEventDestroy(h->staging_free);
     for (int i = 0; i < 2; ++i)
-      if (h->upload_done[i]) (void)hipEventDestroy(h->upload_done[i]);
+      if (h->batch_done[i]) (void)hipEventDestroy(h->batch_done[i]);
     free_batch_buffers(h);
     if (h->records_dev) (void)hipFree(h->records_dev);
   }
@@ -463,8 +464,11 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
   if (rc != MI355_BLIT_SUCCESS) return rc;
 
   // The device-side buffers (records, prefix sums) are shared by consecutive
-  // batches: the next batch waits for the previous one on the stream.
-  if (h->staging_busy) BLIT_HIP(hipStreamWaitEvent(s, h->staging_free, 0));
+  // batches: the next batch waits for the previous one, which stream order
+  // does by itself unless the two are on different streams.
+  const unsigned b = h->next_host;
+  h->next_host ^= 1;
+  if (h->batch_busy[b ^ 1] && h->last_batch_stream != s) BLIT_HIP(hipStreamWaitEvent(s, h->batch_done[b ^ 1], 0));
 
   mi355_blit_plan_t p{};
   p.kernel = MI355_BLIT_KERNEL_COPY_BATCH;
@@ -488,12 +492,10 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
     // piece's first record index) is all the GPU needs to write the records
     // with one lane per piece.  The two staging buffers alternate, so staging
     // one batch overlaps the execution of the one before; a buffer is only
-    // waited for until the kernel that read it, two batches ago, has finished.
-    const unsigned b = h->next_host;
-    h->next_host ^= 1;
-    if (h->upload_busy[b]) {
-      BLIT_HIP(hipEventSynchronize(h->upload_done[b]));
-      h->upload_busy[b] = false;
+    // waited for until the batch that used it, two batches ago, has finished.
+    if (h->batch_busy[b]) {
+      BLIT_HIP(hipEventSynchronize(h->batch_done[b]));
+      h->batch_busy[b] = false;
     }
     const size_t image_bytes = batch_stage_bytes(shape.pieces);
     batch_stage(h->stage_image, h->descs_host[b]);
@@ -508,8 +510,6 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
     hipLaunchKernelGGL(mi355_batch_emit_records, dim3(static_cast<uint32_t>((shape.pieces + 255) / 256)), dim3(256),
                        0, s, er);
     BLIT_HIP(hipGetLastError());
-    BLIT_HIP(hipEventRecord(h->upload_done[b], s));
-    h->upload_busy[b] = true;
 
     p.wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size : 256;
     const uint64_t waves_per_wg = p.wg_size / 64;
@@ -552,8 +552,9 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
     else hipLaunchKernelGGL(mi355_batch_strided_l0_s0, dim3(p.grid), dim3(p.wg_size), 0, s, bs);
   }
   BLIT_HIP(hipGetLastError());
-  BLIT_HIP(hipEventRecord(h->staging_free, s));
-  h->staging_busy = true;
+  BLIT_HIP(hipEventRecord(h->batch_done[b], s));
+  h->batch_busy[b] = true;
+  h->last_batch_stream = s;
   h->last_plan = p;
   return ledger_record(h, s, shape.total_bytes);
 }

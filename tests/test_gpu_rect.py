@@ -139,11 +139,11 @@ def test_rect_random_narrow_rows(capi, fresh_tuning, oracle, rand, seed):
 
 
 def test_rect_plan_shapes(capi, blit, oracle, rand):
-    """What the launch record says: a rect kernel with one wave per 2 KiB of
-    row for aligned rows, a linear copy when the region is one run."""
+    """What the launch record says: a rect kernel with one wave per 1 KiB of
+    row for rows of whole cache lines, a linear copy when the region is one run."""
     p = run_rect_case(capi, blit, oracle, rand, (1, 64, 16384), (1, 64, 16384), (8192, 64, 1), (0, 0, 0), (8192, 0, 0))
-    assert p.kernel == capi.KERNEL_COPY_RECT and p.body_vecs == 64 * 4 and p.unroll == 2
-    assert p.grid * (p.wg_size // 64) == 64 * 4
+    assert p.kernel == capi.KERNEL_COPY_RECT and p.body_vecs == 64 * 8 and p.unroll == 1
+    assert p.grid * (p.wg_size // 64) == 64 * 8
     p = run_rect_case(capi, blit, oracle, rand, (1, 64, 8192), (1, 64, 8192), (8192, 64, 1), (0, 0, 0), (0, 0, 0))
     assert p.kernel == capi.KERNEL_COPY
 

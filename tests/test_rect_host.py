@@ -220,9 +220,13 @@ def test_plan_rect_merges_contiguous_rows(capi_host):
 
 def test_plan_rect_slots_follow_row_alignment(capi_host):
     base_d, base_s = 0x7f0000000000, 0x7f1000000000
-    # 4 KiB rows at 256-byte aligned destinations: two units of 2 KiB each
+    # 4 KiB rows whose every store is a whole cache line: four units of 1 KiB, workgroups of 256
     st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 64, 1))
-    assert st == SUCCESS and (p.slots, p.unroll, p.lanes_per_row) == (2, 2, 0)
+    assert st == SUCCESS and (p.slots, p.unroll, p.lanes_per_row, p.wg_size) == (4, 1, 0, 256)
+    assert p.grid * (p.wg_size // 64) == 64 * 4
+    # 16 bytes off the lines: two units of 2 KiB, workgroups of 128
+    st, p = capi_host.plan_rect((base_d, 8192, 0), (16, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 64, 1))
+    assert st == SUCCESS and (p.slots, p.unroll, p.lanes_per_row, p.wg_size) == (2, 2, 0, 128)
     assert p.grid * (p.wg_size // 64) == 64 * 2
     # the same rows up to 240 bytes further: the last unit absorbs the spill
     for x in (16, 100, 240):
@@ -232,7 +236,7 @@ def test_plan_rect_slots_follow_row_alignment(capi_host):
     st, p = capi_host.plan_rect((base_d, 4100, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 64, 1))
     assert st == SUCCESS and p.slots == 2
     # but 16 vectors more than two units need a third
-    st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096 + 256, 64, 1))
+    st, p = capi_host.plan_rect((base_d, 8192, 0), (16, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096 + 256, 64, 1))
     assert st == SUCCESS and p.slots == 3
     # rows of up to 64 destination slots are packed, as many to a wave as fit
     st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (1024, 64, 1))
@@ -250,6 +254,8 @@ def test_plan_rect_slots_follow_row_alignment(capi_host):
     # streaming policy from 4 MiB of payload
     assert p.nt_load == 0
     st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 1024, 1))
+    assert st == SUCCESS and p.nt_load == 1 and p.store_policy == capi_host.STORE_AGENT_WT   # whole lines
+    st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4100, 1024, 1))
     assert st == SUCCESS and p.nt_load == 1 and p.store_policy == capi_host.STORE_NT
 
 

@@ -116,6 +116,10 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
   out->store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
   if (t && t->store_policy >= 1 && t->store_policy <= 4) out->store_policy = t->store_policy - 1;
 
+  // every store of every row is a whole cache line
+  const bool whole_lines = reinterpret_cast<uintptr_t>(d0) % 128 == 0 && dp % 128 == 0 && width % 128 == 0 &&
+                           (layers == 1 || ds % 128 == 0);
+
   // 16-byte destination slots a row touches, at the worst alignment its rows
   // can have (they differ by multiples of g16 modulo 16)
   uint64_t g16 = rect_gcd(dp % 16, 16);
@@ -141,7 +145,22 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
     n.magic = (65536 + n.lanes_per_row - 1) / n.lanes_per_row;
     n.magic64 = n.lanes_per_row > 1 ? ~0ull / n.lanes_per_row + 1 : 0;  // unused for 1
     out->unroll = 1;
-    out->wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size : 256;
+    // Measured on MI355X with 2^20 rows.  When every store is a whole cache
+    // line, single-wave workgroups and written-through stores are best (1 KiB
+    // rows 312 us against 349 us, 512 B rows 167 against 177).  Waves that share
+    // cache lines with their neighbours want to be in one workgroup, hence on
+    // one CU (520 B rows at a 1 KiB pitch, 33 lanes a row: 241 us with workgroups
+    // of 256, 283 us with single waves, whose neighbours run on other XCDs), and
+    // non-temporal stores.
+    if (whole_lines && streaming && !(t && t->store_policy >= 1 && t->store_policy <= 4))
+      out->store_policy = MI355_BLIT_STORE_AGENT_WT;
+    // No two waves touch the same destination line when rows are whole lines,
+    // or when waves hold whole rows and neighbouring rows are a line apart.
+    const bool rows_apart = dp >= width + 127 && (layers == 1 || ds >= (rows - 1) * dp + width + 127);
+    const bool waves_apart = whole_lines || (64 % n.lanes_per_row == 0 && rows_apart);
+    out->wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size
+                   : waves_apart                                                           ? 64
+                                                                                            : 256;
     const uint64_t waves_per_wg = out->wg_size / 64;
     const uint64_t groups = (rows * layers * n.lanes_per_row + 63) / 64;
     uint64_t wgs = (groups + waves_per_wg - 1) / waves_per_wg;
@@ -160,8 +179,6 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
   // 333-341 us with the shape below.  Any other rows: two vectors per lane,
   // workgroups of 128, non-temporal stores (written-through stores lose 8-15 %
   // there: the rows' cut ends are partial lines).
-  const bool whole_lines = reinterpret_cast<uintptr_t>(d0) % 128 == 0 && dp % 128 == 0 && width % 128 == 0 &&
-                           (layers == 1 || ds % 128 == 0);
   uint32_t unroll = whole_lines ? 1 : 2;
   uint32_t default_wg = whole_lines ? 256 : 128;
   if (whole_lines && streaming && !(t && t->store_policy >= 1 && t->store_policy <= 4))

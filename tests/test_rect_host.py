@@ -251,6 +251,15 @@ def test_plan_rect_slots_follow_row_alignment(capi_host):
     assert st == SUCCESS and p.lanes_per_row == 5 and p.grid * (p.wg_size // 64) == 320   # rows at every alignment mod 4
     st, p = capi_host.plan_rect((base_d, 37, 37 * 9), (3, 0, 0), (base_s, 41, 41 * 9), (0, 0, 0), (1, 9, 5))
     assert st == SUCCESS and (p.lanes_per_row, p.rows, p.layers) == (1, 9, 5)
+    # packed rows: single-wave workgroups when no two waves can touch one destination line
+    st, p = capi_host.plan_rect((base_d, 2048, 0), (0, 0, 0), (base_s, 2048, 0), (0, 0, 0), (1024, 8192, 1))
+    assert st == SUCCESS and (p.lanes_per_row, p.wg_size, p.store_policy) == (64, 64, capi_host.STORE_AGENT_WT)
+    st, p = capi_host.plan_rect((base_d, 2048, 0), (9, 0, 0), (base_s, 2048, 0), (3, 0, 0), (1000, 8192, 1))
+    assert st == SUCCESS and (p.lanes_per_row, p.wg_size, p.store_policy) == (64, 64, capi_host.STORE_NT)
+    st, p = capi_host.plan_rect((base_d, 1024, 0), (0, 0, 0), (base_s, 1024, 0), (0, 0, 0), (520, 8192, 1))
+    assert st == SUCCESS and (p.lanes_per_row, p.wg_size, p.store_policy) == (33, 256, capi_host.STORE_NT)
+    st, p = capi_host.plan_rect((base_d, 260, 0), (0, 0, 0), (base_s, 260, 0), (0, 0, 0), (256, 32768, 1))
+    assert st == SUCCESS and p.wg_size == 256                       # neighbouring rows share lines
     # streaming policy from 4 MiB of payload
     assert p.nt_load == 0
     st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 1024, 1))

@@ -261,7 +261,8 @@ def test_plan_rect_slots_follow_row_alignment(capi_host):
     st, p = capi_host.plan_rect((base_d, 260, 0), (0, 0, 0), (base_s, 260, 0), (0, 0, 0), (256, 32768, 1))
     assert st == SUCCESS and p.wg_size == 256                       # neighbouring rows share lines
     # streaming policy from 4 MiB of payload
-    assert p.nt_load == 0
+    st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 64, 1))
+    assert st == SUCCESS and p.nt_load == 0 and p.store_policy == capi_host.STORE_CACHED
     st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 1024, 1))
     assert st == SUCCESS and p.nt_load == 1 and p.store_policy == capi_host.STORE_AGENT_WT   # whole lines
     st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4100, 1024, 1))

@@ -422,7 +422,7 @@ def reference_gpu_path(r):
 
 def cpu_baseline(ora, budget_s):
     """The reference's host path on this box's cores: memcpy of 256 MiB
-    (BASELINE config 1; what hsa_memory_copy does for host pointers), single
+    (what hsa_memory_copy does for host pointers, core/runtime/runtime.cpp:507-510), single
     thread and T threads, on a bounded number of repetitions."""
     import numpy as np
     n = 256 * MIB

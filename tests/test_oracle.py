@@ -60,7 +60,7 @@ def test_fnv1a64_known_answers(oracle):
 
 # ---- fill ------------------------------------------------------------------
 
-# rocrtst/samples/async_mem_copy/async_mem_copy.cc:62-65 and BASELINE's pattern
+# rocrtst/samples/async_mem_copy/async_mem_copy.cc:62-65 and the benchmark's pattern
 REFERENCE_FILL_VALUES = [0xabcdef12, 0xba5eba11, 0xfeed5a1e, 0xbaadf00d, 0xA5C30F1E]
 
 

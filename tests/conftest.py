@@ -98,7 +98,15 @@ def oracle_validate_rect(oracle, dst, dst_offset, src, src_offset, extent, direc
 
 @pytest.fixture(scope="session")
 def pkg():
-    return entry.load_package()
+    """The package, with its native parts built: a checkout that has not been
+    built yet (the libraries are not kept in the history) is built once here,
+    where hipcc is at hand.  Building is not a fallback: the tests still run the
+    HIP libraries and nothing else."""
+    p = entry.load_package()
+    b = p.build
+    if not all(os.path.exists(f) for f in (b.BLIT_LIB, b.AQL_LIB, b.ROCR_LIB, b.ORACLE_LIB, b.ROCR_TEST)):
+        b.build_all()
+    return p
 
 
 @pytest.fixture(scope="session")

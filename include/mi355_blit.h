@@ -152,6 +152,20 @@ int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwo
 int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n,
                           int descs_on_device, void* stream);
 
+/* The batched path for device-resident descriptors whose sizes the host does
+ * not know but can bound (a previous kernel wrote them): the n copies together
+ * move at most max_total_bytes bytes.  No counterpart in the reference.  The
+ * bound sizes the grid and the record buffer (max_total_bytes / 4096 + 2 n
+ * records of 32 bytes), which lets the copy run one wave per 4 KiB chunk as
+ * with host-resident descriptors instead of on a fixed grid that walks the
+ * prefix sums; a loose bound costs idle waves, not correctness.  Descriptors
+ * that exceed the bound are the caller's error: the copies are then cut short
+ * at the bound (no access outside the described regions is made, and no error
+ * can be reported without a read-back).  max_total_bytes == 0 with n > 0, or
+ * a bound that needs 2^32 records or more -> INVALID_ARGUMENT. */
+int mi355_blit_copy_batch_bounded(mi355_blit_t* h, const mi355_blit_desc_t* device_descs, size_t n,
+                                  uint64_t max_total_bytes, void* stream);
+
 /* Pitched 3-D region copy as a shader: range->z layers of range->y rows of
  * range->x bytes, from src at src_offset to dst at dst_offset.  The reference
  * has this on its SDMA engines only: GpuAgent::DmaCopyRect answers

@@ -68,6 +68,14 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
 int mi355_aql_copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, size_t n,
                                 const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal);
 
+/* Device-resident descriptors that together move at most max_total_bytes
+ * bytes (see mi355_blit_copy_batch_bounded in mi355_blit.h: the bound sizes a
+ * per-chunk grid; copies beyond it are cut short).  Four packets.
+ * max_total_bytes == 0 with n > 0 -> INVALID_ARGUMENT. */
+int mi355_aql_copy_batch_bounded(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, size_t n,
+                                 uint64_t max_total_bytes, const uint64_t* dep_signals, uint32_t num_deps,
+                                 uint64_t completion_signal);
+
 /* Pitched 3-D region copy, asynchronous like mi355_aql_copy: the shader
  * counterpart of BlitSdmaBase::SubmitCopyRectCommand
  * (core/inc/amd_blit_sdma.h:68-73), which the reference reaches through

@@ -16,6 +16,8 @@ SIGNATURES = {
     "mi355_aql_fill32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
     "mi355_aql_copy_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
     "mi355_aql_copy_batch_device": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
+    "mi355_aql_copy_batch_bounded": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint64, _U64P, C.c_uint32,
+                                               C.c_uint64]),
     "mi355_aql_copy_rect": (C.c_int, [C.c_void_p, C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
                                       C.POINTER(Dim3), C.POINTER(Dim3), _U64P, C.c_uint32, C.c_uint64]),
     "mi355_aql_wait_idle": (C.c_int, [C.c_void_p]),
@@ -109,6 +111,12 @@ class AqlBlit:
         if on_device:
             return self.lib.mi355_aql_copy_batch_device(self.handle, addr, n, arr, nd, completion)
         return self.lib.mi355_aql_copy_batch(self.handle, addr, n, arr, nd, completion)
+
+    def copy_batch_bounded(self, device_descs, n, max_total_bytes, *, deps=None, completion=0):
+        """Device-resident descriptors that together move at most max_total_bytes."""
+        arr, nd = _deps(deps)
+        addr = device_descs if isinstance(device_descs, int) or device_descs is None else C.cast(device_descs, C.c_void_p)
+        return self.lib.mi355_aql_copy_batch_bounded(self.handle, addr, n, max_total_bytes, arr, nd, completion)
 
     def copy_rect(self, dst, dst_offset, src, src_offset, extent, *, deps=None, completion=0):
         """dst, src: (base, pitch, slice); offsets and extent: (x bytes, y rows, z layers)."""

@@ -84,6 +84,7 @@ SIGNATURES = {
     "mi355_blit_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "mi355_blit_fill32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t, C.c_void_p]),
     "mi355_blit_copy_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]),
+    "mi355_blit_copy_batch_bounded": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint64, C.c_void_p]),
     "mi355_blit_copy_rect": (C.c_int, [C.c_void_p, C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
                                        C.POINTER(Dim3), C.POINTER(Dim3), C.c_void_p]),
     "mi355_blit_plan_rect": (C.c_int, [C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
@@ -177,6 +178,11 @@ class Blit:
     def copy_batch(self, descs, n, on_device=False, stream=None):
         addr = descs if isinstance(descs, int) else C.cast(descs, C.c_void_p)
         return self.lib.mi355_blit_copy_batch(self.handle, addr, n, 1 if on_device else 0, stream)
+
+    def copy_batch_bounded(self, device_descs, n, max_total_bytes, stream=None):
+        """Device-resident descriptors that together move at most max_total_bytes."""
+        addr = device_descs if isinstance(device_descs, int) or device_descs is None else C.cast(device_descs, C.c_void_p)
+        return self.lib.mi355_blit_copy_batch_bounded(self.handle, addr, n, max_total_bytes, stream)
 
     def copy_rect(self, dst, dst_offset, src, src_offset, extent, stream=None):
         """dst, src: (base, pitch, slice); offsets and extent: (x bytes, y rows, z layers)."""

@@ -107,7 +107,7 @@ struct mi355_aql {
   std::vector<BatchKernel> batch_kernels{MI355_FOR_EACH_BATCH_RECORDS_KERNEL(MI355_BATCH_NAME)};
   std::vector<RectKernel> rect_kernels{MI355_FOR_EACH_RECT_KERNEL(MI355_RECT_NAME)};
   std::vector<RectKernel> rect_narrow_kernels{MI355_FOR_EACH_RECT_NARROW_KERNEL(MI355_RECT_NARROW_NAME)};
-  Kernel scan_local, scan_top, emit_records, finalize, strided_cached, strided_streaming;
+  Kernel scan_local, scan_top, emit_records, emit_records_device, finalize, strided_cached, strided_streaming;
 
   hsa_signal_t idle_signal{};  // completion signal of wait_idle's barrier packet
 
@@ -251,6 +251,7 @@ int load_code_object(mi355_aql* h) {
   if ((rc = lookup(h, "mi355_batch_scan_local", &h->scan_local)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_scan_top", &h->scan_top)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_emit_records", &h->emit_records)) != MI355_BLIT_SUCCESS) return rc;
+  if ((rc = lookup(h, "mi355_batch_emit_records_device", &h->emit_records_device)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_finalize", &h->finalize)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_strided_l0_s0", &h->strided_cached)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_strided_l1_s1", &h->strided_streaming)) != MI355_BLIT_SUCCESS) return rc;
@@ -766,7 +767,7 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   for (const auto& v : h->batch_kernels)
     if (v.split == split && v.nt_load == (streaming ? 1u : 0u) && v.store == p.store_policy) bk = &v.k;
   if (!bk) return MI355_BLIT_ERROR;
-  BatchCopyArgs bc{h->records_dev, total_chunks, static_cast<uint32_t>(waves_per_wg),
+  BatchCopyArgs bc{h->records_dev, total_chunks, nullptr, static_cast<uint32_t>(waves_per_wg),
                    static_cast<uint32_t>(wgs * waves_per_wg)};
   h->last_plan = p;
 
@@ -839,6 +840,72 @@ int mi355_aql_copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_
   write_dispatch(h, i++, h->finalize, &fa, sizeof(fa), static_cast<uint32_t>((n + 255) / 256), 256, 0, true);
   write_dispatch(h, i++, streaming ? h->strided_streaming : h->strided_cached, &bs, sizeof(bs), p.grid, p.wg_size,
                  completion_signal, true);
+  release_write_index(h, index, total);
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_aql_copy_batch_bounded(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, size_t n,
+                                 uint64_t max_total_bytes, const uint64_t* dep_signals, uint32_t num_deps,
+                                 uint64_t completion_signal) {
+  if (!h || (!device_descs && n) || (num_deps && !dep_signals)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (n > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (h->queue_error.load()) return MI355_BLIT_ERROR;
+  if (n == 0) return mi355_aql_copy(h, h, h, 0, dep_signals, num_deps, completion_signal);
+  const uint64_t capacity = max_total_bytes ? batch_bound_chunks(n, max_total_bytes) : 0;
+  if (capacity == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+
+  std::lock_guard<std::mutex> g(h->lock);
+  int rc = ensure_batch_capacity(h, n, capacity);
+  if (rc != MI355_BLIT_SUCCESS) return rc;
+  const mi355_blit_tuning_t* t = h->has_tuning ? &h->tuning : nullptr;
+  const BatchDesc* descs = reinterpret_cast<const BatchDesc*>(device_descs);
+  const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
+  ScanLocalArgs sl{descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
+  ScanTopArgs stp{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
+  EmitRecordsDeviceArgs er{descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n), h->records_dev,
+                           capacity};
+
+  mi355_blit_plan_t p{};
+  p.kernel = MI355_BLIT_KERNEL_COPY_BATCH;
+  p.body_vecs = capacity;
+  bool streaming = true;  // the lengths are only known on the device
+  if (t && t->nt_load) streaming = (t->nt_load == 2);
+  p.nt_load = streaming;
+  p.store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
+  if (t && t->store_policy >= 1 && t->store_policy <= 4) p.store_policy = t->store_policy - 1;
+  p.wg_size = 256;
+  const unsigned split = 4;
+  p.unroll = 4 / split;
+  const uint64_t waves_per_wg = p.wg_size / 64;
+  uint64_t wgs = (capacity * split + waves_per_wg - 1) / waves_per_wg;
+  if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
+  if (wgs * p.wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / p.wg_size;
+  p.grid = static_cast<uint32_t>(wgs);
+  const Kernel* bk = nullptr;
+  for (const auto& v : h->batch_kernels)
+    if (v.split == split && v.nt_load == (streaming ? 1u : 0u) && v.store == p.store_policy) bk = &v.k;
+  if (!bk) return MI355_BLIT_ERROR;
+  // the grid is sized for the bound; the kernel reads the number of records the device counted
+  BatchCopyArgs bc{h->records_dev, capacity, h->chunk_start_dev + n, static_cast<uint32_t>(waves_per_wg),
+                   static_cast<uint32_t>(wgs * waves_per_wg)};
+  h->last_plan = p;
+
+  const uint32_t nb = barrier_packets(num_deps);
+  const uint32_t total = nb + 4;
+  uint64_t index;
+  {
+    std::lock_guard<std::mutex> r(h->reservation_lock);
+    index = acquire_write_index(h, total);
+    record_blit_history(h, max_total_bytes, index + total - 1);
+  }
+  write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
+  uint64_t i = index + nb;
+  // every packet waits for the one before; the first also for whatever still uses the shared buffers
+  write_dispatch(h, i++, h->scan_local, &sl, sizeof(sl), n_blocks, 1024, 0, true);
+  write_dispatch(h, i++, h->scan_top, &stp, sizeof(stp), 1, 1024, 0, true);
+  write_dispatch(h, i++, h->emit_records_device, &er, sizeof(er), static_cast<uint32_t>((n + 255) / 256), 256, 0,
+                 true);
+  write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true);
   release_write_index(h, index, total);
   return MI355_BLIT_SUCCESS;
 }

@@ -92,9 +92,25 @@ struct EmitRecordsArgs {
   ChunkRecord* records;
 };
 
+// Device-resident descriptors with a bound on their total size: the prefix
+// sum was done on the device (chunk_start within each group of 1024 copies,
+// block_sum across groups); one lane per copy, records beyond `capacity` are
+// not written.
+struct EmitRecordsDeviceArgs {
+  const BatchDesc* descs;
+  const uint32_t* chunk_start;
+  const uint32_t* block_sum;
+  uint64_t n;
+  ChunkRecord* records;
+  uint64_t capacity;
+};
+
 struct BatchCopyArgs {
   const ChunkRecord* records;
-  uint64_t total_chunks;
+  uint64_t total_chunks;  // the number of records, or a bound on it when total is given
+  // When not null, the number of records as the device computed it; the grid
+  // was sized for total_chunks and waves beyond *total have nothing to do.
+  const uint32_t* total;
   uint32_t waves_per_wg;
   uint32_t n_waves;
 };

@@ -41,6 +41,15 @@ inline uint64_t batch_desc_chunks(uint64_t dst, uint64_t bytes) {
   return c ? c : 1;
 }
 
+// The most chunks n copies of at most max_total_bytes together can have: a
+// copy of b bytes has at most ceil((b / 16 + 15) / 256) <= b / 4096 + 2 of
+// them (15 = the vectors between the 256-byte line and the copy's first aligned
+// byte).  0 when the record indices would not fit their 32 bits.
+inline uint64_t batch_bound_chunks(uint64_t n, uint64_t max_total_bytes) {
+  const uint64_t c = max_total_bytes / (16 * kBatchChunkVecs) + 2 * n;
+  return c < 0xffffffffull ? c : 0;
+}
+
 // Calls f(dst, src, bytes) for every piece of one copy.
 template <typename F>
 inline void batch_for_each_piece(const mi355_blit_desc_t& d, F f) {

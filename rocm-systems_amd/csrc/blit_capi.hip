@@ -441,8 +441,25 @@ int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwo
   return ledger_record(h, s, num_dwords * 4);
 }
 
+namespace {
+int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int descs_on_device,
+               uint64_t max_total_bytes, void* stream);
+}
+
 int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n,
                           int descs_on_device, void* stream) {
+  return copy_batch(h, descs, n, descs_on_device, 0, stream);
+}
+
+int mi355_blit_copy_batch_bounded(mi355_blit_t* h, const mi355_blit_desc_t* device_descs, size_t n,
+                                  uint64_t max_total_bytes, void* stream) {
+  if (max_total_bytes == 0) return n ? MI355_BLIT_ERROR_INVALID_ARGUMENT : MI355_BLIT_SUCCESS;
+  return copy_batch(h, device_descs, n, 1, max_total_bytes, stream);
+}
+
+namespace {
+int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int descs_on_device,
+               uint64_t max_total_bytes, void* stream) {
   if (!h || (!descs && n)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   if (n == 0) return MI355_BLIT_SUCCESS;
   if (n > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
@@ -459,6 +476,12 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
   } else {
     shape.pieces = n;
     shape.total_bytes = n;  // lengths are only known on the device; keep the record non-zero
+    if (max_total_bytes) {
+      // what the caller vouches for bounds the number of records
+      shape.total_chunks = batch_bound_chunks(n, max_total_bytes);
+      if (shape.total_chunks == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+      shape.total_bytes = max_total_bytes;
+    }
   }
   int rc = ensure_batch_capacity(h, shape.pieces, shape.total_chunks);
   if (rc != MI355_BLIT_SUCCESS) return rc;
@@ -523,7 +546,37 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
     p.unroll = 4 / split;
     batch_kernel_t k = select_batch_kernel(split, streaming, p.store_policy);
     if (!k) return MI355_BLIT_ERROR;
-    BatchCopyArgs bc{h->records_dev, shape.total_chunks, static_cast<uint32_t>(waves_per_wg),
+    BatchCopyArgs bc{h->records_dev, shape.total_chunks, nullptr, static_cast<uint32_t>(waves_per_wg),
+                     static_cast<uint32_t>(wgs * waves_per_wg)};
+    hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, bc);
+  } else if (max_total_bytes) {
+    // Device-resident descriptors whose total size the caller bounds: the
+    // bound sizes the record buffer and a per-chunk grid, so the copy runs in
+    // the kernel of the host-resident path.  The prefix sum and the records
+    // are made on the device; the copy kernel reads the number of records
+    // there too and the waves the bound overestimated end at once.
+    const BatchDesc* dev_descs = reinterpret_cast<const BatchDesc*>(descs);
+    const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
+    ScanLocalArgs sl{dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
+    hipLaunchKernelGGL(mi355_batch_scan_local, dim3(n_blocks), dim3(1024), 0, s, sl);
+    ScanTopArgs st{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
+    hipLaunchKernelGGL(mi355_batch_scan_top, dim3(1), dim3(1024), 0, s, st);
+    EmitRecordsDeviceArgs er{dev_descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n),
+                             h->records_dev, shape.total_chunks};
+    hipLaunchKernelGGL(mi355_batch_emit_records_device, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0,
+                       s, er);
+    BLIT_HIP(hipGetLastError());
+    p.wg_size = 256;
+    const uint64_t waves_per_wg = p.wg_size / 64;
+    const uint64_t waves = shape.total_chunks * kBatchSplit;
+    uint64_t wgs = (waves + waves_per_wg - 1) / waves_per_wg;
+    if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
+    if (wgs * p.wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / p.wg_size;
+    p.grid = static_cast<uint32_t>(wgs);
+    p.unroll = 4 / kBatchSplit;
+    batch_kernel_t k = select_batch_kernel(kBatchSplit, streaming, p.store_policy);
+    if (!k) return MI355_BLIT_ERROR;
+    BatchCopyArgs bc{h->records_dev, shape.total_chunks, h->chunk_start_dev + n, static_cast<uint32_t>(waves_per_wg),
                      static_cast<uint32_t>(wgs * waves_per_wg)};
     hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, bc);
   } else {
@@ -558,6 +611,7 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
   h->last_plan = p;
   return ledger_record(h, s, shape.total_bytes);
 }
+}  // namespace
 
 int mi355_blit_copy_rect(mi355_blit_t* h, const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
                          const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,

@@ -415,6 +415,46 @@ __device__ __forceinline__ ChunkRecord make_record(const BatchDesc& d, uint32_t 
 // records, this takes 11.  The descriptors and the record indices were written
 // by the host, into host memory or across the bus into device memory, behind
 // the GPU's caches: they are read at system scope.
+// Writes the records of one wave's 64 copies: lane l holds copy (dst, src,
+// bytes) with `chunks` records, the wave's records start at out[0] and at most
+// `room` of them are written.
+__device__ __forceinline__ void emit_wave_records(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t chunks,
+                                                  ChunkRecord* out, uint64_t room, unsigned lane) {
+  // exclusive running sum of the chunk counts over the wave's lanes
+  uint32_t incl = chunks;
+#pragma unroll
+  for (unsigned off = 1; off < kWave; off <<= 1) {
+    const uint32_t x = __shfl_up(incl, off, kWave);
+    if (lane >= off) incl += x;
+  }
+  const uint32_t excl = incl - chunks;
+  const uint32_t total = __shfl(incl, kWave - 1, kWave);
+  const uint32_t dst_lo = static_cast<uint32_t>(dst), dst_hi = static_cast<uint32_t>(dst >> 32);
+  const uint32_t src_lo = static_cast<uint32_t>(src), src_hi = static_cast<uint32_t>(src >> 32);
+  const uint32_t len_lo = static_cast<uint32_t>(bytes), len_hi = static_cast<uint32_t>(bytes >> 32);
+  // every lane runs the same number of rounds: the shuffles need all of them
+  for (uint32_t base = 0; base < total; base += kWave) {
+    const uint32_t j = base + lane;
+    // The last lane whose running sum is <= j owns record j: lanes without
+    // chunks share their sum with the next lane and lose to it, and those at
+    // the wave's end have a sum of `total` and never win.
+    unsigned owner = 0;
+#pragma unroll
+    for (unsigned step = kWave / 2; step >= 1; step >>= 1) {
+      const uint32_t e = __shfl(excl, owner + step, kWave);
+      if (e <= j) owner += step;
+    }
+    BatchDesc d;
+    d.dst = reinterpret_cast<uint8_t*>(static_cast<uint64_t>(__shfl(dst_hi, owner, kWave)) << 32 |
+                                       __shfl(dst_lo, owner, kWave));
+    d.src = reinterpret_cast<const uint8_t*>(static_cast<uint64_t>(__shfl(src_hi, owner, kWave)) << 32 |
+                                             __shfl(src_lo, owner, kWave));
+    d.bytes = static_cast<uint64_t>(__shfl(len_hi, owner, kWave)) << 32 | __shfl(len_lo, owner, kWave);
+    const uint32_t k = j - __shfl(excl, owner, kWave);
+    if (j < total && j < room) out[j] = make_record(d, k);
+  }
+}
+
 __device__ __forceinline__ void emit_records_body(const EmitRecordsArgs& a) {
   const unsigned lane = threadIdx.x & (kWave - 1);
   const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
@@ -433,40 +473,30 @@ __device__ __forceinline__ void emit_records_body(const EmitRecordsArgs& a) {
   mine.src = reinterpret_cast<const uint8_t*>(src);
   mine.bytes = bytes;
   const uint32_t chunks = valid ? desc_chunks(mine) : 0;
-  // exclusive running sum of the chunk counts over the wave's lanes
-  uint32_t incl = chunks;
-#pragma unroll
-  for (unsigned off = 1; off < kWave; off <<= 1) {
-    const uint32_t x = __shfl_up(incl, off, kWave);
-    if (lane >= off) incl += x;
-  }
-  const uint32_t excl = incl - chunks;
-  const uint32_t total = __shfl(incl, kWave - 1, kWave);
   // the wave's records are consecutive: lane 0's first record starts them
-  ChunkRecord* out = a.records + __shfl(first, 0, kWave);
-  const uint32_t dst_lo = static_cast<uint32_t>(dst), dst_hi = static_cast<uint32_t>(dst >> 32);
-  const uint32_t src_lo = static_cast<uint32_t>(src), src_hi = static_cast<uint32_t>(src >> 32);
-  const uint32_t len_lo = static_cast<uint32_t>(bytes), len_hi = static_cast<uint32_t>(bytes >> 32);
-  // every lane runs the same number of rounds: the shuffles need all of them
-  for (uint32_t base = 0; base < total; base += kWave) {
-    const uint32_t j = base + lane;
-    // the last lane whose running sum is <= j owns record j (lanes without
-    // chunks, the invalid ones at the end, have a sum of `total` and never win)
-    unsigned owner = 0;
-#pragma unroll
-    for (unsigned step = kWave / 2; step >= 1; step >>= 1) {
-      const uint32_t e = __shfl(excl, owner + step, kWave);
-      if (e <= j) owner += step;
-    }
-    BatchDesc d;
-    d.dst = reinterpret_cast<uint8_t*>(static_cast<uint64_t>(__shfl(dst_hi, owner, kWave)) << 32 |
-                                       __shfl(dst_lo, owner, kWave));
-    d.src = reinterpret_cast<const uint8_t*>(static_cast<uint64_t>(__shfl(src_hi, owner, kWave)) << 32 |
-                                             __shfl(src_lo, owner, kWave));
-    d.bytes = static_cast<uint64_t>(__shfl(len_hi, owner, kWave)) << 32 | __shfl(len_lo, owner, kWave);
-    const uint32_t k = j - __shfl(excl, owner, kWave);
-    if (j < total) out[j] = make_record(d, k);
+  emit_wave_records(dst, src, bytes, chunks, a.records + __shfl(first, 0, kWave), ~0ull, lane);
+}
+
+// The same for device-resident descriptors, behind the two prefix-sum kernels:
+// a copy's first record is its group's sum plus its own running sum within the
+// group.  Copies may be of any length here (nothing has cut them), so a wave
+// may have many rounds to go through.
+__device__ __forceinline__ void emit_records_device_body(const EmitRecordsDeviceArgs& a) {
+  const unsigned lane = threadIdx.x & (kWave - 1);
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+  const bool valid = i < a.n;
+  BatchDesc mine{nullptr, nullptr, 0};
+  uint64_t first = 0;
+  if (valid) {
+    mine = a.descs[i];
+    first = static_cast<uint64_t>(a.block_sum[i / 1024]) + a.chunk_start[i];
   }
+  const uint32_t chunks = valid ? desc_chunks(mine) : 0;
+  const uint64_t wave_first = static_cast<uint64_t>(__shfl(static_cast<uint32_t>(first >> 32), 0, kWave)) << 32 |
+                              __shfl(static_cast<uint32_t>(first), 0, kWave);
+  const uint64_t room = wave_first < a.capacity ? a.capacity - wave_first : 0;
+  emit_wave_records(reinterpret_cast<uint64_t>(mine.dst), reinterpret_cast<uint64_t>(mine.src), mine.bytes, chunks,
+                    a.records + wave_first, room, lane);
 }
 
 // Loads of one wave's share of a chunk: virtual vector indices [v0, v0 + 64 U)
@@ -543,7 +573,12 @@ template <int SPLIT, bool NTL, int NTS>
 __device__ __forceinline__ void batch_copy_records_body(const BatchCopyArgs& a) {
   constexpr int U = kChunkVecs / kWave / SPLIT;
   const ChunkRecord* __restrict__ records = a.records;
-  const uint64_t total_chunks = a.total_chunks;
+  uint64_t total_chunks = a.total_chunks;
+  if (a.total) {
+    // sized for a bound: the device knows how many records there are
+    const uint64_t counted = *a.total;
+    if (counted < total_chunks) total_chunks = counted;
+  }
   const unsigned lane = threadIdx.x & (kWave - 1);
   const uint64_t wave = global_wave(a.waves_per_wg);
   const uint64_t n_waves = a.n_waves;
@@ -854,6 +889,9 @@ extern "C" __global__ void __launch_bounds__(256) mi355_batch_finalize(mi355::Fi
 }
 extern "C" __global__ void __launch_bounds__(256) mi355_batch_emit_records(mi355::EmitRecordsArgs a) {
   mi355::emit_records_body(a);
+}
+extern "C" __global__ void __launch_bounds__(256) mi355_batch_emit_records_device(mi355::EmitRecordsDeviceArgs a) {
+  mi355::emit_records_device_body(a);
 }
 extern "C" __global__ void __launch_bounds__(64) mi355_signal_complete(mi355::SignalArgs a) {
   mi355::signal_complete_body(a);

@@ -127,9 +127,12 @@ class BlitKernelGfx950 : public core::Blit {
 
   /// Batched small copies: n independent copies in one submission, out_signal
   /// decremented once when all are done.  No counterpart in core::Blit.
+  /// For device-resident descriptors, max_total_bytes != 0 vouches that the
+  /// copies together move no more than that, which sizes a per-chunk grid
+  /// (mi355_blit_copy_batch_bounded); 0 = no bound known.
   hsa_status_t SubmitBatchCopyCommand(const void* descs, size_t n, bool descs_on_device,
                                       std::vector<core::Signal*>& dep_signals,
-                                      core::Signal& out_signal);
+                                      core::Signal& out_signal, uint64_t max_total_bytes = 0);
 
   hsa_status_t EnableProfiling(bool enable) override;
 
@@ -149,6 +152,7 @@ class BlitKernelGfx950 : public core::Blit {
     const void* src;
     size_t size;     // bytes, dwords (Fill) or descriptors (Batch)
     uint32_t value;  // Fill pattern / Batch: descriptors are device-resident
+    uint64_t bound = 0;  // Batch, device-resident: most bytes the copies move together, 0 = unknown
     std::vector<hsa_signal_t> deps;
     hsa_signal_t out;
   };
@@ -200,9 +204,10 @@ class BlitKernelGfx950Aql : public core::Blit {
                                        std::vector<core::Signal*>& gang_signals) override;
   hsa_status_t SubmitLinearFillCommand(void* ptr, uint32_t value, size_t count) override;
   /// Batched small copies, descriptors in host or device memory; no counterpart in core::Blit.
+  /// max_total_bytes != 0: a bound on what device-resident descriptors move (0 = none known).
   hsa_status_t SubmitBatchCopyCommand(const void* descs, size_t n, bool descs_on_device,
                                       std::vector<core::Signal*>& dep_signals,
-                                      core::Signal& out_signal);
+                                      core::Signal& out_signal, uint64_t max_total_bytes = 0);
   /// Pitched 3-D region copy with the signature of BlitSdmaBase::SubmitCopyRectCommand
   /// (core/inc/amd_blit_sdma.h:68-73), so that GpuAgent::DmaCopyRect
   /// (core/runtime/amd_gpu_agent.cpp:1255-1283) can call a shader blit where it

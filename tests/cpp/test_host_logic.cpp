@@ -295,6 +295,21 @@ void one_batch_stage() {
   bad.bytes = 8;
   bad.dst = nullptr;
   CHECK(batch_build(&bad, 1, &image, &shape) == MI355_BLIT_ERROR_INVALID_ARGUMENT, "NULL destination accepted");
+
+  // The bound on the records of uncut copies (device-resident descriptors, of
+  // which the host only knows a bound on the total size) must cover their
+  // actual chunk counts, also when the bound on the bytes is exact.
+  uint64_t uncut_chunks = 0, uncut_bytes = 0;
+  for (const auto& d : descs) {
+    uncut_chunks += batch_desc_chunks(reinterpret_cast<uint64_t>(d.dst), d.bytes);
+    uncut_bytes += d.bytes;
+  }
+  if (uncut_bytes) {
+    const uint64_t bound = batch_bound_chunks(n, uncut_bytes);
+    CHECK(bound >= uncut_chunks, "bound of %" PRIu64 " records for %" PRIu64, bound, uncut_chunks);
+    CHECK(bound <= uncut_chunks + 2 * n + 1, "bound of %" PRIu64 " records is loose for %" PRIu64, bound, uncut_chunks);
+  }
+  CHECK(batch_bound_chunks(1, 1ull << 62) == 0, "a bound beyond 32-bit record indices accepted");
 }
 
 }  // namespace

@@ -29,7 +29,7 @@ using rocr::core::Blit;
 using rocr::core::Signal;
 
 // SubmitBatchCopyCommand is not part of core::Blit; each engine supplies it.
-typedef std::function<hsa_status_t(const void*, size_t, std::vector<Signal*>&, Signal&)> BatchFn;
+typedef std::function<hsa_status_t(const void*, size_t, bool, uint64_t, std::vector<Signal*>&, Signal&)> BatchFn;
 
 namespace {
 
@@ -307,10 +307,29 @@ void test_batch(Blit& blit, const BatchFn& submit_batch) {
   hsa_signal_t s = make_signal(1);
   Signal sig(s);
   std::vector<Signal*> none;
-  REQUIRE(submit_batch(descs.data(), ncopy, none, sig) == HSA_STATUS_SUCCESS, "submit");
+  REQUIRE(submit_batch(descs.data(), ncopy, false, 0, none, sig) == HSA_STATUS_SUCCESS, "submit");
   REQUIRE(wait_zero(s, HSA_WAIT_STATE_BLOCKED), "batch never completed");
   REQUIRE(dst.download(got), "download");
   REQUIRE(got == want, "bytes differ");
+  std::printf("PASS %s%s\n", name, g_suffix.c_str());
+
+  // the same descriptors, device-resident: without a bound on their sizes and with one
+  name = "batched_copies_device_resident";
+  std::vector<uint8_t> image(ncopy * sizeof(mi355_blit_desc_t));
+  std::memcpy(image.data(), descs.data(), image.size());
+  DeviceBuf descs_dev(image.size());
+  REQUIRE(descs_dev.p, "hipMalloc");
+  REQUIRE(descs_dev.upload(image), "upload");
+  uint64_t sum = 0;
+  for (size_t i = 0; i < ncopy; ++i) sum += len[i];
+  for (uint64_t bound : {uint64_t(0), sum, 3 * sum}) {
+    REQUIRE(dst.upload(std::vector<uint8_t>(total, kGuardByte)), "upload");
+    hsa_signal_store_relaxed(s, 1);
+    REQUIRE(submit_batch(descs_dev.p, ncopy, true, bound, none, sig) == HSA_STATUS_SUCCESS, "submit");
+    REQUIRE(wait_zero(s, HSA_WAIT_STATE_BLOCKED), "batch never completed");
+    REQUIRE(dst.download(got), "download");
+    REQUIRE(got == want, "bytes differ");
+  }
   hsa_signal_destroy(s);
   std::printf("PASS %s%s\n", name, g_suffix.c_str());
 }
@@ -489,16 +508,16 @@ int main(int argc, char** argv) {
       g_suffix = "_hip";
       auto* b = new BlitKernelGfx950(nullptr);
       init = b->Initialize(agent);
-      batch = [b](const void* d, size_t n, std::vector<Signal*>& deps, Signal& out) {
-        return b->SubmitBatchCopyCommand(d, n, false, deps, out);
+      batch = [b](const void* d, size_t n, bool on_device, uint64_t bound, std::vector<Signal*>& deps, Signal& out) {
+        return b->SubmitBatchCopyCommand(d, n, on_device, deps, out, bound);
       };
       blit = b;
     } else {
       g_suffix = "_aql";
       auto* b = new BlitKernelGfx950Aql(nullptr);
       init = b->Initialize(agent);
-      batch = [b](const void* d, size_t n, std::vector<Signal*>& deps, Signal& out) {
-        return b->SubmitBatchCopyCommand(d, n, false, deps, out);
+      batch = [b](const void* d, size_t n, bool on_device, uint64_t bound, std::vector<Signal*>& deps, Signal& out) {
+        return b->SubmitBatchCopyCommand(d, n, on_device, deps, out, bound);
       };
       blit = b;
     }

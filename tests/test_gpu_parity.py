@@ -510,6 +510,102 @@ def test_batch_device_resident_descriptors(capi, blit, oracle, arenas, torch_cud
     assert np.array_equal(dst.host(0, total), _expect_batch(oracle, src_host, total, lens, offs, so, do))
 
 
+def _to_device(torch, descs):
+    raw = np.frombuffer(bytes(descs), dtype=np.uint8).copy()
+    return torch.from_numpy(raw).to("cuda:0")
+
+
+@pytest.mark.parametrize("n,slack", [(1, 0), (65, 0), (777, 0), (777, 64 * MIB), (3000, 1)])
+def test_batch_bounded_device_resident_descriptors(capi, blit, oracle, arenas, torch_cuda, n, slack):
+    """Device-resident descriptors with a bound on their total size, exact and
+    loose: the per-chunk kernel behind a device-side prefix sum."""
+    torch = torch_cuda
+    src, src_host, dst = arenas
+    rng = np.random.default_rng(5000 + n)
+    descs, lens, offs, so, do, total = _make_batch(capi, rng, src, dst, n, max_len=64 << 10)
+    descs_dev = _to_device(torch, descs)
+    dst.fill(0, total, GUARD_BYTE)
+    torch.cuda.synchronize()
+    check_ok(capi, blit.copy_batch_bounded(descs_dev.data_ptr(), n, int(lens.sum()) + slack), "copy_batch_bounded")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert np.array_equal(dst.host(0, total), _expect_batch(oracle, src_host, total, lens, offs, so, do))
+    assert blit.last_plan().kernel == capi.KERNEL_COPY_BATCH
+
+
+def test_batch_bounded_edge_lengths_and_long_copies(capi, blit, oracle, arenas, torch_cuda):
+    """Zero-length entries (whole waves of them too), lengths around the 16-byte
+    vector and the 4 KiB chunk, and copies of several MiB, which nothing cuts
+    into pieces on this path."""
+    torch = torch_cuda
+    src, src_host, dst = arenas
+    lens = ([0] * 70 + list(range(1, 49)) + [0, 4095, 4096, 4097, 4096 + 15, 8192, 8193, 12288 + 31, 0]
+            + [5 * MIB + 3, 0, 77, MIB + 1, 3 * MIB - 17] + [0] * 130 + [9, 2 * MIB])
+    n = len(lens)
+    rng = np.random.default_rng(4711)
+    so = rng.integers(0, 16, n)
+    do = rng.integers(0, 256, n)
+    lens = np.array(lens, dtype=np.int64)
+    stride = ((lens + 255) // 256) * 256 + 512
+    offs = np.concatenate([[0], np.cumsum(stride)[:-1]]) + 256
+    total = int(offs[-1] + stride[-1] + 256)
+    assert total <= dst.nbytes
+    descs = (capi.Desc * n)()
+    for i in range(n):
+        descs[i].dst = dst.base + int(offs[i] + do[i])
+        descs[i].src = src.base + int(offs[i] + so[i])
+        descs[i].bytes = int(lens[i])
+    descs_dev = _to_device(torch, descs)
+    dst.fill(0, total, GUARD_BYTE)
+    torch.cuda.synchronize()
+    check_ok(capi, blit.copy_batch_bounded(descs_dev.data_ptr(), n, int(lens.sum())), "copy_batch_bounded")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert np.array_equal(dst.host(0, total), _expect_batch(oracle, src_host, total, lens, offs, so, do))
+
+
+def test_batch_bounded_all_empty_and_arguments(capi, blit, arenas, torch_cuda):
+    torch = torch_cuda
+    src, _, dst = arenas
+    n = 100
+    descs = (capi.Desc * n)()
+    for i in range(n):
+        descs[i].dst = dst.base + 512 * i
+        descs[i].src = src.base + 512 * i
+        descs[i].bytes = 0
+    descs_dev = _to_device(torch, descs)
+    dst.fill(0, 512 * n, GUARD_BYTE)
+    torch.cuda.synchronize()
+    check_ok(capi, blit.copy_batch_bounded(descs_dev.data_ptr(), n, 1), "copy_batch_bounded")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert (dst.host(0, 512 * n) == GUARD_BYTE).all()
+    inv = capi.ERROR_INVALID_ARGUMENT
+    assert blit.copy_batch_bounded(descs_dev.data_ptr(), n, 0) == inv
+    assert blit.copy_batch_bounded(None, n, 4096) == inv
+    assert blit.copy_batch_bounded(descs_dev.data_ptr(), n, 1 << 62) == inv   # more records than 32 bits index
+    assert blit.copy_batch_bounded(None, 0, 0) == capi.SUCCESS
+    check_ok(capi, blit.synchronize(), "synchronize")
+
+
+def test_batch_bounded_too_small_a_bound_stays_inside_the_regions(capi, blit, oracle, arenas, torch_cuda):
+    """A bound the descriptors exceed is the caller's error; the engine then
+    leaves the last chunks uncopied, and writes nothing outside the regions:
+    every byte is either the guard or what the full batch would have put there."""
+    torch = torch_cuda
+    src, src_host, dst = arenas
+    n = 64
+    rng = np.random.default_rng(808)
+    descs, lens, offs, so, do, total = _make_batch(capi, rng, src, dst, n, min_len=32 << 10, max_len=64 << 10)
+    descs_dev = _to_device(torch, descs)
+    dst.fill(0, total, GUARD_BYTE)
+    torch.cuda.synchronize()
+    check_ok(capi, blit.copy_batch_bounded(descs_dev.data_ptr(), n, 4096), "copy_batch_bounded")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    got = dst.host(0, total)
+    want = _expect_batch(oracle, src_host, total, lens, offs, so, do)
+    assert ((got == want) | (got == GUARD_BYTE)).all()
+    first = slice(int(offs[0] + do[0]), int(offs[0] + do[0]) + 4096)
+    assert np.array_equal(got[first], want[first]), "the chunks within the bound are copied"
+
+
 def test_batch_65536_copies(capi, blit, oracle, rand, torch_cuda):
     """The benchmark's batch: 65,536 copies, 64 B .. 256 KiB log-uniform, offsets
     0..15 on both sides, carved sequentially out of one arena; all bytes and

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define MI355_BLIT_ABI_VERSION 1
+#define MI355_BLIT_ABI_VERSION 2
 
 /* Same numeric values as HSA_STATUS_* (inc/hsa.h). */
 enum {
@@ -70,6 +70,13 @@ typedef struct {
   uint64_t head_bytes;
   uint64_t body_vecs;
   uint64_t tail_bytes;
+  uint32_t xcd_run;     /* 0: workgroups take tiles in launch order.  N > 1: the
+                           hardware deals consecutive workgroups to the 8 XCDs
+                           (each with its own L2) in turn; the launch is
+                           permuted so that every XCD works on runs of N
+                           neighbouring workgroups' tiles, and a cache line two
+                           neighbouring tiles share is fetched into one L2 */
+  uint32_t reserved;
 } mi355_blit_plan_t;
 
 /* Cache policy of the body's 16-byte stores. */
@@ -82,14 +89,16 @@ enum {
 
 /* Overrides for the sizing heuristics; 0 in a field keeps the heuristic.
  * nt_load: 0 = heuristic, 1 = force off, 2 = force on.
- * store_policy: 0 = heuristic, otherwise MI355_BLIT_STORE_* + 1. */
+ * store_policy: 0 = heuristic, otherwise MI355_BLIT_STORE_* + 1.
+ * xcd_run: 0 = heuristic, 1 = launch order, N > 1 = runs of N workgroups per XCD. */
 typedef struct {
   uint32_t wg_size;
   uint32_t unroll;
   uint32_t max_grid;   /* cap on workgroups; beyond it waves stride over tiles */
   uint32_t nt_load;
   uint32_t store_policy;
-  uint32_t reserved[3];
+  uint32_t xcd_run;
+  uint32_t reserved[2];
 } mi355_blit_tuning_t;
 
 /* One element of a batched submission.  No counterpart in the reference. */
@@ -207,7 +216,7 @@ typedef struct {
   uint32_t slots;
   uint32_t unroll;
   uint32_t lanes_per_row;
-  uint32_t reserved;
+  uint32_t xcd_run; /* as in mi355_blit_plan_t */
   uint32_t wg_size, grid, nt_load, store_policy;
   uint64_t total_bytes;
 } mi355_blit_rect_plan_t;

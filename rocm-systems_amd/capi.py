@@ -31,6 +31,7 @@ class Plan(C.Structure):
         ("unroll", C.c_uint32), ("nt_load", C.c_uint32), ("store_policy", C.c_uint32),
         ("byte_shift", C.c_uint32), ("lead_vecs", C.c_uint32),
         ("head_bytes", C.c_uint64), ("body_vecs", C.c_uint64), ("tail_bytes", C.c_uint64),
+        ("xcd_run", C.c_uint32), ("reserved", C.c_uint32),
     ]
 
     def as_dict(self):
@@ -40,7 +41,8 @@ class Plan(C.Structure):
 class Tuning(C.Structure):
     _fields_ = [
         ("wg_size", C.c_uint32), ("unroll", C.c_uint32), ("max_grid", C.c_uint32),
-        ("nt_load", C.c_uint32), ("store_policy", C.c_uint32), ("reserved", C.c_uint32 * 3),
+        ("nt_load", C.c_uint32), ("store_policy", C.c_uint32), ("xcd_run", C.c_uint32),
+        ("reserved", C.c_uint32 * 2),
     ]
 
 
@@ -62,7 +64,7 @@ class RectPlan(C.Structure):
         ("width", C.c_uint64), ("dst_pitch", C.c_uint64), ("dst_slice", C.c_uint64),
         ("src_pitch", C.c_uint64), ("src_slice", C.c_uint64), ("rows", C.c_uint32), ("layers", C.c_uint32),
         ("slots", C.c_uint32), ("unroll", C.c_uint32), ("lanes_per_row", C.c_uint32),
-        ("reserved", C.c_uint32), ("wg_size", C.c_uint32), ("grid", C.c_uint32),
+        ("xcd_run", C.c_uint32), ("wg_size", C.c_uint32), ("grid", C.c_uint32),
         ("nt_load", C.c_uint32), ("store_policy", C.c_uint32), ("total_bytes", C.c_uint64),
     ]
 

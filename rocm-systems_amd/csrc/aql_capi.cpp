@@ -647,6 +647,8 @@ int mi355_aql_copy(mi355_aql_t* h, void* dst, const void* src, size_t bytes, con
   a.head = static_cast<uint32_t>(p.head_bytes);
   a.lead = p.lead_vecs;
   tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
+  a.xcd_run = p.xcd_run;
+  a.xcd_full = xcd_full(p.grid, p.xcd_run);
   const uint32_t total = nb + 1;
   uint64_t index;
   {
@@ -691,6 +693,8 @@ int mi355_aql_fill32(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dword
   a.lead = p.lead_vecs;
   a.value = value;
   tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
+  a.xcd_run = p.xcd_run;
+  a.xcd_full = xcd_full(p.grid, p.xcd_run);
   const uint32_t nb = barrier_packets(num_deps);
   const uint32_t total = nb + 1;
   uint64_t index;
@@ -763,12 +767,14 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
   if (wgs * p.wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / p.wg_size;
   p.grid = static_cast<uint32_t>(wgs);
+  const uint32_t batch_run = batch_xcd_run(total_bytes, split, static_cast<uint32_t>(waves_per_wg), t);
+  p.xcd_run = batch_run;
   const Kernel* bk = nullptr;
   for (const auto& v : h->batch_kernels)
     if (v.split == split && v.nt_load == (streaming ? 1u : 0u) && v.store == p.store_policy) bk = &v.k;
   if (!bk) return MI355_BLIT_ERROR;
   BatchCopyArgs bc{h->records_dev, total_chunks, nullptr, static_cast<uint32_t>(waves_per_wg),
-                   static_cast<uint32_t>(wgs * waves_per_wg)};
+                   static_cast<uint32_t>(wgs * waves_per_wg), batch_run, xcd_full(p.grid, batch_run)};
   h->last_plan = p;
 
   const uint32_t nb = barrier_packets(num_deps);
@@ -881,13 +887,15 @@ int mi355_aql_copy_batch_bounded(mi355_aql_t* h, const mi355_blit_desc_t* device
   if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
   if (wgs * p.wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / p.wg_size;
   p.grid = static_cast<uint32_t>(wgs);
+  const uint32_t batch_run = batch_xcd_run(max_total_bytes, split, static_cast<uint32_t>(waves_per_wg), t);
+  p.xcd_run = batch_run;
   const Kernel* bk = nullptr;
   for (const auto& v : h->batch_kernels)
     if (v.split == split && v.nt_load == (streaming ? 1u : 0u) && v.store == p.store_policy) bk = &v.k;
   if (!bk) return MI355_BLIT_ERROR;
   // the grid is sized for the bound; the kernel reads the number of records the device counted
   BatchCopyArgs bc{h->records_dev, capacity, h->chunk_start_dev + n, static_cast<uint32_t>(waves_per_wg),
-                   static_cast<uint32_t>(wgs * waves_per_wg)};
+                   static_cast<uint32_t>(wgs * waves_per_wg), batch_run, xcd_full(p.grid, batch_run)};
   h->last_plan = p;
 
   const uint32_t nb = barrier_packets(num_deps);

@@ -3,15 +3,31 @@
 // Each kernel takes exactly one of these structs by value: its bytes are the
 // kernel's kernarg segment.  They take the place of BlitKernel::KernelArgs
 // (projects/rocr-runtime/runtime/hsa-runtime/core/inc/amd_blit_kernel.h:122-154).
-// Plain C++ without any HIP construct.
+// Plain C++; the one function here is also compiled for the device.
 #ifndef MI355_BLIT_ARGS_H_
 #define MI355_BLIT_ARGS_H_
 
 #include <stdint.h>
 
+#ifdef __HIPCC__
+#define MI355_HOST_DEVICE __host__ __device__
+#else
+#define MI355_HOST_DEVICE
+#endif
+
 namespace mi355 {
 
 constexpr unsigned kWave = 64;
+
+// The workgroup whose work workgroup b does when a launch deals runs of `run`
+// neighbouring workgroups to each of the 8 XCDs: the hardware places workgroup
+// b on XCD b % 8, so XCD x takes workgroups [x * run, (x + 1) * run) of every
+// round of 8 * run.  A permutation of [0, m) for every multiple m of 8 * run.
+MI355_HOST_DEVICE inline uint32_t xcd_workgroup(uint32_t b, uint32_t run) {
+  const uint32_t xcd = b & 7, j = b >> 3;
+  const uint32_t q = j / run;
+  return (q * 8 + xcd) * run + (j - q * run);
+}
 constexpr unsigned kChunkVecs = 256;  // vectors of one batched-copy chunk: 4 KiB
 
 struct CopyArgs {
@@ -29,6 +45,13 @@ struct CopyArgs {
   // kernel arguments and can be dispatched from a hand-built AQL packet.
   uint32_t waves_per_wg;
   uint32_t n_waves;  // grid * waves_per_wg
+  // The hardware deals consecutive workgroups to the 8 XCDs in turn.  With
+  // xcd_run != 0, workgroup b < xcd_full does the work of workgroup
+  // xcd_workgroup(b) instead, which gives every XCD runs of xcd_run
+  // neighbouring workgroups (a permutation of [0, xcd_full), a multiple of
+  // 8 * xcd_run).
+  uint32_t xcd_run;
+  uint32_t xcd_full;
 };
 
 struct FillArgs {
@@ -42,6 +65,8 @@ struct FillArgs {
   uint32_t edge_wave;
   uint32_t waves_per_wg;
   uint32_t n_waves;
+  uint32_t xcd_run;
+  uint32_t xcd_full;
 };
 
 struct BatchDesc {
@@ -113,6 +138,8 @@ struct BatchCopyArgs {
   const uint32_t* total;
   uint32_t waves_per_wg;
   uint32_t n_waves;
+  uint32_t xcd_run;   // as in CopyArgs
+  uint32_t xcd_full;
 };
 
 struct BatchStridedArgs {
@@ -141,7 +168,8 @@ struct RectArgs {
   uint32_t total_slots;  // rows * layers * slots
   uint32_t waves_per_wg;
   uint32_t n_waves;
-  uint32_t pad;
+  uint32_t xcd_run;   // as in CopyArgs
+  uint32_t xcd_full;
 };
 
 // The same region copy for rows of up to about 1 KiB: every 16-byte slot of a
@@ -162,7 +190,8 @@ struct RectNarrowArgs {
   uint32_t magic;    // ceil(2^16 / lanes_per_row): n / lanes_per_row == (n * magic) >> 16, n < 128
   uint32_t waves_per_wg;
   uint32_t n_waves;
-  uint32_t pad;
+  uint32_t xcd_run;   // as in CopyArgs
+  uint32_t xcd_full;
 };
 
 // Layout of amd_signal_t (inc/amd_hsa_signal.h, struct amd_signal_s).

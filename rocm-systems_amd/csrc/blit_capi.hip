@@ -407,6 +407,8 @@ int mi355_blit_copy(mi355_blit_t* h, void* dst, const void* src, size_t bytes, v
   a.head = static_cast<uint32_t>(p.head_bytes);
   a.lead = p.lead_vecs;
   set_tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
+  a.xcd_run = p.xcd_run;
+  a.xcd_full = xcd_full(p.grid, p.xcd_run);
   hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
   hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
   BLIT_HIP(hipGetLastError());
@@ -434,6 +436,8 @@ int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwo
   a.lead = p.lead_vecs;
   a.value = value;
   set_tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
+  a.xcd_run = p.xcd_run;
+  a.xcd_full = xcd_full(p.grid, p.xcd_run);
   hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
   hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
   BLIT_HIP(hipGetLastError());
@@ -543,11 +547,13 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
     if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
     if (wgs * p.wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / p.wg_size;
     p.grid = static_cast<uint32_t>(wgs);
+    const uint32_t batch_run = batch_xcd_run(shape.total_bytes, split, static_cast<uint32_t>(waves_per_wg), t);
+    p.xcd_run = batch_run;
     p.unroll = 4 / split;
     batch_kernel_t k = select_batch_kernel(split, streaming, p.store_policy);
     if (!k) return MI355_BLIT_ERROR;
     BatchCopyArgs bc{h->records_dev, shape.total_chunks, nullptr, static_cast<uint32_t>(waves_per_wg),
-                     static_cast<uint32_t>(wgs * waves_per_wg)};
+                     static_cast<uint32_t>(wgs * waves_per_wg), batch_run, xcd_full(p.grid, batch_run)};
     hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, bc);
   } else if (max_total_bytes) {
     // Device-resident descriptors whose total size the caller bounds: the
@@ -573,11 +579,13 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
     if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
     if (wgs * p.wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / p.wg_size;
     p.grid = static_cast<uint32_t>(wgs);
+    const uint32_t batch_run = batch_xcd_run(max_total_bytes, kBatchSplit, static_cast<uint32_t>(waves_per_wg), t);
+    p.xcd_run = batch_run;
     p.unroll = 4 / kBatchSplit;
     batch_kernel_t k = select_batch_kernel(kBatchSplit, streaming, p.store_policy);
     if (!k) return MI355_BLIT_ERROR;
     BatchCopyArgs bc{h->records_dev, shape.total_chunks, h->chunk_start_dev + n, static_cast<uint32_t>(waves_per_wg),
-                     static_cast<uint32_t>(wgs * waves_per_wg)};
+                     static_cast<uint32_t>(wgs * waves_per_wg), batch_run, xcd_full(p.grid, batch_run)};
     hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, bc);
   } else {
     // Device-resident descriptors: the prefix sum runs on the device and, as
@@ -678,6 +686,7 @@ int mi355_blit_plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst
   out->grid = rp.grid;
   out->nt_load = rp.streaming;
   out->store_policy = rp.store_policy;
+  out->xcd_run = rp.xcd_run;
   return MI355_BLIT_SUCCESS;
 }
 

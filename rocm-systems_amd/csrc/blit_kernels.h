@@ -228,10 +228,18 @@ __device__ __forceinline__ uint64_t global_wave(unsigned waves_per_wg) {
   return __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
 }
 
+// global_wave() of a launch permuted that way: workgroups below xcd_full swap
+// places, the others keep theirs.
+__device__ __forceinline__ uint64_t global_wave_xcd(unsigned waves_per_wg, uint32_t xcd_run, uint32_t xcd_full) {
+  uint32_t wg = blockIdx.x;
+  if (wg < xcd_full) wg = xcd_workgroup(wg, xcd_run);
+  return __builtin_amdgcn_readfirstlane(wg * waves_per_wg + threadIdx.x / kWave);
+}
+
 template <int U, bool NTL, int NTS, bool SHIFT>
 __device__ __forceinline__ void copy_body(const CopyArgs& a) {
   const unsigned lane = threadIdx.x & (kWave - 1);
-  const uint64_t wave = global_wave(a.waves_per_wg);
+  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd_run, a.xcd_full);
   const uint64_t n_waves = a.n_waves;
   const uint8_t* sb = a.src + a.head;
   const unsigned r = SHIFT ? static_cast<unsigned>(reinterpret_cast<uintptr_t>(sb) & 3) : 0;
@@ -244,7 +252,7 @@ __device__ __forceinline__ void copy_body(const CopyArgs& a) {
 template <int U, int NTS>
 __device__ __forceinline__ void fill_body(const FillArgs& a) {
   const unsigned lane = threadIdx.x & (kWave - 1);
-  const uint64_t wave = global_wave(a.waves_per_wg);
+  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd_run, a.xcd_full);
   const uint64_t n_waves = a.n_waves;
   const v4u val = {a.value, a.value, a.value, a.value};
   constexpr uint64_t kTile = kWave * U;
@@ -580,7 +588,7 @@ __device__ __forceinline__ void batch_copy_records_body(const BatchCopyArgs& a) 
     if (counted < total_chunks) total_chunks = counted;
   }
   const unsigned lane = threadIdx.x & (kWave - 1);
-  const uint64_t wave = global_wave(a.waves_per_wg);
+  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd_run, a.xcd_full);
   const uint64_t n_waves = a.n_waves;
   for (uint64_t w = wave; w < total_chunks * SPLIT; w += n_waves) {
     const ChunkRecord rec = load_record(records + w / SPLIT);
@@ -656,7 +664,7 @@ template <int U, bool NTL, int NTS>
 __device__ __forceinline__ void rect_copy_body(const RectArgs& a) {
   constexpr unsigned kUnit = kWave * U;
   const unsigned lane = threadIdx.x & (kWave - 1);
-  const uint64_t wave = global_wave(a.waves_per_wg);
+  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd_run, a.xcd_full);
   const uint64_t n_waves = a.n_waves;
   for (uint64_t w = wave; w < a.total_slots; w += n_waves) {
     const uint32_t slot = static_cast<uint32_t>(w);
@@ -761,7 +769,7 @@ __device__ __forceinline__ void copy_partial_slot(uintptr_t slot, unsigned off, 
 template <bool NTL, int NTS>
 __device__ __forceinline__ void rect_narrow_body(const RectNarrowArgs& a) {
   const unsigned lane = threadIdx.x & (kWave - 1);
-  const uint64_t wave = global_wave(a.waves_per_wg);
+  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd_run, a.xcd_full);
   const uint32_t lpr = a.lanes_per_row;
   const uint64_t total = static_cast<uint64_t>(a.lines) * lpr;
   const uint64_t n_groups = (total + kWave - 1) / kWave;

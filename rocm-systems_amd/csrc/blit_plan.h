@@ -30,39 +30,57 @@ struct SizeClass {
   uint32_t unroll;
   uint32_t nt_load;
   uint32_t store_policy;
+  uint32_t xcd_run_bytes;  // bytes of the runs of tiles each XCD works through; 0 = tiles in launch order
 };
 
-// Measured on MI355X (256 CUs), sweeps of 4 KiB .. 4 GiB in powers of 4.
+// Measured on MI355X (256 CUs), sweeps of 4 KiB .. 4 GiB.
 // Up to a few MiB a launch is bound by its fixed cost (~3.5 us back to back)
 // and the shape does not matter.  From there on transfers bypass the caches:
-// loads non-temporal, stores written through L2.  Source and destination
-// equally aligned mod 16: one 1 KiB tile per single-wave workgroup is the
-// fastest shape once the transfer streams from HBM (>= 512 MiB); while the
-// 256 MiB last-level cache still absorbs part of it, 4-wave workgroups are.
-// Tiles are anchored at the destination's 256-byte boundaries, so when source
-// and destination differ mod 128 every wave's 1 KiB of loads straddles a cache
-// line shared with its neighbour; 4-wave workgroups share that line within
-// one CU instead of fetching it twice.  A byte offset adds one dword fetch per tile (the bytes that
-// spill past the last lane), which 2 KiB tiles amortise best.  Fills at one
+// loads non-temporal, stores written through L2.
+//
+// The hardware deals consecutive workgroups to the 8 XCDs in turn, each XCD
+// with an L2 of its own.  From about 100 MiB on it pays to permute the launch
+// so that each XCD works through runs of neighbouring tiles (xcd_run
+// workgroups, 576 KiB): a source line that two tiles share (tiles are anchored
+// at the destination's 256-byte boundaries, so they do whenever source and
+// destination differ mod 128) is then fetched into one L2 instead of two, and
+// single-wave workgroups, the fastest shape for a stream, no longer pay for
+// having their neighbours on another XCD.  The run is 512 KiB + 64 KiB on
+// purpose: with runs of a power of two the 8 streams sit a power of two apart
+// and, depending on where source and destination lie, collide in the memory
+// channels (1 GiB with a byte offset: 315-367 us over 20 placements with runs
+// of 256 KiB, 320-326 us with 576 KiB, 338-344 us in launch order).
+// Measured, 1 GiB: equally aligned 309-312 us against 314-317 us in launch
+// order; source and destination differing mod 128, 311-313 us against 321-327;
+// a byte offset, 320-326 us against 338-344.  At 128-256 MiB, where the
+// last-level cache holds most of the transfer, 59 us against 66 us.  A byte
+// offset adds one dword fetch per tile (the bytes that spill past the last
+// lane), which 2 KiB tiles amortise best; its stores are written through while
+// the last-level cache absorbs them and non-temporal beyond.  Fills at one
 // wave per workgroup are bound by the dispatcher's workgroup rate and want
 // 4-wave workgroups.  Last match wins.
-constexpr SizeClass kCopyClasses[] = {      // (src - dst) % 128 == 0
-    {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
-    {4ull << 20, 256, 1, 1, MI355_BLIT_STORE_AGENT_WT},
-    {512ull << 20, 64, 1, 1, MI355_BLIT_STORE_AGENT_WT},
-};
-constexpr SizeClass kCopyDwordOffsetClasses[] = {  // (src - dst) % 4 == 0, not % 128
-    {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
-    {4ull << 20, 256, 1, 1, MI355_BLIT_STORE_AGENT_WT},
+constexpr uint32_t kXcdRunBytes = 576u << 10;
+// Below this size the permutation gains nothing (the transfer sits in the
+// last-level cache) or loses a little.
+constexpr uint64_t kXcdRunMinBytes = 64ull << 20;
+// The batched copy, whose neighbouring 4 KiB chunks share source lines and cut
+// destination lines: measured with 65,536 copies (2 GB), 698-701 us with runs
+// of 272 chunks or more against 728-730 us in launch order.
+constexpr uint32_t kBatchXcdRunChunks = 528;
+constexpr SizeClass kCopyClasses[] = {      // (src - dst) % 4 == 0
+    {0, 256, 1, 0, MI355_BLIT_STORE_CACHED, 0},
+    {4ull << 20, 256, 1, 1, MI355_BLIT_STORE_AGENT_WT, 0},
+    {128ull << 20, 64, 1, 1, MI355_BLIT_STORE_AGENT_WT, kXcdRunBytes},
 };
 constexpr SizeClass kCopyRealignClasses[] = {  // (src - dst) % 4 != 0
-    {0, 512, 1, 0, MI355_BLIT_STORE_CACHED},
-    {4ull << 20, 256, 2, 1, MI355_BLIT_STORE_AGENT_WT},
-    {512ull << 20, 512, 2, 1, MI355_BLIT_STORE_NT},
+    {0, 512, 1, 0, MI355_BLIT_STORE_CACHED, 0},
+    {4ull << 20, 256, 2, 1, MI355_BLIT_STORE_AGENT_WT, 0},
+    {64ull << 20, 64, 2, 1, MI355_BLIT_STORE_AGENT_WT, kXcdRunBytes},
+    {320ull << 20, 64, 2, 1, MI355_BLIT_STORE_NT, kXcdRunBytes},
 };
 constexpr SizeClass kFillClasses[] = {
-    {0, 256, 1, 0, MI355_BLIT_STORE_CACHED},
-    {16ull << 20, 256, 1, 0, MI355_BLIT_STORE_SYSTEM_WT},
+    {0, 256, 1, 0, MI355_BLIT_STORE_CACHED, 0},
+    {16ull << 20, 256, 1, 0, MI355_BLIT_STORE_SYSTEM_WT, 0},
 };
 
 inline bool valid_unroll(uint32_t u) { return u == 1 || u == 2 || u == 4; }
@@ -73,6 +91,28 @@ inline const SizeClass& pick_class(const SizeClass (&tbl)[N], uint64_t bytes) {
   for (unsigned i = 0; i < N; ++i)
     if (bytes >= tbl[i].min_bytes) c = &tbl[i];
   return *c;
+}
+
+// Runs of workgroups per XCD: the heuristic's choice unless tuning overrides it
+// (1 = launch order, which a plan states as 0).
+inline uint32_t plan_xcd_run(uint32_t heuristic, const mi355_blit_tuning_t* t) {
+  uint32_t run = heuristic;
+  if (t && t->xcd_run) run = t->xcd_run;
+  return run > 1 ? run : 0;
+}
+
+// In workgroups of waves_per_wg waves, `split` waves to a chunk.
+inline uint32_t batch_xcd_run(uint64_t total_bytes, uint32_t split, uint32_t waves_per_wg,
+                              const mi355_blit_tuning_t* t) {
+  return plan_xcd_run(total_bytes >= kXcdRunMinBytes ? kBatchXcdRunChunks * split / waves_per_wg : 0, t);
+}
+
+// Workgroups of a launch of `grid` that the XCD permutation covers: whole
+// rounds of 8 runs; the rest keep their place.
+inline uint32_t xcd_full(uint32_t grid, uint32_t run) {
+  if (run <= 1) return 0;
+  const uint64_t round = 8ull * run;
+  return static_cast<uint32_t>(grid / round * round);
 }
 
 inline void apply_launch_shape(mi355_blit_plan_t* p, const SizeClass& cls, uint32_t num_cus,
@@ -90,6 +130,7 @@ inline void apply_launch_shape(mi355_blit_plan_t* p, const SizeClass& cls, uint3
     if (t->store_policy >= 1 && t->store_policy <= 4) p->store_policy = t->store_policy - 1;
     max_grid = t->max_grid;
   }
+  p->xcd_run = plan_xcd_run(cls.xcd_run_bytes / (p->wg_size / 64 * p->unroll * 1024), t);
   const uint64_t hw_max = kMaxGridWorkItems / p->wg_size;
   if (max_grid == 0 || max_grid > hw_max) max_grid = hw_max;
   // One wave per tile of 64*unroll vectors (tiles anchored at 256-byte
@@ -117,10 +158,7 @@ inline int plan_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t num_cu
   p->lead_vecs = static_cast<uint32_t>(((dst + head) & 255) / 16);
   p->byte_shift = static_cast<uint32_t>((src - dst) & 3);
   p->kernel = p->byte_shift ? MI355_BLIT_KERNEL_COPY_REALIGN : MI355_BLIT_KERNEL_COPY;
-  const uint64_t delta = (src - dst) & 127;
-  const SizeClass& cls = delta == 0         ? pick_class(kCopyClasses, bytes)
-                         : (delta & 3) == 0 ? pick_class(kCopyDwordOffsetClasses, bytes)
-                                            : pick_class(kCopyRealignClasses, bytes);
+  const SizeClass& cls = p->byte_shift ? pick_class(kCopyRealignClasses, bytes) : pick_class(kCopyClasses, bytes);
   apply_launch_shape(p, cls, num_cus, t);
   return MI355_BLIT_SUCCESS;
 }

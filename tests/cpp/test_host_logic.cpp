@@ -312,6 +312,31 @@ void one_batch_stage() {
   CHECK(batch_bound_chunks(1, 1ull << 62) == 0, "a bound beyond 32-bit record indices accepted");
 }
 
+// The XCD permutation of a launch: workgroups below xcd_full(grid, run) swap
+// places among themselves (a bijection), each XCD (b % 8) gets whole runs of
+// neighbouring workgroups in launch order, the rest keep their place.
+void one_xcd_permutation() {
+  const uint32_t run = 2 + static_cast<uint32_t>(below(700));
+  const uint32_t grid = static_cast<uint32_t>(below(40000));
+  const uint32_t full = xcd_full(grid, run);
+  CHECK(full <= grid && full % (8 * run) == 0 && grid - full < 8 * run, "xcd_full(%u, %u) = %u", grid, run, full);
+  CHECK(xcd_full(grid, 0) == 0 && xcd_full(grid, 1) == 0, "no permutation without a run");
+  std::vector<uint8_t> seen(full, 0);
+  std::vector<uint32_t> last(8, 0);
+  for (uint32_t b = 0; b < full; ++b) {
+    const uint32_t w = xcd_workgroup(b, run);
+    CHECK(w < full && !seen[w], "workgroup %u -> %u (run %u) out of range or taken twice", b, w, run);
+    if (w < full) seen[w] = 1;
+    // within a round the work of XCD x is [x * run, (x + 1) * run), taken in launch order
+    CHECK((w % (8 * run)) / run == (b & 7), "workgroup %u works on another XCD's run", b);
+    if (b >= 8) CHECK(w == last[b & 7] + 1 || w == last[b & 7] + 1 + 7 * run, "XCD %u jumps from %u to %u", b & 7, last[b & 7], w);
+    last[b & 7] = w;
+  }
+  const mi355_blit_tuning_t linear{0, 0, 0, 0, 0, 1, {0, 0}}, forced{0, 0, 0, 0, 0, 99, {0, 0}};
+  CHECK(plan_xcd_run(288, nullptr) == 288 && plan_xcd_run(288, &linear) == 0 && plan_xcd_run(0, &forced) == 99,
+        "tuning of the run");
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
@@ -321,6 +346,7 @@ int main(int argc, char** argv) {
     one_fill_plan();
     one_rect_plan();
     if (i % 8 == 0) one_batch_stage();
+    if (i % 64 == 0) one_xcd_permutation();
   }
   std::printf("%s: %ld cases each of copy, fill and region plans, %d failures\n", g_failures ? "FAILED" : "OK", cases,
               g_failures);

@@ -35,14 +35,14 @@ def test_library_exports_every_declared_symbol(capi_host):
 
 def test_abi_version_and_status_strings(capi_host):
     lib = capi_host.load()
-    assert lib.mi355_blit_abi_version() == 1
+    assert lib.mi355_blit_abi_version() == 2
     assert lib.mi355_blit_status_string(0) == b"success"
     assert lib.mi355_blit_status_string(capi_host.ERROR_INVALID_ARGUMENT) == b"invalid argument"
     assert lib.mi355_blit_status_string(12345) == b"unknown status"
 
 
 def test_struct_layouts_match_header(capi_host):
-    assert C.sizeof(capi_host.Plan) == 8 * 4 + 3 * 8
+    assert C.sizeof(capi_host.Plan) == 8 * 4 + 3 * 8 + 2 * 4
     assert capi_host.Plan.lead_vecs.offset == 28
     assert C.sizeof(capi_host.Tuning) == 32
     assert C.sizeof(capi_host.Desc) == 24
@@ -118,6 +118,40 @@ def test_plan_copy_tuning_overrides(capi_host):
     t = capi_host.Tuning(nt_load=1, store_policy=capi_host.STORE_CACHED + 1)
     st, p = capi_host.plan_copy(0x1000, 0x9000, 1 << 30, 256, t)
     assert p.nt_load == 0 and p.store_policy == capi_host.STORE_CACHED
+
+
+def test_plan_copy_shapes_by_size_and_offset(capi_host):
+    """The launch shapes the heuristics pick, and the XCD runs: 576 KiB of
+    neighbouring tiles per XCD once a transfer streams from memory."""
+    MIB = 1 << 20
+    dst = 0x7f0000000000
+
+    def shape(src_off, n):
+        st, p = capi_host.plan_copy(dst, 0x7e0000000000 + src_off, n)
+        assert st == 0
+        return p.wg_size, p.unroll, p.nt_load, p.store_policy, p.xcd_run
+
+    wt, nt, cached = capi_host.STORE_AGENT_WT, capi_host.STORE_NT, capi_host.STORE_CACHED
+    for off in (0, 4, 64):                                   # dword-aligned to one another
+        assert shape(off, MIB) == (256, 1, 0, cached, 0)
+        assert shape(off, 64 * MIB) == (256, 1, 1, wt, 0)
+        assert shape(off, 128 * MIB) == (64, 1, 1, wt, 576)     # 576 tiles of 1 KiB
+        assert shape(off, 1 << 30) == (64, 1, 1, wt, 576)
+    for off in (1, 3, 6):                                    # a byte offset: the realigning kernel
+        assert shape(off, MIB) == (512, 1, 0, cached, 0)
+        assert shape(off, 16 * MIB) == (256, 2, 1, wt, 0)
+        assert shape(off, 64 * MIB) == (64, 2, 1, wt, 288)      # 288 tiles of 2 KiB
+        assert shape(off, 1 << 30) == (64, 2, 1, nt, 288)
+    # the run follows the workgroup the tuning asks for; 1 means launch order
+    st, p = capi_host.plan_copy(dst, 0x7e0000000000, 1 << 30, 256, capi_host.Tuning(wg_size=256))
+    assert p.xcd_run == 144
+    st, p = capi_host.plan_copy(dst, 0x7e0000000000, 1 << 30, 256, capi_host.Tuning(xcd_run=1))
+    assert p.xcd_run == 0
+    st, p = capi_host.plan_copy(dst, 0x7e0000000000, MIB, 256, capi_host.Tuning(xcd_run=40))
+    assert p.xcd_run == 40
+    # fills store whole lines and share nothing: launch order
+    st, p = capi_host.plan_fill(dst, 1 << 28)
+    assert st == 0 and p.xcd_run == 0
 
 
 def test_plan_fill_invariants(capi_host):

@@ -372,6 +372,47 @@ def test_every_fill_variant_is_exact(capi, fresh_tuning, oracle, arenas, unroll)
                     run_fill_case(capi, blit, oracle, dst, GUARD + off, (2 * MIB + 1236) // 4, FILL_VALUE)
 
 
+@pytest.mark.parametrize("xcd_run", [2, 5, 36, 288])
+def test_permuted_launches_are_exact(capi, fresh_tuning, oracle, arenas, xcd_run):
+    """Launches whose workgroups take their tiles in runs per XCD instead of
+    launch order: a permutation of the same tiles, so the same bytes.  Grids
+    that are not whole rounds of 8 runs, capped grids (waves striding over
+    tiles) and the two copy kernels, the fill and the batch."""
+    blit = fresh_tuning
+    src, src_host, dst = arenas
+    for wg, unroll, max_grid in ((64, 1, 0), (256, 2, 0), (64, 2, 0), (128, 1, 1000), (64, 4, 333)):
+        blit.set_tuning(wg_size=wg, unroll=unroll, max_grid=max_grid, xcd_run=xcd_run)
+        for so, do, n in ((0, 0, 5 * MIB + 12345), (3, 9, 7 * MIB + 1), (64, 16, 2 * MIB + 77), (1, 0, 40000)):
+            run_copy_case(capi, blit, oracle, src, src_host, dst, 64 + so, GUARD + do, n)
+            assert blit.last_plan().xcd_run == xcd_run
+        run_fill_case(capi, blit, oracle, dst, GUARD + 4, (3 * MIB + 1236) // 4, FILL_VALUE)
+        assert blit.last_plan().xcd_run == xcd_run
+    blit.set_tuning(xcd_run=xcd_run)
+    rng = np.random.default_rng(77 + xcd_run)
+    n = 4000
+    descs, lens, offs, so, do, total = _make_batch(capi, rng, src, dst, n, max_len=64 << 10)
+    dst.fill(0, total, GUARD_BYTE)
+    check_ok(capi, blit.copy_batch(descs, n), "copy_batch")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert blit.last_plan().xcd_run == xcd_run
+    assert np.array_equal(dst.host(0, total), _expect_batch(oracle, src_host, total, lens, offs, so, do))
+
+
+def test_large_copies_with_the_heuristic_runs(capi, blit, oracle, rand, torch_cuda):
+    """At the sizes where the heuristics permute the launch by themselves
+    (from 64 MiB with a byte offset, from 128 MiB without): every byte and the
+    guards against the oracle."""
+    torch = torch_cuda
+    n = 160 * MIB + 4099
+    src_host = rand(n + 512, 0xB1170077)
+    src = Arena(torch, n + 512, host=src_host)
+    dst = Arena(torch, n + 1024, fill=GUARD_BYTE)
+    for so, do in ((0, 0), (64, 128), (3, 9)):
+        run_copy_case(capi, blit, oracle, src, src_host, dst, so, GUARD + do, n)
+        p = blit.last_plan()
+        assert p.xcd_run == (288 if (so - do) % 4 else 576), p.as_dict()
+
+
 # ---------------------------------------------------------------------- batched
 
 def _make_batch(capi, rng, src, dst, n, min_len=64, max_len=256 << 10):

@@ -138,6 +138,24 @@ def test_rect_random_narrow_rows(capi, fresh_tuning, oracle, rand, seed):
                   int(rng.integers(0, 256)), int(rng.integers(0, 256)), seed=0x7A220000 + seed)
 
 
+@pytest.mark.parametrize("xcd_run", [2, 3, 36])
+def test_rect_permuted_launches_are_exact(capi, fresh_tuning, oracle, rand, xcd_run):
+    """Both region kernels with their workgroups dealt to the XCDs in runs: a
+    permutation of the same row units, so the same bytes.  Grids of a few
+    hundred to a few thousand workgroups, not whole rounds of 8 runs."""
+    blit = fresh_tuning
+    for wg, max_grid in ((64, 0), (256, 0), (128, 50)):
+        blit.set_tuning(wg_size=wg, xcd_run=xcd_run, max_grid=max_grid)
+        # wide rows: 61 rows of 9001 bytes, 9 units of 1 KiB each
+        p = run_rect_case(capi, blit, oracle, rand, (2, 40, 12000), (2, 37, 11003), (9001, 31, 2), (7, 3, 0),
+                          (1001, 2, 0), 3, 77, seed=0x7EC7AA00 + xcd_run)
+        assert p.kernel == capi.KERNEL_COPY_RECT and p.xcd_run == xcd_run
+        # narrow rows: 3 x 500 rows of 333 bytes
+        p = run_rect_case(capi, blit, oracle, rand, (3, 600, 517), (3, 550, 400), (333, 500, 3), (13, 20, 0),
+                          (5, 31, 0), 9, 130, seed=0x7EC7BB00 + xcd_run)
+        assert p.kernel == capi.KERNEL_COPY_RECT and p.xcd_run == xcd_run
+
+
 def test_rect_plan_shapes(capi, blit, oracle, rand):
     """What the launch record says: a rect kernel with one wave per 1 KiB of
     row for rows of whole cache lines, a linear copy when the region is one run."""

@@ -34,6 +34,10 @@ MIB = 1 << 20
 FILL_VALUE = 0xA5C30F1E
 
 
+# Launches that bring the device out of idle before anything is timed (see --warmup).
+WARMUP_AFTER_IDLE = 60
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -41,7 +45,7 @@ def parse_args():
     # After an idle period the first ~50 launches of a streaming kernel run up to 25 % slow (a hump
     # that peaks around the tenth launch and is gone by the fiftieth, whatever the kernel): the
     # default warm-up covers it.
-    ap.add_argument("--warmup", type=int, default=60)
+    ap.add_argument("--warmup", type=int, default=WARMUP_AFTER_IDLE)
     ap.add_argument("--workload", default="copy", choices=["copy", "fill", "misaligned", "batch", "rect", "calib"])
     ap.add_argument("--bytes", type=int, default=GIB, help="transfer size of the copy/fill workloads")
     ap.add_argument("--rect", default="8192,131072,262144,0,0",
@@ -236,7 +240,7 @@ def rect_shapes(r):
     out = {}
     for rows, width, pitch, sx, dx in RECT_SHAPES:
         fn, verify, algo, keep = make_rect(r, rows, width, pitch, sx, dx)
-        _, us = r.time_launches(fn, 10, 3)
+        _, us = r.time_launches(fn, 20, WARMUP_AFTER_IDLE)
         verify()
         out["%dx%d/%d+%d,%d" % (rows, width, pitch, sx, dx)] = {
             "gbs": round(algo / us / 1e3, 1), "us_per_launch": round(us, 2),
@@ -260,9 +264,9 @@ def size_sweep(r):
     for k in range(11):
         n = 4096 * 4 ** k
         iters = 100 if n <= MIB else (30 if n <= 256 * MIB else 8)
-        _, us = r.time_launches(lambda: r.check(r.blit.copy(D, S, n, r.stream), "copy"), iters, 3)
+        _, us = r.time_launches(lambda: r.check(r.blit.copy(D, S, n, r.stream), "copy"), iters, WARMUP_AFTER_IDLE)
         out["copy"][str(n)] = {"us": round(us, 2), "gbs": round(2 * n / us / 1e3, 1)}
-        _, us = r.time_launches(lambda: r.check(r.blit.fill32(D, FILL_VALUE, n // 4, r.stream), "fill32"), iters, 3)
+        _, us = r.time_launches(lambda: r.check(r.blit.fill32(D, FILL_VALUE, n // 4, r.stream), "fill32"), iters, WARMUP_AFTER_IDLE)
         out["fill"][str(n)] = {"us": round(us, 2), "gbs": round(n / us / 1e3, 1)}
     so, do = (-src.data_ptr()) % 256, (-dst.data_ptr()) % 256
     r.check(r.blit.copy(D, S, top, r.stream), "copy")
@@ -314,11 +318,11 @@ def aql_path(r, pkg):
         for key, submit, algo in cases:
             # one command at a time: with the barrier bit clear, commands
             # queued together would overlap and stretch each other's time
-            sigs = [sig.create(1) for _ in range(23)]
+            sigs = [sig.create(1) for _ in range(WARMUP_AFTER_IDLE + 20)]
             for c in sigs:
                 r.check(submit(c), key)
                 sig.wait_below_one(c)
-            us = [eng.command_time_us(c) for c in sigs[3:]]
+            us = [eng.command_time_us(c) for c in sigs[WARMUP_AFTER_IDLE:]]
             for c in sigs:
                 sig.destroy(c)
             avg = sum(us) / len(us)
@@ -349,7 +353,7 @@ def aql_path(r, pkg):
         fn, verify, algo, keep = make_batch(r)
         descs = keep[2]
         n = len(descs)
-        for _ in range(3):
+        for _ in range(WARMUP_AFTER_IDLE // 2):
             r.check(eng.copy_batch(descs, n), "copy_batch")
         r.check(eng.synchronize(), "wait_idle")
         t0 = time.perf_counter()
@@ -524,7 +528,7 @@ def main():
                            ("batch_65536", lambda: make_batch(r)),
                            ("rect_8192x131072_262144", lambda: make_rect(r))):
             f2, v2, a2, k2 = maker()
-            w2, us2 = r.time_launches(f2, 20, 10)
+            w2, us2 = r.time_launches(f2, 30, max(args.warmup, WARMUP_AFTER_IDLE))
             v2()
             also[key] = {"gbs": round(a2 / us2 / 1e3, 1), "frac_of_peak": round(a2 / us2 / 1e3 / HBM_PEAK_GBS, 4),
                          "us_per_launch": round(us2, 2)}

@@ -1,6 +1,6 @@
 // Device kernels of the gfx950 blit engine: linear copy, dword fill, batched
-// small copies, pitched 3-D region copies.  They take the place of ROCr's CopyAligned, CopyMisaligned and
-// Fill shaders (projects/rocr-runtime/runtime/hsa-runtime/core/runtime/
+// small copies, pitched 3-D region copies.  They take the place of ROCr's
+// CopyAligned, CopyMisaligned and Fill shaders (projects/rocr-runtime/runtime/hsa-runtime/core/runtime/
 // blit_shaders/blit_copyAligned.s:76-259, blit_copyMisaligned.s:90-182,
 // blit_fill.s:91-185) but share none of their structure:
 //
@@ -12,6 +12,11 @@
 //    address order as waves retire, which keeps the set of DRAM pages in use
 //    small; measured on MI355X this beats a persistent grid-stride loop by
 //    ~10 % at 1 GiB.  The grid-stride loop remains for capped grids.
+//  * Where neighbouring tiles share cache lines and the transfer is large, the
+//    host asks for the launch to be permuted so that each of the 8 XCDs (each
+//    with its own L2) works through runs of neighbouring workgroups' tiles
+//    (xcd_run / xcd_full in the argument blocks, xcd_workgroup in blit_args.h):
+//    the shared lines then meet in one L2.
 //  * Large transfers bypass the caches: loads carry nt, stores are written
 //    through L2 (sc1 / sc0 sc1), chosen per size by the host.
 //  * Stores are always 16-byte aligned, and tiles are anchored at 256-byte
@@ -228,8 +233,9 @@ __device__ __forceinline__ uint64_t global_wave(unsigned waves_per_wg) {
   return __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
 }
 
-// global_wave() of a launch permuted that way: workgroups below xcd_full swap
-// places, the others keep theirs.
+// global_wave() of a launch whose workgroups take their work in runs per XCD
+// (xcd_workgroup): workgroups below xcd_full swap places among themselves, the
+// others keep theirs.  xcd_full == 0: launch order.
 __device__ __forceinline__ uint64_t global_wave_xcd(unsigned waves_per_wg, uint32_t xcd_run, uint32_t xcd_full) {
   uint32_t wg = blockIdx.x;
   if (wg < xcd_full) wg = xcd_workgroup(wg, xcd_run);

@@ -136,6 +136,57 @@ def test_copy_4gib_properties(capi, blit, oracle, rand, torch_cuda):
     assert p.grid * (p.wg_size // 64) >= -(-p.body_vecs // (64 * p.unroll))
 
 
+def test_copy_and_fill_beyond_the_largest_grid(capi, blit, oracle, rand, torch_cuda):
+    """33 GiB: more 1 KiB tiles than a grid can have workgroups (an AQL packet
+    counts work-items in 32 bits), so the grid is capped and waves take a
+    second tile.  Same properties as at 4 GiB, compared on the device in 1 GiB
+    slices, with the slices around the wrap of the grid also hashed on the host."""
+    torch = torch_cuda
+    gib = 1 << 30
+    n = 33 * gib + 12345 * 16
+    blk = 64 * MIB
+    free, _ = torch.cuda.mem_get_info()
+    if free < 2 * n + 4 * gib:
+        pytest.skip("needs %d GiB of free device memory" % ((2 * n + 4 * gib) >> 30))
+    block_host = rand(blk, 0xB1170034)
+    src = Arena(torch, n)
+    block_dev = torch.from_numpy(block_host).to("cuda:0")
+    for lo in range(0, n, blk):
+        m = min(blk, n - lo)
+        src.view[lo:lo + m].copy_(block_dev[:m])
+    torch.cuda.synchronize()
+    dst = Arena(torch, n + 2 * GUARD, fill=GUARD_BYTE)
+    check_ok(capi, blit.copy(dst.base + GUARD, src.base, n), "copy")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    p = blit.last_plan()
+    tiles = -(-(p.body_vecs + p.lead_vecs) // (64 * p.unroll))
+    waves = p.grid * (p.wg_size // 64)
+    assert waves < tiles, "the case is meant to cap the grid: %s" % p.as_dict()
+    assert bool((dst.view[:GUARD] == GUARD_BYTE).all()) and bool((dst.view[GUARD + n:] == GUARD_BYTE).all())
+    for lo in range(0, n, gib):
+        m = min(gib, n - lo)
+        assert torch.equal(dst.view[GUARD + lo:GUARD + lo + m], src.view[lo:lo + m]), "slice at %d GiB differs" % (lo >> 30)
+    want = np.empty(blk, dtype=np.uint8)
+    oracle.oracle_copy(want.ctypes.data, block_host.ctypes.data, blk)
+    wrap = waves * 64 * p.unroll * 16 // blk      # the 64 MiB block in which the second round of tiles starts
+    for i in (0, wrap - 1, wrap, wrap + 1, n // blk - 1):
+        got = dst.host(GUARD + i * blk, GUARD + (i + 1) * blk)
+        assert np.array_equal(got, want), "block %d differs" % i
+    del src
+    torch.cuda.empty_cache()
+    # the fill, over what the copy left
+    count = n // 4
+    check_ok(capi, blit.fill32(dst.base + GUARD, FILL_VALUE, count), "fill32")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    p = blit.last_plan()
+    assert p.grid * (p.wg_size // 64) < -(-(p.body_vecs + p.lead_vecs) // (64 * p.unroll)), p.as_dict()
+    assert bool((dst.view[:GUARD] == GUARD_BYTE).all()) and bool((dst.view[GUARD + n:] == GUARD_BYTE).all())
+    words = dst.view[GUARD:GUARD + n].view(torch.int32)
+    pattern = FILL_VALUE - (1 << 32)
+    for lo in range(0, count, gib // 4):
+        assert bool((words[lo:lo + gib // 4] == pattern).all()), "fill slice at %d GiB differs" % (lo >> 28)
+
+
 # -------------------------------------------------------------- misaligned copy
 
 def _log_uniform_lengths(rng, k, max_bytes):

@@ -66,6 +66,7 @@ class RectPlan(C.Structure):
         ("slots", C.c_uint32), ("unroll", C.c_uint32), ("lanes_per_row", C.c_uint32),
         ("xcd_run", C.c_uint32), ("wg_size", C.c_uint32), ("grid", C.c_uint32),
         ("nt_load", C.c_uint32), ("store_policy", C.c_uint32), ("total_bytes", C.c_uint64),
+        ("plain_rows", C.c_uint32), ("reserved", C.c_uint32),
     ]
 
 

@@ -19,6 +19,12 @@ namespace mi355 {
 
 constexpr unsigned kWave = 64;
 
+// Division of a 32-bit n by an invariant d without a divide: with m =
+// magic_divisor(d) = ceil(2^64 / d), n / d == (n * m) >> 64 for all n < 2^32
+// (the error n * (m * d - 2^64) stays below 2^64).  d == 1 has no such m in 64
+// bits and is encoded as 0.
+inline uint64_t magic_divisor(uint32_t d) { return d > 1 ? ~0ull / d + 1 : 0; }
+
 // The workgroup whose work workgroup b does when a launch deals runs of `run`
 // neighbouring workgroups to each of the 8 XCDs: the hardware places workgroup
 // b on XCD b % 8, so XCD x takes workgroups [x * run, (x + 1) * run) of every
@@ -170,6 +176,15 @@ struct RectArgs {
   uint32_t n_waves;
   uint32_t xcd_run;   // as in CopyArgs
   uint32_t xcd_full;
+  // n / slots == div_magic(n, magic_slots) and n / rows == div_magic(n,
+  // magic_rows) for every 32-bit n (magic_divisor below).
+  uint64_t magic_slots;
+  uint64_t magic_rows;
+  // Not 0: every row starts at a 256-byte boundary of the destination, is a
+  // whole number of units long and lies a multiple of 4 bytes from its source,
+  // so that no unit has a head, a tail, a cut end or bytes to realign.
+  uint32_t plain_rows;
+  uint32_t pad;
 };
 
 // The same region copy for rows of up to about 1 KiB: every 16-byte slot of a

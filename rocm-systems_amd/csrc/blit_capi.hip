@@ -681,6 +681,7 @@ int mi355_blit_plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst
     out->slots = rp.args.slots;
     out->layers = rp.args.total_slots / (rp.args.slots * rp.args.rows);
     out->unroll = rp.unroll;
+    out->plain_rows = rp.args.plain_rows;
   }
   out->wg_size = rp.wg_size;
   out->grid = rp.grid;

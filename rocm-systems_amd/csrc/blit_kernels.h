@@ -666,17 +666,42 @@ __device__ __forceinline__ uint64_t row_units(uint64_t n_virtual, unsigned unit)
   return n_virtual > kRowOverflowVecs + unit ? (n_virtual - kRowOverflowVecs + unit - 1) / unit : 1;
 }
 
+// n / d for the d that magic is the magic_divisor of.
+__device__ __forceinline__ uint32_t div_magic(uint32_t n, uint64_t magic) {
+  return magic ? static_cast<uint32_t>(__umul64hi(n, magic)) : n;
+}
+
 template <int U, bool NTL, int NTS>
 __device__ __forceinline__ void rect_copy_body(const RectArgs& a) {
   constexpr unsigned kUnit = kWave * U;
   const unsigned lane = threadIdx.x & (kWave - 1);
   const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd_run, a.xcd_full);
   const uint64_t n_waves = a.n_waves;
+  if (a.plain_rows) {
+    // Rows of whole units, aligned like a linear copy's tiles: a unit is U
+    // loads and U stores per lane and nothing else.
+    for (uint64_t w = wave; w < a.total_slots; w += n_waves) {
+      const uint32_t slot = static_cast<uint32_t>(w);
+      const uint32_t line = div_magic(slot, a.magic_slots);
+      const uint32_t kq = slot - line * a.slots;
+      const uint32_t layer = div_magic(line, a.magic_rows);
+      const uint32_t y = line - layer * a.rows;
+      const uint64_t in_row = static_cast<uint64_t>(kq) * (kUnit * 16) + lane * 16;
+      const v4u_a4* sv = reinterpret_cast<const v4u_a4*>(a.src + layer * a.src_slice + y * a.src_pitch + in_row);
+      v4u* dv = reinterpret_cast<v4u*>(a.dst + layer * a.dst_slice + y * a.dst_pitch + in_row);
+      v4u x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) x[u] = ld_v4<NTL>(sv + u * kWave);
+#pragma unroll
+      for (int u = 0; u < U; ++u) st_v4<NTS>(dv + u * kWave, x[u]);
+    }
+    return;
+  }
   for (uint64_t w = wave; w < a.total_slots; w += n_waves) {
     const uint32_t slot = static_cast<uint32_t>(w);
-    const uint32_t line = slot / a.slots;  // row index through all layers
+    const uint32_t line = div_magic(slot, a.magic_slots);  // row index through all layers
     const uint32_t kq = slot - line * a.slots;
-    const uint32_t layer = line / a.rows;
+    const uint32_t layer = div_magic(line, a.magic_rows);
     const uint32_t y = line - layer * a.rows;
     BatchDesc row;
     row.dst = a.dst + layer * a.dst_slice + y * a.dst_pitch;

@@ -190,9 +190,9 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
 
   // Measured on MI355X, 1 GiB moved in rows of 4 KiB and of 128 KiB.  Rows whose
   // every store is a whole cache line (first row, pitches and width multiples
-  // of 128 bytes): one vector per lane, workgroups of 256, stores written
-  // through L2 like the linear copy's, 320-326 us (6.6-6.7 TB/s) against
-  // 333-341 us with the shape below.  Any other rows: two vectors per lane,
+  // of 128 bytes): one vector per lane, workgroups of 256 (of 64 for plain
+  // rows, below), stores written through L2 like the linear copy's, 320-326 us
+  // (6.6-6.7 TB/s) against 333-341 us with the shape below.  Any other rows: two vectors per lane,
   // workgroups of 128, non-temporal stores (written-through stores lose 8-15 %
   // there: the rows' cut ends are partial lines).
   uint32_t unroll = whole_lines ? 1 : 2;
@@ -214,6 +214,25 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
   if (total_slots > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   a.slots = static_cast<uint32_t>(slots);
   a.total_slots = static_cast<uint32_t>(total_slots);
+  a.magic_slots = magic_divisor(a.slots);
+  a.magic_rows = magic_divisor(a.rows);
+  // Rows that are tiled like a linear copy: they start at 256-byte boundaries
+  // of the destination, are whole units long and lie a multiple of 4 bytes
+  // from their source.  The kernel then skips everything a row's ends need.
+  const uint64_t unit_bytes = 1024ull * unroll;
+  const uintptr_t delta = reinterpret_cast<uintptr_t>(s0) - reinterpret_cast<uintptr_t>(d0);
+  a.plain_rows = reinterpret_cast<uintptr_t>(d0) % 256 == 0 && dp % 256 == 0 && (layers == 1 || ds % 256 == 0) &&
+                 width % unit_bytes == 0 && delta % 4 == 0 && sp % 4 == 0 && (layers == 1 || ss % 4 == 0);
+  // Plain rows in XCD runs want single-wave workgroups, like the linear copy.
+  // Measured on 17 shapes of 1 GiB, widths 2 KiB .. 1 MiB at pitches of 1.03 to
+  // 256 times the width: workgroups of 256 in launch order are up to 27 % behind
+  // the best shape found for a region (3 KiB rows at a 4 KiB pitch: 414 us
+  // against 324 us), single waves in launch order up to 20 %, single waves in
+  // runs of 576 units at most 12 % (8 KiB rows at a 16 KiB pitch, 361 us against
+  // 321 us) and within 2 % everywhere else.  Which shape wins for a given pitch
+  // follows the memory channels' interleave, not the kernel.
+  const bool plain_runs = a.plain_rows && out->total_bytes >= kXcdRunMinBytes;
+  if (plain_runs) default_wg = 64;
   out->wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size : default_wg;
   const uint64_t waves_per_wg = out->wg_size / 64;
   uint64_t wgs = (total_slots + waves_per_wg - 1) / waves_per_wg;
@@ -224,10 +243,11 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
   a.n_waves = static_cast<uint32_t>(wgs * waves_per_wg);
   // Units of rows that are not whole lines share source and destination lines
   // with their neighbours: runs of neighbouring units per XCD, as for the
-  // linear copy (131,065-byte rows 344 us against 361 us in launch order;
-  // whole-line rows lose, 347 us against 330 us).
+  // linear copy (131,065-byte rows 344 us against 361 us in launch order).
+  // Whole-line rows that are not plain go through the general path of the
+  // kernel, where runs lose (347 us against 330 us).
   uint32_t run = 0;
-  if (!whole_lines && out->total_bytes >= kXcdRunMinBytes)
+  if ((!whole_lines || plain_runs) && out->total_bytes >= kXcdRunMinBytes)
     run = static_cast<uint32_t>(kXcdRunBytes / (waves_per_wg * 1024 * unroll));
   out->xcd_run = plan_xcd_run(run, t);
   a.xcd_run = out->xcd_run;

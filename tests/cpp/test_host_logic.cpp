@@ -312,6 +312,23 @@ void one_batch_stage() {
   CHECK(batch_bound_chunks(1, 1ull << 62) == 0, "a bound beyond 32-bit record indices accepted");
 }
 
+// Division by an invariant through its magic number must be exact for every
+// 32-bit dividend: divisors and dividends at the extremes and at random.
+void one_magic_division() {
+  const uint32_t ds[] = {1, 2, 3, 5, 7, 255, 256, 257, 65535, 65536, 0x7fffffffu, 0x80000000u, 0xfffffffeu, 0xffffffffu,
+                         static_cast<uint32_t>(1 + below(0xffffffffull)), static_cast<uint32_t>(1 + below(100000))};
+  for (uint32_t d : ds) {
+    const uint64_t m = magic_divisor(d);
+    const uint32_t ns[] = {0, 1, d - 1, d, d + 1, 2 * d - 1, 2 * d, 0x7fffffffu, 0x80000000u, 0xfffffffeu, 0xffffffffu,
+                           static_cast<uint32_t>(below(1ull << 32)), static_cast<uint32_t>(below(1ull << 32)),
+                           0xffffffffu / d * d, 0xffffffffu / d * d - 1};
+    for (uint32_t n : ns) {
+      const uint32_t q = m ? static_cast<uint32_t>((static_cast<unsigned __int128>(n) * m) >> 64) : n;
+      CHECK(q == n / d, "%u / %u through the magic number gives %u", n, d, q);
+    }
+  }
+}
+
 // The XCD permutation of a launch: workgroups below xcd_full(grid, run) swap
 // places among themselves (a bijection), each XCD (b % 8) gets whole runs of
 // neighbouring workgroups in launch order, the rest keep their place.
@@ -347,6 +364,7 @@ int main(int argc, char** argv) {
     one_rect_plan();
     if (i % 8 == 0) one_batch_stage();
     if (i % 64 == 0) one_xcd_permutation();
+    if (i % 16 == 0) one_magic_division();
   }
   std::printf("%s: %ld cases each of copy, fill and region plans, %d failures\n", g_failures ? "FAILED" : "OK", cases,
               g_failures);

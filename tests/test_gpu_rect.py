@@ -156,6 +156,30 @@ def test_rect_permuted_launches_are_exact(capi, fresh_tuning, oracle, rand, xcd_
         assert p.kernel == capi.KERNEL_COPY_RECT and p.xcd_run == xcd_run
 
 
+@pytest.mark.parametrize("unroll", [1, 2, 4])
+def test_rect_plain_rows_are_exact(capi, fresh_tuning, oracle, rand, unroll):
+    """Rows tiled like a linear copy (256-byte aligned destination rows, whole
+    units, source a multiple of 4 bytes away) take the kernel's short path:
+    same bytes, under every launch shape, in launch order and in XCD runs, and
+    a region that misses one of the conditions takes the general path."""
+    blit = fresh_tuning
+    sshape, dshape = (2, 20, 8192), (2, 18, 12288)
+    ext, so, do = (4096, 15, 2), (1028, 3, 0), (512, 2, 0)
+    for wg, xcd_run, max_grid in ((64, 1, 0), (256, 3, 0), (128, 2, 37), (1024, 1, 0)):
+        blit.set_tuning(wg_size=wg, unroll=unroll, xcd_run=xcd_run, max_grid=max_grid)
+        p = run_rect_case(capi, blit, oracle, rand, sshape, dshape, ext, so, do, 0, 0, seed=0x7EC7CC00 + unroll)
+        assert p.kernel == capi.KERNEL_COPY_RECT and p.unroll == unroll
+    t = capi.Tuning(unroll=unroll)
+    st, plan = capi.plan_rect((1 << 40, 12288, 12288 * 18), do, (1 << 41, 8192, 8192 * 20), so, ext, t)
+    assert st == capi.SUCCESS and plan.plain_rows == 1 and plan.slots == 4096 // (1024 * unroll)
+    # one condition off at a time: destination x, source x, width
+    for so2, do2, ext2 in (((1028, 3, 0), (640, 2, 0), ext), ((1030, 3, 0), do, ext), (so, do, (4096 - 256, 15, 2))):
+        st, plan = capi.plan_rect((1 << 40, 12288, 12288 * 18), do2, (1 << 41, 8192, 8192 * 20), so2, ext2, t)
+        assert st == capi.SUCCESS and plan.plain_rows == 0
+        blit.set_tuning(unroll=unroll)
+        run_rect_case(capi, blit, oracle, rand, sshape, dshape, ext2, so2, do2, 0, 0, seed=0x7EC7DD00 + unroll)
+
+
 def test_rect_plan_shapes(capi, blit, oracle, rand):
     """What the launch record says: a rect kernel with one wave per 1 KiB of
     row for rows of whole cache lines, a linear copy when the region is one run."""

@@ -267,12 +267,22 @@ def test_plan_rect_slots_follow_row_alignment(capi_host):
     assert st == SUCCESS and p.nt_load == 1 and p.store_policy == capi_host.STORE_AGENT_WT   # whole lines
     st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4100, 1024, 1))
     assert st == SUCCESS and p.nt_load == 1 and p.store_policy == capi_host.STORE_NT
+    # rows tiled like a linear copy take the kernel's short path
+    st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 1024, 1))
+    assert st == SUCCESS and p.plain_rows == 1
+    st, p = capi_host.plan_rect((base_d, 8192, 0), (256, 0, 0), (base_s, 8192, 0), (4, 0, 0), (4096, 1024, 1))
+    assert st == SUCCESS and p.plain_rows == 1                     # 256-byte aligned destination, dword-aligned source
+    for d_x, s_x, w, dp in ((128, 0, 4096, 8192), (0, 2, 4096, 8192), (0, 0, 4096 + 128, 8192), (0, 0, 4096, 8192 + 128)):
+        st, p = capi_host.plan_rect((base_d, dp, 0), (d_x, 0, 0), (base_s, 8192, 0), (s_x, 0, 0), (w, 1024, 1))
+        assert st == SUCCESS and p.plain_rows == 0, (d_x, s_x, w, dp)
     # XCD runs: only from 64 MiB moved, and only where neighbouring waves share cache lines
     assert p.xcd_run == 0                                                                     # 4 MiB
     st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4100, 32768, 1))
     assert st == SUCCESS and (p.wg_size, p.unroll, p.xcd_run) == (128, 2, 144)               # 144 x 4 KiB
     st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 32768, 1))
-    assert st == SUCCESS and p.xcd_run == 0                                                   # whole lines
+    assert st == SUCCESS and (p.plain_rows, p.wg_size, p.xcd_run) == (1, 64, 576)              # tiled like a linear copy
+    st, p = capi_host.plan_rect((base_d, 8192, 0), (128, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 32768, 1))
+    assert st == SUCCESS and (p.plain_rows, p.wg_size, p.xcd_run) == (0, 256, 0)               # whole lines, not plain
     st, p = capi_host.plan_rect((base_d, 2048, 0), (9, 0, 0), (base_s, 2048, 0), (3, 0, 0), (1000, 1 << 20, 1))
     assert st == SUCCESS and (p.wg_size, p.xcd_run) == (64, 0)                                # waves share no line
     st, p = capi_host.plan_rect((base_d, 1024, 0), (0, 0, 0), (base_s, 1024, 0), (0, 0, 0), (520, 1 << 20, 1))

@@ -647,8 +647,7 @@ int mi355_aql_copy(mi355_aql_t* h, void* dst, const void* src, size_t bytes, con
   a.head = static_cast<uint32_t>(p.head_bytes);
   a.lead = p.lead_vecs;
   tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
-  a.xcd_run = p.xcd_run;
-  a.xcd_full = xcd_full(p.grid, p.xcd_run);
+  a.xcd = make_xcd_runs(p.grid, p.xcd_run);
   const uint32_t total = nb + 1;
   uint64_t index;
   {
@@ -693,8 +692,7 @@ int mi355_aql_fill32(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dword
   a.lead = p.lead_vecs;
   a.value = value;
   tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
-  a.xcd_run = p.xcd_run;
-  a.xcd_full = xcd_full(p.grid, p.xcd_run);
+  a.xcd = make_xcd_runs(p.grid, p.xcd_run);
   const uint32_t nb = barrier_packets(num_deps);
   const uint32_t total = nb + 1;
   uint64_t index;
@@ -774,7 +772,7 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
     if (v.split == split && v.nt_load == (streaming ? 1u : 0u) && v.store == p.store_policy) bk = &v.k;
   if (!bk) return MI355_BLIT_ERROR;
   BatchCopyArgs bc{h->records_dev, total_chunks, nullptr, static_cast<uint32_t>(waves_per_wg),
-                   static_cast<uint32_t>(wgs * waves_per_wg), batch_run, xcd_full(p.grid, batch_run)};
+                   static_cast<uint32_t>(wgs * waves_per_wg), make_xcd_runs(p.grid, batch_run)};
   h->last_plan = p;
 
   const uint32_t nb = barrier_packets(num_deps);
@@ -895,7 +893,7 @@ int mi355_aql_copy_batch_bounded(mi355_aql_t* h, const mi355_blit_desc_t* device
   if (!bk) return MI355_BLIT_ERROR;
   // the grid is sized for the bound; the kernel reads the number of records the device counted
   BatchCopyArgs bc{h->records_dev, capacity, h->chunk_start_dev + n, static_cast<uint32_t>(waves_per_wg),
-                   static_cast<uint32_t>(wgs * waves_per_wg), batch_run, xcd_full(p.grid, batch_run)};
+                   static_cast<uint32_t>(wgs * waves_per_wg), make_xcd_runs(p.grid, batch_run)};
   h->last_plan = p;
 
   const uint32_t nb = barrier_packets(num_deps);

@@ -25,15 +25,46 @@ constexpr unsigned kWave = 64;
 // bits and is encoded as 0.
 inline uint64_t magic_divisor(uint32_t d) { return d > 1 ? ~0ull / d + 1 : 0; }
 
-// The workgroup whose work workgroup b does when a launch deals runs of `run`
-// neighbouring workgroups to each of the 8 XCDs: the hardware places workgroup
-// b on XCD b % 8, so XCD x takes workgroups [x * run, (x + 1) * run) of every
-// round of 8 * run.  A permutation of [0, m) for every multiple m of 8 * run.
-MI355_HOST_DEVICE inline uint32_t xcd_workgroup(uint32_t b, uint32_t run) {
-  const uint32_t xcd = b & 7, j = b >> 3;
-  const uint32_t q = j / run;
-  return (q * 8 + xcd) * run + (j - q * run);
+MI355_HOST_DEVICE inline uint32_t div_magic(uint32_t n, uint64_t magic) {
+#ifdef __HIP_DEVICE_COMPILE__
+  return magic ? static_cast<uint32_t>(__umul64hi(n, magic)) : n;
+#else
+  return magic ? static_cast<uint32_t>((static_cast<unsigned __int128>(n) * magic) >> 64) : n;
+#endif
 }
+
+// XCD-aware launch order.  The hardware deals consecutive workgroups to the 8
+// XCDs in turn (workgroup b runs on XCD b % 8).  With run != 0, workgroup
+// b < full does the work of workgroup xcd_workgroup(b) instead, which gives
+// every XCD runs of `run` neighbouring workgroups: XCD x takes workgroups
+// [x * run, (x + 1) * run) of every round of 8 * run.  A permutation of
+// [0, full); full is a multiple of 8 * run and the workgroups from there on
+// keep their place.
+struct XcdRuns {
+  uint32_t run;    // workgroups per run; 0 = launch order
+  uint32_t full;   // workgroups that take part; 0 when run == 0
+  uint64_t magic;  // magic_divisor(run)
+};
+
+MI355_HOST_DEVICE inline uint32_t xcd_workgroup(uint32_t b, const XcdRuns& x) {
+  const uint32_t xcd = b & 7, j = b >> 3;
+  const uint32_t q = div_magic(j, x.magic);
+  return (q * 8 + xcd) * x.run + (j - q * x.run);
+}
+
+// The permutation of a launch of `grid` workgroups in runs of `run` (0 or 1:
+// launch order): whole rounds of 8 runs take part.
+inline XcdRuns make_xcd_runs(uint32_t grid, uint32_t run) {
+  XcdRuns x{0, 0, 0};
+  if (run > 1) {
+    const uint64_t round = 8ull * run;
+    x.run = run;
+    x.full = static_cast<uint32_t>(grid / round * round);
+    x.magic = magic_divisor(run);
+  }
+  return x;
+}
+
 constexpr unsigned kChunkVecs = 256;  // vectors of one batched-copy chunk: 4 KiB
 
 struct CopyArgs {
@@ -51,13 +82,7 @@ struct CopyArgs {
   // kernel arguments and can be dispatched from a hand-built AQL packet.
   uint32_t waves_per_wg;
   uint32_t n_waves;  // grid * waves_per_wg
-  // The hardware deals consecutive workgroups to the 8 XCDs in turn.  With
-  // xcd_run != 0, workgroup b < xcd_full does the work of workgroup
-  // xcd_workgroup(b) instead, which gives every XCD runs of xcd_run
-  // neighbouring workgroups (a permutation of [0, xcd_full), a multiple of
-  // 8 * xcd_run).
-  uint32_t xcd_run;
-  uint32_t xcd_full;
+  XcdRuns xcd;
 };
 
 struct FillArgs {
@@ -71,8 +96,7 @@ struct FillArgs {
   uint32_t edge_wave;
   uint32_t waves_per_wg;
   uint32_t n_waves;
-  uint32_t xcd_run;
-  uint32_t xcd_full;
+  XcdRuns xcd;
 };
 
 struct BatchDesc {
@@ -144,8 +168,7 @@ struct BatchCopyArgs {
   const uint32_t* total;
   uint32_t waves_per_wg;
   uint32_t n_waves;
-  uint32_t xcd_run;   // as in CopyArgs
-  uint32_t xcd_full;
+  XcdRuns xcd;
 };
 
 struct BatchStridedArgs {
@@ -174,8 +197,7 @@ struct RectArgs {
   uint32_t total_slots;  // rows * layers * slots
   uint32_t waves_per_wg;
   uint32_t n_waves;
-  uint32_t xcd_run;   // as in CopyArgs
-  uint32_t xcd_full;
+  XcdRuns xcd;
   // n / slots == div_magic(n, magic_slots) and n / rows == div_magic(n,
   // magic_rows) for every 32-bit n (magic_divisor below).
   uint64_t magic_slots;
@@ -205,8 +227,7 @@ struct RectNarrowArgs {
   uint32_t magic;    // ceil(2^16 / lanes_per_row): n / lanes_per_row == (n * magic) >> 16, n < 128
   uint32_t waves_per_wg;
   uint32_t n_waves;
-  uint32_t xcd_run;   // as in CopyArgs
-  uint32_t xcd_full;
+  XcdRuns xcd;
 };
 
 // Layout of amd_signal_t (inc/amd_hsa_signal.h, struct amd_signal_s).

@@ -407,8 +407,7 @@ int mi355_blit_copy(mi355_blit_t* h, void* dst, const void* src, size_t bytes, v
   a.head = static_cast<uint32_t>(p.head_bytes);
   a.lead = p.lead_vecs;
   set_tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
-  a.xcd_run = p.xcd_run;
-  a.xcd_full = xcd_full(p.grid, p.xcd_run);
+  a.xcd = make_xcd_runs(p.grid, p.xcd_run);
   hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
   hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
   BLIT_HIP(hipGetLastError());
@@ -436,8 +435,7 @@ int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwo
   a.lead = p.lead_vecs;
   a.value = value;
   set_tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
-  a.xcd_run = p.xcd_run;
-  a.xcd_full = xcd_full(p.grid, p.xcd_run);
+  a.xcd = make_xcd_runs(p.grid, p.xcd_run);
   hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
   hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
   BLIT_HIP(hipGetLastError());
@@ -553,7 +551,7 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
     batch_kernel_t k = select_batch_kernel(split, streaming, p.store_policy);
     if (!k) return MI355_BLIT_ERROR;
     BatchCopyArgs bc{h->records_dev, shape.total_chunks, nullptr, static_cast<uint32_t>(waves_per_wg),
-                     static_cast<uint32_t>(wgs * waves_per_wg), batch_run, xcd_full(p.grid, batch_run)};
+                     static_cast<uint32_t>(wgs * waves_per_wg), make_xcd_runs(p.grid, batch_run)};
     hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, bc);
   } else if (max_total_bytes) {
     // Device-resident descriptors whose total size the caller bounds: the
@@ -585,7 +583,7 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
     batch_kernel_t k = select_batch_kernel(kBatchSplit, streaming, p.store_policy);
     if (!k) return MI355_BLIT_ERROR;
     BatchCopyArgs bc{h->records_dev, shape.total_chunks, h->chunk_start_dev + n, static_cast<uint32_t>(waves_per_wg),
-                     static_cast<uint32_t>(wgs * waves_per_wg), batch_run, xcd_full(p.grid, batch_run)};
+                     static_cast<uint32_t>(wgs * waves_per_wg), make_xcd_runs(p.grid, batch_run)};
     hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, bc);
   } else {
     // Device-resident descriptors: the prefix sum runs on the device and, as

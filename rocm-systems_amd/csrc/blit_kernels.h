@@ -15,7 +15,7 @@
 //  * Where neighbouring tiles share cache lines and the transfer is large, the
 //    host asks for the launch to be permuted so that each of the 8 XCDs (each
 //    with its own L2) works through runs of neighbouring workgroups' tiles
-//    (xcd_run / xcd_full in the argument blocks, xcd_workgroup in blit_args.h):
+//    (XcdRuns in the argument blocks, xcd_workgroup in blit_args.h):
 //    the shared lines then meet in one L2.
 //  * Large transfers bypass the caches: loads carry nt, stores are written
 //    through L2 (sc1 / sc0 sc1), chosen per size by the host.
@@ -234,18 +234,18 @@ __device__ __forceinline__ uint64_t global_wave(unsigned waves_per_wg) {
 }
 
 // global_wave() of a launch whose workgroups take their work in runs per XCD
-// (xcd_workgroup): workgroups below xcd_full swap places among themselves, the
-// others keep theirs.  xcd_full == 0: launch order.
-__device__ __forceinline__ uint64_t global_wave_xcd(unsigned waves_per_wg, uint32_t xcd_run, uint32_t xcd_full) {
+// (xcd_workgroup): workgroups below x.full swap places among themselves, the
+// others keep theirs.  x.full == 0: launch order.
+__device__ __forceinline__ uint64_t global_wave_xcd(unsigned waves_per_wg, const XcdRuns& x) {
   uint32_t wg = blockIdx.x;
-  if (wg < xcd_full) wg = xcd_workgroup(wg, xcd_run);
+  if (wg < x.full) wg = xcd_workgroup(wg, x);
   return __builtin_amdgcn_readfirstlane(wg * waves_per_wg + threadIdx.x / kWave);
 }
 
 template <int U, bool NTL, int NTS, bool SHIFT>
 __device__ __forceinline__ void copy_body(const CopyArgs& a) {
   const unsigned lane = threadIdx.x & (kWave - 1);
-  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd_run, a.xcd_full);
+  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd);
   const uint64_t n_waves = a.n_waves;
   const uint8_t* sb = a.src + a.head;
   const unsigned r = SHIFT ? static_cast<unsigned>(reinterpret_cast<uintptr_t>(sb) & 3) : 0;
@@ -258,7 +258,7 @@ __device__ __forceinline__ void copy_body(const CopyArgs& a) {
 template <int U, int NTS>
 __device__ __forceinline__ void fill_body(const FillArgs& a) {
   const unsigned lane = threadIdx.x & (kWave - 1);
-  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd_run, a.xcd_full);
+  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd);
   const uint64_t n_waves = a.n_waves;
   const v4u val = {a.value, a.value, a.value, a.value};
   constexpr uint64_t kTile = kWave * U;
@@ -594,7 +594,7 @@ __device__ __forceinline__ void batch_copy_records_body(const BatchCopyArgs& a) 
     if (counted < total_chunks) total_chunks = counted;
   }
   const unsigned lane = threadIdx.x & (kWave - 1);
-  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd_run, a.xcd_full);
+  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd);
   const uint64_t n_waves = a.n_waves;
   for (uint64_t w = wave; w < total_chunks * SPLIT; w += n_waves) {
     const ChunkRecord rec = load_record(records + w / SPLIT);
@@ -666,16 +666,11 @@ __device__ __forceinline__ uint64_t row_units(uint64_t n_virtual, unsigned unit)
   return n_virtual > kRowOverflowVecs + unit ? (n_virtual - kRowOverflowVecs + unit - 1) / unit : 1;
 }
 
-// n / d for the d that magic is the magic_divisor of.
-__device__ __forceinline__ uint32_t div_magic(uint32_t n, uint64_t magic) {
-  return magic ? static_cast<uint32_t>(__umul64hi(n, magic)) : n;
-}
-
 template <int U, bool NTL, int NTS>
 __device__ __forceinline__ void rect_copy_body(const RectArgs& a) {
   constexpr unsigned kUnit = kWave * U;
   const unsigned lane = threadIdx.x & (kWave - 1);
-  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd_run, a.xcd_full);
+  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd);
   const uint64_t n_waves = a.n_waves;
   if (a.plain_rows) {
     // Rows of whole units, aligned like a linear copy's tiles: a unit is U
@@ -800,7 +795,7 @@ __device__ __forceinline__ void copy_partial_slot(uintptr_t slot, unsigned off, 
 template <bool NTL, int NTS>
 __device__ __forceinline__ void rect_narrow_body(const RectNarrowArgs& a) {
   const unsigned lane = threadIdx.x & (kWave - 1);
-  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd_run, a.xcd_full);
+  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd);
   const uint32_t lpr = a.lanes_per_row;
   const uint64_t total = static_cast<uint64_t>(a.lines) * lpr;
   const uint64_t n_groups = (total + kWave - 1) / kWave;

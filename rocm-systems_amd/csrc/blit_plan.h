@@ -107,14 +107,6 @@ inline uint32_t batch_xcd_run(uint64_t total_bytes, uint32_t split, uint32_t wav
   return plan_xcd_run(total_bytes >= kXcdRunMinBytes ? kBatchXcdRunChunks * split / waves_per_wg : 0, t);
 }
 
-// Workgroups of a launch of `grid` that the XCD permutation covers: whole
-// rounds of 8 runs; the rest keep their place.
-inline uint32_t xcd_full(uint32_t grid, uint32_t run) {
-  if (run <= 1) return 0;
-  const uint64_t round = 8ull * run;
-  return static_cast<uint32_t>(grid / round * round);
-}
-
 inline void apply_launch_shape(mi355_blit_plan_t* p, const SizeClass& cls, uint32_t num_cus,
                                const mi355_blit_tuning_t* t) {
   (void)num_cus;

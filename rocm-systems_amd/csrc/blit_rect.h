@@ -183,8 +183,7 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
       if (run < 32) run = 32;
     }
     out->xcd_run = plan_xcd_run(run, t);
-    n.xcd_run = out->xcd_run;
-    n.xcd_full = xcd_full(out->grid, out->xcd_run);
+    n.xcd = make_xcd_runs(out->grid, out->xcd_run);
     return MI355_BLIT_SUCCESS;
   }
 
@@ -250,8 +249,7 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
   if ((!whole_lines || plain_runs) && out->total_bytes >= kXcdRunMinBytes)
     run = static_cast<uint32_t>(kXcdRunBytes / (waves_per_wg * 1024 * unroll));
   out->xcd_run = plan_xcd_run(run, t);
-  a.xcd_run = out->xcd_run;
-  a.xcd_full = xcd_full(out->grid, out->xcd_run);
+  a.xcd = make_xcd_runs(out->grid, out->xcd_run);
   return MI355_BLIT_SUCCESS;
 }
 

@@ -323,25 +323,27 @@ void one_magic_division() {
                            static_cast<uint32_t>(below(1ull << 32)), static_cast<uint32_t>(below(1ull << 32)),
                            0xffffffffu / d * d, 0xffffffffu / d * d - 1};
     for (uint32_t n : ns) {
-      const uint32_t q = m ? static_cast<uint32_t>((static_cast<unsigned __int128>(n) * m) >> 64) : n;
+      const uint32_t q = div_magic(n, m);
       CHECK(q == n / d, "%u / %u through the magic number gives %u", n, d, q);
     }
   }
 }
 
-// The XCD permutation of a launch: workgroups below xcd_full(grid, run) swap
+// The XCD permutation of a launch: workgroups below make_xcd_runs(grid, run).full swap
 // places among themselves (a bijection), each XCD (b % 8) gets whole runs of
 // neighbouring workgroups in launch order, the rest keep their place.
 void one_xcd_permutation() {
   const uint32_t run = 2 + static_cast<uint32_t>(below(700));
   const uint32_t grid = static_cast<uint32_t>(below(40000));
-  const uint32_t full = xcd_full(grid, run);
-  CHECK(full <= grid && full % (8 * run) == 0 && grid - full < 8 * run, "xcd_full(%u, %u) = %u", grid, run, full);
-  CHECK(xcd_full(grid, 0) == 0 && xcd_full(grid, 1) == 0, "no permutation without a run");
+  const XcdRuns x = make_xcd_runs(grid, run);
+  const uint32_t full = x.full;
+  CHECK(x.run == run && full <= grid && full % (8 * run) == 0 && grid - full < 8 * run, "runs of %u in a grid of %u: %u take part", run, grid, full);
+  CHECK(make_xcd_runs(grid, 0).full == 0 && make_xcd_runs(grid, 1).full == 0 && make_xcd_runs(grid, 1).run == 0,
+        "no permutation without a run");
   std::vector<uint8_t> seen(full, 0);
   std::vector<uint32_t> last(8, 0);
   for (uint32_t b = 0; b < full; ++b) {
-    const uint32_t w = xcd_workgroup(b, run);
+    const uint32_t w = xcd_workgroup(b, x);
     CHECK(w < full && !seen[w], "workgroup %u -> %u (run %u) out of range or taken twice", b, w, run);
     if (w < full) seen[w] = 1;
     // within a round the work of XCD x is [x * run, (x + 1) * run), taken in launch order

@@ -715,6 +715,26 @@ __device__ __forceinline__ void rect_copy_body(const RectArgs& a) {
     const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(sb)) & 3;
     const v4u_a4* sv = reinterpret_cast<const v4u_a4*>(sb - r) - sh.lead;
     v4u* dv = reinterpret_cast<v4u*>(row.dst + sh.head) - sh.lead;
+    if (kq != 0 && !last) {
+      // A unit inside its row (most are, in a wide row): it lies above the
+      // row's lead and head, every lane has its U vectors, and it is moved
+      // like a tile of the linear copy.
+      const uint64_t base = v0 + lane;
+      v4u x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) x[u] = ld_v4<NTL>(sv + base + u * kWave);
+      // lane 0 fetches the dword behind the unit: with r != 0 it holds the
+      // last r bytes the unit needs, and the row goes on behind it
+      unsigned e = 0;
+      if (r && lane == 0) e = ld_u32<NTL>(reinterpret_cast<const unsigned*>(sv + v0 + kUnit));
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const unsigned nxt = (u + 1 < U) ? x[u + 1 < U ? u + 1 : u].x : e;
+        const unsigned w4 = wave_rotate_down1(lane == 0 ? nxt : x[u].x);
+        st_v4<NTS>(dv + base + u * kWave, realign(x[u], w4, r));
+      }
+      continue;
+    }
     // U vectors per lane, and one more for the overflow of a row's last unit
     v4u x[U + 1];
 #pragma unroll

@@ -164,6 +164,32 @@ int mi355_hsa_amd_memory_async_copy(mi355_aql_t* h, void* dst, const void* src, 
                                     uint32_t num_dep_signals, const uint64_t* dep_signals,
                                     uint64_t completion_signal);
 
+/* hsa_amd_memory_async_copy_on_engine for copies within this GPU's memory
+ * (core/runtime/hsa_ext_amd.cpp:296-339, Runtime::CopyMemoryOnEngine
+ * runtime.cpp:585-601, GpuAgent::DmaCopyOnEngine amd_gpu_agent.cpp:1110-1179).
+ * The argument checks of the asynchronous copy; size 0 -> SUCCESS; engine_id
+ * (hsa_amd_sdma_engine_id_t) must be exactly one bit and name an engine the GPU
+ * has (HSA_AMD_AGENT_INFO_NUM_SDMA_ENG + ..._XGMI_ENG), else INVALID_ARGUMENT.
+ * Within one GPU the reference sets the named engine aside for the blit kernel
+ * unless force_copy_on_sdma: so does this.  With force_copy_on_sdma the copy
+ * would need an SDMA engine, which this library does not drive ->
+ * OUT_OF_RESOURCES. */
+int mi355_hsa_amd_memory_async_copy_on_engine(mi355_aql_t* h, void* dst, const void* src, size_t size,
+                                              uint32_t num_dep_signals, const uint64_t* dep_signals,
+                                              uint64_t completion_signal, uint32_t engine_id,
+                                              int force_copy_on_sdma);
+
+/* hsa_amd_memory_copy_engine_status between this GPU and the host
+ * (core/runtime/hsa_ext_amd.cpp:341-352, Runtime::CopyMemoryStatus
+ * runtime.cpp:603-613, GpuAgent::DmaCopyStatus amd_gpu_agent.cpp:1181-1243).
+ * dst_is_gpu / src_is_gpu say which side is this GPU; both or neither ->
+ * HSA_STATUS_ERROR_INVALID_AGENT (0x1004) as for equal agents.  The mask is
+ * what the reference answers on an agent whose SDMA engines are all unused
+ * (this library never occupies one): the H2D and the D2H engine and every
+ * xGMI engine; OUT_OF_RESOURCES with a mask of 0 on a GPU without engines. */
+int mi355_hsa_amd_memory_copy_engine_status(mi355_aql_t* h, int dst_is_gpu, int src_is_gpu,
+                                            uint32_t* engine_ids_mask);
+
 /* hsa_amd_memory_async_copy_rect for copies this GPU executes
  * (core/runtime/hsa_ext_amd.cpp:367-410): NULL pointers, a dependency count
  * that disagrees with the array pointer, a zero completion signal or

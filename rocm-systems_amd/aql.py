@@ -34,6 +34,9 @@ SIGNATURES = {
     "mi355_hsa_amd_memory_fill": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t]),
     "mi355_hsa_amd_memory_async_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint32,
                                                   _U64P, C.c_uint64]),
+    "mi355_hsa_amd_memory_async_copy_on_engine": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint32,
+                                                            _U64P, C.c_uint64, C.c_uint32, C.c_int]),
+    "mi355_hsa_amd_memory_copy_engine_status": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_uint32)]),
     "mi355_hsa_amd_memory_async_copy_rect": (C.c_int, [C.c_void_p, C.POINTER(PitchedPtr), C.POINTER(Dim3),
                                                        C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(Dim3),
                                                        C.c_int, C.c_uint32, _U64P, C.c_uint64]),
@@ -159,6 +162,19 @@ class AqlBlit:
     def hsa_amd_memory_async_copy(self, dst, src, nbytes, deps=None, completion=0):
         arr, n = _deps(deps)
         return self.lib.mi355_hsa_amd_memory_async_copy(self.handle, dst, src, nbytes, n, arr, completion)
+
+    def hsa_amd_memory_async_copy_on_engine(self, dst, src, nbytes, engine_id, force_copy_on_sdma=False, deps=None,
+                                            completion=0):
+        arr, n = _deps(deps)
+        return self.lib.mi355_hsa_amd_memory_async_copy_on_engine(self.handle, dst, src, nbytes, n, arr, completion,
+                                                                  engine_id, 1 if force_copy_on_sdma else 0)
+
+    def hsa_amd_memory_copy_engine_status(self, dst_is_gpu, src_is_gpu):
+        """(status, engine_ids_mask)"""
+        mask = C.c_uint32(0xdeadbeef)
+        st = self.lib.mi355_hsa_amd_memory_copy_engine_status(self.handle, 1 if dst_is_gpu else 0,
+                                                              1 if src_is_gpu else 0, C.byref(mask))
+        return st, mask.value
 
     def hsa_amd_memory_async_copy_rect(self, dst, dst_offset, src, src_offset, extent, direction=3, deps=None,
                                        completion=0):

@@ -168,3 +168,84 @@ def test_async_copy_api_edge_and_completion(eng, signals, oracle, rand, torch_cu
     assert np.array_equal(dst.cpu().numpy(), want)
     signals.destroy(done)
     signals.destroy(dep)
+
+
+def _stock_agents():
+    """(hsa library, GPU agent handles, CPU agent handles) of the runtime the process runs on."""
+    hsa = C.CDLL("libhsa-runtime64.so.1")
+    gpus, cpus = [], []
+    CB = C.CFUNCTYPE(C.c_int, C.c_uint64, C.c_void_p)
+
+    def visit(agent, _):
+        dev = C.c_int(-1)
+        hsa.hsa_agent_get_info(C.c_uint64(agent), 17, C.byref(dev))     # HSA_AGENT_INFO_DEVICE
+        (gpus if dev.value == 1 else cpus).append(agent)                 # HSA_DEVICE_TYPE_GPU == 1
+        return 0
+    cb = CB(visit)
+    hsa.hsa_agent_get_info.argtypes = [C.c_uint64, C.c_int, C.c_void_p]
+    hsa.hsa_iterate_agents.argtypes = [CB, C.c_void_p]
+    assert hsa.hsa_iterate_agents(cb, None) == 0
+    return hsa, gpus, cpus
+
+
+def test_copy_engine_status_matches_the_installed_runtime(eng, torch_cuda):
+    """hsa_amd_memory_copy_engine_status (hsa_ext_amd.cpp:341-352, runtime.cpp:603-613,
+    amd_gpu_agent.cpp:1181-1243): the same statuses and, with no copy in flight,
+    the same mask of free engines as the runtime itself reports for this GPU."""
+    torch_cuda.cuda.synchronize()
+    inv_agent = 0x1004
+    assert eng.hsa_amd_memory_copy_engine_status(True, True) == (inv_agent, 0)
+    assert eng.hsa_amd_memory_copy_engine_status(False, False) == (inv_agent, 0)
+    assert eng.lib.mi355_hsa_amd_memory_copy_engine_status(eng.handle, 1, 0, None) == 0x1001
+    h2d = eng.hsa_amd_memory_copy_engine_status(True, False)
+    d2h = eng.hsa_amd_memory_copy_engine_status(False, True)
+    assert h2d == d2h
+    try:
+        hsa, gpus, cpus = _stock_agents()
+        f = hsa.hsa_amd_memory_copy_engine_status
+    except (OSError, AttributeError) as e:
+        pytest.skip("no loadable libhsa-runtime64 with the entry point: %s" % e)
+    f.argtypes = [C.c_uint64, C.c_uint64, C.POINTER(C.c_uint32)]
+    gpu = eng.lib.mi355_aql_gpu_agent(eng.handle)
+    assert gpu in gpus and cpus
+    mask = C.c_uint32(0)
+    st = f(gpu, cpus[0], C.byref(mask))                                   # destination GPU, source host
+    assert (st, mask.value) == h2d
+    st = f(cpus[0], gpu, C.byref(mask))
+    assert (st, mask.value) == d2h
+    assert f(gpu, gpu, C.byref(mask)) == inv_agent
+
+
+def test_async_copy_on_engine(eng, signals, oracle, rand, torch_cuda):
+    """hsa_amd_memory_async_copy_on_engine within the GPU (hsa_ext_amd.cpp:296-339,
+    runtime.cpp:585-601, amd_gpu_agent.cpp:1110-1179): the engine must be one
+    existing engine, and the copy then runs on the blit kernel all the same."""
+    torch = torch_cuda
+    n = MIB + 77
+    payload = rand(n, 0xB1170009)
+    src = torch.from_numpy(payload).to("cuda:0")
+    dst = torch.full((n + 2 * GUARD,), 0xEE, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    inv = 0x1001
+    done = signals.create(1)
+    st, free_mask = eng.hsa_amd_memory_copy_engine_status(True, False)
+    assert st == 0 and free_mask & 1
+    d, s = dst.data_ptr() + GUARD, src.data_ptr()
+    f = eng.hsa_amd_memory_async_copy_on_engine
+    assert f(None, s, n, 1, completion=done) == inv
+    assert f(d, None, n, 1, completion=done) == inv
+    assert f(d, s, n, 1, completion=0) == inv
+    assert f(d, s, n, 0, completion=done) == inv                    # no engine named
+    assert f(d, s, n, 3, completion=done) == inv                    # two engines named
+    assert f(d, s, n, 1 << 31, completion=done) == inv              # an engine the GPU does not have
+    assert f(d, s, 0, 3, completion=done) == 0                      # size 0 succeeds before the engine is looked at
+    assert f(d, s, n, 1, force_copy_on_sdma=True, completion=done) == 0x1008   # no SDMA behind this library
+    assert signals.load(done) == 1
+    torch.cuda.synchronize()
+    assert bool((dst == 0xEE).all())
+    assert f(d, s, n, 1, completion=done) == 0
+    signals.wait_below_one(done, active=False)
+    want = _host(n + 2 * GUARD)
+    oracle.oracle_copy(want.ctypes.data + GUARD, payload.ctypes.data, n)
+    assert np.array_equal(dst.cpu().numpy(), want)
+    signals.destroy(done)

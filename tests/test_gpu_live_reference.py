@@ -5,7 +5,8 @@ pointers go through AMD::BlitKernel and the CopyAligned / CopyMisaligned / Fill
 shaders (core/runtime/runtime.cpp:513, amd_gpu_agent.cpp:951, 1285).  Both are
 given the same seeded inputs, misaligned offsets and odd lengths included
 (cases no test of the reference holds a vector for), and must leave the same
-bytes, which must also be the CPU oracle's."""
+bytes, which must also be the CPU oracle's.  Its hsa_amd_memory_async_copy_rect
+(SDMA engines) is the reference for the region copy in the same way."""
 import ctypes as C
 
 import numpy as np
@@ -112,3 +113,64 @@ def test_api_edge_answers_match_the_installed_runtime(capi, blit, stock, torch_c
     assert stock.hsa_amd_memory_fill(p + 2, 1, 4) == blit.fill32(p + 2, 1, 4) == capi.ERROR_INVALID_ARGUMENT
     assert stock.hsa_amd_memory_fill(p, 1, 0) == blit.fill32(p, 1, 0) == capi.SUCCESS
     assert blit.synchronize() == capi.SUCCESS
+
+
+RECT_CASES = [
+    # source shape (layers, rows, pitch), destination shape, extent (x bytes, y, z), source offset, destination offset:
+    # bases, pitches, offsets and widths multiples of 4, which is all the reference's SDMA packet accepts
+    ((1, 16, 512), (1, 12, 1024), (256, 7, 1), (64, 2, 0), (128, 3, 0)),
+    ((4, 9, 1032), (5, 11, 1500), (1000, 5, 3), (32, 4, 1), (496, 6, 2)),
+    ((1, 64, 131072), (1, 64, 131072), (65536, 64, 1), (0, 0, 0), (65536, 0, 0)),
+    ((3, 300, 516), (3, 310, 400), (332, 250, 3), (12, 20, 0), (4, 31, 0)),
+    ((2, 40, 12000), (2, 37, 11004), (9000, 31, 2), (8, 3, 0), (1000, 2, 0)),
+]
+
+
+@pytest.mark.parametrize("case", range(len(RECT_CASES)))
+def test_rect_copy_leaves_the_bytes_the_installed_runtime_leaves(capi, blit, oracle, rand, torch_cuda, pkg, case):
+    """hsa_amd_memory_async_copy_rect of the installed runtime (SDMA engines:
+    amd_gpu_agent.cpp:1255-1283, amd_blit_sdma.cpp:564-636) beside this engine's
+    shader on the same seeded surfaces: both destination surfaces, everything
+    outside the region included, must be equal, and equal to the oracle's.  The
+    reference's tests hold no vector for region copies; this is the check
+    against its own implementation."""
+    from conftest import PitchedPtr, Dim3, oracle_rect
+    torch = torch_cuda
+    try:
+        hsa = C.CDLL("libhsa-runtime64.so.1")
+        f = hsa.hsa_amd_memory_async_copy_rect
+    except (OSError, AttributeError) as e:
+        pytest.skip("no loadable libhsa-runtime64 with the entry point: %s" % e)
+    f.restype = C.c_int
+    f.argtypes = [C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(Dim3),
+                  C.c_uint64, C.c_int, C.c_uint32, C.c_void_p, C.c_uint64]
+    sshape, dshape, ext, so, do = RECT_CASES[case]
+    src_h = rand(int(np.prod(sshape)), 0x11FE7000 + case)
+    src = torch.from_numpy(src_h).to("cuda:0")
+    ours = torch.full((int(np.prod(dshape)),), GUARD_BYTE, dtype=torch.uint8, device="cuda:0")
+    theirs = torch.full((int(np.prod(dshape)),), GUARD_BYTE, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    assert src.data_ptr() % 4 == 0 and ours.data_ptr() % 4 == 0 and theirs.data_ptr() % 4 == 0
+    sp = (src.data_ptr(), sshape[2], sshape[1] * sshape[2])
+    signals = pkg.aql.HsaSignals()
+    done = signals.create(1)
+    # the GPU agent of the installed runtime: the one that owns the destination
+    aql = pkg.aql.AqlBlit(0)
+    gpu = aql.lib.mi355_aql_gpu_agent(aql.handle)
+    aql.close()
+    dp_t = (theirs.data_ptr(), dshape[2], dshape[1] * dshape[2])
+    st = f(PitchedPtr(*dp_t), Dim3(*do), PitchedPtr(*sp), Dim3(*so), Dim3(*ext), gpu, 3, 0, None, done)
+    if st != 0:
+        signals.destroy(done)
+        pytest.skip("the installed runtime has no engine for region copies here: status 0x%x" % st)
+    signals.wait_below_one(done, active=False)
+    signals.destroy(done)
+    dp_o = (ours.data_ptr(), dshape[2], dshape[1] * dshape[2])
+    assert blit.copy_rect(dp_o, do, sp, so, ext) == capi.SUCCESS
+    assert blit.synchronize() == capi.SUCCESS
+    torch.cuda.synchronize()
+    got, ref = ours.cpu().numpy(), theirs.cpu().numpy()
+    assert np.array_equal(got, ref), "differs from the installed runtime's region copy"
+    want = np.full(got.size, GUARD_BYTE, dtype=np.uint8)
+    oracle_rect(oracle, (want.ctypes.data,) + dp_o[1:], do, (src_h.ctypes.data,) + sp[1:], so, ext)
+    assert np.array_equal(ref, want), "the installed runtime's region copy differs from the oracle"

@@ -420,8 +420,48 @@ def reference_gpu_path(r):
     t = best(lambda: hsa.hsa_memory_copy(D, S, MIB), 200)
     if t:
         out["copy_1MiB_us"] = round(t * 1e6, 2)
-    out["how"] = "blocking hsa_memory_copy / hsa_amd_memory_fill of the loaded libhsa-runtime64, host clock, best of n"
+    rect = reference_rect(r, hsa, S, D)
+    if rect:
+        out["rect_4096x128KiB_gbs"] = rect
+    out["how"] = ("blocking hsa_memory_copy / hsa_amd_memory_fill of the loaded libhsa-runtime64, host clock, best of n; "
+                  "region copy: hsa_amd_memory_async_copy_rect (SDMA engines), submit to completion signal")
     return out or None
+
+
+def reference_rect(r, hsa, S, D):
+    """The reference's region copy (SDMA engines, amd_gpu_agent.cpp:1255-1283):
+    4096 rows of 128 KiB out of 256 KiB-pitch surfaces inside the 1 GiB
+    buffers, device to device; GB/s of bytes read plus written."""
+    try:
+        import __graft_entry__ as entry
+        f = hsa.hsa_amd_memory_async_copy_rect
+        aql = entry.load_package().aql
+        sig = aql.HsaSignals()
+        eng = aql.AqlBlit(0)
+        gpu = eng.lib.mi355_aql_gpu_agent(eng.handle)
+        eng.close()
+    except (OSError, AttributeError, RuntimeError):
+        return None
+    capi = r.capi
+    f.restype = C.c_int
+    f.argtypes = [C.POINTER(capi.PitchedPtr), C.POINTER(capi.Dim3), C.POINTER(capi.PitchedPtr), C.POINTER(capi.Dim3),
+                  C.POINTER(capi.Dim3), C.c_uint64, C.c_int, C.c_uint32, C.c_void_p, C.c_uint64]
+    rows, width, pitch = 4096, 128 * 1024, 256 * 1024
+    sp, dp = capi.PitchedPtr(S, pitch, rows * pitch), capi.PitchedPtr(D, pitch, rows * pitch)
+    zero, ext = capi.Dim3(0, 0, 0), capi.Dim3(width, rows, 1)
+    done = sig.create(1)
+    best = None
+    for _ in range(4):
+        sig.store(done, 1)
+        t0 = time.perf_counter()
+        if f(dp, zero, sp, zero, ext, gpu, 3, 0, None, done) != 0:   # 3 = hsaDeviceToDevice
+            best = None
+            break
+        sig.wait_below_one(done)
+        t = time.perf_counter() - t0
+        best = t if best is None else min(best, t)
+    sig.destroy(done)
+    return round(2 * rows * width / best / 1e9, 1) if best else None
 
 
 def cpu_baseline(ora, budget_s):

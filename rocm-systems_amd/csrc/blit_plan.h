@@ -39,7 +39,7 @@ struct SizeClass {
 // loads non-temporal, stores written through L2.
 //
 // The hardware deals consecutive workgroups to the 8 XCDs in turn, each XCD
-// with an L2 of its own.  From about 100 MiB on it pays to permute the launch
+// with an L2 of its own.  From 50-80 MiB on it pays to permute the launch
 // so that each XCD works through runs of neighbouring tiles (xcd_run
 // workgroups, 576 KiB): a source line that two tiles share (tiles are anchored
 // at the destination's 256-byte boundaries, so they do whenever source and
@@ -56,7 +56,9 @@ struct SizeClass {
 // last-level cache holds most of the transfer, 59 us against 66 us.  A byte
 // offset adds one dword fetch per tile (the bytes that spill past the last
 // lane), which 2 KiB tiles amortise best; its stores are written through while
-// the last-level cache absorbs them and non-temporal beyond.  Fills at one
+// the 256 MiB last-level cache absorbs them and non-temporal beyond (256 MiB:
+// 61 us against 79 us, 288 MiB: 93 us against 89 us).  The thresholds are where
+// the shapes cross in a sweep in steps of 16-32 MiB.  Fills at one
 // wave per workgroup are bound by the dispatcher's workgroup rate and want
 // 4-wave workgroups.  Last match wins.
 constexpr uint32_t kXcdRunBytes = 576u << 10;
@@ -70,13 +72,13 @@ constexpr uint32_t kBatchXcdRunChunks = 528;
 constexpr SizeClass kCopyClasses[] = {      // (src - dst) % 4 == 0
     {0, 256, 1, 0, MI355_BLIT_STORE_CACHED, 0},
     {4ull << 20, 256, 1, 1, MI355_BLIT_STORE_AGENT_WT, 0},
-    {128ull << 20, 64, 1, 1, MI355_BLIT_STORE_AGENT_WT, kXcdRunBytes},
+    {80ull << 20, 64, 1, 1, MI355_BLIT_STORE_AGENT_WT, kXcdRunBytes},
 };
 constexpr SizeClass kCopyRealignClasses[] = {  // (src - dst) % 4 != 0
     {0, 512, 1, 0, MI355_BLIT_STORE_CACHED, 0},
     {4ull << 20, 256, 2, 1, MI355_BLIT_STORE_AGENT_WT, 0},
-    {64ull << 20, 64, 2, 1, MI355_BLIT_STORE_AGENT_WT, kXcdRunBytes},
-    {320ull << 20, 64, 2, 1, MI355_BLIT_STORE_NT, kXcdRunBytes},
+    {48ull << 20, 64, 2, 1, MI355_BLIT_STORE_AGENT_WT, kXcdRunBytes},
+    {272ull << 20, 64, 2, 1, MI355_BLIT_STORE_NT, kXcdRunBytes},
 };
 constexpr SizeClass kFillClasses[] = {
     {0, 256, 1, 0, MI355_BLIT_STORE_CACHED, 0},

@@ -135,12 +135,14 @@ def test_plan_copy_shapes_by_size_and_offset(capi_host):
     for off in (0, 4, 64):                                   # dword-aligned to one another
         assert shape(off, MIB) == (256, 1, 0, cached, 0)
         assert shape(off, 64 * MIB) == (256, 1, 1, wt, 0)
-        assert shape(off, 128 * MIB) == (64, 1, 1, wt, 576)     # 576 tiles of 1 KiB
+        assert shape(off, 80 * MIB) == (64, 1, 1, wt, 576)      # 576 tiles of 1 KiB
         assert shape(off, 1 << 30) == (64, 1, 1, wt, 576)
     for off in (1, 3, 6):                                    # a byte offset: the realigning kernel
         assert shape(off, MIB) == (512, 1, 0, cached, 0)
         assert shape(off, 16 * MIB) == (256, 2, 1, wt, 0)
-        assert shape(off, 64 * MIB) == (64, 2, 1, wt, 288)      # 288 tiles of 2 KiB
+        assert shape(off, 48 * MIB) == (64, 2, 1, wt, 288)      # 288 tiles of 2 KiB
+        assert shape(off, 256 * MIB) == (64, 2, 1, wt, 288)     # the last-level cache still absorbs the stores
+        assert shape(off, 272 * MIB) == (64, 2, 1, nt, 288)
         assert shape(off, 1 << 30) == (64, 2, 1, nt, 288)
     # the run follows the workgroup the tuning asks for; 1 means launch order
     st, p = capi_host.plan_copy(dst, 0x7e0000000000, 1 << 30, 256, capi_host.Tuning(wg_size=256))

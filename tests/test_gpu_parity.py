@@ -451,7 +451,7 @@ def test_permuted_launches_are_exact(capi, fresh_tuning, oracle, arenas, xcd_run
 
 def test_large_copies_with_the_heuristic_runs(capi, blit, oracle, rand, torch_cuda):
     """At the sizes where the heuristics permute the launch by themselves
-    (from 64 MiB with a byte offset, from 128 MiB without): every byte and the
+    (from 48 MiB with a byte offset, from 80 MiB without): every byte and the
     guards against the oracle."""
     torch = torch_cuda
     n = 160 * MIB + 4099

@@ -464,6 +464,19 @@ def test_large_copies_with_the_heuristic_runs(capi, blit, oracle, rand, torch_cu
         assert p.xcd_run == (288 if (so - do) % 4 else 576), p.as_dict()
 
 
+@pytest.mark.parametrize("so", [0, 1, 2, 3, 7, 64])
+def test_offsets_at_the_sizes_of_the_heuristic_runs(capi, blit, oracle, arenas, so):
+    """50-60 MiB, where the byte-offset copies (and from 80 MiB the others) are
+    launched in XCD runs by the heuristics: every byte shift against destination
+    residues that give the first tile a head, a lead or neither."""
+    src, src_host, dst = arenas
+    for do, n in ((0, 50 * MIB + 1), (5, 49 * MIB + 4321), (16 * 9 + 3, 60 * MIB - 7)):
+        run_copy_case(capi, blit, oracle, src, src_host, dst, 256 + so, GUARD + do, n)
+        p = blit.last_plan()
+        assert p.byte_shift == (so - do) % 4
+        assert p.xcd_run == (288 if p.byte_shift else 0), p.as_dict()
+
+
 # ---------------------------------------------------------------------- batched
 
 def _make_batch(capi, rng, src, dst, n, min_len=64, max_len=256 << 10):

@@ -460,6 +460,41 @@ int mi355_blit_copy_batch_bounded(mi355_blit_t* h, const mi355_blit_desc_t* devi
 }
 
 namespace {
+// The two launches of the device-side prefix sum over the copies' chunk
+// counts: chunk_start within groups of 1024 copies, block_sum across groups.
+void launch_scans(mi355_blit* h, hipStream_t s, const BatchDesc* dev_descs, size_t n) {
+  const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
+  ScanLocalArgs sl{dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
+  hipLaunchKernelGGL(mi355_batch_scan_local, dim3(n_blocks), dim3(1024), 0, s, sl);
+  ScanTopArgs st{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
+  hipLaunchKernelGGL(mi355_batch_scan_top, dim3(1), dim3(1024), 0, s, st);
+}
+
+// The copy over h->records_dev: one wave per quarter chunk unless tuning says
+// otherwise.  total_chunks is the number of records, or a bound on it when
+// `counted` points at the number the device computed.  Fills in the launch
+// shape of *p.
+int launch_records_copy(mi355_blit* h, hipStream_t s, const mi355_blit_tuning_t* t, mi355_blit_plan_t* p,
+                        uint64_t total_chunks, const uint32_t* counted, uint64_t total_bytes, bool streaming) {
+  p->wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size : 256;
+  const uint64_t waves_per_wg = p->wg_size / 64;
+  unsigned split = kBatchSplit;
+  if (t && (t->unroll == 1 || t->unroll == 2 || t->unroll == 4)) split = 4 / t->unroll;
+  const uint64_t waves = total_chunks * split;
+  uint64_t wgs = (waves + waves_per_wg - 1) / waves_per_wg;
+  if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
+  if (wgs * p->wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / p->wg_size;
+  p->grid = static_cast<uint32_t>(wgs);
+  p->xcd_run = batch_xcd_run(total_bytes, split, static_cast<uint32_t>(waves_per_wg), t);
+  p->unroll = 4 / split;
+  batch_kernel_t k = select_batch_kernel(split, streaming, p->store_policy);
+  if (!k) return MI355_BLIT_ERROR;
+  BatchCopyArgs bc{h->records_dev, total_chunks, counted, static_cast<uint32_t>(waves_per_wg),
+                   static_cast<uint32_t>(wgs * waves_per_wg), make_xcd_runs(p->grid, p->xcd_run)};
+  hipLaunchKernelGGL(k, dim3(p->grid), dim3(p->wg_size), 0, s, bc);
+  return MI355_BLIT_SUCCESS;
+}
+
 int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int descs_on_device,
                uint64_t max_total_bytes, void* stream) {
   if (!h || (!descs && n)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
@@ -536,23 +571,8 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
                        0, s, er);
     BLIT_HIP(hipGetLastError());
 
-    p.wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size : 256;
-    const uint64_t waves_per_wg = p.wg_size / 64;
-    unsigned split = kBatchSplit;
-    if (t && (t->unroll == 1 || t->unroll == 2 || t->unroll == 4)) split = 4 / t->unroll;
-    const uint64_t waves = shape.total_chunks * split;
-    uint64_t wgs = (waves + waves_per_wg - 1) / waves_per_wg;
-    if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
-    if (wgs * p.wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / p.wg_size;
-    p.grid = static_cast<uint32_t>(wgs);
-    const uint32_t batch_run = batch_xcd_run(shape.total_bytes, split, static_cast<uint32_t>(waves_per_wg), t);
-    p.xcd_run = batch_run;
-    p.unroll = 4 / split;
-    batch_kernel_t k = select_batch_kernel(split, streaming, p.store_policy);
-    if (!k) return MI355_BLIT_ERROR;
-    BatchCopyArgs bc{h->records_dev, shape.total_chunks, nullptr, static_cast<uint32_t>(waves_per_wg),
-                     static_cast<uint32_t>(wgs * waves_per_wg), make_xcd_runs(p.grid, batch_run)};
-    hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, bc);
+    rc = launch_records_copy(h, s, t, &p, shape.total_chunks, nullptr, shape.total_bytes, streaming);
+    if (rc != MI355_BLIT_SUCCESS) return rc;
   } else if (max_total_bytes) {
     // Device-resident descriptors whose total size the caller bounds: the
     // bound sizes the record buffer and a per-chunk grid, so the copy runs in
@@ -560,41 +580,27 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
     // are made on the device; the copy kernel reads the number of records
     // there too and the waves the bound overestimated end at once.
     const BatchDesc* dev_descs = reinterpret_cast<const BatchDesc*>(descs);
-    const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
-    ScanLocalArgs sl{dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
-    hipLaunchKernelGGL(mi355_batch_scan_local, dim3(n_blocks), dim3(1024), 0, s, sl);
-    ScanTopArgs st{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
-    hipLaunchKernelGGL(mi355_batch_scan_top, dim3(1), dim3(1024), 0, s, st);
+    launch_scans(h, s, dev_descs, n);
     EmitRecordsDeviceArgs er{dev_descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n),
                              h->records_dev, shape.total_chunks};
     hipLaunchKernelGGL(mi355_batch_emit_records_device, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0,
                        s, er);
     BLIT_HIP(hipGetLastError());
-    p.wg_size = 256;
-    const uint64_t waves_per_wg = p.wg_size / 64;
-    const uint64_t waves = shape.total_chunks * kBatchSplit;
-    uint64_t wgs = (waves + waves_per_wg - 1) / waves_per_wg;
-    if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
-    if (wgs * p.wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / p.wg_size;
-    p.grid = static_cast<uint32_t>(wgs);
-    const uint32_t batch_run = batch_xcd_run(max_total_bytes, kBatchSplit, static_cast<uint32_t>(waves_per_wg), t);
-    p.xcd_run = batch_run;
-    p.unroll = 4 / kBatchSplit;
-    batch_kernel_t k = select_batch_kernel(kBatchSplit, streaming, p.store_policy);
-    if (!k) return MI355_BLIT_ERROR;
-    BatchCopyArgs bc{h->records_dev, shape.total_chunks, h->chunk_start_dev + n, static_cast<uint32_t>(waves_per_wg),
-                     static_cast<uint32_t>(wgs * waves_per_wg), make_xcd_runs(p.grid, batch_run)};
-    hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, bc);
+    // the shape of the copy is not open to tuning here, only its grid cap and cache policy
+    mi355_blit_tuning_t fixed{};
+    if (t) {
+      fixed.max_grid = t->max_grid;
+      fixed.xcd_run = t->xcd_run;
+    }
+    rc = launch_records_copy(h, s, t ? &fixed : nullptr, &p, shape.total_chunks, h->chunk_start_dev + n,
+                             max_total_bytes, streaming);
+    if (rc != MI355_BLIT_SUCCESS) return rc;
   } else {
     // Device-resident descriptors: the prefix sum runs on the device and, as
     // the host cannot size a per-chunk grid without a read-back, the copy runs
     // on a device-filling grid whose waves share the chunks out evenly.
     const BatchDesc* dev_descs = reinterpret_cast<const BatchDesc*>(descs);
-    const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
-    ScanLocalArgs sl{dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
-    hipLaunchKernelGGL(mi355_batch_scan_local, dim3(n_blocks), dim3(1024), 0, s, sl);
-    ScanTopArgs st{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
-    hipLaunchKernelGGL(mi355_batch_scan_top, dim3(1), dim3(1024), 0, s, st);
+    launch_scans(h, s, dev_descs, n);
     FinalizeArgs fa{static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
     hipLaunchKernelGGL(mi355_batch_finalize, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, s, fa);
     p.wg_size = 256;

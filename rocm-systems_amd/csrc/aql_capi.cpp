@@ -462,6 +462,12 @@ const Kernel* find_copy(mi355_aql* h, const mi355_blit_plan_t& p) {
   return nullptr;
 }
 
+const Kernel* find_batch(mi355_aql* h, const BatchLaunch& l, const mi355_blit_plan_t& p) {
+  for (const auto& v : h->batch_kernels)
+    if (v.split == l.split && v.nt_load == p.nt_load && v.store == p.store_policy) return &v.k;
+  return nullptr;
+}
+
 }  // namespace
 
 extern "C" {
@@ -748,31 +754,11 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
                      h->records_dev};
 
   // 2. the copy
-  mi355_blit_plan_t p{};
-  p.kernel = MI355_BLIT_KERNEL_COPY_BATCH;
-  p.body_vecs = total_chunks;
-  bool streaming = total_bytes >= (4ull << 20);
-  if (t && t->nt_load) streaming = (t->nt_load == 2);
-  p.nt_load = streaming;
-  p.store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
-  if (t && t->store_policy >= 1 && t->store_policy <= 4) p.store_policy = t->store_policy - 1;
-  p.wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size : 256;
-  unsigned split = 4;
-  if (t && (t->unroll == 1 || t->unroll == 2 || t->unroll == 4)) split = 4 / t->unroll;
-  p.unroll = 4 / split;
-  const uint64_t waves_per_wg = p.wg_size / 64;
-  uint64_t wgs = (total_chunks * split + waves_per_wg - 1) / waves_per_wg;
-  if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
-  if (wgs * p.wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / p.wg_size;
-  p.grid = static_cast<uint32_t>(wgs);
-  const uint32_t batch_run = batch_xcd_run(total_bytes, split, static_cast<uint32_t>(waves_per_wg), t);
-  p.xcd_run = batch_run;
-  const Kernel* bk = nullptr;
-  for (const auto& v : h->batch_kernels)
-    if (v.split == split && v.nt_load == (streaming ? 1u : 0u) && v.store == p.store_policy) bk = &v.k;
+  mi355_blit_plan_t p;
+  const BatchLaunch l = plan_batch_records(total_chunks, total_bytes, total_bytes >= (4ull << 20), t, true, &p);
+  const Kernel* bk = find_batch(h, l, p);
   if (!bk) return MI355_BLIT_ERROR;
-  BatchCopyArgs bc{h->records_dev, total_chunks, nullptr, static_cast<uint32_t>(waves_per_wg),
-                   static_cast<uint32_t>(wgs * waves_per_wg), make_xcd_runs(p.grid, batch_run)};
+  BatchCopyArgs bc{h->records_dev, total_chunks, nullptr, l.waves_per_wg, l.n_waves, make_xcd_runs(p.grid, p.xcd_run)};
   h->last_plan = p;
 
   const uint32_t nb = barrier_packets(num_deps);
@@ -869,31 +855,14 @@ int mi355_aql_copy_batch_bounded(mi355_aql_t* h, const mi355_blit_desc_t* device
   EmitRecordsDeviceArgs er{descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n), h->records_dev,
                            capacity};
 
-  mi355_blit_plan_t p{};
-  p.kernel = MI355_BLIT_KERNEL_COPY_BATCH;
-  p.body_vecs = capacity;
-  bool streaming = true;  // the lengths are only known on the device
-  if (t && t->nt_load) streaming = (t->nt_load == 2);
-  p.nt_load = streaming;
-  p.store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
-  if (t && t->store_policy >= 1 && t->store_policy <= 4) p.store_policy = t->store_policy - 1;
-  p.wg_size = 256;
-  const unsigned split = 4;
-  p.unroll = 4 / split;
-  const uint64_t waves_per_wg = p.wg_size / 64;
-  uint64_t wgs = (capacity * split + waves_per_wg - 1) / waves_per_wg;
-  if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
-  if (wgs * p.wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / p.wg_size;
-  p.grid = static_cast<uint32_t>(wgs);
-  const uint32_t batch_run = batch_xcd_run(max_total_bytes, split, static_cast<uint32_t>(waves_per_wg), t);
-  p.xcd_run = batch_run;
-  const Kernel* bk = nullptr;
-  for (const auto& v : h->batch_kernels)
-    if (v.split == split && v.nt_load == (streaming ? 1u : 0u) && v.store == p.store_policy) bk = &v.k;
+  // the lengths are only known on the device: a large batch, in the fixed shape
+  mi355_blit_plan_t p;
+  const BatchLaunch l = plan_batch_records(capacity, max_total_bytes, true, t, false, &p);
+  const Kernel* bk = find_batch(h, l, p);
   if (!bk) return MI355_BLIT_ERROR;
   // the grid is sized for the bound; the kernel reads the number of records the device counted
-  BatchCopyArgs bc{h->records_dev, capacity, h->chunk_start_dev + n, static_cast<uint32_t>(waves_per_wg),
-                   static_cast<uint32_t>(wgs * waves_per_wg), make_xcd_runs(p.grid, batch_run)};
+  BatchCopyArgs bc{h->records_dev, capacity, h->chunk_start_dev + n, l.waves_per_wg, l.n_waves,
+                   make_xcd_runs(p.grid, p.xcd_run)};
   h->last_plan = p;
 
   const uint32_t nb = barrier_packets(num_deps);

@@ -34,10 +34,6 @@ using namespace mi355;
 // queue has 64 (amd_gpu_agent.h:507-508).
 constexpr unsigned kLedgerSlots = 64;
 
-// Waves that share one 4 KiB chunk of the batched copy: with 4, a 4-wave
-// workgroup moves one chunk, 1 KiB per wave (measured best on MI355X).
-constexpr unsigned kBatchSplit = 4;
-
 struct LedgerSlot {
   hipEvent_t done = nullptr;
   uint64_t bytes = 0;  // submitted between the previous marker and this one
@@ -470,28 +466,15 @@ void launch_scans(mi355_blit* h, hipStream_t s, const BatchDesc* dev_descs, size
   hipLaunchKernelGGL(mi355_batch_scan_top, dim3(1), dim3(1024), 0, s, st);
 }
 
-// The copy over h->records_dev: one wave per quarter chunk unless tuning says
-// otherwise.  total_chunks is the number of records, or a bound on it when
-// `counted` points at the number the device computed.  Fills in the launch
-// shape of *p.
-int launch_records_copy(mi355_blit* h, hipStream_t s, const mi355_blit_tuning_t* t, mi355_blit_plan_t* p,
-                        uint64_t total_chunks, const uint32_t* counted, uint64_t total_bytes, bool streaming) {
-  p->wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size : 256;
-  const uint64_t waves_per_wg = p->wg_size / 64;
-  unsigned split = kBatchSplit;
-  if (t && (t->unroll == 1 || t->unroll == 2 || t->unroll == 4)) split = 4 / t->unroll;
-  const uint64_t waves = total_chunks * split;
-  uint64_t wgs = (waves + waves_per_wg - 1) / waves_per_wg;
-  if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
-  if (wgs * p->wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / p->wg_size;
-  p->grid = static_cast<uint32_t>(wgs);
-  p->xcd_run = batch_xcd_run(total_bytes, split, static_cast<uint32_t>(waves_per_wg), t);
-  p->unroll = 4 / split;
-  batch_kernel_t k = select_batch_kernel(split, streaming, p->store_policy);
+// The copy over h->records_dev, launched as *p says (plan_batch_records).
+// total_chunks is the number of records, or a bound on it when `counted`
+// points at the number the device computed.
+int launch_records_copy(mi355_blit* h, hipStream_t s, const mi355_blit_plan_t& p, const BatchLaunch& l,
+                        uint64_t total_chunks, const uint32_t* counted) {
+  batch_kernel_t k = select_batch_kernel(l.split, p.nt_load != 0, p.store_policy);
   if (!k) return MI355_BLIT_ERROR;
-  BatchCopyArgs bc{h->records_dev, total_chunks, counted, static_cast<uint32_t>(waves_per_wg),
-                   static_cast<uint32_t>(wgs * waves_per_wg), make_xcd_runs(p->grid, p->xcd_run)};
-  hipLaunchKernelGGL(k, dim3(p->grid), dim3(p->wg_size), 0, s, bc);
+  BatchCopyArgs bc{h->records_dev, total_chunks, counted, l.waves_per_wg, l.n_waves, make_xcd_runs(p.grid, p.xcd_run)};
+  hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, bc);
   return MI355_BLIT_SUCCESS;
 }
 
@@ -530,20 +513,13 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
   h->next_host ^= 1;
   if (h->batch_busy[b ^ 1] && h->last_batch_stream != s) BLIT_HIP(hipStreamWaitEvent(s, h->batch_done[b ^ 1], 0));
 
-  mi355_blit_plan_t p{};
-  p.kernel = MI355_BLIT_KERNEL_COPY_BATCH;
-  p.unroll = kBatchChunkVecs / 64;
-  p.body_vecs = shape.total_chunks;  // chunks, when known
   const mi355_blit_tuning_t* t = h->has_tuning ? &h->tuning : nullptr;
-  // Measured on MI355X with 65,536 copies of 64 B..256 KiB: non-temporal loads
-  // and stores are best (739 us against 824 us cached); written-through
-  // stores are worst (958 us), because a chunk's first and last cache line
-  // are shared with its neighbours and written through in halves.
-  bool streaming = descs_on_device || shape.total_bytes >= (4ull << 20);
-  if (t && t->nt_load) streaming = (t->nt_load == 2);
-  p.nt_load = streaming;
-  p.store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
-  if (t && t->store_policy >= 1 && t->store_policy <= 4) p.store_policy = t->store_policy - 1;
+  // Device-resident descriptors are taken to be a large batch: their lengths
+  // are only known on the device.  Only host-resident ones leave the copy's
+  // shape open to tuning.
+  mi355_blit_plan_t p;
+  const BatchLaunch l = plan_batch_records(shape.total_chunks, shape.total_bytes,
+                                           descs_on_device || shape.total_bytes >= (4ull << 20), t, !descs_on_device, &p);
 
   if (!descs_on_device) {
     // Host-resident descriptors.  The host has walked them to validate them
@@ -571,7 +547,7 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
                        0, s, er);
     BLIT_HIP(hipGetLastError());
 
-    rc = launch_records_copy(h, s, t, &p, shape.total_chunks, nullptr, shape.total_bytes, streaming);
+    rc = launch_records_copy(h, s, p, l, shape.total_chunks, nullptr);
     if (rc != MI355_BLIT_SUCCESS) return rc;
   } else if (max_total_bytes) {
     // Device-resident descriptors whose total size the caller bounds: the
@@ -586,14 +562,7 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
     hipLaunchKernelGGL(mi355_batch_emit_records_device, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0,
                        s, er);
     BLIT_HIP(hipGetLastError());
-    // the shape of the copy is not open to tuning here, only its grid cap and cache policy
-    mi355_blit_tuning_t fixed{};
-    if (t) {
-      fixed.max_grid = t->max_grid;
-      fixed.xcd_run = t->xcd_run;
-    }
-    rc = launch_records_copy(h, s, t ? &fixed : nullptr, &p, shape.total_chunks, h->chunk_start_dev + n,
-                             max_total_bytes, streaming);
+    rc = launch_records_copy(h, s, p, l, shape.total_chunks, h->chunk_start_dev + n);
     if (rc != MI355_BLIT_SUCCESS) return rc;
   } else {
     // Device-resident descriptors: the prefix sum runs on the device and, as
@@ -604,6 +573,8 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
     FinalizeArgs fa{static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
     hipLaunchKernelGGL(mi355_batch_finalize, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, s, fa);
     p.wg_size = 256;
+    p.unroll = kBatchChunkVecs / 64;
+    p.xcd_run = 0;
     uint32_t max_grid = h->num_cus * kWgPerCu;
     if (t && t->max_grid) max_grid = t->max_grid;
     // A copy has at least one chunk and, at the sizes this path is meant for,
@@ -611,6 +582,7 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
     // idle waves.
     const uint64_t wgs = static_cast<uint64_t>(n) * 16;
     p.grid = static_cast<uint32_t>(wgs < max_grid ? wgs : max_grid);
+    const bool streaming = p.nt_load != 0;
     p.store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
     BatchStridedArgs bs{dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, 4u, p.grid * 4u};
     if (streaming) hipLaunchKernelGGL(mi355_batch_strided_l1_s1, dim3(p.grid), dim3(p.wg_size), 0, s, bs);

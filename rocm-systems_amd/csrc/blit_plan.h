@@ -109,6 +109,49 @@ inline uint32_t batch_xcd_run(uint64_t total_bytes, uint32_t split, uint32_t wav
   return plan_xcd_run(total_bytes >= kXcdRunMinBytes ? kBatchXcdRunChunks * split / waves_per_wg : 0, t);
 }
 
+// Launch shape of the batched copy over chunk records, shared by the two
+// submission paths.  Measured on MI355X with 65,536 copies of 64 B..256 KiB:
+// one 4 KiB chunk per 4-wave workgroup, 1 KiB per wave, is the fastest shape;
+// non-temporal loads and stores are best (739 us against 824 us cached), and
+// written-through stores are worst (958 us) because the copies' cut ends are
+// partial lines.
+struct BatchLaunch {
+  uint32_t split;         // waves per chunk
+  uint32_t waves_per_wg;
+  uint32_t n_waves;
+};
+
+// total_chunks: the number of records, or a bound on it.  streaming: whether
+// the batch is large enough to bypass the caches (tuning may override).  With
+// shape_tunable false only the grid cap, the XCD runs and the cache policies
+// follow the tuning.  Fills in *p.
+inline BatchLaunch plan_batch_records(uint64_t total_chunks, uint64_t total_bytes, bool streaming,
+                                      const mi355_blit_tuning_t* t, bool shape_tunable, mi355_blit_plan_t* p) {
+  *p = mi355_blit_plan_t{};
+  p->kernel = MI355_BLIT_KERNEL_COPY_BATCH;
+  p->body_vecs = total_chunks;
+  if (t && t->nt_load) streaming = (t->nt_load == 2);
+  p->nt_load = streaming;
+  p->store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
+  if (t && t->store_policy >= 1 && t->store_policy <= 4) p->store_policy = t->store_policy - 1;
+  BatchLaunch l;
+  p->wg_size = 256;
+  l.split = 4;
+  if (t && shape_tunable) {
+    if (t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) p->wg_size = t->wg_size;
+    if (valid_unroll(t->unroll)) l.split = 4 / t->unroll;
+  }
+  p->unroll = 4 / l.split;
+  l.waves_per_wg = p->wg_size / 64;
+  uint64_t wgs = (total_chunks * l.split + l.waves_per_wg - 1) / l.waves_per_wg;
+  if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
+  if (wgs * p->wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / p->wg_size;
+  p->grid = static_cast<uint32_t>(wgs);
+  l.n_waves = static_cast<uint32_t>(wgs * l.waves_per_wg);
+  p->xcd_run = batch_xcd_run(total_bytes, l.split, l.waves_per_wg, t);
+  return l;
+}
+
 inline void apply_launch_shape(mi355_blit_plan_t* p, const SizeClass& cls, uint32_t num_cus,
                                const mi355_blit_tuning_t* t) {
   (void)num_cus;

@@ -329,6 +329,30 @@ void one_magic_division() {
   }
 }
 
+// Launch shape of the batched copy: a wave for every quarter chunk (or what the
+// tuning says) unless the grid is capped; the fixed shape ignores the tuning's
+// workgroup and unroll but keeps its grid cap and cache policy.
+void one_batch_launch() {
+  const uint64_t chunks = 1 + below(3000000);
+  const uint64_t bytes = chunks * 4096;
+  mi355_blit_tuning_t t = random_tuning();
+  const bool tuned = below(2), tunable = below(2);
+  mi355_blit_plan_t p;
+  const BatchLaunch l = plan_batch_records(chunks, bytes, bytes >= (4ull << 20), tuned ? &t : nullptr, tunable, &p);
+  CHECK(p.kernel == MI355_BLIT_KERNEL_COPY_BATCH && p.body_vecs == chunks, "kernel / chunk count");
+  CHECK(l.split * p.unroll == 4 && l.waves_per_wg == p.wg_size / 64, "split %u unroll %u", l.split, p.unroll);
+  CHECK(l.n_waves == static_cast<uint64_t>(p.grid) * l.waves_per_wg, "wave count");
+  const bool capped = tuned && t.max_grid && t.max_grid < (chunks * l.split + l.waves_per_wg - 1) / l.waves_per_wg;
+  if (capped) CHECK(p.grid == t.max_grid, "grid cap");
+  else CHECK(l.n_waves >= chunks * l.split && l.n_waves < chunks * l.split + l.waves_per_wg, "one wave per part of a chunk");
+  if (!tuned || !tunable) CHECK(p.wg_size == 256 && l.split == 4, "fixed shape");
+  if (!tuned) {
+    CHECK(p.nt_load == (bytes >= (4ull << 20)) && p.store_policy == (p.nt_load ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED),
+          "cache policy by size");
+    CHECK(p.xcd_run == (bytes >= (64ull << 20) ? 528u : 0u), "XCD runs by size: %u", p.xcd_run);
+  }
+}
+
 // The XCD permutation of a launch: workgroups below make_xcd_runs(grid, run).full swap
 // places among themselves (a bijection), each XCD (b % 8) gets whole runs of
 // neighbouring workgroups in launch order, the rest keep their place.
@@ -367,6 +391,7 @@ int main(int argc, char** argv) {
     if (i % 8 == 0) one_batch_stage();
     if (i % 64 == 0) one_xcd_permutation();
     if (i % 16 == 0) one_magic_division();
+    if (i % 8 == 0) one_batch_launch();
   }
   std::printf("%s: %ld cases each of copy, fill and region plans, %d failures\n", g_failures ? "FAILED" : "OK", cases,
               g_failures);

@@ -49,40 +49,75 @@ typedef unsigned v4u __attribute__((ext_vector_type(4)));
 typedef v4u v4u_a4 __attribute__((aligned(4)));
 
 
+// Every pointer these kernels dereference points into global memory, but one
+// that was itself loaded from memory (the chunk records of a batch) reaches the
+// compiler as a generic pointer and would be accessed with flat_* instructions,
+// which go through the aperture check and count against both memory counters.
+// The accessors below therefore state the address space.
+#define MI355_GLOBAL __attribute__((address_space(1)))
+
+template <typename T>
+__device__ __forceinline__ const T MI355_GLOBAL* as_global(const T* p) {
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wold-style-cast"
+  return (const T MI355_GLOBAL*)(p);
+#pragma clang diagnostic pop
+}
+template <typename T>
+__device__ __forceinline__ T MI355_GLOBAL* as_global(T* p) {
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wold-style-cast"
+  return (T MI355_GLOBAL*)(p);
+#pragma clang diagnostic pop
+}
+
 template <bool NT>
 __device__ __forceinline__ v4u ld_v4(const v4u_a4* p) {
-  if constexpr (NT) return __builtin_nontemporal_load(p);
-  else return *p;
+  if constexpr (NT) return __builtin_nontemporal_load(as_global(p));
+  else return *as_global(p);
 }
 template <bool NT>
 __device__ __forceinline__ unsigned ld_u32(const unsigned* p) {
-  if constexpr (NT) return __builtin_nontemporal_load(p);
-  else return *p;
+  if constexpr (NT) return __builtin_nontemporal_load(as_global(p));
+  else return *as_global(p);
 }
+__device__ __forceinline__ uint8_t ld_u8(const uint8_t* p) { return *as_global(p); }
+__device__ __forceinline__ void st_u8(uint8_t* p, uint8_t v) { *as_global(p) = v; }
+__device__ __forceinline__ void st_u32(unsigned* p, unsigned v) { *as_global(p) = v; }
+
 // Store cache policies (values of mi355_blit_plan_t::store_policy).
 constexpr int kStoreCached = 0;   // plain write-back L2
 constexpr int kStoreNt = 1;       // non-temporal hint
 constexpr int kStoreAgentWt = 2;  // sc1: written through L2 at agent scope
 constexpr int kStoreSystemWt = 3; // sc0 sc1: written through at system scope
 
-// The write-through forms have no builtin for a 16-byte store, hence the asm.
-// A store needs no wait of its own, and on gfx9 the extra outstanding store
-// only makes a compiler-placed s_waitcnt vmcnt(n) wait longer, never shorter.
-// A store of more than 8 bytes reads its data registers after issue: a VALU
-// write to them within the next 2 wait states (gfx940 and later) corrupts the
-// data.  The compiler pads its own stores but cannot see into the asm, so the
-// s_nop is part of it.
+// The policies are spelled out in asm: the write-through forms have no builtin
+// for a 16-byte store, and the non-temporal builtin's hint was seen to get lost
+// on the way through the optimizer (the body store of one realigning variant
+// came out as a plain store).  A store needs no wait of its own, and on gfx9
+// the extra outstanding store only makes a compiler-placed s_waitcnt vmcnt(n)
+// wait longer, never shorter.  A store of more than 8 bytes reads its data
+// registers after issue: a VALU write to them within the next 2 wait states
+// (gfx940 and later) corrupts the data.  The compiler pads its own stores but
+// cannot see into the asm, so the s_nop is part of it.  The asm forms take any
+// byte address.
 template <int POLICY>
-__device__ __forceinline__ void st_v4(v4u* p, v4u v) {
+__device__ __forceinline__ void st_v4_at(uintptr_t p, v4u v) {
   if constexpr (POLICY == kStoreNt) {
-    __builtin_nontemporal_store(v, p);
+    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
   } else if constexpr (POLICY == kStoreAgentWt) {
     asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
   } else if constexpr (POLICY == kStoreSystemWt) {
     asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
   } else {
-    *p = v;
+    typedef v4u v4u_any __attribute__((aligned(1)));
+    *as_global(reinterpret_cast<v4u_any*>(p)) = v;
   }
+}
+template <int POLICY>
+__device__ __forceinline__ void st_v4(v4u* p, v4u v) {
+  if constexpr (POLICY == kStoreCached) *as_global(p) = v;
+  else st_v4_at<POLICY>(reinterpret_cast<uintptr_t>(p), v);
 }
 
 // 16-byte accesses at any byte address: gfx950 under HSA runs with unaligned
@@ -91,19 +126,13 @@ typedef v4u v4u_a1 __attribute__((aligned(1)));
 
 template <bool NT>
 __device__ __forceinline__ v4u ld_v4_any(const uint8_t* p) {
-  if constexpr (NT) return __builtin_nontemporal_load(reinterpret_cast<const v4u_a1*>(p));
-  else return *reinterpret_cast<const v4u_a1*>(p);
+  if constexpr (NT) return __builtin_nontemporal_load(as_global(reinterpret_cast<const v4u_a1*>(p)));
+  else return *as_global(reinterpret_cast<const v4u_a1*>(p));
 }
 
 template <int POLICY>
 __device__ __forceinline__ void st_v4_any(uintptr_t p, v4u v) {
-  if constexpr (POLICY == kStoreNt) {
-    __builtin_nontemporal_store(v, reinterpret_cast<v4u_a1*>(p));
-  } else if constexpr (POLICY == kStoreAgentWt || POLICY == kStoreSystemWt) {
-    st_v4<POLICY>(reinterpret_cast<v4u*>(p), v);  // the asm forms take any address
-  } else {
-    *reinterpret_cast<v4u_a1*>(p) = v;
-  }
+  st_v4_at<POLICY>(p, v);
 }
 
 // Lane i receives the value lane (i + 1) % 64 passed in (DPP wave_rol:1).
@@ -555,10 +584,10 @@ __device__ __forceinline__ void record_store(const ChunkRecord& rec, unsigned v0
 __device__ __forceinline__ void record_edges(const ChunkRecord& rec, bool do_head, bool do_tail,
                                              unsigned lane) {
   if (do_head && lane < rec.head) {
-    (rec.dst - rec.head)[lane] = (rec.src - rec.head)[lane];
+    st_u8(rec.dst - rec.head + lane, ld_u8(rec.src - rec.head + lane));
   } else if (do_tail && lane >= 16 && lane - 16 < rec.tail) {
     const uint64_t off = 16ull * rec.n_vec + lane - 16;
-    rec.dst[off] = rec.src[off];
+    st_u8(rec.dst + off, ld_u8(rec.src + off));
   }
 }
 
@@ -791,12 +820,12 @@ __device__ __forceinline__ void copy_partial_slot(uintptr_t slot, unsigned off, 
     const unsigned b_hi = 4u * q + 4 < end ? 4u * q + 4 : end;
     if (b_hi <= b_lo) continue;
     if (b_hi - b_lo == 4) {
-      *reinterpret_cast<unsigned*>(slot + 4 * q) = o[q];
+      st_u32(reinterpret_cast<unsigned*>(slot + 4 * q), o[q]);
     } else {
 #pragma unroll
       for (unsigned b = 0; b < 4; ++b)
         if (4u * q + b >= b_lo && 4u * q + b < b_hi)
-          *reinterpret_cast<uint8_t*>(slot + 4 * q + b) = static_cast<uint8_t>(o[q] >> (8 * b));
+          st_u8(reinterpret_cast<uint8_t*>(slot + 4 * q + b), static_cast<uint8_t>(o[q] >> (8 * b)));
     }
   }
 }

@@ -48,14 +48,17 @@ struct SizeClass {
 // having their neighbours on another XCD.  The run is 512 KiB + 64 KiB on
 // purpose: with runs of a power of two the 8 streams sit a power of two apart
 // and, depending on where source and destination lie, collide in the memory
-// channels (1 GiB with a byte offset: 315-367 us over 20 placements with runs
-// of 256 KiB, 320-326 us with 576 KiB, 338-344 us in launch order).
+// channels (1 GiB with a byte offset, 2 KiB tiles: 315-367 us over 20
+// placements with runs of 256 KiB, 320-326 us with 576 KiB, 338-344 us in
+// launch order).
 // Measured, 1 GiB: equally aligned 309-312 us against 314-317 us in launch
 // order; source and destination differing mod 128, 311-313 us against 321-327;
-// a byte offset, 320-326 us against 338-344.  At 128-256 MiB, where the
+// a byte offset, 310-314 us against 338-344.  At 128-256 MiB, where the
 // last-level cache holds most of the transfer, 59 us against 66 us.  A byte
 // offset adds one dword fetch per tile (the bytes that spill past the last
-// lane), which 2 KiB tiles amortise best; its stores are written through while
+// lane); while the transfer sits in the last-level cache 2 KiB tiles amortise
+// it best, beyond that 1 KiB tiles with non-temporal stores run like the
+// aligned copy.  Its stores are written through while
 // the 256 MiB last-level cache absorbs them and non-temporal beyond (256 MiB:
 // 61 us against 79 us, 288 MiB: 93 us against 89 us).  The thresholds are where
 // the shapes cross in a sweep in steps of 16-32 MiB.  Fills at one
@@ -78,7 +81,7 @@ constexpr SizeClass kCopyRealignClasses[] = {  // (src - dst) % 4 != 0
     {0, 512, 1, 0, MI355_BLIT_STORE_CACHED, 0},
     {4ull << 20, 256, 2, 1, MI355_BLIT_STORE_AGENT_WT, 0},
     {48ull << 20, 64, 2, 1, MI355_BLIT_STORE_AGENT_WT, kXcdRunBytes},
-    {272ull << 20, 64, 2, 1, MI355_BLIT_STORE_NT, kXcdRunBytes},
+    {272ull << 20, 64, 1, 1, MI355_BLIT_STORE_NT, kXcdRunBytes},
 };
 constexpr SizeClass kFillClasses[] = {
     {0, 256, 1, 0, MI355_BLIT_STORE_CACHED, 0},

@@ -142,8 +142,8 @@ def test_plan_copy_shapes_by_size_and_offset(capi_host):
         assert shape(off, 16 * MIB) == (256, 2, 1, wt, 0)
         assert shape(off, 48 * MIB) == (64, 2, 1, wt, 288)      # 288 tiles of 2 KiB
         assert shape(off, 256 * MIB) == (64, 2, 1, wt, 288)     # the last-level cache still absorbs the stores
-        assert shape(off, 272 * MIB) == (64, 2, 1, nt, 288)
-        assert shape(off, 1 << 30) == (64, 2, 1, nt, 288)
+        assert shape(off, 272 * MIB) == (64, 1, 1, nt, 576)
+        assert shape(off, 1 << 30) == (64, 1, 1, nt, 576)
     # the run follows the workgroup the tuning asks for; 1 means launch order
     st, p = capi_host.plan_copy(dst, 0x7e0000000000, 1 << 30, 256, capi_host.Tuning(wg_size=256))
     assert p.xcd_run == 144

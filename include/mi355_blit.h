@@ -157,7 +157,8 @@ int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwo
  * No counterpart in the reference (it submits one AQL packet per copy).
  * descs may live in host memory (descs_on_device == 0: the library stages
  * them) or be device-resident (descs_on_device != 0: read in place, must stay
- * valid until completion).  Regions must not overlap one another. */
+ * valid until completion).  Regions must not overlap one another.  A stream
+ * under HIP graph capture -> INVALID_ARGUMENT (both batched entry points). */
 int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n,
                           int descs_on_device, void* stream);
 

@@ -199,16 +199,18 @@ int ledger_mark(mi355_blit* h) {
   return MI355_BLIT_SUCCESS;
 }
 
+bool stream_is_capturing(hipStream_t s) {
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  return hipStreamIsCapturing(s, &capture) == hipSuccess && capture == hipStreamCaptureStatusActive;
+}
+
 // Notes `bytes` as queued on `s`.  Caller holds h->lock.
 int ledger_record(mi355_blit* h, hipStream_t s, uint64_t bytes) {
-  if (s != h->stream) {
-    // A command recorded into a graph under stream capture is not queued
-    // anywhere: nothing is pending because of it, and no marker event may be
-    // recorded on the capturing stream.
-    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(s, &capture) == hipSuccess && capture == hipStreamCaptureStatusActive)
-      return MI355_BLIT_SUCCESS;
-  }
+  // A command recorded into a graph under stream capture is not queued
+  // anywhere: nothing is pending because of it, and no marker event may be
+  // recorded on the capturing stream.  (The handle's own stream is never
+  // captured by a caller that does not know it.)
+  if (s != h->stream && stream_is_capturing(s)) return MI355_BLIT_SUCCESS;
   if (h->unmarked && h->last_stream != s) {
     // a marker only orders against its own stream
     int rc = ledger_mark(h);
@@ -487,6 +489,12 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
   DeviceScope scope(h->device);
   if (scope.err != hipSuccess) return status_of(scope.err);
   hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
+  if (stream_is_capturing(s)) {
+    // A batch stages descriptors, may allocate, and shares its record buffer
+    // with the batches around it through events: none of that can be
+    // recorded into a graph.
+    return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  }
 
   BatchShape shape;
   if (!descs_on_device) {

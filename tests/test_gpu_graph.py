@@ -62,3 +62,34 @@ def test_captured_commands_replay_exactly(capi, oracle, rand, torch_cuda):
             assert blit.copy(dst.data_ptr(), src.data_ptr(), 4096) == capi.SUCCESS
             assert blit.synchronize() == capi.SUCCESS
         del graph
+
+
+def test_batches_refuse_a_capturing_stream(capi, torch_cuda):
+    """The batched copy stages descriptors and orders batches with events, so it
+    cannot be recorded into a graph: it must say so instead of recording half of
+    itself.  Nothing is launched by the refused calls."""
+    torch = torch_cuda
+    src = torch.arange(8192, dtype=torch.uint8, device="cuda:0")
+    dst = torch.zeros(8192, dtype=torch.uint8, device="cuda:0")
+    descs = (capi.Desc * 2)()
+    for i in range(2):
+        descs[i].dst, descs[i].src, descs[i].bytes = dst.data_ptr() + 4096 * i, src.data_ptr() + 4096 * i, 4000
+    dev = torch.from_numpy(np.frombuffer(bytes(descs), dtype=np.uint8).copy()).to("cuda:0")
+    with capi.Blit(0) as blit:
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            s = torch.cuda.current_stream().cuda_stream
+            assert blit.copy_batch(descs, 2, False, s) == capi.ERROR_INVALID_ARGUMENT
+            assert blit.copy_batch(dev.data_ptr(), 2, True, s) == capi.ERROR_INVALID_ARGUMENT
+            assert blit.copy_batch_bounded(dev.data_ptr(), 2, 8000, s) == capi.ERROR_INVALID_ARGUMENT
+            assert blit.copy(dst.data_ptr(), src.data_ptr(), 64, s) == capi.SUCCESS
+        graph.replay()
+        torch.cuda.synchronize()
+        assert int(dst[:64].sum()) == sum(range(64)) and int(dst[64:].sum()) == 0
+        # the same batch outside a capture goes through
+        assert blit.copy_batch(descs, 2, False, None) == capi.SUCCESS
+        assert blit.synchronize() == capi.SUCCESS
+        assert torch.equal(dst[:4000], src[:4000]) and torch.equal(dst[4096:8096], src[4096:8096])
+        del graph

@@ -372,6 +372,52 @@ def aql_path(r, pkg):
     return out
 
 
+def host_link(r, pkg):
+    """Host <-> device through the blit kernel over the host link (pinned host
+    memory, the routes of include/mi355_blit.h), with the runtime's own
+    hsa_memory_copy beside it, which sends such copies to its DMA engines
+    (amd_gpu_agent.cpp:2370-2377).  Blocking calls, host clock, best of 5;
+    GB/s of bytes moved (not read plus written: the link carries them once)."""
+    eng = pkg.aql.AqlBlit(0)
+    out = {}
+    try:
+        hsa = C.CDLL("libhsa-runtime64.so.1")
+        hsa.hsa_memory_copy.restype = C.c_int
+        hsa.hsa_memory_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+    except (OSError, AttributeError):
+        hsa = None
+    try:
+        for n in (16 * MIB, 256 * MIB):
+            host = r.torch.empty(n, dtype=r.torch.uint8, pin_memory=True)
+            host.numpy()[:] = seeded_bytes(n, 0xB1170006)
+            back = r.torch.zeros(n, dtype=r.torch.uint8, pin_memory=True)
+            dev = r.torch.zeros(n, dtype=r.torch.uint8, device="cuda:0")
+            r.torch.cuda.synchronize()
+            legs = [("h2d", lambda: eng.hsa_memory_copy(dev.data_ptr(), host.data_ptr(), n)),
+                    ("d2h", lambda: eng.hsa_memory_copy(back.data_ptr(), dev.data_ptr(), n))]
+            if hsa is not None:
+                legs += [("reference_h2d", lambda: hsa.hsa_memory_copy(dev.data_ptr(), host.data_ptr(), n)),
+                         ("reference_d2h", lambda: hsa.hsa_memory_copy(back.data_ptr(), dev.data_ptr(), n))]
+            for name, fn in legs:
+                best = None
+                for _ in range(6):
+                    t0 = time.perf_counter()
+                    st = fn()
+                    t = time.perf_counter() - t0
+                    if st != 0:
+                        best = None
+                        break
+                    best = t if best is None else min(best, t)
+                if best:
+                    out["%s_%dMiB_gbs" % (name, n // MIB)] = round(n / best / 1e9, 2)
+            assert r.torch.equal(back, host), "host -> device -> host differs"
+            del host, back, dev
+    finally:
+        eng.close()
+    out["how"] = "pinned host memory, blocking calls, host clock, best of 6; reference = hsa_memory_copy of the loaded runtime (DMA engines)"
+    return out
+
+
 def reference_gpu_path(r):
     """The reference's own blit kernels on this GPU, for orientation: the ROCr
     this process already runs on (libhsa-runtime64, the binary build of the same
@@ -580,6 +626,7 @@ def main():
         r.torch.cuda.empty_cache()
         also["aql_submission"] = aql_path(r, pkg)
         also["reference_gpu_path"] = reference_gpu_path(r)
+        also["host_link"] = host_link(r, pkg)
 
     line = {
         "metric": "D2D copy & fill GB/s (R+W) at 1 GiB on 1 MI355X",

@@ -76,8 +76,22 @@ typedef struct {
                            permuted so that every XCD works on runs of N
                            neighbouring workgroups' tiles, and a cache line two
                            neighbouring tiles share is fetched into one L2 */
-  uint32_t reserved;
+  uint32_t route;       /* MI355_BLIT_ROUTE_* the launch was shaped for */
 } mi355_blit_plan_t;
+
+/* Which memories a linear copy connects.  The reference keeps one blit object
+ * per direction (core/inc/amd_gpu_agent.h:588, BlitDevToDev / BlitHostToDev /
+ * BlitDevToHost; amd_gpu_agent.cpp:846-867, GetPcieBlit :2370-2377) and may put
+ * a blit kernel behind each; here the direction shapes the launch.  A copy
+ * one side of which is host memory is bound by the host link (64 GB/s
+ * nominal), not by HBM: it wants a few hundred waves walking the buffer in
+ * address order, not a wave per KiB.  The kernels and the results are the
+ * same on every route. */
+enum {
+  MI355_BLIT_ROUTE_DEVICE = 0,         /* both sides in the GPU's memory */
+  MI355_BLIT_ROUTE_HOST_TO_DEVICE = 1, /* src is host memory the GPU can read */
+  MI355_BLIT_ROUTE_DEVICE_TO_HOST = 2  /* dst is host memory the GPU can write */
+};
 
 /* Cache policy of the body's 16-byte stores. */
 enum {
@@ -145,6 +159,15 @@ int mi355_blit_destroy(mi355_blit_t* h);
  * are not counted by mi355_blit_pending_bytes.  The batched copy stages its
  * descriptors and may not. */
 int mi355_blit_copy(mi355_blit_t* h, void* dst, const void* src, size_t bytes, void* stream);
+
+/* mi355_blit_copy for a copy that crosses the host link: what the reference
+ * submits to blits_[BlitHostToDev] / blits_[BlitDevToHost] when a blit kernel
+ * serves them (amd_gpu_agent.cpp:761-841 DmaCopy, :2370-2377).  route is
+ * MI355_BLIT_ROUTE_*; MI355_BLIT_ROUTE_DEVICE is mi355_blit_copy itself, any
+ * other value -> INVALID_ARGUMENT.  The host side must be memory the GPU can
+ * access (allocated through the runtime or locked). */
+int mi355_blit_copy_route(mi355_blit_t* h, void* dst, const void* src, size_t bytes, uint32_t route,
+                          void* stream);
 
 /* Replaces the dispatch half of BlitKernel::SubmitLinearFillCommand
  * (amd_blit_kernel.cpp:787-837) and the Fill shader (blit_shaders/blit_fill.s).
@@ -265,6 +288,9 @@ int mi355_blit_plan_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t nu
                          const mi355_blit_tuning_t* tuning, mi355_blit_plan_t* out);
 int mi355_blit_plan_fill(uint64_t ptr, uint64_t num_dwords, uint32_t num_cus,
                          const mi355_blit_tuning_t* tuning, mi355_blit_plan_t* out);
+/* mi355_blit_plan_copy for a route other than within the device. */
+int mi355_blit_plan_copy_route(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t num_cus,
+                               const mi355_blit_tuning_t* tuning, uint32_t route, mi355_blit_plan_t* out);
 
 /* Installs overrides used by every later command on the handle (NULL clears).
  * For tuning sweeps; replaces the reference's string-parsed kernel parameters

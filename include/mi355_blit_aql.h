@@ -49,6 +49,14 @@ int mi355_aql_destroy(mi355_aql_t* h);
 int mi355_aql_copy(mi355_aql_t* h, void* dst, const void* src, size_t bytes,
                    const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal);
 
+/* mi355_aql_copy for a copy that crosses the host link, launched in the
+ * shape that suits the link (mi355_blit.h, MI355_BLIT_ROUTE_*): what the
+ * reference submits to blits_[BlitHostToDev] / blits_[BlitDevToHost]
+ * (amd_gpu_agent.cpp:761-841, :2370-2377).  MI355_BLIT_ROUTE_DEVICE is
+ * mi355_aql_copy itself; any other value -> INVALID_ARGUMENT. */
+int mi355_aql_copy_route(mi355_aql_t* h, void* dst, const void* src, size_t bytes, uint32_t route,
+                         const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal);
+
 /* Replaces the dispatch half of BlitKernel::SubmitLinearFillCommand
  * (amd_blit_kernel.cpp:787-837), asynchronous like the copy.  ptr NULL or not
  * 4-byte aligned -> INVALID_ARGUMENT. */
@@ -143,7 +151,9 @@ int mi355_aql_staging(mi355_aql_t* h, size_t* half_bytes, void** half0, void** h
  * one side is host memory unknown to the runtime it is locked for the GPU for
  * the duration of the copy (:521-537), or, where the system refuses to lock
  * existing memory, bounced through the engine's staging buffers in 4 MiB
- * pieces; everything else goes to the blit. */
+ * pieces; everything else goes to the blit, on the route the two placements
+ * give (the reference picks blits_[BlitHostToDev] or blits_[BlitDevToHost]
+ * there, amd_gpu_agent.cpp:2370-2377). */
 int mi355_hsa_memory_copy(mi355_aql_t* h, void* dst, const void* src, size_t size);
 
 /* hsa_amd_memory_fill (core/runtime/hsa_ext_amd.cpp:237-251 + Runtime::FillMemory,
@@ -159,7 +169,11 @@ int mi355_hsa_amd_memory_fill(mi355_aql_t* h, void* ptr, uint32_t value, size_t 
  * that disagrees with the array pointer, or a zero completion signal ->
  * INVALID_ARGUMENT; size 0 -> SUCCESS without touching the signal (:285-291);
  * both ranges must already be accessible to the GPU (device memory, or host
- * memory allocated or locked through the runtime), as the API demands. */
+ * memory allocated or locked through the runtime), as the API demands.  The
+ * reference learns the direction from the two agents it is handed
+ * (GetBlitObject, amd_gpu_agent.cpp:2379-2442); this signature has none, so
+ * copies of 1 MiB and more, the sizes whose launch shape depends on it, look
+ * the two pointers up (hsa_amd_pointer_info) and take the route they give. */
 int mi355_hsa_amd_memory_async_copy(mi355_aql_t* h, void* dst, const void* src, size_t size,
                                     uint32_t num_dep_signals, const uint64_t* dep_signals,
                                     uint64_t completion_signal);

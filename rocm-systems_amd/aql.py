@@ -13,6 +13,8 @@ SIGNATURES = {
     "mi355_aql_create": (C.c_int, [C.c_int, C.POINTER(C.c_void_p)]),
     "mi355_aql_destroy": (C.c_int, [C.c_void_p]),
     "mi355_aql_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
+    "mi355_aql_copy_route": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint32, _U64P, C.c_uint32,
+                                       C.c_uint64]),
     "mi355_aql_fill32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
     "mi355_aql_copy_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
     "mi355_aql_copy_batch_device": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
@@ -100,8 +102,10 @@ class AqlBlit:
     def __exit__(self, *exc):
         self.close()
 
-    def copy(self, dst, src, nbytes, *, deps=None, completion=0):
+    def copy(self, dst, src, nbytes, *, deps=None, completion=0, route=None):
         arr, n = _deps(deps)
+        if route is not None:
+            return self.lib.mi355_aql_copy_route(self.handle, dst, src, nbytes, route, arr, n, completion)
         return self.lib.mi355_aql_copy(self.handle, dst, src, nbytes, arr, n, completion)
 
     def fill32(self, ptr, value, num_dwords, *, deps=None, completion=0):

@@ -23,6 +23,9 @@ STORE_CACHED = 0
 STORE_NT = 1
 STORE_AGENT_WT = 2
 STORE_SYSTEM_WT = 3
+ROUTE_DEVICE = 0
+ROUTE_HOST_TO_DEVICE = 1
+ROUTE_DEVICE_TO_HOST = 2
 
 
 class Plan(C.Structure):
@@ -31,7 +34,7 @@ class Plan(C.Structure):
         ("unroll", C.c_uint32), ("nt_load", C.c_uint32), ("store_policy", C.c_uint32),
         ("byte_shift", C.c_uint32), ("lead_vecs", C.c_uint32),
         ("head_bytes", C.c_uint64), ("body_vecs", C.c_uint64), ("tail_bytes", C.c_uint64),
-        ("xcd_run", C.c_uint32), ("reserved", C.c_uint32),
+        ("xcd_run", C.c_uint32), ("route", C.c_uint32),
     ]
 
     def as_dict(self):
@@ -85,6 +88,7 @@ SIGNATURES = {
     "mi355_blit_create": (C.c_int, [C.c_int, C.POINTER(C.c_void_p)]),
     "mi355_blit_destroy": (C.c_int, [C.c_void_p]),
     "mi355_blit_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "mi355_blit_copy_route": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint32, C.c_void_p]),
     "mi355_blit_fill32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t, C.c_void_p]),
     "mi355_blit_copy_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]),
     "mi355_blit_copy_batch_bounded": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint64, C.c_void_p]),
@@ -99,6 +103,8 @@ SIGNATURES = {
     "mi355_blit_last_launch_info": (C.c_int, [C.c_void_p, C.POINTER(Plan)]),
     "mi355_blit_plan_copy": (C.c_int, [C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint32,
                                        C.POINTER(Tuning), C.POINTER(Plan)]),
+    "mi355_blit_plan_copy_route": (C.c_int, [C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint32,
+                                             C.POINTER(Tuning), C.c_uint32, C.POINTER(Plan)]),
     "mi355_blit_plan_fill": (C.c_int, [C.c_uint64, C.c_uint64, C.c_uint32,
                                        C.POINTER(Tuning), C.POINTER(Plan)]),
     "mi355_blit_set_tuning": (C.c_int, [C.c_void_p, C.POINTER(Tuning)]),
@@ -172,7 +178,9 @@ class Blit:
     def __exit__(self, *exc):
         self.close()
 
-    def copy(self, dst, src, nbytes, stream=None):
+    def copy(self, dst, src, nbytes, stream=None, route=None):
+        if route is not None:
+            return self.lib.mi355_blit_copy_route(self.handle, dst, src, nbytes, route, stream)
         return self.lib.mi355_blit_copy(self.handle, dst, src, nbytes, stream)
 
     def fill32(self, ptr, value, num_dwords, stream=None):
@@ -220,10 +228,13 @@ class Blit:
         return self.lib.mi355_blit_stream(self.handle)
 
 
-def plan_copy(dst, src, nbytes, num_cus=256, tuning=None):
+def plan_copy(dst, src, nbytes, num_cus=256, tuning=None, route=None):
     p = Plan()
-    st = load().mi355_blit_plan_copy(dst, src, nbytes, num_cus,
-                                     C.byref(tuning) if tuning is not None else None, C.byref(p))
+    t = C.byref(tuning) if tuning is not None else None
+    if route is not None:
+        st = load().mi355_blit_plan_copy_route(dst, src, nbytes, num_cus, t, route, C.byref(p))
+    else:
+        st = load().mi355_blit_plan_copy(dst, src, nbytes, num_cus, t, C.byref(p))
     return st, p
 
 

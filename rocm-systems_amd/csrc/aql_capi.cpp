@@ -615,7 +615,13 @@ int mi355_aql_get_command_time(mi355_aql_t* h, uint64_t completion_signal, uint6
 
 int mi355_aql_copy(mi355_aql_t* h, void* dst, const void* src, size_t bytes, const uint64_t* dep_signals,
                    uint32_t num_deps, uint64_t completion_signal) {
-  if (!h || !dst || !src || (num_deps && !dep_signals)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  return mi355_aql_copy_route(h, dst, src, bytes, MI355_BLIT_ROUTE_DEVICE, dep_signals, num_deps, completion_signal);
+}
+
+int mi355_aql_copy_route(mi355_aql_t* h, void* dst, const void* src, size_t bytes, uint32_t route,
+                         const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal) {
+  if (!h || !dst || !src || (num_deps && !dep_signals) || route > MI355_BLIT_ROUTE_DEVICE_TO_HOST)
+    return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   if (h->queue_error.load()) return MI355_BLIT_ERROR;
   mi355_blit_plan_t p;
   const Kernel* k = nullptr;
@@ -624,7 +630,7 @@ int mi355_aql_copy(mi355_aql_t* h, void* dst, const void* src, size_t bytes, con
     std::lock_guard<std::mutex> g(h->lock);
     if (bytes) {
       int rc = plan_copy(reinterpret_cast<uint64_t>(dst), reinterpret_cast<uint64_t>(src), bytes, h->num_cus,
-                         h->has_tuning ? &h->tuning : nullptr, &p);
+                         h->has_tuning ? &h->tuning : nullptr, &p, route);
       if (rc != MI355_BLIT_SUCCESS) return rc;
       k = find_copy(h, p);
       if (!k) return MI355_BLIT_ERROR;

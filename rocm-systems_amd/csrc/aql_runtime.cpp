@@ -54,6 +54,18 @@ int classify(mi355_aql_t* h, const void* ptr, size_t size, Placement* out) {
   return MI355_BLIT_SUCCESS;
 }
 
+// The blit a GPU<->host copy goes to (GetPcieBlit, amd_gpu_agent.cpp:2370-2377):
+// host to device when the source is the host's, device to host otherwise.
+uint32_t route_of(bool src_is_host, bool dst_is_host) {
+  if (src_is_host && !dst_is_host) return MI355_BLIT_ROUTE_HOST_TO_DEVICE;
+  if (dst_is_host) return MI355_BLIT_ROUTE_DEVICE_TO_HOST;
+  return MI355_BLIT_ROUTE_DEVICE;
+}
+
+// Sizes from which the route changes the launch: below it a copy has too few
+// tiles for the shapes to differ, and a pointer lookup would only add latency.
+constexpr size_t kRouteLookupMinBytes = 1u << 20;
+
 // Locks [ptr, ptr+size) for the GPU when it is host memory the runtime does
 // not know (runtime.cpp:521-535); unlocks on destruction.
 class ScopedLock {
@@ -116,10 +128,10 @@ int bounced_copy(mi355_aql_t* h, void* dst, const void* src, size_t size, bool t
     if (to_device) {
       std::memcpy(buf[b], s + off, len);
       hsa_signal_store_relaxed(done[b], 1);
-      rc = mi355_aql_copy(h, d + off, buf[b], len, nullptr, 0, done[b].handle);
+      rc = mi355_aql_copy_route(h, d + off, buf[b], len, MI355_BLIT_ROUTE_HOST_TO_DEVICE, nullptr, 0, done[b].handle);
     } else {
       hsa_signal_store_relaxed(done[b], 1);
-      rc = mi355_aql_copy(h, buf[b], s + off, len, nullptr, 0, done[b].handle);
+      rc = mi355_aql_copy_route(h, buf[b], s + off, len, MI355_BLIT_ROUTE_DEVICE_TO_HOST, nullptr, 0, done[b].handle);
       // drain the previous piece while this one is in flight
       if (piece > 0) {
         wait(b ^ 1);
@@ -171,7 +183,8 @@ int mi355_hsa_memory_copy(mi355_aql_t* h, void* dst, const void* src, size_t siz
     if (lock_dst.Lock(h, dst, size, &mapped) != MI355_BLIT_SUCCESS) return bounced_copy(h, dst, src, size, false);
     d = mapped;
   }
-  if ((rc = mi355_aql_copy(h, d, s, size, nullptr, 0, 0)) != MI355_BLIT_SUCCESS) return rc;
+  if ((rc = mi355_aql_copy_route(h, d, s, size, route_of(src_sys, dst_sys), nullptr, 0, 0)) != MI355_BLIT_SUCCESS)
+    return rc;
   return mi355_aql_wait_idle(h);
 }
 
@@ -207,7 +220,13 @@ int mi355_hsa_amd_memory_async_copy(mi355_aql_t* h, void* dst, const void* src, 
   if (completion_signal == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   // hsa_ext_amd.cpp:285-293: size 0 succeeds and leaves the signal alone
   if (size == 0) return MI355_BLIT_SUCCESS;
-  return mi355_aql_copy(h, dst, src, size, dep_signals, num_dep_signals, completion_signal);
+  uint32_t route = MI355_BLIT_ROUTE_DEVICE;
+  if (size >= kRouteLookupMinBytes) {
+    Placement ps, pd;
+    if (classify(h, src, size, &ps) == MI355_BLIT_SUCCESS && classify(h, dst, size, &pd) == MI355_BLIT_SUCCESS)
+      route = route_of(ps.where != Where::kGpu, pd.where != Where::kGpu);
+  }
+  return mi355_aql_copy_route(h, dst, src, size, route, dep_signals, num_dep_signals, completion_signal);
 }
 
 namespace {

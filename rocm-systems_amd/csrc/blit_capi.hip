@@ -301,6 +301,11 @@ int mi355_blit_plan_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t nu
   return plan_copy(dst, src, bytes, num_cus, tuning, out);
 }
 
+int mi355_blit_plan_copy_route(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t num_cus,
+                               const mi355_blit_tuning_t* tuning, uint32_t route, mi355_blit_plan_t* out) {
+  return plan_copy(dst, src, bytes, num_cus, tuning, out, route);
+}
+
 int mi355_blit_plan_fill(uint64_t ptr, uint64_t num_dwords, uint32_t num_cus,
                          const mi355_blit_tuning_t* tuning, mi355_blit_plan_t* out) {
   return plan_fill(ptr, num_dwords, num_cus, tuning, out);
@@ -386,14 +391,19 @@ int mi355_blit_last_launch_info(mi355_blit_t* h, mi355_blit_plan_t* out) {
 }
 
 int mi355_blit_copy(mi355_blit_t* h, void* dst, const void* src, size_t bytes, void* stream) {
-  if (!h || !dst || !src) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  return mi355_blit_copy_route(h, dst, src, bytes, MI355_BLIT_ROUTE_DEVICE, stream);
+}
+
+int mi355_blit_copy_route(mi355_blit_t* h, void* dst, const void* src, size_t bytes, uint32_t route,
+                          void* stream) {
+  if (!h || !dst || !src || route > MI355_BLIT_ROUTE_DEVICE_TO_HOST) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   if (bytes == 0) return MI355_BLIT_SUCCESS;
   std::lock_guard<std::mutex> g(h->lock);
   DeviceScope scope(h->device);
   if (scope.err != hipSuccess) return status_of(scope.err);
   mi355_blit_plan_t p;
   int rc = plan_copy(reinterpret_cast<uint64_t>(dst), reinterpret_cast<uint64_t>(src), bytes,
-                     h->num_cus, h->has_tuning ? &h->tuning : nullptr, &p);
+                     h->num_cus, h->has_tuning ? &h->tuning : nullptr, &p, route);
   if (rc != MI355_BLIT_SUCCESS) return rc;
   copy_kernel_t k = select_copy_kernel(p);
   if (!k) return MI355_BLIT_ERROR;

@@ -192,7 +192,13 @@ class BlitKernelGfx950 : public core::Blit {
 // thread, no HIP.  This is the class that replaces AMD::BlitKernel in tree.
 class BlitKernelGfx950Aql : public core::Blit {
  public:
-  explicit BlitKernelGfx950Aql(core::Queue* queue);
+  /// Which of GpuAgent's blits_ slots the object fills
+  /// (core/inc/amd_gpu_agent.h:588): the linear copies of an object made for
+  /// BlitHostToDev or BlitDevToHost are launched in the shape that suits the
+  /// host link (MI355_BLIT_ROUTE_* in include/mi355_blit.h).
+  enum class Slot : uint32_t { kDevToDev = 0, kHostToDev = 1, kDevToHost = 2 };
+
+  explicit BlitKernelGfx950Aql(core::Queue* queue, Slot slot = Slot::kDevToDev);
   ~BlitKernelGfx950Aql() override;
 
   hsa_status_t Initialize(const core::Agent& agent);
@@ -224,6 +230,7 @@ class BlitKernelGfx950Aql : public core::Blit {
 
  private:
   core::Queue* queue_;
+  Slot slot_;
   mi355_aql* blit_;
   /// Completion signal of the blocking calls; guarded by lock_.
   hsa_signal_t completion_signal_;

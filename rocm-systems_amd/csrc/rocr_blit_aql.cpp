@@ -22,7 +22,12 @@ std::vector<uint64_t> handles(const std::vector<core::Signal*>& signals) {
 
 }  // namespace
 
-BlitKernelGfx950Aql::BlitKernelGfx950Aql(core::Queue* queue) : core::Blit(), queue_(queue), blit_(nullptr) {
+static_assert(static_cast<uint32_t>(BlitKernelGfx950Aql::Slot::kHostToDev) == MI355_BLIT_ROUTE_HOST_TO_DEVICE &&
+                  static_cast<uint32_t>(BlitKernelGfx950Aql::Slot::kDevToHost) == MI355_BLIT_ROUTE_DEVICE_TO_HOST,
+              "slots and routes count alike");
+
+BlitKernelGfx950Aql::BlitKernelGfx950Aql(core::Queue* queue, Slot slot)
+    : core::Blit(), queue_(queue), slot_(slot), blit_(nullptr) {
   completion_signal_.handle = 0;
 }
 
@@ -56,7 +61,8 @@ hsa_status_t BlitKernelGfx950Aql::SubmitLinearCopyCommand(void* dst, const void*
   std::lock_guard<std::mutex> guard(lock_);
   if (blit_ == nullptr) return HSA_STATUS_ERROR_NOT_INITIALIZED;
   hsa_signal_store_relaxed(completion_signal_, 1);
-  int st = mi355_aql_copy(blit_, dst, src, size, nullptr, 0, completion_signal_.handle);
+  int st = mi355_aql_copy_route(blit_, dst, src, size, static_cast<uint32_t>(slot_), nullptr, 0,
+                                completion_signal_.handle);
   if (st != MI355_BLIT_SUCCESS) return to_hsa(st);
   if (hsa_signal_wait_scacquire(completion_signal_, HSA_SIGNAL_CONDITION_LT, 1, uint64_t(-1),
                                 HSA_WAIT_STATE_ACTIVE) != 0) {
@@ -71,8 +77,9 @@ hsa_status_t BlitKernelGfx950Aql::SubmitLinearCopyCommand(void* dst, const void*
                                                           std::vector<core::Signal*>& /*gang_signals*/) {
   if (blit_ == nullptr) return HSA_STATUS_ERROR_NOT_INITIALIZED;
   const std::vector<uint64_t> deps = handles(dep_signals);
-  return to_hsa(mi355_aql_copy(blit_, dst, src, size, deps.empty() ? nullptr : deps.data(),
-                               static_cast<uint32_t>(deps.size()), core::Signal::Convert(&out_signal).handle));
+  return to_hsa(mi355_aql_copy_route(blit_, dst, src, size, static_cast<uint32_t>(slot_),
+                                     deps.empty() ? nullptr : deps.data(), static_cast<uint32_t>(deps.size()),
+                                     core::Signal::Convert(&out_signal).handle));
 }
 
 hsa_status_t BlitKernelGfx950Aql::SubmitLinearFillCommand(void* ptr, uint32_t value, size_t count) {

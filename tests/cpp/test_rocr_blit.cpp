@@ -369,6 +369,47 @@ void test_copy_rect(BlitKernelGfx950Aql& blit) {
   std::printf("PASS %s%s\n", name, g_suffix.c_str());
 }
 
+// Objects made for GpuAgent's BlitHostToDev / BlitDevToHost slots
+// (amd_gpu_agent.cpp:864-867) move a payload from pinned host memory into the
+// device and back out, blocking and with a signal.
+void test_host_link_slots(const rocr::core::Agent& agent) {
+  const char* name = "host_link_slots";
+  const size_t n = (6u << 20) + 13;
+  uint8_t *in = nullptr, *out = nullptr;
+  HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&in), n + 64, hipHostMallocDefault));
+  HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&out), n + 2 * kGuard, hipHostMallocDefault));
+  const std::vector<uint8_t> payload = seeded(n + 64, 0xB1170031);
+  std::memcpy(in, payload.data(), n + 64);
+  std::memset(out, kGuardByte, n + 2 * kGuard);
+  DeviceBuf dev(n + 2 * kGuard);
+  REQUIRE(dev.p, "hipMalloc");
+  std::vector<uint8_t> want(dev.n, kGuardByte), got;
+  REQUIRE(dev.upload(want), "upload");
+  BlitKernelGfx950Aql h2d(nullptr, BlitKernelGfx950Aql::Slot::kHostToDev);
+  BlitKernelGfx950Aql d2h(nullptr, BlitKernelGfx950Aql::Slot::kDevToHost);
+  REQUIRE(h2d.Initialize(agent) == HSA_STATUS_SUCCESS && d2h.Initialize(agent) == HSA_STATUS_SUCCESS, "Initialize");
+  hsa_status_t st = h2d.SubmitLinearCopyCommand(dev.p + kGuard + 5, in + 3, n);
+  REQUIRE(st == HSA_STATUS_SUCCESS, "host to device: status 0x%x", st);
+  oracle_copy(want.data() + kGuard + 5, payload.data() + 3, n);
+  REQUIRE(dev.download(got), "download");
+  REQUIRE(got == want, "host to device: bytes differ");
+  hsa_signal_t done = make_signal(1);
+  REQUIRE(done.handle, "signal");
+  std::vector<Signal*> none;
+  Signal out_signal(done);
+  st = d2h.SubmitLinearCopyCommand(out + kGuard + 1, dev.p + kGuard + 5, n, none, out_signal, none);
+  REQUIRE(st == HSA_STATUS_SUCCESS, "device to host: status 0x%x", st);
+  REQUIRE(wait_zero(done, HSA_WAIT_STATE_ACTIVE), "device to host: signal never reached 0");
+  std::vector<uint8_t> want_out(n + 2 * kGuard, kGuardByte);
+  oracle_copy(want_out.data() + kGuard + 1, payload.data() + 3, n);
+  REQUIRE(std::memcmp(out, want_out.data(), want_out.size()) == 0, "device to host: bytes differ");
+  hsa_signal_destroy(done);
+  REQUIRE(h2d.Destroy(agent) == HSA_STATUS_SUCCESS && d2h.Destroy(agent) == HSA_STATUS_SUCCESS, "Destroy");
+  (void)hipHostFree(in);
+  (void)hipHostFree(out);
+  std::printf("PASS %s%s\n", name, g_suffix.c_str());
+}
+
 void test_threads(Blit& blit) {
   const char* name = "concurrent_submitters";
   const int kThreads = 4, kPer = 6;
@@ -471,7 +512,7 @@ int main(int argc, char** argv) {
     for (const char* engine : {"_hip", "_aql"})
       for (const char* c : cases) std::printf("%s%s\n", c, engine);
     std::printf("async_copy_blocked_wait_hip_callback\nchain_a_to_b_to_c_hip_callback\n"
-                "profiling_timestamps_aql\ncopy_rect_with_signal_aql\n");
+                "profiling_timestamps_aql\ncopy_rect_with_signal_aql\nhost_link_slots_aql\n");
     return 0;
   }
   if (hsa_init() != HSA_STATUS_SUCCESS) {
@@ -538,6 +579,7 @@ int main(int argc, char** argv) {
     if (engine == 1) {
       test_profiling_timestamps(*blit);
       test_copy_rect(*static_cast<BlitKernelGfx950Aql*>(blit));
+      test_host_link_slots(agent);
     }
     latency_report(*blit, engine == 0 ? "hip_device_signal" : "aql");
     hsa_status_t st = blit->Destroy(agent);

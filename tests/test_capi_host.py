@@ -156,6 +156,39 @@ def test_plan_copy_shapes_by_size_and_offset(capi_host):
     assert st == 0 and p.xcd_run == 0
 
 
+def test_plan_copy_routes_across_the_host_link(capi_host):
+    """A copy one side of which is host memory is cut up like any other (the same
+    head / body / tail, the same kernel choice) but launched for the link: 128
+    workgroups of 256 at most, in launch order, stores to the host written
+    through.  The route of a plan within the device is 0 and changes nothing."""
+    MIB = 1 << 20
+    dst, src = 0x7f0000000000, 0x7e0000000000
+    wt, sys_wt, cached = capi_host.STORE_AGENT_WT, capi_host.STORE_SYSTEM_WT, capi_host.STORE_CACHED
+    h2d, d2h = capi_host.ROUTE_HOST_TO_DEVICE, capi_host.ROUTE_DEVICE_TO_HOST
+    for off in (0, 3):
+        for n in (1, 4096, 512 * 1024 + 5, 3 * MIB, 4 * MIB, 256 * MIB + 1, 1 << 32):
+            st, dev = capi_host.plan_copy(dst + 9, src + 9 + off, n)
+            assert st == 0 and dev.route == capi_host.ROUTE_DEVICE
+            st, same = capi_host.plan_copy(dst + 9, src + 9 + off, n, route=capi_host.ROUTE_DEVICE)
+            assert st == 0 and same.as_dict() == dev.as_dict()
+            for route, store_small, store_large in ((h2d, cached, wt), (d2h, sys_wt, sys_wt)):
+                st, p = capi_host.plan_copy(dst + 9, src + 9 + off, n, route=route)
+                assert st == 0 and p.route == route
+                # the cut and the kernel do not depend on the route
+                for f in ("kernel", "byte_shift", "lead_vecs", "head_bytes", "body_vecs", "tail_bytes"):
+                    assert getattr(p, f) == getattr(dev, f), f
+                assert (p.wg_size, p.unroll, p.xcd_run) == (256, 1, 0)
+                assert p.nt_load == (1 if n >= 4 * MIB else 0)
+                assert p.store_policy == (store_large if n >= 4 * MIB else store_small)
+                tiles = (p.body_vecs + p.lead_vecs + 63) // 64
+                assert p.grid == min(128, (tiles + 1 + 3) // 4)
+    # tuning still overrides the cap; an unknown route is refused
+    st, p = capi_host.plan_copy(dst, src, 1 << 30, 256, capi_host.Tuning(max_grid=512), route=h2d)
+    assert st == 0 and p.grid == 512
+    st, p = capi_host.plan_copy(dst, src, 1 << 30, route=3)
+    assert st == capi_host.ERROR_INVALID_ARGUMENT
+
+
 def test_plan_fill_invariants(capi_host):
     for off in (0, 4, 8, 12):
         ptr = 0x7f0000000000 + off

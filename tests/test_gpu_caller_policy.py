@@ -83,6 +83,73 @@ def test_memory_copy_pinned_host(eng, oracle, rand, torch_cuda):
     assert np.array_equal(out.numpy()[2:2 + n], payload[1:1 + n]) and out.numpy()[0] == 0xEE
 
 
+@pytest.mark.parametrize("n,s_off,d_off", [(1, 0, 0), (4099, 3, 9), (MIB + 3, 5, 0), (5 * MIB + 77, 0, 4),
+                                          (40 * MIB + 1, 13, 6)])
+def test_copies_across_the_host_link_are_exact(eng, capi, oracle, rand, torch_cuda, n, s_off, d_off):
+    """Host to device and device to host on the routes made for the link (pinned
+    host memory, both submission paths): the launch is the link's shape, the bytes
+    are the oracle's and the guard bytes stay."""
+    torch = torch_cuda
+    h2d, d2h = capi.ROUTE_HOST_TO_DEVICE, capi.ROUTE_DEVICE_TO_HOST
+    payload = rand(n + 64, 0xB1170021)
+    pinned = torch.empty(n + 64, dtype=torch.uint8, pin_memory=True)
+    pinned.numpy()[:] = payload
+    want_dev = _host(n + 2 * GUARD)
+    oracle.oracle_copy(want_dev.ctypes.data + GUARD + d_off, payload.ctypes.data + s_off, n)
+    want_out = _host(n + 2 * GUARD)
+    oracle.oracle_copy(want_out.ctypes.data + GUARD + s_off, want_dev.ctypes.data + GUARD + d_off, n)
+    with capi.Blit(0) as blit:
+        for path in ("aql", "hip"):
+            dev = torch.full((n + 2 * GUARD,), 0xEE, dtype=torch.uint8, device="cuda:0")
+            out = torch.full((n + 2 * GUARD,), 0xEE, dtype=torch.uint8).pin_memory()
+            torch.cuda.synchronize()
+            for route, dst, src in ((h2d, dev.data_ptr() + GUARD + d_off, pinned.data_ptr() + s_off),
+                                    (d2h, out.data_ptr() + GUARD + s_off, dev.data_ptr() + GUARD + d_off)):
+                if path == "aql":
+                    assert eng.copy(dst, src, n, route=route) == 0
+                    assert eng.synchronize() == 0
+                    p = eng.last_plan()
+                else:
+                    assert blit.copy(dst, src, n, route=route) == 0
+                    assert blit.synchronize() == 0
+                    p = blit.last_plan()
+                assert p.route == route and p.wg_size == 256 and p.grid <= 128 and p.xcd_run == 0
+                assert p.byte_shift == ((s_off - d_off) & 3 if route == h2d else (d_off - s_off) & 3)
+            assert np.array_equal(dev.cpu().numpy(), want_dev), path
+            assert np.array_equal(out.numpy(), want_out), path
+    assert eng.copy(dev.data_ptr(), pinned.data_ptr(), 16, route=3) == capi.ERROR_INVALID_ARGUMENT
+
+
+def test_caller_policy_takes_the_route_the_placements_give(eng, signals, capi, rand, torch_cuda):
+    """hsa_memory_copy classifies both pointers anyway and routes every size; the
+    asynchronous copy has no agents in its signature and looks the pointers up
+    from 1 MiB on, where the launch shape starts to depend on the route."""
+    torch = torch_cuda
+    n = 2 * MIB
+    pinned = torch.empty(n, dtype=torch.uint8, pin_memory=True)
+    pinned.numpy()[:] = rand(n, 0xB1170022)
+    dev = torch.zeros(n, dtype=torch.uint8, device="cuda:0")
+    dev2 = torch.zeros(n, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    assert eng.hsa_memory_copy(dev.data_ptr(), pinned.data_ptr(), n) == 0
+    assert eng.last_plan().route == capi.ROUTE_HOST_TO_DEVICE
+    assert eng.hsa_memory_copy(pinned.data_ptr(), dev.data_ptr(), 4096) == 0
+    assert eng.last_plan().route == capi.ROUTE_DEVICE_TO_HOST
+    assert eng.hsa_memory_copy(dev2.data_ptr(), dev.data_ptr(), n) == 0
+    assert eng.last_plan().route == capi.ROUTE_DEVICE
+    done = signals.create(1)
+    for dst, src, size, route in ((dev2.data_ptr(), pinned.data_ptr(), n, capi.ROUTE_HOST_TO_DEVICE),
+                                  (pinned.data_ptr(), dev.data_ptr(), n, capi.ROUTE_DEVICE_TO_HOST),
+                                  (dev2.data_ptr(), dev.data_ptr(), n, capi.ROUTE_DEVICE),
+                                  (dev2.data_ptr(), pinned.data_ptr(), n // 4, capi.ROUTE_DEVICE)):
+        signals.store(done, 1)
+        assert eng.hsa_amd_memory_async_copy(dst, src, size, None, done) == 0
+        signals.wait_below_one(done)
+        assert eng.last_plan().route == route
+    signals.destroy(done)
+    assert torch.equal(dev2.cpu(), pinned) and torch.equal(dev.cpu(), pinned)
+
+
 def test_memory_copy_api_edge(eng, torch_cuda):
     """hsa.cpp:1174-1180"""
     torch = torch_cuda

@@ -218,6 +218,14 @@ int mi355_blit_copy_rect(mi355_blit_t* h, const mi355_pitched_ptr_t* dst, const 
                          const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
                          const mi355_dim3_t* range, void* stream);
 
+/* mi355_blit_copy_rect for a region one side of which is host memory the GPU
+ * can access: route is MI355_BLIT_ROUTE_*, the hsa_amd_copy_direction_t of
+ * hsa_amd_memory_async_copy_rect (inc/hsa_ext_amd.h, hsaHostToDevice = 1,
+ * hsaDeviceToHost = 2) with 0 for a copy within the device. */
+int mi355_blit_copy_rect_route(mi355_blit_t* h, const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
+                               const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
+                               const mi355_dim3_t* range, uint32_t route, void* stream);
+
 /* How mi355_blit_copy_rect launches a region: pure host arithmetic, for
  * harnesses.  Rows (and layers) that are contiguous on both sides are merged
  * first; a region that merges into one run is a linear copy (linear = 1,
@@ -246,13 +254,17 @@ typedef struct {
   uint32_t plain_rows; /* rows tiled like a linear copy (256-byte aligned on the
                           destination side, whole units long, a multiple of 4
                           bytes from their source): the kernel's short path */
-  uint32_t reserved;
+  uint32_t route;      /* MI355_BLIT_ROUTE_* the launch was shaped for */
 } mi355_blit_rect_plan_t;
 
 int mi355_blit_plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
                          const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
                          const mi355_dim3_t* range, const mi355_blit_tuning_t* tuning,
                          mi355_blit_rect_plan_t* out);
+int mi355_blit_plan_rect_route(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
+                               const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
+                               const mi355_dim3_t* range, const mi355_blit_tuning_t* tuning, uint32_t route,
+                               mi355_blit_rect_plan_t* out);
 
 /* Decrements an HSA signal by 1 from the GPU once every command submitted
  * before it on the stream has completed, and wakes its waiters: replaces the

@@ -97,6 +97,16 @@ int mi355_aql_copy_rect(mi355_aql_t* h, const mi355_pitched_ptr_t* dst, const mi
                         const mi355_dim3_t* range, const uint64_t* dep_signals, uint32_t num_deps,
                         uint64_t completion_signal);
 
+/* mi355_aql_copy_rect for a region one side of which is host memory
+ * (mi355_blit_copy_rect_route in mi355_blit.h): the direction argument of
+ * hsa_amd_memory_async_copy_rect, which GpuAgent::DmaCopyRect turns into the
+ * choice between blits_[BlitHostToDev] and blits_[BlitDevToHost]
+ * (amd_gpu_agent.cpp:1265-1266). */
+int mi355_aql_copy_rect_route(mi355_aql_t* h, const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
+                              const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
+                              const mi355_dim3_t* range, uint32_t route, const uint64_t* dep_signals,
+                              uint32_t num_deps, uint64_t completion_signal);
+
 /* Blocks until the queue has drained: the wait BlitKernel's blocking calls do
  * on their completion signal (amd_blit_kernel.cpp:632, 830). */
 int mi355_aql_wait_idle(mi355_aql_t* h);
@@ -209,7 +219,9 @@ int mi355_hsa_amd_memory_copy_engine_status(mi355_aql_t* h, int dst_is_gpu, int 
  * that disagrees with the array pointer, a zero completion signal or
  * dir == 0 (hsaHostToHost) -> INVALID_ARGUMENT; a zero in range -> SUCCESS
  * without touching the signal (:400-402).  Where the reference then fails with
- * OUT_OF_RESOURCES unless an SDMA engine is available, this runs the shader. */
+ * OUT_OF_RESOURCES unless an SDMA engine is available, this runs the shader,
+ * on the route dir names (hsaHostToDevice = 1, hsaDeviceToHost = 2; any other
+ * value, hsaDeviceToDevice = 3 included, within the device). */
 int mi355_hsa_amd_memory_async_copy_rect(mi355_aql_t* h, const mi355_pitched_ptr_t* dst,
                                          const mi355_dim3_t* dst_offset, const mi355_pitched_ptr_t* src,
                                          const mi355_dim3_t* src_offset, const mi355_dim3_t* range, int dir,

@@ -22,6 +22,9 @@ SIGNATURES = {
                                                C.c_uint64]),
     "mi355_aql_copy_rect": (C.c_int, [C.c_void_p, C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
                                       C.POINTER(Dim3), C.POINTER(Dim3), _U64P, C.c_uint32, C.c_uint64]),
+    "mi355_aql_copy_rect_route": (C.c_int, [C.c_void_p, C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
+                                            C.POINTER(Dim3), C.POINTER(Dim3), C.c_uint32, _U64P, C.c_uint32,
+                                            C.c_uint64]),
     "mi355_aql_wait_idle": (C.c_int, [C.c_void_p]),
     "mi355_aql_pending_bytes": (C.c_uint64, [C.c_void_p]),
     "mi355_aql_enable_profiling": (C.c_int, [C.c_void_p, C.c_int]),
@@ -125,10 +128,12 @@ class AqlBlit:
         addr = device_descs if isinstance(device_descs, int) or device_descs is None else C.cast(device_descs, C.c_void_p)
         return self.lib.mi355_aql_copy_batch_bounded(self.handle, addr, n, max_total_bytes, arr, nd, completion)
 
-    def copy_rect(self, dst, dst_offset, src, src_offset, extent, *, deps=None, completion=0):
+    def copy_rect(self, dst, dst_offset, src, src_offset, extent, *, deps=None, completion=0, route=None):
         """dst, src: (base, pitch, slice); offsets and extent: (x bytes, y rows, z layers)."""
         arr, n = _deps(deps)
         a = rect_args(dst, dst_offset, src, src_offset, extent)
+        if route is not None:
+            return self.lib.mi355_aql_copy_rect_route(self.handle, *a, route, arr, n, completion)
         return self.lib.mi355_aql_copy_rect(self.handle, *a, arr, n, completion)
 
     def synchronize(self):

@@ -69,7 +69,7 @@ class RectPlan(C.Structure):
         ("slots", C.c_uint32), ("unroll", C.c_uint32), ("lanes_per_row", C.c_uint32),
         ("xcd_run", C.c_uint32), ("wg_size", C.c_uint32), ("grid", C.c_uint32),
         ("nt_load", C.c_uint32), ("store_policy", C.c_uint32), ("total_bytes", C.c_uint64),
-        ("plain_rows", C.c_uint32), ("reserved", C.c_uint32),
+        ("plain_rows", C.c_uint32), ("route", C.c_uint32),
     ]
 
 
@@ -96,6 +96,11 @@ SIGNATURES = {
                                        C.POINTER(Dim3), C.POINTER(Dim3), C.c_void_p]),
     "mi355_blit_plan_rect": (C.c_int, [C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
                                        C.POINTER(Dim3), C.POINTER(Dim3), C.POINTER(Tuning), C.POINTER(RectPlan)]),
+    "mi355_blit_copy_rect_route": (C.c_int, [C.c_void_p, C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
+                                             C.POINTER(Dim3), C.POINTER(Dim3), C.c_uint32, C.c_void_p]),
+    "mi355_blit_plan_rect_route": (C.c_int, [C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
+                                             C.POINTER(Dim3), C.POINTER(Dim3), C.POINTER(Tuning), C.c_uint32,
+                                             C.POINTER(RectPlan)]),
     "mi355_blit_signal_complete": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p]),
     "mi355_blit_add_callback": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "mi355_blit_synchronize": (C.c_int, [C.c_void_p]),
@@ -195,9 +200,11 @@ class Blit:
         addr = device_descs if isinstance(device_descs, int) or device_descs is None else C.cast(device_descs, C.c_void_p)
         return self.lib.mi355_blit_copy_batch_bounded(self.handle, addr, n, max_total_bytes, stream)
 
-    def copy_rect(self, dst, dst_offset, src, src_offset, extent, stream=None):
+    def copy_rect(self, dst, dst_offset, src, src_offset, extent, stream=None, route=None):
         """dst, src: (base, pitch, slice); offsets and extent: (x bytes, y rows, z layers)."""
         a = rect_args(dst, dst_offset, src, src_offset, extent)
+        if route is not None:
+            return self.lib.mi355_blit_copy_rect_route(self.handle, *a, route, stream)
         return self.lib.mi355_blit_copy_rect(self.handle, *a, stream)
 
     def synchronize(self):
@@ -238,11 +245,14 @@ def plan_copy(dst, src, nbytes, num_cus=256, tuning=None, route=None):
     return st, p
 
 
-def plan_rect(dst, dst_offset, src, src_offset, extent, tuning=None):
+def plan_rect(dst, dst_offset, src, src_offset, extent, tuning=None, route=None):
     """(status, RectPlan) for a region given as in Blit.copy_rect."""
     out = RectPlan()
     a = rect_args(dst, dst_offset, src, src_offset, extent)
-    st = load().mi355_blit_plan_rect(*a, tuning, C.byref(out))
+    if route is not None:
+        st = load().mi355_blit_plan_rect_route(*a, tuning, route, C.byref(out))
+    else:
+        st = load().mi355_blit_plan_rect(*a, tuning, C.byref(out))
     return st, out
 
 

@@ -895,13 +895,21 @@ int mi355_aql_copy_rect(mi355_aql_t* h, const mi355_pitched_ptr_t* dst, const mi
                         const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
                         const mi355_dim3_t* range, const uint64_t* dep_signals, uint32_t num_deps,
                         uint64_t completion_signal) {
+  return mi355_aql_copy_rect_route(h, dst, dst_offset, src, src_offset, range, MI355_BLIT_ROUTE_DEVICE, dep_signals,
+                                   num_deps, completion_signal);
+}
+
+int mi355_aql_copy_rect_route(mi355_aql_t* h, const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
+                              const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
+                              const mi355_dim3_t* range, uint32_t route, const uint64_t* dep_signals,
+                              uint32_t num_deps, uint64_t completion_signal) {
   if (!h || (num_deps && !dep_signals)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   if (h->queue_error.load()) return MI355_BLIT_ERROR;
   RectPlan rp;
   const Kernel* k = nullptr;
   {
     std::lock_guard<std::mutex> g(h->lock);
-    int rc = plan_rect(dst, dst_offset, src, src_offset, range, h->has_tuning ? &h->tuning : nullptr, &rp);
+    int rc = plan_rect(dst, dst_offset, src, src_offset, range, h->has_tuning ? &h->tuning : nullptr, &rp, route);
     if (rc != MI355_BLIT_SUCCESS) return rc;
     if (!rp.empty && !rp.linear) {
       if (rp.narrow) {
@@ -916,7 +924,9 @@ int mi355_aql_copy_rect(mi355_aql_t* h, const mi355_pitched_ptr_t* dst, const mi
     }
   }
   if (rp.empty) return mi355_aql_copy(h, h, h, 0, dep_signals, num_deps, completion_signal);
-  if (rp.linear) return mi355_aql_copy(h, rp.args.dst, rp.args.src, rp.args.width, dep_signals, num_deps, completion_signal);
+  if (rp.linear)
+    return mi355_aql_copy_route(h, rp.args.dst, rp.args.src, rp.args.width, route, dep_signals, num_deps,
+                                completion_signal);
   const uint32_t nb = barrier_packets(num_deps);
   const uint32_t total = nb + 1;
   uint64_t index;

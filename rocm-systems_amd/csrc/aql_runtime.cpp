@@ -307,8 +307,12 @@ int mi355_hsa_amd_memory_async_copy_rect(mi355_aql_t* h, const mi355_pitched_ptr
   if (completion_signal == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   // hsa_ext_amd.cpp:400-405: an empty range succeeds and leaves the signal alone
   if (range->x == 0 || range->y == 0 || range->z == 0) return MI355_BLIT_SUCCESS;
-  return mi355_aql_copy_rect(h, dst, dst_offset, src, src_offset, range, dep_signals, num_dep_signals,
-                             completion_signal);
+  // hsa_amd_copy_direction_t: amd_gpu_agent.cpp:1265-1266 picks the blit by it
+  const uint32_t route = dir == 1 /* hsaHostToDevice */   ? MI355_BLIT_ROUTE_HOST_TO_DEVICE
+                         : dir == 2 /* hsaDeviceToHost */ ? MI355_BLIT_ROUTE_DEVICE_TO_HOST
+                                                          : MI355_BLIT_ROUTE_DEVICE;
+  return mi355_aql_copy_rect_route(h, dst, dst_offset, src, src_offset, range, route, dep_signals, num_dep_signals,
+                                   completion_signal);
 }
 
 }  // extern "C"

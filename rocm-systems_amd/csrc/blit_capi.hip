@@ -618,15 +618,21 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
 int mi355_blit_copy_rect(mi355_blit_t* h, const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
                          const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
                          const mi355_dim3_t* range, void* stream) {
+  return mi355_blit_copy_rect_route(h, dst, dst_offset, src, src_offset, range, MI355_BLIT_ROUTE_DEVICE, stream);
+}
+
+int mi355_blit_copy_rect_route(mi355_blit_t* h, const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
+                               const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
+                               const mi355_dim3_t* range, uint32_t route, void* stream) {
   if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   RectPlan rp;
   {
     std::lock_guard<std::mutex> g(h->lock);
-    int rc = plan_rect(dst, dst_offset, src, src_offset, range, h->has_tuning ? &h->tuning : nullptr, &rp);
+    int rc = plan_rect(dst, dst_offset, src, src_offset, range, h->has_tuning ? &h->tuning : nullptr, &rp, route);
     if (rc != MI355_BLIT_SUCCESS) return rc;
   }
   if (rp.empty) return MI355_BLIT_SUCCESS;
-  if (rp.linear) return mi355_blit_copy(h, rp.args.dst, rp.args.src, rp.args.width, stream);
+  if (rp.linear) return mi355_blit_copy_route(h, rp.args.dst, rp.args.src, rp.args.width, route, stream);
   std::lock_guard<std::mutex> g(h->lock);
   DeviceScope scope(h->device);
   if (scope.err != hipSuccess) return status_of(scope.err);
@@ -651,9 +657,16 @@ int mi355_blit_plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst
                          const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
                          const mi355_dim3_t* range, const mi355_blit_tuning_t* tuning,
                          mi355_blit_rect_plan_t* out) {
+  return mi355_blit_plan_rect_route(dst, dst_offset, src, src_offset, range, tuning, MI355_BLIT_ROUTE_DEVICE, out);
+}
+
+int mi355_blit_plan_rect_route(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
+                               const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,
+                               const mi355_dim3_t* range, const mi355_blit_tuning_t* tuning, uint32_t route,
+                               mi355_blit_rect_plan_t* out) {
   if (!out) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   RectPlan rp;
-  int rc = plan_rect(dst, dst_offset, src, src_offset, range, tuning, &rp);
+  int rc = plan_rect(dst, dst_offset, src, src_offset, range, tuning, &rp, route);
   if (rc != MI355_BLIT_SUCCESS) return rc;
   *out = mi355_blit_rect_plan_t{};
   out->empty = rp.empty;
@@ -662,6 +675,7 @@ int mi355_blit_plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst
   out->src = reinterpret_cast<uint64_t>(rp.args.src);
   out->width = rp.args.width;
   out->total_bytes = rp.total_bytes;
+  out->route = rp.route;
   if (rp.empty || rp.linear) return MI355_BLIT_SUCCESS;
   out->dst_pitch = rp.args.dst_pitch;
   out->dst_slice = rp.args.dst_slice;

@@ -34,6 +34,7 @@ struct RectPlan {
   uint32_t wg_size;
   uint32_t grid;
   uint32_t xcd_run;    // runs of workgroups per XCD, 0 = launch order
+  uint32_t route;      // MI355_BLIT_ROUTE_*
 };
 
 // Units of `unit` vectors that a row of `width` bytes is cut into when its
@@ -57,9 +58,20 @@ inline uint64_t rect_gcd(uint64_t a, uint64_t b) {
 
 inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset, const mi355_pitched_ptr_t* src,
                      const mi355_dim3_t* src_offset, const mi355_dim3_t* range, const mi355_blit_tuning_t* t,
-                     RectPlan* out) {
-  if (!dst || !dst_offset || !src || !src_offset || !range || !out) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+                     RectPlan* out, uint32_t route = MI355_BLIT_ROUTE_DEVICE) {
+  if (!dst || !dst_offset || !src || !src_offset || !range || !out || route > MI355_BLIT_ROUTE_DEVICE_TO_HOST)
+    return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   *out = RectPlan{};
+  out->route = route;
+  // A region one side of which is host memory moves at the host link's rate:
+  // as for a linear copy (kHostLinkMaxGrid), at most 128 workgroups of 256
+  // walk the rows in address order, and stores to the host are written through
+  // at once.  Measured with pinned memory, 256 MiB in rows of 64 KiB, 4 KiB and
+  // 256 bytes: 57.2 GB/s from the host and 57.0 GB/s to it (the runtime's DMA
+  // engines: 57.5 / 57.0, and 43.7 for the 256-byte rows) against 54-55 GB/s
+  // in the shapes made for HBM.
+  const bool link = route != MI355_BLIT_ROUTE_DEVICE;
+  const uint64_t link_max_grid = link ? kHostLinkMaxGrid : 0;
   if (range->x == 0 || range->y == 0 || range->z == 0) {
     out->empty = true;
     return MI355_BLIT_SUCCESS;
@@ -115,7 +127,10 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
   if (t && t->nt_load) streaming = (t->nt_load == 2);
   out->streaming = streaming;
   out->store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
-  if (t && t->store_policy >= 1 && t->store_policy <= 4) out->store_policy = t->store_policy - 1;
+  const bool store_tuned = t && t->store_policy >= 1 && t->store_policy <= 4;
+  if (store_tuned) out->store_policy = t->store_policy - 1;
+  const bool to_host = route == MI355_BLIT_ROUTE_DEVICE_TO_HOST && !store_tuned;
+  if (to_host) out->store_policy = MI355_BLIT_STORE_SYSTEM_WT;
 
   // every store of every row is a whole cache line
   const bool whole_lines = reinterpret_cast<uintptr_t>(d0) % 128 == 0 && dp % 128 == 0 && width % 128 == 0 &&
@@ -153,19 +168,19 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
     // one CU (520 B rows at a 1 KiB pitch, 33 lanes a row: 241 us with workgroups
     // of 256, 283 us with single waves, whose neighbours run on other XCDs), and
     // non-temporal stores.
-    if (whole_lines && streaming && !(t && t->store_policy >= 1 && t->store_policy <= 4))
-      out->store_policy = MI355_BLIT_STORE_AGENT_WT;
+    if (whole_lines && streaming && !store_tuned && !to_host) out->store_policy = MI355_BLIT_STORE_AGENT_WT;
     // No two waves touch the same destination line when rows are whole lines,
     // or when waves hold whole rows and neighbouring rows are a line apart.
     const bool rows_apart = dp >= width + 127 && (layers == 1 || ds >= (rows - 1) * dp + width + 127);
     const bool waves_apart = whole_lines || (64 % n.lanes_per_row == 0 && rows_apart);
     out->wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size
-                   : waves_apart                                                           ? 64
+                   : waves_apart && !link                                                  ? 64
                                                                                             : 256;
     const uint64_t waves_per_wg = out->wg_size / 64;
     const uint64_t groups = (rows * layers * n.lanes_per_row + 63) / 64;
     uint64_t wgs = (groups + waves_per_wg - 1) / waves_per_wg;
-    if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
+    const uint64_t max_grid = (t && t->max_grid) ? t->max_grid : link_max_grid;
+    if (max_grid && wgs > max_grid) wgs = max_grid;
     if (wgs * out->wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / out->wg_size;
     out->grid = static_cast<uint32_t>(wgs);
     n.waves_per_wg = static_cast<uint32_t>(waves_per_wg);
@@ -176,7 +191,7 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
     // 520-byte rows at 1 KiB 455-462 against 489-501); waves that share none
     // gain nothing from it.
     uint32_t run = 0;
-    if (!waves_apart && out->total_bytes >= kXcdRunMinBytes) {
+    if (!waves_apart && !link && out->total_bytes >= kXcdRunMinBytes) {
       const uint64_t rows_per_wave = 64 / n.lanes_per_row;  // >= 1
       const uint64_t span = waves_per_wg * (rows_per_wave * dp > 1024 ? rows_per_wave * dp : 1024);
       run = static_cast<uint32_t>(kXcdRunBytes / span);
@@ -196,8 +211,11 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
   // there: the rows' cut ends are partial lines).
   uint32_t unroll = whole_lines ? 1 : 2;
   uint32_t default_wg = whole_lines ? 256 : 128;
-  if (whole_lines && streaming && !(t && t->store_policy >= 1 && t->store_policy <= 4))
-    out->store_policy = MI355_BLIT_STORE_AGENT_WT;
+  if (link) {
+    unroll = 1;
+    default_wg = 256;
+  }
+  if (whole_lines && streaming && !store_tuned && !to_host) out->store_policy = MI355_BLIT_STORE_AGENT_WT;
   if (t && (t->unroll == 1 || t->unroll == 2 || t->unroll == 4)) unroll = t->unroll;
   out->unroll = unroll;
   // Row destinations differ by multiples of g modulo 256: the largest unit
@@ -230,12 +248,13 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
   // runs of 576 units at most 12 % (8 KiB rows at a 16 KiB pitch, 361 us against
   // 321 us) and within 2 % everywhere else.  Which shape wins for a given pitch
   // follows the memory channels' interleave, not the kernel.
-  const bool plain_runs = a.plain_rows && out->total_bytes >= kXcdRunMinBytes;
+  const bool plain_runs = a.plain_rows && !link && out->total_bytes >= kXcdRunMinBytes;
   if (plain_runs) default_wg = 64;
   out->wg_size = (t && t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) ? t->wg_size : default_wg;
   const uint64_t waves_per_wg = out->wg_size / 64;
   uint64_t wgs = (total_slots + waves_per_wg - 1) / waves_per_wg;
-  if (t && t->max_grid && wgs > t->max_grid) wgs = t->max_grid;
+  const uint64_t max_grid = (t && t->max_grid) ? t->max_grid : link_max_grid;
+  if (max_grid && wgs > max_grid) wgs = max_grid;
   if (wgs * out->wg_size > kMaxGridWorkItems) wgs = kMaxGridWorkItems / out->wg_size;
   out->grid = static_cast<uint32_t>(wgs);
   a.waves_per_wg = static_cast<uint32_t>(waves_per_wg);
@@ -246,7 +265,7 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
   // Whole-line rows that are not plain go through the general path of the
   // kernel, where runs lose (347 us against 330 us).
   uint32_t run = 0;
-  if ((!whole_lines || plain_runs) && out->total_bytes >= kXcdRunMinBytes)
+  if ((!whole_lines || plain_runs) && !link && out->total_bytes >= kXcdRunMinBytes)
     run = static_cast<uint32_t>(kXcdRunBytes / (waves_per_wg * 1024 * unroll));
   out->xcd_run = plan_xcd_run(run, t);
   a.xcd = make_xcd_runs(out->grid, out->xcd_run);
@@ -262,6 +281,7 @@ inline void rect_launch_info(const RectPlan& rp, mi355_blit_plan_t* p) {
   p->nt_load = rp.streaming;
   p->store_policy = rp.store_policy;
   p->xcd_run = rp.xcd_run;
+  p->route = rp.route;
   p->body_vecs = rp.narrow ? rp.nargs.lines : rp.args.total_slots;  // rows, or chunk slots
 }
 

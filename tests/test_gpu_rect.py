@@ -312,3 +312,61 @@ def test_async_copy_rect_stand_in(capi, pkg, oracle, rand, torch_cuda):
         sig.destroy(done)
     finally:
         eng.close()
+
+
+LINK_CASES = [
+    # (z, y, pitch) of both surfaces, extent (x, y, z), src offset, dst offset
+    ((1, 600, 8192), (4096, 600, 1), (0, 0, 0), (4096, 0, 0)),       # plain rows
+    ((2, 90, 20000), (16385, 80, 2), (3001, 3, 0), (17, 9, 0)),      # any alignment, wide rows
+    ((1, 5000, 512), (256, 5000, 1), (0, 0, 0), (256, 0, 0)),        # narrow rows of whole lines
+    ((3, 700, 261), (100, 650, 3), (13, 20, 0), (150, 1, 0)),        # narrow rows, every alignment
+    ((2, 50, 4096), (4096, 50, 2), (0, 0, 0), (0, 0, 0)),            # merges into one run: a linear copy
+]
+
+
+@pytest.mark.parametrize("case", range(len(LINK_CASES)))
+def test_rect_across_the_host_link(capi, blit, pkg, oracle, rand, torch_cuda, case):
+    """Regions between pinned host surfaces and device surfaces on the routes made
+    for the host link, over the HIP path (route argument) and over the stand-in
+    for hsa_amd_memory_async_copy_rect (its direction argument): the launch is the
+    link's shape and both destination surfaces, guard bytes included, are the
+    oracle's."""
+    torch = torch_cuda
+    shape, ext, so, do = LINK_CASES[case]
+    nbytes = int(np.prod(shape))
+    pitched = lambda base: (base, shape[2], shape[1] * shape[2])
+    payload = rand(nbytes, 0x11CC0000 + case)
+    host_in = torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+    host_in.numpy()[:] = payload
+    want_dev = np.full(nbytes, GUARD_BYTE, dtype=np.uint8)
+    oracle_rect(oracle, pitched(want_dev.ctypes.data), do, pitched(payload.ctypes.data), so, ext)
+    want_out = np.full(nbytes, GUARD_BYTE, dtype=np.uint8)
+    oracle_rect(oracle, pitched(want_out.ctypes.data), so, pitched(want_dev.ctypes.data), do, ext)
+    eng = pkg.aql.AqlBlit(0)
+    sig = pkg.aql.HsaSignals()
+    done = sig.create(1)
+    try:
+        for path in ("hip", "aql"):
+            dev = torch.full((nbytes,), GUARD_BYTE, dtype=torch.uint8, device="cuda:0")
+            host_out = torch.full((nbytes,), GUARD_BYTE, dtype=torch.uint8).pin_memory()
+            torch.cuda.synchronize()
+            legs = ((capi.ROUTE_HOST_TO_DEVICE, pitched(dev.data_ptr()), do, pitched(host_in.data_ptr()), so),
+                    (capi.ROUTE_DEVICE_TO_HOST, pitched(host_out.data_ptr()), so, pitched(dev.data_ptr()), do))
+            for route, dp, d_at, sp, s_at in legs:
+                if path == "hip":
+                    assert blit.copy_rect(dp, d_at, sp, s_at, ext, route=route) == capi.SUCCESS
+                    assert blit.synchronize() == capi.SUCCESS
+                    p = blit.last_plan()
+                else:
+                    sig.store(done, 1)
+                    assert eng.hsa_amd_memory_async_copy_rect(dp, d_at, sp, s_at, ext, route, None, done) == capi.SUCCESS
+                    sig.wait_below_one(done)
+                    p = eng.last_plan()
+                assert p.route == route and p.wg_size == 256 and p.grid <= 128 and p.xcd_run == 0
+                if route == capi.ROUTE_DEVICE_TO_HOST and nbytes >= 4 * MIB:
+                    assert p.store_policy == capi.STORE_SYSTEM_WT
+            assert np.array_equal(dev.cpu().numpy(), want_dev), path
+            assert np.array_equal(host_out.numpy(), want_out), path
+    finally:
+        sig.destroy(done)
+        eng.close()

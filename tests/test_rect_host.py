@@ -289,6 +289,44 @@ def test_plan_rect_slots_follow_row_alignment(capi_host):
     assert st == SUCCESS and (p.lanes_per_row, p.wg_size, p.xcd_run) == (33, 256, 144)        # 4 waves x 1 KiB
 
 
+def test_plan_rect_routes_across_the_host_link(capi_host):
+    """A region one side of which is host memory: the same rows, slots and
+    merging, launched as at most 128 workgroups of 256 in launch order, stores
+    to the host written through at system scope."""
+    h2d, d2h = capi_host.ROUTE_HOST_TO_DEVICE, capi_host.ROUTE_DEVICE_TO_HOST
+    d, s = 0x7f0000000000, 0x7e0000000000
+    regions = [
+        ((d, 262144, 0), (0, 0, 0), (s, 262144, 0), (0, 0, 0), (131072, 8192, 1)),       # plain rows, 1 GiB
+        ((d, 20000, 0), (17, 1, 0), (s, 21000, 0), (3001, 0, 0), (16385, 4000, 1)),     # wide rows, any alignment
+        ((d, 512, 0), (256, 0, 0), (s, 512, 0), (0, 0, 0), (256, 1 << 20, 1)),          # narrow, whole lines
+        ((d, 1024, 0), (3, 0, 0), (s, 1024, 0), (9, 0, 0), (1000, 1 << 18, 1)),         # narrow, sharing lines
+    ]
+    for dst, do, src, so, ext in regions:
+        st, dev = capi_host.plan_rect(dst, do, src, so, ext)
+        assert st == 0 and dev.route == capi_host.ROUTE_DEVICE
+        for route in (h2d, d2h):
+            st, p = capi_host.plan_rect(dst, do, src, so, ext, route=route)
+            assert st == 0 and p.route == route
+            for f in ("empty", "linear", "dst", "src", "width", "rows", "layers", "lanes_per_row", "total_bytes",
+                      "dst_pitch", "src_pitch", "nt_load"):
+                assert getattr(p, f) == getattr(dev, f), f
+            assert (p.wg_size, p.xcd_run) == (256, 0) and p.grid <= 128
+            if p.lanes_per_row == 0:
+                assert p.unroll == 1
+            if route == d2h:
+                assert p.store_policy == capi_host.STORE_SYSTEM_WT
+            else:
+                assert p.store_policy in (capi_host.STORE_NT, capi_host.STORE_AGENT_WT)
+    # a region that merges into one run is a linear copy on the same route
+    st, p = capi_host.plan_rect((d, 4096, 4096 * 50), (0, 0, 0), (s, 4096, 4096 * 50), (0, 0, 0), (4096, 50, 2), route=h2d)
+    assert st == 0 and p.linear and p.route == h2d
+    # tuning still overrides, an unknown route is refused
+    st, p = capi_host.plan_rect(*regions[0], capi_host.Tuning(max_grid=1000, wg_size=64, store_policy=2), route=d2h)
+    assert st == 0 and (p.wg_size, p.grid, p.store_policy) == (64, 1000, capi_host.STORE_NT)
+    st, p = capi_host.plan_rect(*regions[0], route=3)
+    assert st == capi_host.ERROR_INVALID_ARGUMENT
+
+
 def test_plan_rect_validation_matches_reference(capi_host, oracle):
     """Same verdict as the reference's checks on every case, except that the
     SDMA packet's dword alignment is not demanded."""

@@ -127,12 +127,13 @@ hsa_status_t BlitKernelGfx950Aql::SubmitCopyRectCommand(const hsa_pitched_ptr_t*
                                                         core::Signal& out_signal) {
   if (blit_ == nullptr) return HSA_STATUS_ERROR_NOT_INITIALIZED;
   const std::vector<uint64_t> deps = handles(dep_signals);
-  return to_hsa(mi355_aql_copy_rect(blit_, reinterpret_cast<const mi355_pitched_ptr_t*>(dst),
-                                    reinterpret_cast<const mi355_dim3_t*>(dst_offset),
-                                    reinterpret_cast<const mi355_pitched_ptr_t*>(src),
-                                    reinterpret_cast<const mi355_dim3_t*>(src_offset),
-                                    reinterpret_cast<const mi355_dim3_t*>(range), deps.empty() ? nullptr : deps.data(),
-                                    static_cast<uint32_t>(deps.size()), core::Signal::Convert(&out_signal).handle));
+  // DmaCopyRect has picked this object by the copy's direction
+  // (amd_gpu_agent.cpp:1265-1266): the slot is the route.
+  return to_hsa(mi355_aql_copy_rect_route(
+      blit_, reinterpret_cast<const mi355_pitched_ptr_t*>(dst), reinterpret_cast<const mi355_dim3_t*>(dst_offset),
+      reinterpret_cast<const mi355_pitched_ptr_t*>(src), reinterpret_cast<const mi355_dim3_t*>(src_offset),
+      reinterpret_cast<const mi355_dim3_t*>(range), static_cast<uint32_t>(slot_), deps.empty() ? nullptr : deps.data(),
+      static_cast<uint32_t>(deps.size()), core::Signal::Convert(&out_signal).handle));
 }
 
 hsa_status_t BlitKernelGfx950Aql::EnableProfiling(bool enable) {

@@ -180,7 +180,12 @@ int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwo
  * No counterpart in the reference (it submits one AQL packet per copy).
  * descs may live in host memory (descs_on_device == 0: the library stages
  * them) or be device-resident (descs_on_device != 0: read in place, must stay
- * valid until completion).  Regions must not overlap one another.  A stream
+ * valid until completion).  The host cannot see the lengths of
+ * device-resident descriptors: it sizes the launch for copies of 32 KiB on
+ * average, the kernels read the real chunk count on the device, and a batch
+ * of longer copies is slower, never wrong (a caller that knows a bound says
+ * so through mi355_blit_copy_batch_bounded).  A batch may have at most 2^32-1
+ * chunks of 4 KiB.  Regions must not overlap one another.  A stream
  * under HIP graph capture -> INVALID_ARGUMENT (both batched entry points). */
 int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n,
                           int descs_on_device, void* stream);
@@ -188,14 +193,13 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
 /* The batched path for device-resident descriptors whose sizes the host does
  * not know but can bound (a previous kernel wrote them): the n copies together
  * move at most max_total_bytes bytes.  No counterpart in the reference.  The
- * bound sizes the grid and the record buffer (max_total_bytes / 4096 + 2 n
- * records of 32 bytes), which lets the copy run one wave per 4 KiB chunk as
- * with host-resident descriptors instead of on a fixed grid that walks the
- * prefix sums; a loose bound costs idle waves, not correctness.  Descriptors
- * that exceed the bound are the caller's error: the copies are then cut short
- * at the bound (no access outside the described regions is made, and no error
- * can be reported without a read-back).  max_total_bytes == 0 with n > 0, or
- * a bound that needs 2^32 records or more -> INVALID_ARGUMENT. */
+ * bound sizes the record buffer (max_total_bytes / 4096 + 2 n records of 32
+ * bytes, 512 MiB at most) and the grid (a workgroup per likely chunk) in
+ * place of the library's assumption.  It is a hint, not a contract: a loose
+ * bound costs idle waves, and chunks beyond a bound that the descriptors
+ * exceed have no record and are found through the prefix sums by the copy
+ * kernel itself, several times slower but complete.  max_total_bytes == 0
+ * with n > 0, or a bound that needs 2^32 records or more -> INVALID_ARGUMENT. */
 int mi355_blit_copy_batch_bounded(mi355_blit_t* h, const mi355_blit_desc_t* device_descs, size_t n,
                                   uint64_t max_total_bytes, void* stream);
 

@@ -71,14 +71,15 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
 
 /* The same with device-resident descriptors (read in place; they must stay
  * valid until completion and be ready when the dependencies are).  The host
- * cannot know the work's size, so the copy runs on a device-filling grid
- * whose waves share the chunks out evenly.  Four packets. */
+ * cannot know the work's size: see mi355_blit_copy_batch in mi355_blit.h.
+ * Four packets (two for the prefix sum, the records, the copy). */
 int mi355_aql_copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, size_t n,
                                 const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal);
 
 /* Device-resident descriptors that together move at most max_total_bytes
- * bytes (see mi355_blit_copy_batch_bounded in mi355_blit.h: the bound sizes a
- * per-chunk grid; copies beyond it are cut short).  Four packets.
+ * bytes (see mi355_blit_copy_batch_bounded in mi355_blit.h: the bound sizes
+ * the grid and the record buffer; what exceeds it is slower, not lost).  Four
+ * packets.
  * max_total_bytes == 0 with n > 0 -> INVALID_ARGUMENT. */
 int mi355_aql_copy_batch_bounded(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, size_t n,
                                  uint64_t max_total_bytes, const uint64_t* dep_signals, uint32_t num_deps,

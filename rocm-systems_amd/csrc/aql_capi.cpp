@@ -60,6 +60,7 @@ struct RectKernel { unsigned unroll, nt_load, store; const char* name; Kernel k;
 #define MI355_FILL_NAME(U, S) {U, S, "mi355_fill_u" #U "_s" #S, {}},
 #define MI355_BATCH_NAME(P, L, S) {P, L, S, "mi355_batch_records_p" #P "_l" #L "_s" #S, {}},
 #define MI355_RECT_NAME(U, L, S) {U, L, S, "mi355_rect_u" #U "_l" #L "_s" #S, {}},
+#define MI355_BATCH_LOOKUP_NAME(L, S) {0, L, S, "mi355_batch_lookup_l" #L "_s" #S, {}},
 #define MI355_RECT_NARROW_NAME(L, S) {0, L, S, "mi355_rect_narrow_l" #L "_s" #S, {}},
 
 struct BytesWritten {
@@ -107,7 +108,8 @@ struct mi355_aql {
   std::vector<BatchKernel> batch_kernels{MI355_FOR_EACH_BATCH_RECORDS_KERNEL(MI355_BATCH_NAME)};
   std::vector<RectKernel> rect_kernels{MI355_FOR_EACH_RECT_KERNEL(MI355_RECT_NAME)};
   std::vector<RectKernel> rect_narrow_kernels{MI355_FOR_EACH_RECT_NARROW_KERNEL(MI355_RECT_NARROW_NAME)};
-  Kernel scan_local, scan_top, emit_records, emit_records_device, finalize, strided_cached, strided_streaming;
+  std::vector<RectKernel> batch_lookup_kernels{MI355_FOR_EACH_BATCH_LOOKUP_KERNEL(MI355_BATCH_LOOKUP_NAME)};
+  Kernel scan_local, scan_top, emit_records, emit_records_device;
 
   hsa_signal_t idle_signal{};  // completion signal of wait_idle's barrier packet
 
@@ -252,9 +254,8 @@ int load_code_object(mi355_aql* h) {
   if ((rc = lookup(h, "mi355_batch_scan_top", &h->scan_top)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_emit_records", &h->emit_records)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_emit_records_device", &h->emit_records_device)) != MI355_BLIT_SUCCESS) return rc;
-  if ((rc = lookup(h, "mi355_batch_finalize", &h->finalize)) != MI355_BLIT_SUCCESS) return rc;
-  if ((rc = lookup(h, "mi355_batch_strided_l0_s0", &h->strided_cached)) != MI355_BLIT_SUCCESS) return rc;
-  if ((rc = lookup(h, "mi355_batch_strided_l1_s1", &h->strided_streaming)) != MI355_BLIT_SUCCESS) return rc;
+  for (auto& k : h->batch_lookup_kernels)
+    if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
   return MI355_BLIT_SUCCESS;
 }
 
@@ -787,71 +788,23 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   return MI355_BLIT_SUCCESS;
 }
 
-int mi355_aql_copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, size_t n,
-                                const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal) {
+namespace {
+// Device-resident descriptors, with a bound on the bytes they move or without
+// (max_total_bytes == 0): four packets, each waiting for the one before --
+// the two launches of the prefix sum, the records, and the copy, whose grid
+// and record buffer follow batch_device_sizing and which reads the number of
+// chunks on the device.
+int copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, size_t n, uint64_t max_total_bytes,
+                      const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal) {
   if (!h || (!device_descs && n) || (num_deps && !dep_signals)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   if (n > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   if (h->queue_error.load()) return MI355_BLIT_ERROR;
   if (n == 0) return mi355_aql_copy(h, h, h, 0, dep_signals, num_deps, completion_signal);
+  const BatchDeviceSizing sizing = batch_device_sizing(n, max_total_bytes);
+  if (sizing.records == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
 
   std::lock_guard<std::mutex> g(h->lock);
-  int rc = ensure_batch_capacity(h, n, 0);
-  if (rc != MI355_BLIT_SUCCESS) return rc;
-  const mi355_blit_tuning_t* t = h->has_tuning ? &h->tuning : nullptr;
-  const BatchDesc* descs = reinterpret_cast<const BatchDesc*>(device_descs);
-  const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
-  ScanLocalArgs sl{descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
-  ScanTopArgs stp{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
-  FinalizeArgs fa{static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
-
-  mi355_blit_plan_t p{};
-  p.kernel = MI355_BLIT_KERNEL_COPY_BATCH;
-  p.unroll = kBatchChunkVecs / 64;
-  bool streaming = true;  // the lengths are only known on the device
-  if (t && t->nt_load) streaming = (t->nt_load == 2);
-  p.nt_load = streaming;
-  p.store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
-  p.wg_size = 256;
-  uint32_t max_grid = h->num_cus * kWgPerCu;
-  if (t && t->max_grid) max_grid = t->max_grid;
-  // a copy has at least one chunk; with few copies a full-device grid would be mostly idle waves
-  const uint64_t wgs = static_cast<uint64_t>(n) * 16;
-  p.grid = static_cast<uint32_t>(wgs < max_grid ? wgs : max_grid);
-  BatchStridedArgs bs{descs, static_cast<uint64_t>(n), h->chunk_start_dev, 4u, p.grid * 4u};
-  h->last_plan = p;
-
-  const uint32_t nb = barrier_packets(num_deps);
-  const uint32_t total = nb + 4;
-  uint64_t index;
-  {
-    std::lock_guard<std::mutex> r(h->reservation_lock);
-    index = acquire_write_index(h, total);
-    record_blit_history(h, n, index + total - 1);  // lengths unknown here: keep the record non-zero
-  }
-  write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
-  uint64_t i = index + nb;
-  // every packet waits for the one before; the first also for whatever still uses the shared buffers
-  write_dispatch(h, i++, h->scan_local, &sl, sizeof(sl), n_blocks, 1024, 0, true);
-  write_dispatch(h, i++, h->scan_top, &stp, sizeof(stp), 1, 1024, 0, true);
-  write_dispatch(h, i++, h->finalize, &fa, sizeof(fa), static_cast<uint32_t>((n + 255) / 256), 256, 0, true);
-  write_dispatch(h, i++, streaming ? h->strided_streaming : h->strided_cached, &bs, sizeof(bs), p.grid, p.wg_size,
-                 completion_signal, true);
-  release_write_index(h, index, total);
-  return MI355_BLIT_SUCCESS;
-}
-
-int mi355_aql_copy_batch_bounded(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, size_t n,
-                                 uint64_t max_total_bytes, const uint64_t* dep_signals, uint32_t num_deps,
-                                 uint64_t completion_signal) {
-  if (!h || (!device_descs && n) || (num_deps && !dep_signals)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
-  if (n > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
-  if (h->queue_error.load()) return MI355_BLIT_ERROR;
-  if (n == 0) return mi355_aql_copy(h, h, h, 0, dep_signals, num_deps, completion_signal);
-  const uint64_t capacity = max_total_bytes ? batch_bound_chunks(n, max_total_bytes) : 0;
-  if (capacity == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
-
-  std::lock_guard<std::mutex> g(h->lock);
-  int rc = ensure_batch_capacity(h, n, capacity);
+  int rc = ensure_batch_capacity(h, n, sizing.records);
   if (rc != MI355_BLIT_SUCCESS) return rc;
   const mi355_blit_tuning_t* t = h->has_tuning ? &h->tuning : nullptr;
   const BatchDesc* descs = reinterpret_cast<const BatchDesc*>(device_descs);
@@ -859,16 +812,18 @@ int mi355_aql_copy_batch_bounded(mi355_aql_t* h, const mi355_blit_desc_t* device
   ScanLocalArgs sl{descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
   ScanTopArgs stp{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
   EmitRecordsDeviceArgs er{descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n), h->records_dev,
-                           capacity};
+                           sizing.records};
 
   // the lengths are only known on the device: a large batch, in the fixed shape
   mi355_blit_plan_t p;
-  const BatchLaunch l = plan_batch_records(capacity, max_total_bytes, true, t, false, &p);
-  const Kernel* bk = find_batch(h, l, p);
-  if (!bk) return MI355_BLIT_ERROR;
-  // the grid is sized for the bound; the kernel reads the number of records the device counted
-  BatchCopyArgs bc{h->records_dev, capacity, h->chunk_start_dev + n, l.waves_per_wg, l.n_waves,
-                   make_xcd_runs(p.grid, p.xcd_run)};
+  const BatchLaunch l = plan_batch_records(sizing.grid_chunks, sizing.bytes, true, t, false, &p);
+  const Kernel* bk = nullptr;
+  for (const auto& v : h->batch_lookup_kernels)
+    if (v.nt_load == p.nt_load && v.store == p.store_policy) bk = &v.k;
+  if (!bk || l.split != 4) return MI355_BLIT_ERROR;
+  BatchLookupArgs bc{{h->records_dev, sizing.records, h->chunk_start_dev + n, l.waves_per_wg, l.n_waves,
+                      make_xcd_runs(p.grid, p.xcd_run)},
+                     descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n)};
   h->last_plan = p;
 
   const uint32_t nb = barrier_packets(num_deps);
@@ -877,7 +832,8 @@ int mi355_aql_copy_batch_bounded(mi355_aql_t* h, const mi355_blit_desc_t* device
   {
     std::lock_guard<std::mutex> r(h->reservation_lock);
     index = acquire_write_index(h, total);
-    record_blit_history(h, max_total_bytes, index + total - 1);
+    // without a bound the lengths are unknown here: keep the record non-zero
+    record_blit_history(h, max_total_bytes ? max_total_bytes : n, index + total - 1);
   }
   write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
   uint64_t i = index + nb;
@@ -889,6 +845,19 @@ int mi355_aql_copy_batch_bounded(mi355_aql_t* h, const mi355_blit_desc_t* device
   write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true);
   release_write_index(h, index, total);
   return MI355_BLIT_SUCCESS;
+}
+}  // namespace
+
+int mi355_aql_copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, size_t n,
+                                const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal) {
+  return copy_batch_device(h, device_descs, n, 0, dep_signals, num_deps, completion_signal);
+}
+
+int mi355_aql_copy_batch_bounded(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, size_t n,
+                                 uint64_t max_total_bytes, const uint64_t* dep_signals, uint32_t num_deps,
+                                 uint64_t completion_signal) {
+  if (max_total_bytes == 0 && n != 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  return copy_batch_device(h, device_descs, n, max_total_bytes, dep_signals, num_deps, completion_signal);
 }
 
 int mi355_aql_copy_rect(mi355_aql_t* h, const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,

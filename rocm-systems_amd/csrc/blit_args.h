@@ -132,12 +132,6 @@ struct ScanTopArgs {
   uint32_t n_blocks;
 };
 
-struct FinalizeArgs {
-  uint64_t n;
-  uint32_t* chunk_start;
-  const uint32_t* block_sum;
-};
-
 // Host-resident descriptors: the host has cut them into pieces and summed
 // their chunk counts; one lane per piece writes the piece's records.
 struct EmitRecordsArgs {
@@ -147,10 +141,9 @@ struct EmitRecordsArgs {
   ChunkRecord* records;
 };
 
-// Device-resident descriptors with a bound on their total size: the prefix
-// sum was done on the device (chunk_start within each group of 1024 copies,
-// block_sum across groups); one lane per copy, records beyond `capacity` are
-// not written.
+// Device-resident descriptors: the prefix sum was done on the device
+// (chunk_start within each group of 1024 copies, block_sum across groups); one
+// lane per copy, records beyond `capacity` are not written.
 struct EmitRecordsDeviceArgs {
   const BatchDesc* descs;
   const uint32_t* chunk_start;
@@ -162,21 +155,26 @@ struct EmitRecordsDeviceArgs {
 
 struct BatchCopyArgs {
   const ChunkRecord* records;
-  uint64_t total_chunks;  // the number of records, or a bound on it when total is given
-  // When not null, the number of records as the device computed it; the grid
-  // was sized for total_chunks and waves beyond *total have nothing to do.
+  uint64_t total_chunks;  // the number of records
+  // Device-resident descriptors only (BatchLookupArgs): where the device has
+  // put the number of chunks.  Null when the host knows it.
   const uint32_t* total;
   uint32_t waves_per_wg;
   uint32_t n_waves;
   XcdRuns xcd;
 };
 
-struct BatchStridedArgs {
+// The copy over records for device-resident descriptors, whose number of
+// chunks only the device knows: copy.total points at it, copy.total_chunks is
+// the number of records there was room for, and a chunk beyond that is looked
+// up in the prefix sums instead (a batch larger than the caller's bound, or
+// than the library assumed, is slower, not wrong).
+struct BatchLookupArgs {
+  BatchCopyArgs copy;
   const BatchDesc* descs;
+  const uint32_t* chunk_start;  // within each group of 1024 copies
+  const uint32_t* block_sum;    // chunks in front of each group
   uint64_t n;
-  const uint32_t* chunk_start;
-  uint32_t waves_per_wg;
-  uint32_t n_waves;
 };
 
 // A pitched 3-D region copy: `layers` slices of `rows` rows of `width` bytes.

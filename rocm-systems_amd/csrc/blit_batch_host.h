@@ -50,6 +50,50 @@ inline uint64_t batch_bound_chunks(uint64_t n, uint64_t max_total_bytes) {
   return c < 0xffffffffull ? c : 0;
 }
 
+// Device-resident descriptors: the host sizes the record buffer and the grid
+// without knowing the lengths.  With a bound from the caller both follow the
+// bound.  Without one the library assumes copies of 32 KiB on average for the
+// grid (one 4-wave workgroup per chunk; waves beyond the real total end at
+// once, and waves stride when there are more chunks) and makes room for twice
+// that many records.  Either way a chunk beyond the records is found through
+// the prefix sums by the copy kernel itself: a wrong guess or a bound that is
+// exceeded costs speed, not correctness.  Records are capped at 512 MiB.
+constexpr uint64_t kBatchMaxDeviceRecords = 1ull << 24;
+constexpr uint64_t kBatchMinDeviceRecords = 1ull << 16;
+constexpr uint64_t kBatchAssumedChunksPerCopy = 8;
+
+struct BatchDeviceSizing {
+  uint64_t records;      // capacity of the record buffer
+  uint64_t grid_chunks;  // chunks the grid has a workgroup for
+  uint64_t bytes;        // what the launch heuristics take the batch's size to be
+};
+
+inline BatchDeviceSizing batch_device_sizing(uint64_t n, uint64_t max_total_bytes) {
+  BatchDeviceSizing z;
+  if (max_total_bytes) {
+    // 0: a bound beyond what 32-bit record indices can count, which no batch
+    // can need (the caller answers INVALID_ARGUMENT)
+    uint64_t c = batch_bound_chunks(n, max_total_bytes);
+    if (c > kBatchMaxDeviceRecords) c = kBatchMaxDeviceRecords;
+    z.records = c;
+    // Room for the most chunks the bound allows (two more than bytes / 4096
+    // per copy), a grid for what is likely (one more): waves without a chunk
+    // cost their dispatch (65,536 copies of 2 GB: 715 us with a workgroup for
+    // every possible chunk, 698 us with 4 % fewer workgroups than chunks).
+    z.grid_chunks = max_total_bytes / (16 * kBatchChunkVecs) + n;
+    if (z.grid_chunks > c) z.grid_chunks = c;
+    z.bytes = max_total_bytes;
+  } else {
+    z.grid_chunks = kBatchAssumedChunksPerCopy * n;
+    z.records = 2 * z.grid_chunks;
+    if (z.records < kBatchMinDeviceRecords) z.records = kBatchMinDeviceRecords;
+    if (z.records > kBatchMaxDeviceRecords) z.records = kBatchMaxDeviceRecords;
+    if (z.grid_chunks > z.records) z.grid_chunks = z.records;
+    z.bytes = z.grid_chunks * (16 * kBatchChunkVecs);
+  }
+  return z;
+}
+
 // Calls f(dst, src, bytes) for every piece of one copy.
 template <typename F>
 inline void batch_for_each_piece(const mi355_blit_desc_t& d, F f) {

@@ -119,6 +119,7 @@ struct DeviceScope {
 typedef void (*copy_kernel_t)(CopyArgs);
 typedef void (*fill_kernel_t)(FillArgs);
 typedef void (*batch_kernel_t)(BatchCopyArgs);
+typedef void (*batch_lookup_kernel_t)(BatchLookupArgs);
 typedef void (*rect_kernel_t)(RectArgs);
 typedef void (*rect_narrow_kernel_t)(RectNarrowArgs);
 
@@ -126,6 +127,7 @@ typedef void (*rect_narrow_kernel_t)(RectNarrowArgs);
 struct CopyVariant { unsigned unroll, nt_load, store, realign; copy_kernel_t fn; };
 struct FillVariant { unsigned unroll, store; fill_kernel_t fn; };
 struct BatchVariant { unsigned split, nt_load, store; batch_kernel_t fn; };
+struct BatchLookupVariant { unsigned nt_load, store; batch_lookup_kernel_t fn; };
 struct RectVariant { unsigned unroll, nt_load, store; rect_kernel_t fn; };
 struct RectNarrowVariant { unsigned nt_load, store; rect_narrow_kernel_t fn; };
 
@@ -135,6 +137,8 @@ const CopyVariant kCopyVariants[] = {MI355_FOR_EACH_COPY_KERNEL(MI355_COPY_ROW)}
 const FillVariant kFillVariants[] = {MI355_FOR_EACH_FILL_KERNEL(MI355_FILL_ROW)};
 #define MI355_BATCH_ROW(P, L, S) {P, L, S, mi355_batch_records_p##P##_l##L##_s##S},
 const BatchVariant kBatchVariants[] = {MI355_FOR_EACH_BATCH_RECORDS_KERNEL(MI355_BATCH_ROW)};
+#define MI355_BATCH_LOOKUP_ROW(L, S) {L, S, mi355_batch_lookup_l##L##_s##S},
+const BatchLookupVariant kBatchLookupVariants[] = {MI355_FOR_EACH_BATCH_LOOKUP_KERNEL(MI355_BATCH_LOOKUP_ROW)};
 #define MI355_RECT_ROW(U, L, S) {U, L, S, mi355_rect_u##U##_l##L##_s##S},
 const RectVariant kRectVariants[] = {MI355_FOR_EACH_RECT_KERNEL(MI355_RECT_ROW)};
 #define MI355_RECT_NARROW_ROW(L, S) {L, S, mi355_rect_narrow_l##L##_s##S},
@@ -479,14 +483,27 @@ void launch_scans(mi355_blit* h, hipStream_t s, const BatchDesc* dev_descs, size
 }
 
 // The copy over h->records_dev, launched as *p says (plan_batch_records).
-// total_chunks is the number of records, or a bound on it when `counted`
-// points at the number the device computed.
 int launch_records_copy(mi355_blit* h, hipStream_t s, const mi355_blit_plan_t& p, const BatchLaunch& l,
-                        uint64_t total_chunks, const uint32_t* counted) {
+                        uint64_t total_chunks) {
   batch_kernel_t k = select_batch_kernel(l.split, p.nt_load != 0, p.store_policy);
   if (!k) return MI355_BLIT_ERROR;
-  BatchCopyArgs bc{h->records_dev, total_chunks, counted, l.waves_per_wg, l.n_waves, make_xcd_runs(p.grid, p.xcd_run)};
+  BatchCopyArgs bc{h->records_dev, total_chunks, nullptr, l.waves_per_wg, l.n_waves, make_xcd_runs(p.grid, p.xcd_run)};
   hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, bc);
+  return MI355_BLIT_SUCCESS;
+}
+
+// The same for device-resident descriptors: `records` is what the record
+// buffer has room for, the number of chunks is behind the prefix sums.
+int launch_lookup_copy(mi355_blit* h, hipStream_t s, const mi355_blit_plan_t& p, const BatchLaunch& l,
+                       uint64_t records, const BatchDesc* dev_descs, size_t n) {
+  batch_lookup_kernel_t k = nullptr;
+  for (const BatchLookupVariant& v : kBatchLookupVariants)
+    if (v.nt_load == p.nt_load && v.store == p.store_policy) k = v.fn;
+  if (!k || l.split != 4) return MI355_BLIT_ERROR;
+  BatchLookupArgs a{{h->records_dev, records, h->chunk_start_dev + n, l.waves_per_wg, l.n_waves,
+                     make_xcd_runs(p.grid, p.xcd_run)},
+                    dev_descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n)};
+  hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
   return MI355_BLIT_SUCCESS;
 }
 
@@ -507,21 +524,20 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
   }
 
   BatchShape shape;
+  BatchDeviceSizing sizing{};
   if (!descs_on_device) {
     int rc = batch_build(descs, n, &h->stage_image, &shape);
     if (rc != MI355_BLIT_SUCCESS) return rc;
     if (shape.total_chunks == 0) return MI355_BLIT_SUCCESS;
   } else {
+    // lengths are only known on the device
+    sizing = batch_device_sizing(n, max_total_bytes);
+    if (sizing.records == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
     shape.pieces = n;
-    shape.total_bytes = n;  // lengths are only known on the device; keep the record non-zero
-    if (max_total_bytes) {
-      // what the caller vouches for bounds the number of records
-      shape.total_chunks = batch_bound_chunks(n, max_total_bytes);
-      if (shape.total_chunks == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
-      shape.total_bytes = max_total_bytes;
-    }
+    shape.total_chunks = sizing.grid_chunks;
+    shape.total_bytes = sizing.bytes;
   }
-  int rc = ensure_batch_capacity(h, shape.pieces, shape.total_chunks);
+  int rc = ensure_batch_capacity(h, shape.pieces, descs_on_device ? sizing.records : shape.total_chunks);
   if (rc != MI355_BLIT_SUCCESS) return rc;
 
   // The device-side buffers (records, prefix sums) are shared by consecutive
@@ -565,46 +581,24 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
                        0, s, er);
     BLIT_HIP(hipGetLastError());
 
-    rc = launch_records_copy(h, s, p, l, shape.total_chunks, nullptr);
+    rc = launch_records_copy(h, s, p, l, shape.total_chunks);
     if (rc != MI355_BLIT_SUCCESS) return rc;
-  } else if (max_total_bytes) {
-    // Device-resident descriptors whose total size the caller bounds: the
-    // bound sizes the record buffer and a per-chunk grid, so the copy runs in
-    // the kernel of the host-resident path.  The prefix sum and the records
-    // are made on the device; the copy kernel reads the number of records
-    // there too and the waves the bound overestimated end at once.
+  } else {
+    // Device-resident descriptors.  The prefix sum over the chunk counts and
+    // the records are made on the device; the grid and the record buffer are
+    // sized by the caller's bound or, without one, by an assumption
+    // (batch_device_sizing).  The copy kernel reads the number of chunks on the
+    // device: surplus waves end at once, missing ones are made up for by
+    // striding, and chunks without a record are looked up in the prefix sums.
     const BatchDesc* dev_descs = reinterpret_cast<const BatchDesc*>(descs);
     launch_scans(h, s, dev_descs, n);
     EmitRecordsDeviceArgs er{dev_descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n),
-                             h->records_dev, shape.total_chunks};
+                             h->records_dev, sizing.records};
     hipLaunchKernelGGL(mi355_batch_emit_records_device, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0,
                        s, er);
     BLIT_HIP(hipGetLastError());
-    rc = launch_records_copy(h, s, p, l, shape.total_chunks, h->chunk_start_dev + n);
+    rc = launch_lookup_copy(h, s, p, l, sizing.records, dev_descs, n);
     if (rc != MI355_BLIT_SUCCESS) return rc;
-  } else {
-    // Device-resident descriptors: the prefix sum runs on the device and, as
-    // the host cannot size a per-chunk grid without a read-back, the copy runs
-    // on a device-filling grid whose waves share the chunks out evenly.
-    const BatchDesc* dev_descs = reinterpret_cast<const BatchDesc*>(descs);
-    launch_scans(h, s, dev_descs, n);
-    FinalizeArgs fa{static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
-    hipLaunchKernelGGL(mi355_batch_finalize, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, s, fa);
-    p.wg_size = 256;
-    p.unroll = kBatchChunkVecs / 64;
-    p.xcd_run = 0;
-    uint32_t max_grid = h->num_cus * kWgPerCu;
-    if (t && t->max_grid) max_grid = t->max_grid;
-    // A copy has at least one chunk and, at the sizes this path is meant for,
-    // at most a few dozen; with few copies a full-device grid would be mostly
-    // idle waves.
-    const uint64_t wgs = static_cast<uint64_t>(n) * 16;
-    p.grid = static_cast<uint32_t>(wgs < max_grid ? wgs : max_grid);
-    const bool streaming = p.nt_load != 0;
-    p.store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
-    BatchStridedArgs bs{dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, 4u, p.grid * 4u};
-    if (streaming) hipLaunchKernelGGL(mi355_batch_strided_l1_s1, dim3(p.grid), dim3(p.wg_size), 0, s, bs);
-    else hipLaunchKernelGGL(mi355_batch_strided_l0_s0, dim3(p.grid), dim3(p.wg_size), 0, s, bs);
   }
   BLIT_HIP(hipGetLastError());
   BLIT_HIP(hipEventRecord(h->batch_done[b], s));

@@ -19,6 +19,10 @@
 #define MI355_BATCH_L_(X, P) MI355_BATCH_S_(X, P, 0) MI355_BATCH_S_(X, P, 1)
 #define MI355_FOR_EACH_BATCH_RECORDS_KERNEL(X) MI355_BATCH_L_(X, 1) MI355_BATCH_L_(X, 2) MI355_BATCH_L_(X, 4)
 
+// X(nt_load, store_policy): the batched copy over records for device-resident
+// descriptors (four waves per chunk)
+#define MI355_FOR_EACH_BATCH_LOOKUP_KERNEL(X) MI355_RECT_NARROW_S_(X, 0) MI355_RECT_NARROW_S_(X, 1)
+
 // X(unroll, nt_load, store_policy): the pitched-region copy
 #define MI355_FOR_EACH_RECT_KERNEL(X) MI355_BATCH_L_(X, 1) MI355_BATCH_L_(X, 2) MI355_BATCH_L_(X, 4)
 

@@ -378,17 +378,16 @@ __device__ __forceinline__ uint32_t block_scan_1024(uint32_t v, uint32_t* lds, u
   return (w ? lds[w - 1] : 0) + incl - v;
 }
 
-// Prefix sum of the chunk counts in three small launches (no workgroup ever
+// Prefix sum of the chunk counts in two small launches (no workgroup ever
 // waits for another):
 //  1. mi355_batch_scan_local, one workgroup per 1024 copies: chunk_start[i] =
 //     chunks of the copies before i in the same workgroup, block_sum[b] = all
 //     chunks of workgroup b;
 //  2. mi355_batch_scan_top, one workgroup: block_sum becomes its own exclusive
-//     prefix, chunk_start[n] = all chunks;
-//  3. mi355_batch_finalize, one lane per copy: chunk_start[i] +=
-//     block_sum[i / 1024], for the kernel that walks chunk_start itself.
-// This is the path of device-resident descriptors; for host-resident ones the
-// host does the sum (mi355_batch_emit_records).
+//     prefix, chunk_start[n] = all chunks.
+// A copy's first chunk is block_sum[i / 1024] + chunk_start[i].  This is the
+// path of device-resident descriptors; for host-resident ones the host does
+// the sum (mi355_batch_emit_records).
 __device__ __forceinline__ void scan_local_body(const ScanLocalArgs& a) {
   const BatchDesc* __restrict__ descs = a.descs;
   const uint64_t n = a.n;
@@ -420,12 +419,6 @@ __device__ __forceinline__ void scan_top_body(const ScanTopArgs& a) {
     __syncthreads();  // lds is reused by the next round
   }
   if (threadIdx.x == 0) chunk_start[n] = carry;
-}
-
-// launched with workgroups of 256
-__device__ __forceinline__ void finalize_body(const FinalizeArgs& a) {
-  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (i < a.n) a.chunk_start[i] += a.block_sum[i / 1024];
 }
 
 // Chunk k of a copy.
@@ -608,6 +601,21 @@ __device__ __forceinline__ ChunkRecord load_record(const ChunkRecord* p) {
   return r;
 }
 
+// A descriptor at an address that is the same for every lane, through the
+// constant address space like a record.
+__device__ __forceinline__ BatchDesc load_desc(const BatchDesc* p) {
+  typedef const uint64_t __attribute__((address_space(4))) * ConstPtr;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wold-style-cast"
+  ConstPtr q = (ConstPtr)(p);
+#pragma clang diagnostic pop
+  BatchDesc d;
+  d.dst = reinterpret_cast<uint8_t*>(q[0]);
+  d.src = reinterpret_cast<const uint8_t*>(q[1]);
+  d.bytes = q[2];
+  return d;
+}
+
 // SPLIT waves per 4 KiB chunk, chunks in global order and waves in address
 // order within a chunk: the dispatcher then walks memory densely, the shape
 // that streams best for a single large copy.  Each wave reads its chunk's
@@ -616,12 +624,7 @@ template <int SPLIT, bool NTL, int NTS>
 __device__ __forceinline__ void batch_copy_records_body(const BatchCopyArgs& a) {
   constexpr int U = kChunkVecs / kWave / SPLIT;
   const ChunkRecord* __restrict__ records = a.records;
-  uint64_t total_chunks = a.total_chunks;
-  if (a.total) {
-    // sized for a bound: the device knows how many records there are
-    const uint64_t counted = *a.total;
-    if (counted < total_chunks) total_chunks = counted;
-  }
+  const uint64_t total_chunks = a.total_chunks;
   const unsigned lane = threadIdx.x & (kWave - 1);
   const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd);
   const uint64_t n_waves = a.n_waves;
@@ -637,46 +640,55 @@ __device__ __forceinline__ void batch_copy_records_body(const BatchCopyArgs& a) 
   }
 }
 
-// Device-filling grid, every wave takes an equal contiguous share of all
-// chunks and finds its first copy by bisection.  Used when the descriptors
-// are device-resident and the host cannot know the chunk total.
-template <bool NTL, int NTS>
-__device__ __forceinline__ void batch_copy_strided_body(const BatchStridedArgs& a) {
-  constexpr int U = kChunkVecs / kWave;
-  const BatchDesc* __restrict__ descs = a.descs;
-  const uint64_t n = a.n;
+// Chunk c of a batch of device-resident descriptors, from the prefix sums: the
+// group of 1024 copies it falls into, then the copy within the group (the last
+// one that starts at or before c: copies without chunks share their start with
+// their successor and lose to it).  c is below the batch's chunk total.
+__device__ __forceinline__ ChunkRecord lookup_record(const BatchLookupArgs& a, uint32_t c) {
+  const uint32_t* __restrict__ block_sum = a.block_sum;
   const uint32_t* __restrict__ chunk_start = a.chunk_start;
-  const unsigned lane = threadIdx.x & (kWave - 1);
-  const uint64_t wave = global_wave(a.waves_per_wg);
-  const uint64_t n_waves = a.n_waves;
-  const uint64_t total = chunk_start[n];
-  const uint64_t c0 = total * wave / n_waves;
-  const uint64_t c1 = total * (wave + 1) / n_waves;
-  if (c0 >= c1) return;
-  // largest i with chunk_start[i] <= c0 (copies without chunks share a start
-  // with their successor; they are stepped over below)
-  uint64_t lo = 0, hi = n;
+  uint64_t lo = 0, hi = (a.n + 1023) / 1024 - 1;
   while (lo < hi) {
-    const uint64_t mid = (lo + hi + 1) / 2;
-    if (chunk_start[mid] <= c0) lo = mid; else hi = mid - 1;
+    const uint64_t mid = lo + (hi - lo + 1) / 2;
+    if (ld_u32<false>(block_sum + mid) <= c) lo = mid; else hi = mid - 1;
   }
-  uint64_t i = lo;
-  uint64_t c = c0;
-  while (c < c1 && i < n) {
-    const uint64_t cs = chunk_start[i];
-    const uint64_t ce = chunk_start[i + 1];
-    if (ce <= c) { ++i; continue; }
-    const BatchDesc dsc = descs[i];
-    const uint64_t stop = ce < c1 ? ce : c1;
-    for (; c < stop; ++c) {
-      const ChunkRecord rec = make_record(dsc, static_cast<uint32_t>(c - cs));
-      v4u x[U];
-      unsigned e;
-      record_load<U, NTL>(rec, 0, lane, x, e);
-      record_store<U, NTS>(rec, 0, lane, x, e);
-      record_edges(rec, true, true, lane);
-    }
-    ++i;
+  const uint32_t rem = c - ld_u32<false>(block_sum + lo);
+  lo *= 1024;
+  hi = lo + 1023 < a.n ? lo + 1023 : a.n - 1;
+  while (lo < hi) {
+    const uint64_t mid = lo + (hi - lo + 1) / 2;
+    if (ld_u32<false>(chunk_start + mid) <= rem) lo = mid; else hi = mid - 1;
+  }
+  // Every lane has found the same copy: say so, and its descriptor comes in
+  // through scalar loads like a record.
+  const uint32_t i = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(lo));
+  return make_record(load_desc(a.descs + i), rem - ld_u32<false>(chunk_start + i));
+}
+
+// The copy over records when only the device knows how many chunks there are:
+// the grid was sized for a bound or an assumption, waves beyond the real total
+// end at once, and waves stride when there are more chunks than waves.  One
+// 4 KiB chunk per four waves, as above.
+template <bool NTL, int NTS>
+__device__ __forceinline__ void batch_copy_lookup_body(const BatchLookupArgs& a) {
+  constexpr int SPLIT = 4;
+  constexpr int U = kChunkVecs / kWave / SPLIT;
+  const ChunkRecord* __restrict__ records = a.copy.records;
+  const uint64_t capacity = a.copy.total_chunks;
+  const uint64_t total_chunks = *a.copy.total;
+  const unsigned lane = threadIdx.x & (kWave - 1);
+  const uint64_t wave = global_wave_xcd(a.copy.waves_per_wg, a.copy.xcd);
+  const uint64_t n_waves = a.copy.n_waves;
+  for (uint64_t w = wave; w < total_chunks * SPLIT; w += n_waves) {
+    const uint64_t c = w / SPLIT;
+    const ChunkRecord rec = c < capacity ? load_record(records + c) : lookup_record(a, static_cast<uint32_t>(c));
+    const unsigned q = static_cast<unsigned>(w % SPLIT);
+    const unsigned v0 = q * (kChunkVecs / SPLIT);
+    v4u x[U];
+    unsigned e;
+    record_load<U, NTL>(rec, v0, lane, x, e);
+    record_store<U, NTS>(rec, v0, lane, x, e);
+    record_edges(rec, q == 0, q == SPLIT - 1, lane);
   }
 }
 
@@ -916,6 +928,7 @@ __device__ __forceinline__ void signal_complete_body(const SignalArgs& a) {
 //   mi355_copy_u<unroll>_l<nt loads>_s<store policy>_r<realign>
 //   mi355_fill_u<unroll>_s<store policy>
 //   mi355_batch_records_p<waves per chunk>_l<nt loads>_s<store policy>
+//   mi355_batch_lookup_l<nt loads>_s<store policy>
 //   mi355_rect_u<unroll>_l<nt loads>_s<store policy>
 //   mi355_rect_narrow_l<nt loads>_s<store policy>
 // ---------------------------------------------------------------------------
@@ -955,20 +968,18 @@ MI355_FOR_EACH_RECT_KERNEL(MI355_DEFINE_RECT)
   }
 MI355_FOR_EACH_RECT_NARROW_KERNEL(MI355_DEFINE_RECT_NARROW)
 
-extern "C" __global__ void __launch_bounds__(256) mi355_batch_strided_l0_s0(mi355::BatchStridedArgs a) {
-  mi355::batch_copy_strided_body<false, mi355::kStoreCached>(a);
-}
-extern "C" __global__ void __launch_bounds__(256) mi355_batch_strided_l1_s1(mi355::BatchStridedArgs a) {
-  mi355::batch_copy_strided_body<true, mi355::kStoreNt>(a);
-}
+#define MI355_DEFINE_BATCH_LOOKUP(L, S)                                                \
+  extern "C" __global__ void __launch_bounds__(1024)                                   \
+      mi355_batch_lookup_l##L##_s##S(mi355::BatchLookupArgs a) {                       \
+    mi355::batch_copy_lookup_body<L != 0, S>(a);                                       \
+  }
+MI355_FOR_EACH_BATCH_LOOKUP_KERNEL(MI355_DEFINE_BATCH_LOOKUP)
+
 extern "C" __global__ void __launch_bounds__(1024) mi355_batch_scan_local(mi355::ScanLocalArgs a) {
   mi355::scan_local_body(a);
 }
 extern "C" __global__ void __launch_bounds__(1024) mi355_batch_scan_top(mi355::ScanTopArgs a) {
   mi355::scan_top_body(a);
-}
-extern "C" __global__ void __launch_bounds__(256) mi355_batch_finalize(mi355::FinalizeArgs a) {
-  mi355::finalize_body(a);
 }
 extern "C" __global__ void __launch_bounds__(256) mi355_batch_emit_records(mi355::EmitRecordsArgs a) {
   mi355::emit_records_body(a);

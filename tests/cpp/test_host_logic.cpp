@@ -312,6 +312,33 @@ void one_batch_stage() {
   CHECK(batch_bound_chunks(1, 1ull << 62) == 0, "a bound beyond 32-bit record indices accepted");
 }
 
+// What the host sizes for device-resident descriptors, whose lengths it cannot
+// see: never more records than the cap, never a grid without a record behind
+// each of its chunks, a bound followed exactly while it fits.
+void one_batch_device_sizing() {
+  const uint64_t n = 1 + below(1ull << (1 + below(32)));
+  const BatchDeviceSizing u = batch_device_sizing(n, 0);
+  CHECK(u.records >= kBatchMinDeviceRecords && u.records <= kBatchMaxDeviceRecords, "records %" PRIu64, u.records);
+  CHECK(u.grid_chunks >= 1 && u.grid_chunks <= u.records, "grid of %" PRIu64 " chunks, %" PRIu64 " records",
+        u.grid_chunks, u.records);
+  CHECK(u.grid_chunks == 8 * n || u.grid_chunks == kBatchMaxDeviceRecords, "grid of %" PRIu64 " chunks for %" PRIu64,
+        u.grid_chunks, n);
+  CHECK(u.bytes == u.grid_chunks * 4096, "assumed bytes");
+  const uint64_t bytes = 1 + below(1ull << (1 + below(50)));
+  const BatchDeviceSizing b = batch_device_sizing(n, bytes);
+  const uint64_t want = batch_bound_chunks(n, bytes);
+  if (want == 0) {  // more chunks than 32-bit record indices count
+    CHECK(b.records == 0, "records %" PRIu64 " for a bound beyond the record indices", b.records);
+    return;
+  }
+  CHECK(b.grid_chunks >= 1 && b.grid_chunks <= b.records && b.bytes == bytes, "grid of %" PRIu64 " chunks, %" PRIu64 " records",
+        b.grid_chunks, b.records);
+  CHECK(b.grid_chunks == b.records || b.grid_chunks == bytes / 4096 + n, "grid of %" PRIu64 " chunks for a bound", b.grid_chunks);
+  CHECK(b.records == (want < kBatchMaxDeviceRecords ? want : kBatchMaxDeviceRecords),
+        "records %" PRIu64 " for a bound of %" PRIu64 " chunks", b.records, want);
+  CHECK(batch_device_sizing(1, 1ull << 62).records == 0, "a bound beyond 32-bit record indices accepted");
+}
+
 // Division by an invariant through its magic number must be exact for every
 // 32-bit dividend: divisors and dividends at the extremes and at random.
 void one_magic_division() {
@@ -392,6 +419,7 @@ int main(int argc, char** argv) {
     if (i % 64 == 0) one_xcd_permutation();
     if (i % 16 == 0) one_magic_division();
     if (i % 8 == 0) one_batch_launch();
+    if (i % 8 == 0) one_batch_device_sizing();
   }
   std::printf("%s: %ld cases each of copy, fill and region plans, %d failures\n", g_failures ? "FAILED" : "OK", cases,
               g_failures);

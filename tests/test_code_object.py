@@ -50,7 +50,7 @@ def test_store_policies_are_what_the_names_say(kernels):
     checked = 0
     for name, body in kernels.items():
         m = re.search(r"_s([0-3])(_r[01])?$", name)
-        if not m or not name.startswith(("mi355_copy_", "mi355_fill_", "mi355_batch_records_", "mi355_batch_strided_",
+        if not m or not name.startswith(("mi355_copy_", "mi355_fill_", "mi355_batch_records_", "mi355_batch_lookup_",
                                          "mi355_rect_")):
             continue
         stores = [i for i in body if i.startswith("global_store_dwordx4")]
@@ -65,8 +65,8 @@ def test_store_policies_are_what_the_names_say(kernels):
 def test_load_policies_are_what_the_names_say(kernels):
     for name, body in kernels.items():
         m = re.search(r"_l([01])_s[0-3]", name)
-        if not m or name.startswith("mi355_batch_strided_"):
-            continue   # the strided batch kernel also fetches descriptors, 16 bytes at a time and cached
+        if not m:
+            continue
         loads = [i for i in body if i.startswith("global_load_dwordx4")]
         assert loads, name
         for i in loads:

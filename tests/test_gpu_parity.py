@@ -690,25 +690,56 @@ def test_batch_bounded_all_empty_and_arguments(capi, blit, arenas, torch_cuda):
     check_ok(capi, blit.synchronize(), "synchronize")
 
 
-def test_batch_bounded_too_small_a_bound_stays_inside_the_regions(capi, blit, oracle, arenas, torch_cuda):
-    """A bound the descriptors exceed is the caller's error; the engine then
-    leaves the last chunks uncopied, and writes nothing outside the regions:
-    every byte is either the guard or what the full batch would have put there."""
+@pytest.mark.parametrize("n,min_len,max_len,bound", [(64, 32 << 10, 64 << 10, 4096), (2100, 8 << 10, 24 << 10, 1),
+                                                     (1030, 64, 200 << 10, 50000)])
+def test_batch_bound_exceeded_costs_speed_not_bytes(capi, blit, oracle, arenas, torch_cuda, n, min_len, max_len, bound):
+    """A bound the descriptors exceed leaves most chunks without a record: the
+    copy kernel then finds them through the prefix sums (across groups of 1024
+    copies, around copies of no bytes), with fewer waves than chunks.  The
+    result is still the full batch, and the guards."""
     torch = torch_cuda
     src, src_host, dst = arenas
-    n = 64
-    rng = np.random.default_rng(808)
-    descs, lens, offs, so, do, total = _make_batch(capi, rng, src, dst, n, min_len=32 << 10, max_len=64 << 10)
+    rng = np.random.default_rng(808 + n)
+    descs, lens, offs, so, do, total = _make_batch(capi, rng, src, dst, n, min_len=min_len, max_len=max_len)
+    for i in range(0, n, 7):       # copies of no bytes share their first chunk with their successor
+        descs[i].bytes = 0
+        lens[i] = 0
+    if n > 1024:
+        for i in range(1024 - 3, 1024 + 2):   # also at the end of a group and the start of the next
+            descs[i].bytes = 0
+            lens[i] = 0
     descs_dev = _to_device(torch, descs)
     dst.fill(0, total, GUARD_BYTE)
     torch.cuda.synchronize()
-    check_ok(capi, blit.copy_batch_bounded(descs_dev.data_ptr(), n, 4096), "copy_batch_bounded")
+    check_ok(capi, blit.copy_batch_bounded(descs_dev.data_ptr(), n, bound), "copy_batch_bounded")
     check_ok(capi, blit.synchronize(), "synchronize")
+    p = blit.last_plan()
+    assert p.grid < int((lens // 4096).sum()), "the case is meant to leave chunks without a wave of their own"
+    assert np.array_equal(dst.host(0, total), _expect_batch(oracle, src_host, total, lens, offs, so, do))
+
+
+def test_batch_unbounded_beyond_what_the_library_assumes(capi, blit, oracle, rand, torch_cuda):
+    """Device-resident descriptors without a bound: the grid assumes 32 KiB a
+    copy and the record buffer twice that (65,536 records at least).  Four
+    copies of 70-80 MiB have 17 times the records: the rest is looked up."""
+    torch = torch_cuda
+    n = 4
+    size = n * 80 * MIB + MIB
+    src_host = rand(size, 0xB1170909)
+    src = Arena(torch, size, host=src_host)
+    dst = Arena(torch, size, fill=GUARD_BYTE)
+    rng = np.random.default_rng(909)
+    descs, lens, offs, so, do, total = _make_batch(capi, rng, src, dst, n, min_len=70 * MIB, max_len=80 * MIB)
+    assert int((lens // 4096).sum()) > 65536
+    descs_dev = _to_device(torch, descs)
+    dst.fill(0, total, GUARD_BYTE)
+    torch.cuda.synchronize()
+    check_ok(capi, blit.copy_batch(descs_dev.data_ptr(), n, on_device=True), "copy_batch")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert blit.last_plan().grid == 32
     got = dst.host(0, total)
     want = _expect_batch(oracle, src_host, total, lens, offs, so, do)
-    assert ((got == want) | (got == GUARD_BYTE)).all()
-    first = slice(int(offs[0] + do[0]), int(offs[0] + do[0]) + 4096)
-    assert np.array_equal(got[first], want[first]), "the chunks within the bound are copied"
+    assert np.array_equal(got, want)
 
 
 def test_batch_65536_copies(capi, blit, oracle, rand, torch_cuda):

@@ -195,6 +195,18 @@ def make_batch(r, n=65536, arena=8 * GIB):
     return fn, verify, int(2 * lens.sum()), (src, dst, descs)
 
 
+def make_batch_device(r):
+    """The same 65,536 copies with the descriptors resident in device memory
+    (as a kernel would have left them) and no bound on their sizes given."""
+    import numpy as np
+    fn, verify, algo, (src, dst, descs) = make_batch(r)
+    n = len(descs)
+    dev = r.torch.from_numpy(np.frombuffer(bytes(descs), dtype=np.uint8).copy()).to("cuda:0")
+    r.torch.cuda.synchronize()
+    fn_dev = lambda: r.check(r.blit.copy_batch(dev.data_ptr(), n, True, r.stream), "copy_batch, device descriptors")
+    return fn_dev, verify, algo, (src, dst, descs, dev)
+
+
 def make_rect(r, rows=8192, width=128 * 1024, pitch=256 * 1024, s_x=0, d_x=0):
     """rows x width bytes out of two pitched 2-D surfaces (rows x pitch each),
     the region starting s_x / d_x bytes into each row."""
@@ -612,6 +624,7 @@ def main():
                            ("fill_1GiB", lambda: make_fill(r, GIB)),
                            ("misaligned_1GiB", lambda: make_copy(r, GIB - 64, s_off=3, d_off=9)),
                            ("batch_65536", lambda: make_batch(r)),
+                           ("batch_65536_device_descriptors", lambda: make_batch_device(r)),
                            ("rect_8192x131072_262144", lambda: make_rect(r))):
             f2, v2, a2, k2 = maker()
             w2, us2 = r.time_launches(f2, 30, max(args.warmup, WARMUP_AFTER_IDLE))

@@ -146,6 +146,7 @@ struct mi355_aql {
   uint32_t* block_sum_dev = nullptr;
   ChunkRecord* records_dev = nullptr;
   size_t batch_capacity = 0, records_capacity = 0;
+  uint64_t* batch_seen = nullptr;  // host memory: copies << 32 | chunks of the last device-resident batch
 
   // bounce buffers of host<->device copies (mi355_aql_staging)
   void* bounce[2] = {nullptr, nullptr};
@@ -542,6 +543,7 @@ int mi355_aql_destroy(mi355_aql_t* h) {
     free_device(h->chunk_start_dev);
     free_device(h->block_sum_dev);
     free_device(h->records_dev);
+    free_device(h->batch_seen);
     free_device(h->bounce[0]);
     free_device(h->bounce[1]);
     if (h->idle_signal.handle) hsa_signal_destroy(h->idle_signal);
@@ -800,11 +802,19 @@ int copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, siz
   if (n > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   if (h->queue_error.load()) return MI355_BLIT_ERROR;
   if (n == 0) return mi355_aql_copy(h, h, h, 0, dep_signals, num_deps, completion_signal);
-  const BatchDeviceSizing sizing = batch_device_sizing(n, max_total_bytes);
-  if (sizing.records == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
 
   std::lock_guard<std::mutex> g(h->lock);
-  int rc = ensure_batch_capacity(h, n, sizing.records);
+  int rc;
+  if (!h->batch_seen) {
+    // where the copy kernel leaves its numbers of copies and chunks (batch_device_sizing)
+    if ((rc = alloc(h, h->host_pool, 64, reinterpret_cast<void**>(&h->batch_seen), true)) != MI355_BLIT_SUCCESS)
+      return rc;
+    *h->batch_seen = 0;
+  }
+  const BatchDeviceSizing sizing =
+      batch_device_sizing(n, max_total_bytes, *static_cast<volatile uint64_t*>(h->batch_seen));
+  if (sizing.records == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  rc = ensure_batch_capacity(h, n, sizing.records);
   if (rc != MI355_BLIT_SUCCESS) return rc;
   const mi355_blit_tuning_t* t = h->has_tuning ? &h->tuning : nullptr;
   const BatchDesc* descs = reinterpret_cast<const BatchDesc*>(device_descs);
@@ -823,7 +833,7 @@ int copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, siz
   if (!bk || l.split != 4) return MI355_BLIT_ERROR;
   BatchLookupArgs bc{{h->records_dev, sizing.records, h->chunk_start_dev + n, l.waves_per_wg, l.n_waves,
                       make_xcd_runs(p.grid, p.xcd_run)},
-                     descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n)};
+                     descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n), h->batch_seen};
   h->last_plan = p;
 
   const uint32_t nb = barrier_packets(num_deps);

@@ -175,6 +175,9 @@ struct BatchLookupArgs {
   const uint32_t* chunk_start;  // within each group of 1024 copies
   const uint32_t* block_sum;    // chunks in front of each group
   uint64_t n;
+  // Host memory where one lane leaves n << 32 | chunks for the host to size
+  // the next such batch by; may be null.
+  uint64_t* seen;
 };
 
 // A pitched 3-D region copy: `layers` slices of `rows` rows of `width` bytes.

@@ -79,6 +79,10 @@ struct mi355_blit {
   uint32_t* chunk_start_dev = nullptr;
   uint32_t* block_sum_dev = nullptr;
   ChunkRecord* records_dev = nullptr;  // one per chunk
+  // Pinned host memory where the copy kernel of a device-resident batch leaves
+  // its numbers of copies and chunks (batch_device_sizing); made with the
+  // first such batch.
+  uint64_t* batch_seen = nullptr;
   size_t records_capacity = 0;
   size_t batch_capacity = 0;
 };
@@ -370,6 +374,7 @@ int mi355_blit_destroy(mi355_blit_t* h) {
       if (h->batch_done[i]) (void)hipEventDestroy(h->batch_done[i]);
     free_batch_buffers(h);
     if (h->records_dev) (void)hipFree(h->records_dev);
+    if (h->batch_seen) (void)hipHostFree(h->batch_seen);
   }
   delete h;
   return rc;
@@ -502,7 +507,7 @@ int launch_lookup_copy(mi355_blit* h, hipStream_t s, const mi355_blit_plan_t& p,
   if (!k || l.split != 4) return MI355_BLIT_ERROR;
   BatchLookupArgs a{{h->records_dev, records, h->chunk_start_dev + n, l.waves_per_wg, l.n_waves,
                      make_xcd_runs(p.grid, p.xcd_run)},
-                    dev_descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n)};
+                    dev_descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n), h->batch_seen};
   hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
   return MI355_BLIT_SUCCESS;
 }
@@ -531,7 +536,11 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
     if (shape.total_chunks == 0) return MI355_BLIT_SUCCESS;
   } else {
     // lengths are only known on the device
-    sizing = batch_device_sizing(n, max_total_bytes);
+    if (!h->batch_seen) {
+      BLIT_HIP(hipHostMalloc(reinterpret_cast<void**>(&h->batch_seen), 64, hipHostMallocDefault));
+      *h->batch_seen = 0;
+    }
+    sizing = batch_device_sizing(n, max_total_bytes, *static_cast<volatile uint64_t*>(h->batch_seen));
     if (sizing.records == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
     shape.pieces = n;
     shape.total_chunks = sizing.grid_chunks;

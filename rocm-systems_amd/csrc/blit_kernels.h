@@ -679,6 +679,8 @@ __device__ __forceinline__ void batch_copy_lookup_body(const BatchLookupArgs& a)
   const unsigned lane = threadIdx.x & (kWave - 1);
   const uint64_t wave = global_wave_xcd(a.copy.waves_per_wg, a.copy.xcd);
   const uint64_t n_waves = a.copy.n_waves;
+  if (wave == 0 && lane == 0 && a.seen)
+    __hip_atomic_store(a.seen, a.n << 32 | total_chunks, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   for (uint64_t w = wave; w < total_chunks * SPLIT; w += n_waves) {
     const uint64_t c = w / SPLIT;
     const ChunkRecord rec = c < capacity ? load_record(records + c) : lookup_record(a, static_cast<uint32_t>(c));

@@ -736,10 +736,54 @@ def test_batch_unbounded_beyond_what_the_library_assumes(capi, blit, oracle, ran
     torch.cuda.synchronize()
     check_ok(capi, blit.copy_batch(descs_dev.data_ptr(), n, on_device=True), "copy_batch")
     check_ok(capi, blit.synchronize(), "synchronize")
-    assert blit.last_plan().grid == 32
+    assert blit.last_plan().grid * 2 < int((lens // 4096).sum())
     got = dst.host(0, total)
     want = _expect_batch(oracle, src_host, total, lens, offs, so, do)
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("path", ["hip", "aql"])
+def test_batch_unbounded_sizes_itself_by_the_batch_before(capi, pkg, oracle, arenas, torch_cuda, path):
+    """Without a bound the first device-resident batch on an engine is launched
+    for 8 chunks a copy; its copy kernel leaves the numbers of copies and chunks
+    in host memory and the next batch is launched for the same chunks per copy
+    plus 3 %.  Bytes are the oracle's whatever the guess."""
+    torch = torch_cuda
+    src, src_host, dst = arenas
+    eng = capi.Blit(0) if path == "hip" else pkg.aql.AqlBlit(0)
+    try:
+        rng = np.random.default_rng(4711)
+        n = 512
+        descs, lens, offs, so, do, total = _make_batch(capi, rng, src, dst, n, min_len=60 << 10, max_len=68 << 10)
+        chunks = sum((int(d.dst) % 4096 % 256 // 16 * 16 + int(d.bytes) + 4095) // 4096 for d in descs)
+        dev = _to_device(torch, descs)
+        want = _expect_batch(oracle, src_host, total, lens, offs, so, do)
+        grids = []
+        for call in range(3):
+            dst.fill(0, total, GUARD_BYTE)
+            torch.cuda.synchronize()
+            check_ok(capi, eng.copy_batch(dev.data_ptr(), n, on_device=True), "copy_batch")
+            check_ok(capi, eng.synchronize(), "synchronize")
+            grids.append(eng.last_plan().grid)
+            assert np.array_equal(dst.host(0, total), want), "call %d" % call
+        assert grids[0] == 8 * n
+        # 16 or 17 chunks a copy: the second and third launches follow what the first one counted
+        assert grids[1] == grids[2] and abs(grids[1] - chunks * 33 // 32 - 16) <= n // 4, (grids, chunks)
+        # a batch of short copies next: sized by the long ones once, by itself afterwards
+        n2 = 300
+        descs2, lens2, offs2, so2, do2, total2 = _make_batch(capi, rng, src, dst, n2, min_len=64, max_len=512)
+        dev2 = _to_device(torch, descs2)
+        want2 = _expect_batch(oracle, src_host, total2, lens2, offs2, so2, do2)
+        for call in range(2):
+            dst.fill(0, total2, GUARD_BYTE)
+            torch.cuda.synchronize()
+            check_ok(capi, eng.copy_batch(dev2.data_ptr(), n2, on_device=True), "copy_batch")
+            check_ok(capi, eng.synchronize(), "synchronize")
+            grids.append(eng.last_plan().grid)
+            assert np.array_equal(dst.host(0, total2), want2), "short copies, call %d" % call
+        assert grids[3] > 10 * n2 and grids[4] <= 2 * n2 + 32, grids
+    finally:
+        eng.close()
 
 
 def test_batch_65536_copies(capi, blit, oracle, rand, torch_cuda):

@@ -186,9 +186,7 @@ int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwo
  * memory; 32 KiB a copy before any has run), the kernels read the real chunk
  * count on the device, and a batch that differs from the guess is slower,
  * never wrong (a caller that knows a bound says so through
- * mi355_blit_copy_batch_bounded).  This is a path for many small copies:
- * copies of megabytes are not split among waves when their records are
- * written.  A batch may have at most 2^32-1
+ * mi355_blit_copy_batch_bounded).  A batch may have at most 2^32-1
  * chunks of 4 KiB.  Regions must not overlap one another.  A stream
  * under HIP graph capture -> INVALID_ARGUMENT (both batched entry points). */
 int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n,

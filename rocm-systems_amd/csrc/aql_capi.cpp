@@ -109,7 +109,7 @@ struct mi355_aql {
   std::vector<RectKernel> rect_kernels{MI355_FOR_EACH_RECT_KERNEL(MI355_RECT_NAME)};
   std::vector<RectKernel> rect_narrow_kernels{MI355_FOR_EACH_RECT_NARROW_KERNEL(MI355_RECT_NARROW_NAME)};
   std::vector<RectKernel> batch_lookup_kernels{MI355_FOR_EACH_BATCH_LOOKUP_KERNEL(MI355_BATCH_LOOKUP_NAME)};
-  Kernel scan_local, scan_top, emit_records, emit_records_device;
+  Kernel scan_local, scan_top, emit_records, emit_records_lookup;
 
   hsa_signal_t idle_signal{};  // completion signal of wait_idle's barrier packet
 
@@ -254,7 +254,7 @@ int load_code_object(mi355_aql* h) {
   if ((rc = lookup(h, "mi355_batch_scan_local", &h->scan_local)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_scan_top", &h->scan_top)) != MI355_BLIT_SUCCESS) return rc;
   if ((rc = lookup(h, "mi355_batch_emit_records", &h->emit_records)) != MI355_BLIT_SUCCESS) return rc;
-  if ((rc = lookup(h, "mi355_batch_emit_records_device", &h->emit_records_device)) != MI355_BLIT_SUCCESS) return rc;
+  if ((rc = lookup(h, "mi355_batch_emit_records_lookup", &h->emit_records_lookup)) != MI355_BLIT_SUCCESS) return rc;
   for (auto& k : h->batch_lookup_kernels)
     if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
   return MI355_BLIT_SUCCESS;
@@ -850,8 +850,8 @@ int copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, siz
   // every packet waits for the one before; the first also for whatever still uses the shared buffers
   write_dispatch(h, i++, h->scan_local, &sl, sizeof(sl), n_blocks, 1024, 0, true);
   write_dispatch(h, i++, h->scan_top, &stp, sizeof(stp), 1, 1024, 0, true);
-  write_dispatch(h, i++, h->emit_records_device, &er, sizeof(er), static_cast<uint32_t>((n + 255) / 256), 256, 0,
-                 true);
+  write_dispatch(h, i++, h->emit_records_lookup, &er, sizeof(er),
+                 static_cast<uint32_t>((sizing.records + 255) / 256), 256, 0, true);
   write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true);
   release_write_index(h, index, total);
   return MI355_BLIT_SUCCESS;

@@ -143,7 +143,7 @@ struct EmitRecordsArgs {
 
 // Device-resident descriptors: the prefix sum was done on the device
 // (chunk_start within each group of 1024 copies, block_sum across groups); one
-// lane per copy, records beyond `capacity` are not written.
+// lane per record, records beyond `capacity` are not written.
 struct EmitRecordsDeviceArgs {
   const BatchDesc* descs;
   const uint32_t* chunk_start;

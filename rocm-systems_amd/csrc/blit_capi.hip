@@ -603,8 +603,8 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
     launch_scans(h, s, dev_descs, n);
     EmitRecordsDeviceArgs er{dev_descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n),
                              h->records_dev, sizing.records};
-    hipLaunchKernelGGL(mi355_batch_emit_records_device, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0,
-                       s, er);
+    hipLaunchKernelGGL(mi355_batch_emit_records_lookup, dim3(static_cast<uint32_t>((sizing.records + 255) / 256)),
+                       dim3(256), 0, s, er);
     BLIT_HIP(hipGetLastError());
     rc = launch_lookup_copy(h, s, p, l, sizing.records, dev_descs, n);
     if (rc != MI355_BLIT_SUCCESS) return rc;

@@ -452,10 +452,9 @@ __device__ __forceinline__ ChunkRecord make_record(const BatchDesc& d, uint32_t 
 // by the host, into host memory or across the bus into device memory, behind
 // the GPU's caches: they are read at system scope.
 // Writes the records of one wave's 64 copies: lane l holds copy (dst, src,
-// bytes) with `chunks` records, the wave's records start at out[0] and at most
-// `room` of them are written.
+// bytes) with `chunks` records, the wave's records start at out[0].
 __device__ __forceinline__ void emit_wave_records(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t chunks,
-                                                  ChunkRecord* out, uint64_t room, unsigned lane) {
+                                                  ChunkRecord* out, unsigned lane) {
   // exclusive running sum of the chunk counts over the wave's lanes
   uint32_t incl = chunks;
 #pragma unroll
@@ -487,7 +486,7 @@ __device__ __forceinline__ void emit_wave_records(uint64_t dst, uint64_t src, ui
                                              __shfl(src_lo, owner, kWave));
     d.bytes = static_cast<uint64_t>(__shfl(len_hi, owner, kWave)) << 32 | __shfl(len_lo, owner, kWave);
     const uint32_t k = j - __shfl(excl, owner, kWave);
-    if (j < total && j < room) out[j] = make_record(d, k);
+    if (j < total) out[j] = make_record(d, k);
   }
 }
 
@@ -510,29 +509,7 @@ __device__ __forceinline__ void emit_records_body(const EmitRecordsArgs& a) {
   mine.bytes = bytes;
   const uint32_t chunks = valid ? desc_chunks(mine) : 0;
   // the wave's records are consecutive: lane 0's first record starts them
-  emit_wave_records(dst, src, bytes, chunks, a.records + __shfl(first, 0, kWave), ~0ull, lane);
-}
-
-// The same for device-resident descriptors, behind the two prefix-sum kernels:
-// a copy's first record is its group's sum plus its own running sum within the
-// group.  Copies may be of any length here (nothing has cut them), so a wave
-// may have many rounds to go through.
-__device__ __forceinline__ void emit_records_device_body(const EmitRecordsDeviceArgs& a) {
-  const unsigned lane = threadIdx.x & (kWave - 1);
-  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
-  const bool valid = i < a.n;
-  BatchDesc mine{nullptr, nullptr, 0};
-  uint64_t first = 0;
-  if (valid) {
-    mine = a.descs[i];
-    first = static_cast<uint64_t>(a.block_sum[i / 1024]) + a.chunk_start[i];
-  }
-  const uint32_t chunks = valid ? desc_chunks(mine) : 0;
-  const uint64_t wave_first = static_cast<uint64_t>(__shfl(static_cast<uint32_t>(first >> 32), 0, kWave)) << 32 |
-                              __shfl(static_cast<uint32_t>(first), 0, kWave);
-  const uint64_t room = wave_first < a.capacity ? a.capacity - wave_first : 0;
-  emit_wave_records(reinterpret_cast<uint64_t>(mine.dst), reinterpret_cast<uint64_t>(mine.src), mine.bytes, chunks,
-                    a.records + wave_first, room, lane);
+  emit_wave_records(dst, src, bytes, chunks, a.records + __shfl(first, 0, kWave), lane);
 }
 
 // Loads of one wave's share of a chunk: virtual vector indices [v0, v0 + 64 U)
@@ -640,29 +617,53 @@ __device__ __forceinline__ void batch_copy_records_body(const BatchCopyArgs& a) 
   }
 }
 
-// Chunk c of a batch of device-resident descriptors, from the prefix sums: the
-// group of 1024 copies it falls into, then the copy within the group (the last
-// one that starts at or before c: copies without chunks share their start with
-// their successor and lose to it).  c is below the batch's chunk total.
-__device__ __forceinline__ ChunkRecord lookup_record(const BatchLookupArgs& a, uint32_t c) {
-  const uint32_t* __restrict__ block_sum = a.block_sum;
-  const uint32_t* __restrict__ chunk_start = a.chunk_start;
-  uint64_t lo = 0, hi = (a.n + 1023) / 1024 - 1;
+// The copy that chunk c of a batch of device-resident descriptors belongs to,
+// from the prefix sums: the group of 1024 copies it falls into, then the copy
+// within the group (the last one that starts at or before c: copies without
+// chunks share their start with their successor and lose to it).  c is below
+// the batch's chunk total; *k is the chunk's index within its copy.
+__device__ __forceinline__ uint64_t find_copy_of_chunk(const uint32_t* __restrict__ block_sum,
+                                                       const uint32_t* __restrict__ chunk_start, uint64_t n,
+                                                       uint32_t c, uint32_t* k) {
+  uint64_t lo = 0, hi = (n + 1023) / 1024 - 1;
   while (lo < hi) {
     const uint64_t mid = lo + (hi - lo + 1) / 2;
     if (ld_u32<false>(block_sum + mid) <= c) lo = mid; else hi = mid - 1;
   }
   const uint32_t rem = c - ld_u32<false>(block_sum + lo);
   lo *= 1024;
-  hi = lo + 1023 < a.n ? lo + 1023 : a.n - 1;
+  hi = lo + 1023 < n ? lo + 1023 : n - 1;
   while (lo < hi) {
     const uint64_t mid = lo + (hi - lo + 1) / 2;
     if (ld_u32<false>(chunk_start + mid) <= rem) lo = mid; else hi = mid - 1;
   }
+  *k = rem - ld_u32<false>(chunk_start + lo);
+  return lo;
+}
+
+// The record of chunk c, the same for every lane of the wave.
+__device__ __forceinline__ ChunkRecord lookup_record(const BatchLookupArgs& a, uint32_t c) {
+  uint32_t k;
+  const uint64_t found = find_copy_of_chunk(a.block_sum, a.chunk_start, a.n, c, &k);
   // Every lane has found the same copy: say so, and its descriptor comes in
   // through scalar loads like a record.
-  const uint32_t i = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(lo));
-  return make_record(load_desc(a.descs + i), rem - ld_u32<false>(chunk_start + i));
+  const uint32_t i = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(found));
+  return make_record(load_desc(a.descs + i), __builtin_amdgcn_readfirstlane(k));
+}
+
+// Records for device-resident descriptors, one lane per record: the lane finds
+// its copy through the prefix sums.  Launched with workgroups of 256 over the
+// record buffer's capacity; lanes beyond the batch's chunk total have nothing
+// to do.  Costs the same whatever the copies' lengths (a wave writing the
+// records of its own 64 copies stalls on a long copy: 100 copies of 4 MiB took
+// 300 us that way).
+__device__ __forceinline__ void emit_records_lookup_body(const EmitRecordsDeviceArgs& a) {
+  const uint64_t j = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+  const uint64_t total = ld_u32<false>(a.chunk_start + a.n);
+  if (j >= total || j >= a.capacity) return;
+  uint32_t k;
+  const uint64_t i = find_copy_of_chunk(a.block_sum, a.chunk_start, a.n, static_cast<uint32_t>(j), &k);
+  a.records[j] = make_record(a.descs[i], k);
 }
 
 // The copy over records when only the device knows how many chunks there are:
@@ -986,8 +987,8 @@ extern "C" __global__ void __launch_bounds__(1024) mi355_batch_scan_top(mi355::S
 extern "C" __global__ void __launch_bounds__(256) mi355_batch_emit_records(mi355::EmitRecordsArgs a) {
   mi355::emit_records_body(a);
 }
-extern "C" __global__ void __launch_bounds__(256) mi355_batch_emit_records_device(mi355::EmitRecordsDeviceArgs a) {
-  mi355::emit_records_device_body(a);
+extern "C" __global__ void __launch_bounds__(256) mi355_batch_emit_records_lookup(mi355::EmitRecordsDeviceArgs a) {
+  mi355::emit_records_lookup_body(a);
 }
 extern "C" __global__ void __launch_bounds__(64) mi355_signal_complete(mi355::SignalArgs a) {
   mi355::signal_complete_body(a);

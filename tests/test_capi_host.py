@@ -252,7 +252,7 @@ def test_aql_code_object_holds_every_kernel_variant(pkg):
         for s in range(4):
             assert "mi355_batch_lookup_l%d_s%d" % (l, s) in names
     for n in ("mi355_batch_scan_local", "mi355_batch_scan_top", "mi355_batch_emit_records",
-              "mi355_batch_emit_records_device", "mi355_signal_complete"):
+              "mi355_batch_emit_records_lookup", "mi355_signal_complete"):
         assert n in names
 
 

@@ -741,7 +741,7 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   const mi355_blit_tuning_t* t = h->has_tuning ? &h->tuning : nullptr;
 
   // Stage what the GPU needs: the descriptors, cut into pieces of at most
-  // 1 MiB, and each piece's first record index (the host, which walks the
+  // 64 chunks, and each piece's first record index (the host, which walks the
   // descriptors anyway, does the prefix sum).  The buffer is free again when
   // the kernel that read it last has finished.
   const unsigned b = h->next_stage;

@@ -3,11 +3,11 @@
 // copy, and the staging image the GPU reads.  Pure host code.
 //
 // The host walks the descriptors anyway to validate them, so it also does the
-// prefix sum over their chunk counts: the GPU then needs one small kernel (one
-// lane per copy writes that copy's chunk records) before the copy kernel.
-// Copies longer than 1 MiB are cut at 1 MiB boundaries of the destination into
-// pieces that are copies in their own right, so that no lane has more than
-// 257 records to write.  No counterpart in the reference.
+// prefix sum over their chunk counts: the GPU then needs one small kernel (a
+// wave writes the chunk records of its 64 copies) before the copy kernel.
+// Copies of more than 64 chunks are cut into pieces of 64 chunks that are
+// copies in their own right, so that no wave has more than 64 rounds of
+// records to write.  No counterpart in the reference.
 #ifndef MI355_BLIT_BATCH_HOST_H_
 #define MI355_BLIT_BATCH_HOST_H_
 
@@ -22,7 +22,13 @@
 
 namespace mi355 {
 
-constexpr uint64_t kBatchPieceBytes = 1ull << 20;
+// A long copy is handed to the GPU as pieces of 64 chunks, copies in their
+// own right: the record kernel gives a wave 64 pieces, whose records it writes
+// 64 at a time, so a wave has at most 64 rounds to go through however long the
+// copies are (100 copies of 4 MiB: 164 us, 228 us with pieces of 1 MiB).  Pieces
+// end where the copy's own chunks end, so cutting adds no chunk.
+constexpr uint64_t kBatchPieceChunks = 64;
+constexpr uint64_t kBatchPieceBytes = kBatchPieceChunks * 16 * kBatchChunkVecs;  // plus up to 15 bytes at either end
 
 struct BatchShape {
   uint64_t pieces = 0;        // descriptors after cutting
@@ -111,10 +117,16 @@ inline BatchDeviceSizing batch_device_sizing(uint64_t n, uint64_t max_total_byte
 template <typename F>
 inline void batch_for_each_piece(const mi355_blit_desc_t& d, F f) {
   const uint64_t dst = reinterpret_cast<uintptr_t>(d.dst), src = reinterpret_cast<uintptr_t>(d.src);
+  // the copy's chunks are 4 KiB steps from the 256-byte boundary at or below
+  // its first 16-byte aligned destination byte
+  uint64_t head = (16 - (dst & 15)) & 15;
+  if (head > d.bytes) head = d.bytes;
+  const uint64_t anchor = (dst + head) & ~255ull;
   uint64_t at = 0;
-  while (at < d.bytes) {
-    uint64_t end = ((dst + at) / kBatchPieceBytes + 1) * kBatchPieceBytes - dst;
-    if (end > d.bytes) end = d.bytes;
+  for (uint64_t piece = 1; at < d.bytes; ++piece) {
+    uint64_t end = anchor + piece * kBatchPieceBytes - dst;
+    // fewer than 16 bytes left over are the tail of this piece's last chunk
+    if (end > d.bytes || d.bytes - end < 16) end = d.bytes;
     f(dst + at, src + at, end - at);
     at = end;
   }
@@ -134,7 +146,6 @@ struct BatchImage {
 // 3.6 ns per descriptor (236 us for 65,536), which is what bounds a batch of
 // many tiny copies: the GPU finishes 65,536 copies of 256 bytes in 67 us.
 inline int batch_build(const mi355_blit_desc_t* descs, size_t n, BatchImage* image, BatchShape* out) {
-  static_assert((kBatchPieceBytes & (kBatchPieceBytes - 1)) == 0, "pieces end at multiples of a power of two");
   BatchShape s;
   image->count = 0;
   size_t cap = image->pieces.size();
@@ -168,8 +179,8 @@ inline int batch_build(const mi355_blit_desc_t* descs, size_t n, BatchImage* ima
     if (!d.dst || !d.src) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
     bytes += d.bytes;
     const uint64_t dst = reinterpret_cast<uintptr_t>(d.dst);
-    if (((dst ^ (dst + d.bytes - 1)) / kBatchPieceBytes) == 0)
-      add(dst, reinterpret_cast<uintptr_t>(d.src), d.bytes);  // the usual case: no boundary inside the copy
+    if (d.bytes <= kBatchPieceBytes - 256)
+      add(dst, reinterpret_cast<uintptr_t>(d.src), d.bytes);  // the usual case: one piece wherever it starts
     else
       batch_for_each_piece(d, add);
     if (chunks > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;

@@ -567,7 +567,7 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
   if (!descs_on_device) {
     // Host-resident descriptors.  The host has walked them to validate them
     // and does the prefix sum over their chunk counts on the way; the image it
-    // stages (the descriptors, cut into pieces of at most 1 MiB, and each
+    // stages (the descriptors, cut into pieces of at most 64 chunks, and each
     // piece's first record index) is all the GPU needs to write the records
     // with one lane per piece.  The two staging buffers alternate, so staging
     // one batch overlaps the execution of the one before; a buffer is only

@@ -241,9 +241,10 @@ void one_rect_plan() {
   }
 }
 
-// The staging image of a batch: the pieces must tile every copy in order, no
-// piece may be longer than 1 MiB or cross a 1 MiB boundary of the destination,
-// and the record indices must be the running sum of the pieces' chunk counts.
+// The staging image of a batch: the pieces must tile every copy in order, a
+// piece has at most 64 chunks and every piece but a copy's last has exactly 64,
+// cutting adds no chunk to the copy, and the record indices must be the
+// running sum of the pieces' chunk counts.
 void one_batch_stage() {
   const size_t n = 1 + below(40);
   std::vector<mi355_blit_desc_t> descs(n);
@@ -266,16 +267,14 @@ void one_batch_stage() {
   CHECK(image.count == shape.pieces && pieces.size() >= image.count && starts.size() >= image.count, "image size");
   uint64_t p = 0, chunks = 0, bytes = 0;
   for (const auto& d : descs) {
-    uint64_t at = 0;
+    uint64_t at = 0, copy_chunks = 0;
     while (at < d.bytes) {
       CHECK(p < shape.pieces, "more pieces than counted");
       const BatchDesc& q = pieces[p];
       const uint64_t qd = reinterpret_cast<uint64_t>(q.dst), qs = reinterpret_cast<uint64_t>(q.src);
       CHECK(qd == reinterpret_cast<uint64_t>(d.dst) + at && qs == reinterpret_cast<uint64_t>(d.src) + at,
             "piece %" PRIu64 " does not continue its copy", p);
-      CHECK(q.bytes >= 1 && q.bytes <= kBatchPieceBytes && at + q.bytes <= d.bytes, "piece length %" PRIu64, q.bytes);
-      CHECK(qd / kBatchPieceBytes == (qd + q.bytes - 1) / kBatchPieceBytes, "piece crosses a 1 MiB boundary");
-      CHECK(at + q.bytes == d.bytes || (qd + q.bytes) % kBatchPieceBytes == 0, "piece stops short of the boundary");
+      CHECK(q.bytes >= 1 && q.bytes <= kBatchPieceBytes + 30 && at + q.bytes <= d.bytes, "piece length %" PRIu64, q.bytes);
       CHECK(starts[p] == chunks, "record index of piece %" PRIu64, p);
       // the chunk count, from the geometry of 256-byte anchored 4 KiB chunks
       const uint64_t head = q.bytes < ((16 - (qd & 15)) & 15) ? q.bytes : ((16 - (qd & 15)) & 15);
@@ -283,12 +282,18 @@ void one_batch_stage() {
       // 4 KiB steps from the 256-byte boundary below the body's first vector
       const uint64_t anchor = body_lo & ~255ull;
       const uint64_t c = body_hi > body_lo ? (body_hi - anchor + 4095) / 4096 : 1;
-      CHECK(c <= 257, "a piece with %" PRIu64 " chunks", c);
+      CHECK(c <= kBatchPieceChunks, "a piece with %" PRIu64 " chunks", c);
+      CHECK(at + q.bytes == d.bytes || (c == kBatchPieceChunks && (qd + q.bytes) % 256 == 0),
+            "a piece of %" PRIu64 " chunks in the middle of a copy", c);
+      CHECK(c == batch_desc_chunks(qd, q.bytes), "chunk count of a piece");
+      copy_chunks += c;
       chunks += c;
       bytes += q.bytes;
       at += q.bytes;
       ++p;
     }
+    CHECK(d.bytes == 0 || copy_chunks == batch_desc_chunks(reinterpret_cast<uint64_t>(d.dst), d.bytes),
+          "cutting changed a copy's chunk count: %" PRIu64, copy_chunks);
   }
   CHECK(p == shape.pieces && chunks == shape.total_chunks && bytes == shape.total_bytes, "shape totals");
   mi355_blit_desc_t bad = descs[0];

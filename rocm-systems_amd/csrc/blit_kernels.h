@@ -622,29 +622,46 @@ __device__ __forceinline__ void batch_copy_records_body(const BatchCopyArgs& a) 
 // within the group (the last one that starts at or before c: copies without
 // chunks share their start with their successor and lose to it).  c is below
 // the batch's chunk total; *k is the chunk's index within its copy.
+// UNIFORM: c is the same for every lane of the wave, and the prefix sums come
+// in through scalar loads (the constant address space, as for a record).
+template <bool UNIFORM>
+__device__ __forceinline__ uint32_t ld_prefix(const uint32_t* p) {
+  if constexpr (UNIFORM) {
+    typedef const uint32_t __attribute__((address_space(4))) * ConstPtr;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wold-style-cast"
+    return *(ConstPtr)(p);
+#pragma clang diagnostic pop
+  } else {
+    return ld_u32<false>(p);
+  }
+}
+
+template <bool UNIFORM>
 __device__ __forceinline__ uint64_t find_copy_of_chunk(const uint32_t* __restrict__ block_sum,
                                                        const uint32_t* __restrict__ chunk_start, uint64_t n,
                                                        uint32_t c, uint32_t* k) {
   uint64_t lo = 0, hi = (n + 1023) / 1024 - 1;
   while (lo < hi) {
     const uint64_t mid = lo + (hi - lo + 1) / 2;
-    if (ld_u32<false>(block_sum + mid) <= c) lo = mid; else hi = mid - 1;
+    if (ld_prefix<UNIFORM>(block_sum + mid) <= c) lo = mid; else hi = mid - 1;
   }
-  const uint32_t rem = c - ld_u32<false>(block_sum + lo);
+  const uint32_t rem = c - ld_prefix<UNIFORM>(block_sum + lo);
   lo *= 1024;
   hi = lo + 1023 < n ? lo + 1023 : n - 1;
   while (lo < hi) {
     const uint64_t mid = lo + (hi - lo + 1) / 2;
-    if (ld_u32<false>(chunk_start + mid) <= rem) lo = mid; else hi = mid - 1;
+    if (ld_prefix<UNIFORM>(chunk_start + mid) <= rem) lo = mid; else hi = mid - 1;
   }
-  *k = rem - ld_u32<false>(chunk_start + lo);
+  *k = rem - ld_prefix<UNIFORM>(chunk_start + lo);
   return lo;
 }
 
 // The record of chunk c, the same for every lane of the wave.
 __device__ __forceinline__ ChunkRecord lookup_record(const BatchLookupArgs& a, uint32_t c) {
   uint32_t k;
-  const uint64_t found = find_copy_of_chunk(a.block_sum, a.chunk_start, a.n, c, &k);
+  const uint64_t found = find_copy_of_chunk<true>(a.block_sum, a.chunk_start, a.n,
+                                                  __builtin_amdgcn_readfirstlane(c), &k);
   // Every lane has found the same copy: say so, and its descriptor comes in
   // through scalar loads like a record.
   const uint32_t i = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(found));
@@ -662,7 +679,7 @@ __device__ __forceinline__ void emit_records_lookup_body(const EmitRecordsDevice
   const uint64_t total = ld_u32<false>(a.chunk_start + a.n);
   if (j >= total || j >= a.capacity) return;
   uint32_t k;
-  const uint64_t i = find_copy_of_chunk(a.block_sum, a.chunk_start, a.n, static_cast<uint32_t>(j), &k);
+  const uint64_t i = find_copy_of_chunk<false>(a.block_sum, a.chunk_start, a.n, static_cast<uint32_t>(j), &k);
   a.records[j] = make_record(a.descs[i], k);
 }
 

@@ -211,6 +211,15 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
   // there: the rows' cut ends are partial lines).
   uint32_t unroll = whole_lines ? 1 : 2;
   uint32_t default_wg = whole_lines ? 256 : 128;
+  // Long rows that are not whole lines behave like the linear copy with a byte
+  // offset: single waves with one vector per lane, in XCD runs (1 GiB moved, any
+  // alignment: rows of 64 KiB 345 us against 347 us, of 128 KiB 336 against 341,
+  // of 512 KiB 328 against 335, of 8 MiB 323 against 358; rows of 32 KiB equal,
+  // of 16 KiB 341 against 329, hence the threshold).
+  if (!whole_lines && width >= (48u << 10) && out->total_bytes >= kXcdRunMinBytes) {
+    unroll = 1;
+    default_wg = 64;
+  }
   if (link) {
     unroll = 1;
     default_wg = 256;

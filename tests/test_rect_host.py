@@ -279,6 +279,13 @@ def test_plan_rect_slots_follow_row_alignment(capi_host):
     assert p.xcd_run == 0                                                                     # 4 MiB
     st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4100, 32768, 1))
     assert st == SUCCESS and (p.wg_size, p.unroll, p.xcd_run) == (128, 2, 144)               # 144 x 4 KiB
+    # ragged rows of 48 KiB and more: the shape of the linear copy with a byte offset
+    st, p = capi_host.plan_rect((base_d, 262148, 0), (9, 0, 0), (base_s, 262148, 0), (3, 0, 0), (48 * 1024 - 1, 8192, 1))
+    assert st == SUCCESS and (p.wg_size, p.unroll, p.xcd_run, p.store_policy) == (128, 2, 144, capi_host.STORE_NT)
+    st, p = capi_host.plan_rect((base_d, 262148, 0), (9, 0, 0), (base_s, 262148, 0), (3, 0, 0), (131065, 8192, 1))
+    assert st == SUCCESS and (p.wg_size, p.unroll, p.xcd_run, p.store_policy) == (64, 1, 576, capi_host.STORE_NT)
+    st, p = capi_host.plan_rect((base_d, 262148, 0), (9, 0, 0), (base_s, 262148, 0), (3, 0, 0), (131065, 128, 1))
+    assert st == SUCCESS and (p.wg_size, p.unroll, p.xcd_run) == (128, 2, 0)                  # 16 MiB: no runs yet
     st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 32768, 1))
     assert st == SUCCESS and (p.plain_rows, p.wg_size, p.xcd_run) == (1, 64, 576)              # tiled like a linear copy
     st, p = capi_host.plan_rect((base_d, 8192, 0), (128, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 32768, 1))

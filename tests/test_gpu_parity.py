@@ -808,6 +808,17 @@ def test_batch_65536_copies(capi, blit, oracle, rand, torch_cuda):
     want = np.full(total, GUARD_BYTE, dtype=np.uint8)
     want[:total2] = _expect_batch(oracle, src_host, total2, lens, offs, so, do)
     assert np.array_equal(got, want)
+    # the same descriptors resident in device memory: sized by the library's
+    # assumption, by the batch before, and by the caller's bound
+    descs_dev = _to_device(torch, descs)
+    for submit in (lambda: blit.copy_batch(descs_dev.data_ptr(), n, on_device=True),
+                   lambda: blit.copy_batch(descs_dev.data_ptr(), n, on_device=True),
+                   lambda: blit.copy_batch_bounded(descs_dev.data_ptr(), n, int(lens.sum()))):
+        dst.fill(0, total, GUARD_BYTE)
+        torch.cuda.synchronize()
+        check_ok(capi, submit(), "copy_batch, device-resident descriptors")
+        check_ok(capi, blit.synchronize(), "synchronize")
+        assert np.array_equal(dst.host(), want)
 
 
 def test_batch_back_to_back_reuses_staging(capi, blit, oracle, arenas):

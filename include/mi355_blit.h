@@ -178,8 +178,9 @@ int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwo
 
 /* Batched small-copy descriptor path: n independent copies in one submission.
  * No counterpart in the reference (it submits one AQL packet per copy).
- * descs may live in host memory (descs_on_device == 0: the library stages
- * them) or be device-resident (descs_on_device != 0: read in place, must stay
+ * descs may live in host memory (descs_on_device == 0: the library checks and
+ * stages them before it returns, so the array may be reused at once) or be
+ * device-resident (descs_on_device != 0: read in place, must stay
  * valid until completion).  The host cannot see the lengths of
  * device-resident descriptors: it sizes the launch by the bytes per copy of
  * the last such batch on the handle (which the copy kernel leaves in host

@@ -144,6 +144,7 @@ struct mi355_aql {
   unsigned next_stage = 0;
   uint32_t* chunk_start_dev = nullptr;
   uint32_t* block_sum_dev = nullptr;
+  BatchDesc* descs_private_dev = nullptr;  // the GPU's own copy of descriptors the host staged as they were
   ChunkRecord* records_dev = nullptr;
   size_t batch_capacity = 0, records_capacity = 0;
   uint64_t* batch_seen = nullptr;  // host memory: copies << 32 | chunks of the last device-resident batch
@@ -431,8 +432,10 @@ int ensure_batch_capacity(mi355_aql* h, size_t n, size_t n_records) {
     }
     free_device(h->chunk_start_dev);
     free_device(h->block_sum_dev);
+    free_device(h->descs_private_dev);
     h->chunk_start_dev = nullptr;
     h->block_sum_dev = nullptr;
+    h->descs_private_dev = nullptr;
     h->batch_capacity = 0;
     for (int i = 0; i < 2; ++i) {
       if ((rc = alloc_stage(h, batch_stage_bytes(cap), i)) != MI355_BLIT_SUCCESS) return rc;
@@ -441,6 +444,8 @@ int ensure_batch_capacity(mi355_aql* h, size_t n, size_t n_records) {
     if ((rc = alloc(h, h->local_pool, (cap + 1) * sizeof(uint32_t), reinterpret_cast<void**>(&h->chunk_start_dev), false)))
       return rc;
     if ((rc = alloc(h, h->local_pool, (cap / 1024 + 1) * sizeof(uint32_t), reinterpret_cast<void**>(&h->block_sum_dev), false)))
+      return rc;
+    if ((rc = alloc(h, h->local_pool, cap * sizeof(BatchDesc), reinterpret_cast<void**>(&h->descs_private_dev), false)))
       return rc;
     h->batch_capacity = cap;
   }
@@ -542,6 +547,7 @@ int mi355_aql_destroy(mi355_aql_t* h) {
     }
     free_device(h->chunk_start_dev);
     free_device(h->block_sum_dev);
+    free_device(h->descs_private_dev);
     free_device(h->records_dev);
     free_device(h->batch_seen);
     free_device(h->bounce[0]);
@@ -722,12 +728,46 @@ int mi355_aql_fill32(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dword
   return MI355_BLIT_SUCCESS;
 }
 
+namespace {
+int copy_batch_device_locked(mi355_aql_t* h, const BatchDesc* scanned, size_t n, uint64_t max_total_bytes,
+                             uint64_t staged_free, const uint64_t* dep_signals, uint32_t num_deps,
+                             uint64_t completion_signal);
+}
+
 int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t n, const uint64_t* dep_signals,
                          uint32_t num_deps, uint64_t completion_signal) {
   if (!h || (!descs && n) || (num_deps && !dep_signals)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   if (n > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   if (h->queue_error.load()) return MI355_BLIT_ERROR;
   std::unique_lock<std::mutex> g(h->lock);
+  if (batch_prefers_raw_staging(descs, n)) {
+    // The walk below would take longer than the copies: stage the descriptors
+    // as they are and take them from there like device-resident ones.
+    int rc = ensure_batch_capacity(h, n, 0);
+    if (rc != MI355_BLIT_SUCCESS) return rc;
+    const unsigned b = h->next_stage;
+    while (hsa_signal_wait_scacquire(h->stage_free[b], HSA_SIGNAL_CONDITION_LT, 1, UINT64_MAX, HSA_WAIT_STATE_ACTIVE) >= 1) {
+      if (h->queue_error.load()) return MI355_BLIT_ERROR;
+    }
+    uint64_t total_bytes = 0;
+    rc = batch_stage_raw(descs, n, h->stage[b], &total_bytes);
+    if (rc != MI355_BLIT_SUCCESS) return rc;
+    if (total_bytes == 0) {
+      g.unlock();
+      return mi355_aql_copy(h, h, h, 0, dep_signals, num_deps, completion_signal);
+    }
+    if (h->stage_in_device_memory[b]) {
+      _mm_sfence();
+      (void)*(reinterpret_cast<volatile uint32_t*>(h->stage[b] + n) - 1);
+    }
+    h->next_stage ^= 1;
+    hsa_signal_store_relaxed(h->stage_free[b], 1);
+    // the bytes are known exactly: they size the launch as a caller's bound would
+    rc = copy_batch_device_locked(h, h->stage[b], n, total_bytes, h->stage_free[b].handle, dep_signals, num_deps,
+                                  completion_signal);
+    if (rc != MI355_BLIT_SUCCESS) hsa_signal_store_relaxed(h->stage_free[b], 0);
+    return rc;
+  }
   BatchShape shape;
   int rc = batch_build(descs, n, &h->stage_image, &shape);
   if (rc != MI355_BLIT_SUCCESS) return rc;
@@ -796,14 +836,12 @@ namespace {
 // the two launches of the prefix sum, the records, and the copy, whose grid
 // and record buffer follow batch_device_sizing and which reads the number of
 // chunks on the device.
-int copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, size_t n, uint64_t max_total_bytes,
-                      const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal) {
-  if (!h || (!device_descs && n) || (num_deps && !dep_signals)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
-  if (n > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
-  if (h->queue_error.load()) return MI355_BLIT_ERROR;
-  if (n == 0) return mi355_aql_copy(h, h, h, 0, dep_signals, num_deps, completion_signal);
-
-  std::lock_guard<std::mutex> g(h->lock);
+// With h->lock held.  staged_free != 0: the descriptors are ones the host
+// staged; the first kernel, their only reader, leaves a copy for the others
+// and sets that signal to 0 when it is done.
+int copy_batch_device_locked(mi355_aql_t* h, const BatchDesc* scanned, size_t n, uint64_t max_total_bytes,
+                             uint64_t staged_free, const uint64_t* dep_signals, uint32_t num_deps,
+                             uint64_t completion_signal) {
   int rc;
   if (!h->batch_seen) {
     // where the copy kernel leaves its numbers of copies and chunks (batch_device_sizing)
@@ -817,9 +855,10 @@ int copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, siz
   rc = ensure_batch_capacity(h, n, sizing.records);
   if (rc != MI355_BLIT_SUCCESS) return rc;
   const mi355_blit_tuning_t* t = h->has_tuning ? &h->tuning : nullptr;
-  const BatchDesc* descs = reinterpret_cast<const BatchDesc*>(device_descs);
+  const BatchDesc* descs = staged_free ? h->descs_private_dev : scanned;
   const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
-  ScanLocalArgs sl{descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
+  ScanLocalArgs sl{scanned, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev,
+                   staged_free ? h->descs_private_dev : nullptr};
   ScanTopArgs stp{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
   EmitRecordsDeviceArgs er{descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n), h->records_dev,
                            sizing.records};
@@ -848,13 +887,24 @@ int copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, siz
   write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
   uint64_t i = index + nb;
   // every packet waits for the one before; the first also for whatever still uses the shared buffers
-  write_dispatch(h, i++, h->scan_local, &sl, sizeof(sl), n_blocks, 1024, 0, true);
+  write_dispatch(h, i++, h->scan_local, &sl, sizeof(sl), n_blocks, 1024, staged_free, true);
   write_dispatch(h, i++, h->scan_top, &stp, sizeof(stp), 1, 1024, 0, true);
   write_dispatch(h, i++, h->emit_records_lookup, &er, sizeof(er),
                  static_cast<uint32_t>((sizing.records + 255) / 256), 256, 0, true);
   write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true);
   release_write_index(h, index, total);
   return MI355_BLIT_SUCCESS;
+}
+
+int copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, size_t n, uint64_t max_total_bytes,
+                      const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal) {
+  if (!h || (!device_descs && n) || (num_deps && !dep_signals)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (n > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (h->queue_error.load()) return MI355_BLIT_ERROR;
+  if (n == 0) return mi355_aql_copy(h, h, h, 0, dep_signals, num_deps, completion_signal);
+  std::lock_guard<std::mutex> g(h->lock);
+  return copy_batch_device_locked(h, reinterpret_cast<const BatchDesc*>(device_descs), n, max_total_bytes, 0,
+                                  dep_signals, num_deps, completion_signal);
 }
 }  // namespace
 

@@ -123,6 +123,10 @@ struct ScanLocalArgs {
   uint64_t n;
   uint32_t* chunk_start;
   uint32_t* block_sum;
+  // Not null: descs were staged by the host (into host memory, or across the
+  // bus into device memory, behind the GPU's caches); they are read at system
+  // scope and copied here for the kernels that follow.
+  BatchDesc* private_copy;
 };
 
 struct ScanTopArgs {

@@ -78,6 +78,7 @@ struct mi355_blit {
   hipStream_t last_batch_stream = nullptr;
   uint32_t* chunk_start_dev = nullptr;
   uint32_t* block_sum_dev = nullptr;
+  BatchDesc* descs_private_dev = nullptr;  // the GPU's own copy of descriptors the host staged as they were
   ChunkRecord* records_dev = nullptr;  // one per chunk
   // Pinned host memory where the copy kernel of a device-resident batch leaves
   // its numbers of copies and chunks (batch_device_sizing); made with the
@@ -240,8 +241,10 @@ void free_batch_buffers(mi355_blit* h) {
   }
   if (h->chunk_start_dev) (void)hipFree(h->chunk_start_dev);
   if (h->block_sum_dev) (void)hipFree(h->block_sum_dev);
+  if (h->descs_private_dev) (void)hipFree(h->descs_private_dev);
   h->chunk_start_dev = nullptr;
   h->block_sum_dev = nullptr;
+  h->descs_private_dev = nullptr;
   h->batch_capacity = 0;
 }
 
@@ -268,6 +271,7 @@ int ensure_batch_capacity(mi355_blit* h, size_t n, size_t n_records) {
     }
     BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->chunk_start_dev), (cap + 1) * sizeof(uint32_t)));
     BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->block_sum_dev), (cap / 1024 + 1) * sizeof(uint32_t)));
+    BLIT_HIP(hipMalloc(reinterpret_cast<void**>(&h->descs_private_dev), cap * sizeof(BatchDesc)));
     h->batch_capacity = cap;
   }
   if (n_records > h->records_capacity) {
@@ -479,9 +483,9 @@ int mi355_blit_copy_batch_bounded(mi355_blit_t* h, const mi355_blit_desc_t* devi
 namespace {
 // The two launches of the device-side prefix sum over the copies' chunk
 // counts: chunk_start within groups of 1024 copies, block_sum across groups.
-void launch_scans(mi355_blit* h, hipStream_t s, const BatchDesc* dev_descs, size_t n) {
+void launch_scans(mi355_blit* h, hipStream_t s, const BatchDesc* dev_descs, size_t n, BatchDesc* private_copy) {
   const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
-  ScanLocalArgs sl{dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev};
+  ScanLocalArgs sl{dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev, private_copy};
   hipLaunchKernelGGL(mi355_batch_scan_local, dim3(n_blocks), dim3(1024), 0, s, sl);
   ScanTopArgs st{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
   hipLaunchKernelGGL(mi355_batch_scan_top, dim3(1), dim3(1024), 0, s, st);
@@ -528,12 +532,46 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
     return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   }
 
+  // Host-resident descriptors go one of two ways: the host walks them (the
+  // exact chunk total, one small kernel before the copy), or, when the walk
+  // would take longer than the copies themselves, they are staged as they are
+  // and taken from there like device-resident ones.
+  const bool raw = !descs_on_device && batch_prefers_raw_staging(descs, n);
+  const bool walk = !descs_on_device && !raw;
   BatchShape shape;
   BatchDeviceSizing sizing{};
-  if (!descs_on_device) {
-    int rc = batch_build(descs, n, &h->stage_image, &shape);
+  int rc;
+  if (walk) {
+    rc = batch_build(descs, n, &h->stage_image, &shape);
     if (rc != MI355_BLIT_SUCCESS) return rc;
     if (shape.total_chunks == 0) return MI355_BLIT_SUCCESS;
+    rc = ensure_batch_capacity(h, shape.pieces, shape.total_chunks);
+    if (rc != MI355_BLIT_SUCCESS) return rc;
+  } else {
+    rc = ensure_batch_capacity(h, n, 0);
+    if (rc != MI355_BLIT_SUCCESS) return rc;
+  }
+
+  // The two staging buffers alternate, so staging one batch overlaps the
+  // execution of the one before; a buffer is only waited for until the batch
+  // that used it, two batches ago, has finished.
+  const unsigned b = h->next_host;
+  if (!descs_on_device && h->batch_busy[b]) {
+    BLIT_HIP(hipEventSynchronize(h->batch_done[b]));
+    h->batch_busy[b] = false;
+  }
+  size_t staged_bytes = 0;
+  if (walk) {
+    staged_bytes = batch_stage_bytes(shape.pieces);
+    batch_stage(h->stage_image, h->descs_host[b]);
+  } else if (raw) {
+    uint64_t total_bytes = 0;
+    rc = batch_stage_raw(descs, n, h->descs_host[b], &total_bytes);
+    if (rc != MI355_BLIT_SUCCESS) return rc;
+    if (total_bytes == 0) return MI355_BLIT_SUCCESS;
+    staged_bytes = n * sizeof(BatchDesc);
+    // the bytes are known exactly: they size the launch as a caller's bound would
+    sizing = batch_device_sizing(n, total_bytes);
   } else {
     // lengths are only known on the device
     if (!h->batch_seen) {
@@ -541,49 +579,39 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
       *h->batch_seen = 0;
     }
     sizing = batch_device_sizing(n, max_total_bytes, *static_cast<volatile uint64_t*>(h->batch_seen));
+  }
+  if (!walk) {
     if (sizing.records == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
     shape.pieces = n;
     shape.total_chunks = sizing.grid_chunks;
     shape.total_bytes = sizing.bytes;
+    rc = ensure_batch_capacity(h, n, sizing.records);
+    if (rc != MI355_BLIT_SUCCESS) return rc;
   }
-  int rc = ensure_batch_capacity(h, shape.pieces, descs_on_device ? sizing.records : shape.total_chunks);
-  if (rc != MI355_BLIT_SUCCESS) return rc;
+  if (staged_bytes && h->stage_in_device_memory) {
+    // posted writes across the bus: order them, then read one back so that
+    // they have landed before the launch below can reach the GPU
+    _mm_sfence();
+    (void)*(reinterpret_cast<volatile uint32_t*>(reinterpret_cast<uint8_t*>(h->descs_host[b]) + staged_bytes) - 1);
+  }
 
   // The device-side buffers (records, prefix sums) are shared by consecutive
   // batches: the next batch waits for the previous one, which stream order
   // does by itself unless the two are on different streams.
-  const unsigned b = h->next_host;
   h->next_host ^= 1;
   if (h->batch_busy[b ^ 1] && h->last_batch_stream != s) BLIT_HIP(hipStreamWaitEvent(s, h->batch_done[b ^ 1], 0));
 
   const mi355_blit_tuning_t* t = h->has_tuning ? &h->tuning : nullptr;
-  // Device-resident descriptors are taken to be a large batch: their lengths
-  // are only known on the device.  Only host-resident ones leave the copy's
-  // shape open to tuning.
+  // Descriptors whose lengths the host has not walked are taken to be a large
+  // batch.  Only walked ones leave the copy's shape open to tuning.
   mi355_blit_plan_t p;
   const BatchLaunch l = plan_batch_records(shape.total_chunks, shape.total_bytes,
-                                           descs_on_device || shape.total_bytes >= (4ull << 20), t, !descs_on_device, &p);
+                                           !walk || shape.total_bytes >= (4ull << 20), t, walk, &p);
 
-  if (!descs_on_device) {
-    // Host-resident descriptors.  The host has walked them to validate them
-    // and does the prefix sum over their chunk counts on the way; the image it
-    // stages (the descriptors, cut into pieces of at most 64 chunks, and each
-    // piece's first record index) is all the GPU needs to write the records
-    // with one lane per piece.  The two staging buffers alternate, so staging
-    // one batch overlaps the execution of the one before; a buffer is only
-    // waited for until the batch that used it, two batches ago, has finished.
-    if (h->batch_busy[b]) {
-      BLIT_HIP(hipEventSynchronize(h->batch_done[b]));
-      h->batch_busy[b] = false;
-    }
-    const size_t image_bytes = batch_stage_bytes(shape.pieces);
-    batch_stage(h->stage_image, h->descs_host[b]);
-    if (h->stage_in_device_memory) {
-      // posted writes across the bus: order them, then read one back so that
-      // they have landed before the launch below can reach the GPU
-      _mm_sfence();
-      (void)*(reinterpret_cast<volatile uint32_t*>(reinterpret_cast<uint8_t*>(h->descs_host[b]) + image_bytes) - 1);
-    }
+  if (walk) {
+    // The image the host staged (the descriptors, cut into pieces of at most 64
+    // chunks, and each piece's first record index) is all the GPU needs to
+    // write the records, a wave for 64 pieces.
     const BatchDesc* staged = h->descs_host[b];
     EmitRecordsArgs er{staged, reinterpret_cast<const uint32_t*>(staged + shape.pieces), shape.pieces, h->records_dev};
     hipLaunchKernelGGL(mi355_batch_emit_records, dim3(static_cast<uint32_t>((shape.pieces + 255) / 256)), dim3(256),
@@ -593,14 +621,17 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
     rc = launch_records_copy(h, s, p, l, shape.total_chunks);
     if (rc != MI355_BLIT_SUCCESS) return rc;
   } else {
-    // Device-resident descriptors.  The prefix sum over the chunk counts and
-    // the records are made on the device; the grid and the record buffer are
-    // sized by the caller's bound or, without one, by an assumption
+    // The prefix sum over the chunk counts and the records are made on the
+    // device; the grid and the record buffer are sized by the bytes the host
+    // added up, by the caller's bound or, without either, by an assumption
     // (batch_device_sizing).  The copy kernel reads the number of chunks on the
     // device: surplus waves end at once, missing ones are made up for by
     // striding, and chunks without a record are looked up in the prefix sums.
-    const BatchDesc* dev_descs = reinterpret_cast<const BatchDesc*>(descs);
-    launch_scans(h, s, dev_descs, n);
+    // Descriptors the host staged are read once, by the first kernel, which
+    // leaves a copy of them for the others.
+    const BatchDesc* scanned = raw ? h->descs_host[b] : reinterpret_cast<const BatchDesc*>(descs);
+    const BatchDesc* dev_descs = raw ? h->descs_private_dev : scanned;
+    launch_scans(h, s, scanned, n, raw ? h->descs_private_dev : nullptr);
     EmitRecordsDeviceArgs er{dev_descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n),
                              h->records_dev, sizing.records};
     hipLaunchKernelGGL(mi355_batch_emit_records_lookup, dim3(static_cast<uint32_t>((sizing.records + 255) / 256)),

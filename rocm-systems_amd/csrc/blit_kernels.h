@@ -395,7 +395,19 @@ __device__ __forceinline__ void scan_local_body(const ScanLocalArgs& a) {
   uint32_t* __restrict__ block_sum = a.block_sum;
   __shared__ uint32_t lds[16];
   const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 1024 + threadIdx.x;
-  const uint32_t c = i < n ? desc_chunks(descs[i]) : 0;
+  BatchDesc d{nullptr, nullptr, 0};
+  if (i < n) {
+    if (a.private_copy) {
+      const uint64_t* w = reinterpret_cast<const uint64_t*>(descs + i);
+      d.dst = reinterpret_cast<uint8_t*>(__hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM));
+      d.src = reinterpret_cast<const uint8_t*>(__hip_atomic_load(w + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM));
+      d.bytes = __hip_atomic_load(w + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      a.private_copy[i] = d;
+    } else {
+      d = descs[i];
+    }
+  }
+  const uint32_t c = i < n ? desc_chunks(d) : 0;
   uint32_t total;
   const uint32_t excl = block_scan_1024(c, lds, &total);
   if (i < n) chunk_start[i] = excl;

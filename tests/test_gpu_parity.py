@@ -786,6 +786,41 @@ def test_batch_unbounded_sizes_itself_by_the_batch_before(capi, pkg, oracle, are
         eng.close()
 
 
+def test_batch_of_many_short_copies_is_staged_as_it_is(capi, blit, oracle, arenas, torch_cuda):
+    """From 4096 host-resident descriptors of a few KiB on average the host does
+    not walk them but stages them as they are, and the GPU takes them from there
+    like device-resident ones (sized by the bytes the host added up).  Three
+    batches in a row with different descriptors (the two staging buffers and
+    the GPU's own copy are reused), copies of no bytes among them; then the
+    argument check such a batch still gets."""
+    src, src_host, dst = arenas
+    for seed, n, max_len in ((1, 4096, 6000), (2, 6001, 3000), (3, 5000, 9000)):
+        rng = np.random.default_rng(6100 + seed)
+        descs, lens, offs, so, do, total = _make_batch(capi, rng, src, dst, n, min_len=1, max_len=max_len)
+        for i in range(0, n, 5):
+            descs[i].bytes = 0
+            lens[i] = 0
+        dst.fill(0, total, GUARD_BYTE)
+        check_ok(capi, blit.copy_batch(descs, n), "copy_batch")
+        check_ok(capi, blit.synchronize(), "synchronize")
+        p = blit.last_plan()
+        assert p.kernel == capi.KERNEL_COPY_BATCH and p.grid == int(lens.sum()) // 4096 + n, p.as_dict()
+        assert np.array_equal(dst.host(0, total), _expect_batch(oracle, src_host, total, lens, offs, so, do)), seed
+    # a copy of bytes without a source: refused before anything is launched
+    descs[n // 2].src = None
+    descs[n // 2].bytes = 8
+    dst.fill(0, total, GUARD_BYTE)
+    assert blit.copy_batch(descs, n) == capi.ERROR_INVALID_ARGUMENT
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert (dst.host(0, total) == GUARD_BYTE).all()
+    # all empty: nothing to do
+    for i in range(n):
+        descs[i].bytes = 0
+    check_ok(capi, blit.copy_batch(descs, n), "copy_batch")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    assert (dst.host(0, total) == GUARD_BYTE).all()
+
+
 def test_batch_65536_copies(capi, blit, oracle, rand, torch_cuda):
     """The benchmark's batch: 65,536 copies, 64 B .. 256 KiB log-uniform, offsets
     0..15 on both sides, carved sequentially out of one arena; all bytes and

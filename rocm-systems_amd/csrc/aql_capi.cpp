@@ -314,8 +314,18 @@ void write_barriers(mi355_aql* h, uint64_t index, const uint64_t* deps, uint32_t
 
 // One KERNEL_DISPATCH packet (amd_blit_kernel.cpp:863-924): 1-D grid, kernarg
 // slot of the same index, acquire and release fences at the configured scope.
+// Where a dispatch stands in a command made of several packets, each waiting
+// for the one before: what one packet leaves for the next is only read on this
+// GPU, so only the command's first acquire and its last release need the
+// configured (system) scope and the fences between its packets are at agent
+// scope (the reference's commands are one packet each, amd_blit_kernel.cpp:
+// 870-873).  The caller's data is covered as for a single packet: acquired
+// before the first kernel, released behind the last.
+enum class Chain { kAlone, kFirst, kMiddle, kLast };
+
 void write_dispatch(mi355_aql* h, uint64_t index, const Kernel& k, const void* args, size_t args_size,
-                    uint32_t grid_wgs, uint32_t wg_size, uint64_t completion, bool barrier_bit) {
+                    uint32_t grid_wgs, uint32_t wg_size, uint64_t completion, bool barrier_bit,
+                    Chain chain = Chain::kAlone) {
   uint8_t* karg = h->kernargs + (index & h->queue_mask) * kKernargSlotBytes;
   std::memcpy(karg, args, args_size);
   if (h->kernargs_in_device_memory) {
@@ -340,9 +350,12 @@ void write_dispatch(mi355_aql* h, uint64_t index, const Kernel& k, const void* a
   auto* ring = static_cast<hsa_kernel_dispatch_packet_t*>(h->queue->base_address);
   hsa_kernel_dispatch_packet_t* slot = &ring[index & h->queue_mask];
   std::memcpy(reinterpret_cast<uint8_t*>(slot) + 4, reinterpret_cast<uint8_t*>(&pkt) + 4, sizeof(pkt) - 4);
+  const uint16_t outer = h->fence_scope, inner = HSA_FENCE_SCOPE_AGENT;
+  const uint16_t acquire = (chain == Chain::kAlone || chain == Chain::kFirst) ? outer : inner;
+  const uint16_t release = (chain == Chain::kAlone || chain == Chain::kLast) ? outer : inner;
   uint16_t header = (HSA_PACKET_TYPE_KERNEL_DISPATCH << HSA_PACKET_HEADER_TYPE) |
-                    (h->fence_scope << HSA_PACKET_HEADER_SCACQUIRE_FENCE_SCOPE) |
-                    (h->fence_scope << HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE);
+                    (acquire << HSA_PACKET_HEADER_SCACQUIRE_FENCE_SCOPE) |
+                    (release << HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE);
   if (barrier_bit) header |= 1 << HSA_PACKET_HEADER_BARRIER;
   publish(slot, header, 1 << HSA_KERNEL_DISPATCH_PACKET_SETUP_DIMENSIONS);
 }
@@ -824,8 +837,8 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   // whatever still reads the shared record buffer; it frees the staging buffer
   // when it is done with it.
   write_dispatch(h, i++, h->emit_records, &er, sizeof(er), static_cast<uint32_t>((shape.pieces + 255) / 256), 256,
-                 h->stage_free[b].handle, true);
-  write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true);
+                 h->stage_free[b].handle, true, Chain::kFirst);
+  write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true, Chain::kLast);
   release_write_index(h, index, total);
   return MI355_BLIT_SUCCESS;
 }
@@ -887,11 +900,11 @@ int copy_batch_device_locked(mi355_aql_t* h, const BatchDesc* scanned, size_t n,
   write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
   uint64_t i = index + nb;
   // every packet waits for the one before; the first also for whatever still uses the shared buffers
-  write_dispatch(h, i++, h->scan_local, &sl, sizeof(sl), n_blocks, 1024, staged_free, true);
-  write_dispatch(h, i++, h->scan_top, &stp, sizeof(stp), 1, 1024, 0, true);
+  write_dispatch(h, i++, h->scan_local, &sl, sizeof(sl), n_blocks, 1024, staged_free, true, Chain::kFirst);
+  write_dispatch(h, i++, h->scan_top, &stp, sizeof(stp), 1, 1024, 0, true, Chain::kMiddle);
   write_dispatch(h, i++, h->emit_records_lookup, &er, sizeof(er),
-                 static_cast<uint32_t>((sizing.records + 255) / 256), 256, 0, true);
-  write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true);
+                 static_cast<uint32_t>((sizing.records + 255) / 256), 256, 0, true, Chain::kMiddle);
+  write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true, Chain::kLast);
   release_write_index(h, index, total);
   return MI355_BLIT_SUCCESS;
 }

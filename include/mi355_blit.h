@@ -258,8 +258,8 @@ typedef struct {
   uint32_t xcd_run; /* as in mi355_blit_plan_t */
   uint32_t wg_size, grid, nt_load, store_policy;
   uint64_t total_bytes;
-  uint32_t plain_rows; /* rows tiled like a linear copy (256-byte aligned on the
-                          destination side, whole units long, a multiple of 4
+  uint32_t plain_rows; /* rows tiled like a linear copy (128-byte aligned on the
+                          destination side, whole lines long, a multiple of 4
                           bytes from their source): the kernel's short path */
   uint32_t route;      /* MI355_BLIT_ROUTE_* the launch was shaped for */
 } mi355_blit_rect_plan_t;

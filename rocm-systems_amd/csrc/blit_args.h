@@ -207,9 +207,10 @@ struct RectArgs {
   // magic_rows) for every 32-bit n (magic_divisor below).
   uint64_t magic_slots;
   uint64_t magic_rows;
-  // Not 0: every row starts at a 256-byte boundary of the destination, is a
-  // whole number of units long and lies a multiple of 4 bytes from its source,
-  // so that no unit has a head, a tail, a cut end or bytes to realign.
+  // Not 0: every row starts at a cache-line boundary of the destination, is a
+  // whole number of lines long and lies a multiple of 4 bytes from its source,
+  // so that no unit has a head, a tail or bytes to realign: unit k of a row is
+  // the row's bytes [k, k + 1) * 1024 * U, cut at the row's end.
   uint32_t plain_rows;
   uint32_t pad;
 };

@@ -746,8 +746,11 @@ __device__ __forceinline__ void rect_copy_body(const RectArgs& a) {
   const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd);
   const uint64_t n_waves = a.n_waves;
   if (a.plain_rows) {
-    // Rows of whole units, aligned like a linear copy's tiles: a unit is U
-    // loads and U stores per lane and nothing else.
+    // Rows of whole vectors, aligned like a linear copy's tiles: a unit is U
+    // loads and U stores per lane and nothing else.  A row's last unit may be
+    // a partial one, whose lanes beyond the row's end have nothing to do, or
+    // have up to kRowOverflowVecs vectors more than a unit, which its first
+    // lanes take.
     for (uint64_t w = wave; w < a.total_slots; w += n_waves) {
       const uint32_t slot = static_cast<uint32_t>(w);
       const uint32_t line = div_magic(slot, a.magic_slots);
@@ -757,11 +760,16 @@ __device__ __forceinline__ void rect_copy_body(const RectArgs& a) {
       const uint64_t in_row = static_cast<uint64_t>(kq) * (kUnit * 16) + lane * 16;
       const v4u_a4* sv = reinterpret_cast<const v4u_a4*>(a.src + layer * a.src_slice + y * a.src_pitch + in_row);
       v4u* dv = reinterpret_cast<v4u*>(a.dst + layer * a.dst_slice + y * a.dst_pitch + in_row);
-      v4u x[U];
+      const bool over = kq + 1 == a.slots && in_row + U * (kWave * 16) < a.width;
+      v4u x[U + 1];
 #pragma unroll
-      for (int u = 0; u < U; ++u) x[u] = ld_v4<NTL>(sv + u * kWave);
+      for (int u = 0; u < U; ++u)
+        if (in_row + u * (kWave * 16) < a.width) x[u] = ld_v4<NTL>(sv + u * kWave);
+      if (over) x[U] = ld_v4<NTL>(sv + U * kWave);
 #pragma unroll
-      for (int u = 0; u < U; ++u) st_v4<NTS>(dv + u * kWave, x[u]);
+      for (int u = 0; u < U; ++u)
+        if (in_row + u * (kWave * 16) < a.width) st_v4<NTS>(dv + u * kWave, x[u]);
+      if (over) st_v4<NTS>(dv + U * kWave, x[U]);
     }
     return;
   }

@@ -236,19 +236,26 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
     const uint64_t c = rect_row_units(r, width, 64 * unroll);
     if (c > slots) slots = c;
   }
+  // Rows that are tiled like a linear copy: they start at cache-line
+  // boundaries of the destination, are whole lines long and lie a multiple of
+  // 4 bytes from their source.  The kernel then skips everything a row's ends
+  // need: a unit is a plain tile of the row from its first byte on, the last
+  // one possibly a partial one (1 GiB in rows of 4224 bytes: 328 us, 368 us
+  // through the general path).
+  const uint64_t unit_bytes = 1024ull * unroll;
+  const uintptr_t delta = reinterpret_cast<uintptr_t>(s0) - reinterpret_cast<uintptr_t>(d0);
+  a.plain_rows = whole_lines && delta % 4 == 0 && sp % 4 == 0 && (layers == 1 || ss % 4 == 0);
+  // A row of one unit and a few vectors is one wave's (1 GiB in rows of 1152
+  // bytes: 354 us, 422 us with a second wave for the last 128 bytes); longer
+  // rows end in a partial unit (rows of 4224 bytes: 328 us, 343 us with the 8
+  // vectors added to the fourth unit).
+  if (a.plain_rows) slots = width <= unit_bytes + 16 * 15 ? 1 : (width + unit_bytes - 1) / unit_bytes;
   const uint64_t total_slots = rows * layers * slots;
   if (total_slots > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   a.slots = static_cast<uint32_t>(slots);
   a.total_slots = static_cast<uint32_t>(total_slots);
   a.magic_slots = magic_divisor(a.slots);
   a.magic_rows = magic_divisor(a.rows);
-  // Rows that are tiled like a linear copy: they start at 256-byte boundaries
-  // of the destination, are whole units long and lie a multiple of 4 bytes
-  // from their source.  The kernel then skips everything a row's ends need.
-  const uint64_t unit_bytes = 1024ull * unroll;
-  const uintptr_t delta = reinterpret_cast<uintptr_t>(s0) - reinterpret_cast<uintptr_t>(d0);
-  a.plain_rows = reinterpret_cast<uintptr_t>(d0) % 256 == 0 && dp % 256 == 0 && (layers == 1 || ds % 256 == 0) &&
-                 width % unit_bytes == 0 && delta % 4 == 0 && sp % 4 == 0 && (layers == 1 || ss % 4 == 0);
   // Plain rows in XCD runs want single-wave workgroups, like the linear copy.
   // Measured on 17 shapes of 1 GiB, widths 2 KiB .. 1 MiB at pitches of 1.03 to
   // 256 times the width: workgroups of 256 in launch order are up to 27 % behind

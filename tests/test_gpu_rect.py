@@ -172,8 +172,19 @@ def test_rect_plain_rows_are_exact(capi, fresh_tuning, oracle, rand, unroll):
     t = capi.Tuning(unroll=unroll)
     st, plan = capi.plan_rect((1 << 40, 12288, 12288 * 18), do, (1 << 41, 8192, 8192 * 20), so, ext, t)
     assert st == capi.SUCCESS and plan.plain_rows == 1 and plan.slots == 4096 // (1024 * unroll)
+    # rows of whole lines whose last unit is a partial one are plain too
+    for width in (4096 - 256, 4096 + 128, 128, 1024 * unroll + 128, 1024 * unroll + 256, 7 * 1024 - 128):
+        ext3 = (width, 15, 2)
+        st, plan = capi.plan_rect((1 << 40, 12288, 12288 * 18), do, (1 << 41, 8192, 8192 * 20), so, ext3, t)
+        if width > 1024:   # narrower rows go to the kernel that packs rows into waves
+            n_vec, unit = width // 16, 64 * unroll
+            assert st == capi.SUCCESS and plan.plain_rows == 1
+            assert plan.slots == (-(-n_vec // unit) if n_vec > 15 + unit else 1)
+        for wg, xcd_run in ((64, 1), (256, 3)):
+            blit.set_tuning(wg_size=wg, unroll=unroll, xcd_run=xcd_run)
+            run_rect_case(capi, blit, oracle, rand, sshape, dshape, ext3, so, do, 0, 0, seed=0x7EC7EE00 + width)
     # one condition off at a time: destination x, source x, width
-    for so2, do2, ext2 in (((1028, 3, 0), (640, 2, 0), ext), ((1030, 3, 0), do, ext), (so, do, (4096 - 256, 15, 2))):
+    for so2, do2, ext2 in (((1028, 3, 0), (576, 2, 0), ext), ((1030, 3, 0), do, ext), (so, do, (4096 - 64, 15, 2))):
         st, plan = capi.plan_rect((1 << 40, 12288, 12288 * 18), do2, (1 << 41, 8192, 8192 * 20), so2, ext2, t)
         assert st == capi.SUCCESS and plan.plain_rows == 0
         blit.set_tuning(unroll=unroll)

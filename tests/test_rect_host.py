@@ -131,6 +131,19 @@ def replay_rect_plan(p, dst_bytes, src_bytes, dst_base, src_base):
         layer, y = divmod(line, p.rows)
         d = p.dst + layer * p.dst_slice + y * p.dst_pitch
         s = p.src + layer * p.src_slice + y * p.src_pitch
+        if p.plain_rows:
+            # every unit is a plain tile of the row, the last one possibly a partial one
+            assert d % 128 == 0 and p.width % 128 == 0 and (s - d) % 4 == 0
+            n_vec = p.width // 16
+            assert p.slots == (-(-n_vec // unit) if n_vec > 15 + unit else 1)
+            for kq in range(p.slots):
+                b0 = kq * 16 * unit
+                b1 = p.width if kq + 1 == p.slots else (kq + 1) * 16 * unit
+                assert b1 - b0 <= 16 * (unit + 15), "the last unit's overflow is at most 15 vectors" 
+                do, so = d - dst_base + b0, s - src_base + b0
+                dst_bytes[do:do + b1 - b0] = src_bytes[so:so + b1 - b0]
+                written[do:do + b1 - b0] += 1
+            continue
         head = min((16 - d % 16) % 16, p.width)
         n_vec = (p.width - head) // 16
         lead = ((d + head) % 256) // 16
@@ -194,6 +207,28 @@ def test_plan_rect_writes_every_byte_once(capi_host, oracle, rand, seed):
         written = replay_rect_plan(p, got, src, dst.ctypes.data, src.ctypes.data)
     assert np.array_equal(got, want)
     assert written.max() == 1 and int(written.sum()) == p.total_bytes
+
+
+@pytest.mark.parametrize("width", [1152, 4096, 4224, 7040, 128 * 77])
+def test_plan_rect_plain_rows_write_every_byte_once(capi_host, oracle, rand, width):
+    """Rows at 256-byte boundaries of the destination, whole lines wide: the
+    short path's tiles cover each row exactly, a partial last unit included."""
+    rows, pitch = 9, 16384
+    src = rand(rows * pitch + 512, width)
+    dst = np.full(rows * pitch + 512, 0xEE, dtype=np.uint8)
+    d_base = dst.ctypes.data + (-dst.ctypes.data) % 256
+    s_base = src.ctypes.data + (-src.ctypes.data) % 256 + 4
+    sp, dp = (s_base, pitch, 0), (d_base, pitch, 0)
+    for unroll in (1, 2, 4):
+        st, p = capi_host.plan_rect(dp, (256, 1, 0), sp, (8, 0, 0), (width, rows - 1, 1), capi_host.Tuning(unroll=unroll))
+        assert st == SUCCESS and p.plain_rows == 1 and p.unroll == unroll
+        want = dst.copy()
+        oracle_rect(oracle, (want.ctypes.data + d_base - dst.ctypes.data,) + dp[1:], (256, 1, 0), sp, (8, 0, 0),
+                    (width, rows - 1, 1))
+        got = dst.copy()
+        written = replay_rect_plan(p, got, src, dst.ctypes.data, src.ctypes.data)
+        assert np.array_equal(got, want)
+        assert written.max() == 1 and int(written.sum()) == p.total_bytes
 
 
 def test_plan_rect_merges_contiguous_rows(capi_host):
@@ -272,7 +307,13 @@ def test_plan_rect_slots_follow_row_alignment(capi_host):
     assert st == SUCCESS and p.plain_rows == 1
     st, p = capi_host.plan_rect((base_d, 8192, 0), (256, 0, 0), (base_s, 8192, 0), (4, 0, 0), (4096, 1024, 1))
     assert st == SUCCESS and p.plain_rows == 1                     # 256-byte aligned destination, dword-aligned source
-    for d_x, s_x, w, dp in ((128, 0, 4096, 8192), (0, 2, 4096, 8192), (0, 0, 4096 + 128, 8192), (0, 0, 4096, 8192 + 128)):
+    st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096 + 128, 1024, 1))
+    assert st == SUCCESS and (p.plain_rows, p.slots) == (1, 5)     # whole lines: the last unit is a partial one
+    st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (1024 + 128, 1024, 1))
+    assert st == SUCCESS and (p.plain_rows, p.slots) == (1, 1)     # a unit and 8 vectors: one wave's
+    st, p = capi_host.plan_rect((base_d, 8192 + 128, 0), (128, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 1024, 1))
+    assert st == SUCCESS and p.plain_rows == 1                     # rows at cache-line boundaries
+    for d_x, s_x, w, dp in ((64, 0, 4096, 8192), (0, 2, 4096, 8192), (0, 0, 4096 + 64, 8192), (0, 0, 4096, 8192 + 64)):
         st, p = capi_host.plan_rect((base_d, dp, 0), (d_x, 0, 0), (base_s, 8192, 0), (s_x, 0, 0), (w, 1024, 1))
         assert st == SUCCESS and p.plain_rows == 0, (d_x, s_x, w, dp)
     # XCD runs: only from 64 MiB moved, and only where neighbouring waves share cache lines
@@ -289,7 +330,9 @@ def test_plan_rect_slots_follow_row_alignment(capi_host):
     st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 32768, 1))
     assert st == SUCCESS and (p.plain_rows, p.wg_size, p.xcd_run) == (1, 64, 576)              # tiled like a linear copy
     st, p = capi_host.plan_rect((base_d, 8192, 0), (128, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 32768, 1))
-    assert st == SUCCESS and (p.plain_rows, p.wg_size, p.xcd_run) == (0, 256, 0)               # whole lines, not plain
+    assert st == SUCCESS and (p.plain_rows, p.wg_size, p.xcd_run) == (1, 64, 576)              # at a line boundary: plain too
+    st, p = capi_host.plan_rect((base_d, 8192, 0), (128, 0, 0), (base_s, 8192, 0), (1, 0, 0), (4096, 32768, 1))
+    assert st == SUCCESS and (p.plain_rows, p.wg_size, p.xcd_run) == (0, 256, 0)               # whole lines, bytes to realign
     st, p = capi_host.plan_rect((base_d, 2048, 0), (9, 0, 0), (base_s, 2048, 0), (3, 0, 0), (1000, 1 << 20, 1))
     assert st == SUCCESS and (p.wg_size, p.xcd_run) == (64, 0)                                # waves share no line
     st, p = capi_host.plan_rect((base_d, 1024, 0), (0, 0, 0), (base_s, 1024, 0), (0, 0, 0), (520, 1 << 20, 1))

@@ -230,7 +230,7 @@ struct RectNarrowArgs {
   uint32_t rows;     // rows per layer
   uint32_t lines;    // rows * layers
   uint32_t lanes_per_row;
-  uint32_t magic;    // ceil(2^16 / lanes_per_row): n / lanes_per_row == (n * magic) >> 16, n < 128
+  uint32_t pad;
   uint32_t waves_per_wg;
   uint32_t n_waves;
   XcdRuns xcd;

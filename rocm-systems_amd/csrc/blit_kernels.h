@@ -904,8 +904,8 @@ __device__ __forceinline__ void rect_narrow_body(const RectNarrowArgs& a) {
     // row and slot of this lane's number 64 w + lane
     const uint64_t first = w * kWave;
     const uint64_t line0 = lpr == 1 ? first : __umul64hi(first, a.magic64);  // first / lpr
-    const unsigned t = static_cast<unsigned>(first - line0 * lpr) + lane;    // < 128
-    const unsigned g = (t * a.magic) >> 16;                                  // t / lpr
+    const unsigned t = static_cast<unsigned>(first - line0 * lpr) + lane;    // < lpr + 64
+    const unsigned g = div_magic(t, a.magic64);                              // t / lpr
     const unsigned j = t - g * lpr;
     const uint64_t line = line0 + g;
     if (line >= a.lines) continue;

@@ -20,6 +20,12 @@ namespace mi355 {
 // Rows that touch at most this many 16-byte destination slots go to the
 // kernel that packs several rows into a wave.
 constexpr uint32_t kRectNarrowSlots = 64;
+// Rows that are not whole lines stay with that kernel up to this many slots:
+// one lane per slot wastes nothing on a row of one unit and a bit, where the
+// unit kernel runs a second, nearly empty wave (1 GiB in rows of 1100 bytes at
+// odd offsets: 5.3 TB/s against 3.9, rows of 2000 bytes 4.7 against 4.1; rows of
+// 3000 bytes 5.6 against 5.9, hence the limit).
+constexpr uint32_t kRectNarrowRaggedSlots = 128;
 
 struct RectPlan {
   bool empty;    // a zero in the range: nothing to move
@@ -145,7 +151,7 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
     const uint64_t c = (r + width + 15) / 16;
     if (c > row_slots) row_slots = c;
   }
-  if (row_slots <= kRectNarrowSlots) {
+  if (row_slots <= kRectNarrowSlots || (!whole_lines && row_slots <= kRectNarrowRaggedSlots)) {
     out->narrow = true;
     RectNarrowArgs& n = out->nargs;
     n.dst = d0;
@@ -158,8 +164,8 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
     n.rows = a.rows;
     n.lines = static_cast<uint32_t>(rows * layers);
     n.lanes_per_row = static_cast<uint32_t>(row_slots);
-    n.magic = (65536 + n.lanes_per_row - 1) / n.lanes_per_row;
-    n.magic64 = n.lanes_per_row > 1 ? ~0ull / n.lanes_per_row + 1 : 0;  // unused for 1
+    n.pad = 0;
+    n.magic64 = magic_divisor(n.lanes_per_row);
     out->unroll = 1;
     // Measured on MI355X with 2^20 rows.  When every store is a whole cache
     // line, single-wave workgroups and written-through stores are best (1 KiB

@@ -188,7 +188,7 @@ void one_rect_plan() {
     if (per > 1) CHECK(dst.pitch == range.x && src.pitch == range.x, "rows merged across a gap");
     if (rp.narrow) {
       const uint64_t lpr = rp.nargs.lanes_per_row;
-      CHECK(lpr >= 1 && lpr <= 64, "lanes per row %" PRIu64, lpr);
+      CHECK(lpr >= 1 && lpr <= kRectNarrowRaggedSlots, "lanes per row %" PRIu64, lpr);
       uint64_t covered = d;  // bytes of the row below this address have been written
       for (uint64_t j = 0; j < lpr; ++j) {
         const uint64_t slot = (d & ~15ull) + 16 * j;
@@ -207,7 +207,7 @@ void one_rect_plan() {
       }
       CHECK(covered == d + width, "row not covered by its %" PRIu64 " slots", lpr);
       // the host's magic numbers divide as the kernel needs them to
-      for (uint64_t n = 0; n < 128; ++n) CHECK(((n * rp.nargs.magic) >> 16) == n / lpr, "16-bit magic");
+      for (uint32_t n = 0; n < lpr + 64; ++n) CHECK(div_magic(n, rp.nargs.magic64) == n / lpr, "lane's row within the wave");
       if (lpr > 1) {
         const uint64_t probe = below(1ull << 38);
         CHECK(static_cast<uint64_t>((static_cast<unsigned __int128>(probe) * rp.nargs.magic64) >> 64) == probe / lpr,

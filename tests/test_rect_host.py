@@ -277,7 +277,11 @@ def test_plan_rect_slots_follow_row_alignment(capi_host):
     st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (1024, 64, 1))
     assert st == SUCCESS and (p.lanes_per_row, p.slots, p.unroll) == (64, 0, 0)
     st, p = capi_host.plan_rect((base_d, 8192, 0), (1, 0, 0), (base_s, 8192, 0), (0, 0, 0), (1024, 64, 1))
-    assert st == SUCCESS and p.lanes_per_row == 0 and p.slots == 1   # 65 slots: not packed
+    assert st == SUCCESS and (p.lanes_per_row, p.slots) == (65, 0)   # ragged rows are packed up to 128 slots
+    st, p = capi_host.plan_rect((base_d, 8192, 0), (1, 0, 0), (base_s, 8192, 0), (0, 0, 0), (2048, 64, 1))
+    assert st == SUCCESS and (p.lanes_per_row, p.slots) == (0, 1)    # 129 slots: one unit of two vectors per lane
+    st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (1, 0, 0), (1024 + 128, 64, 1))
+    assert st == SUCCESS and (p.lanes_per_row, p.slots) == (0, 1)    # whole lines with bytes to realign: units
     st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (0, 0, 0), (512, 64, 1))
     assert st == SUCCESS and p.lanes_per_row == 32 and p.grid * (p.wg_size // 64) == 32
     st, p = capi_host.plan_rect((base_d, 256, 0), (128, 0, 0), (base_s, 256, 0), (64, 0, 0), (64, 4096, 1))

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define MI355_BLIT_ABI_VERSION 2
+#define MI355_BLIT_ABI_VERSION 3
 
 /* Same numeric values as HSA_STATUS_* (inc/hsa.h). */
 enum {
@@ -205,6 +205,29 @@ int mi355_blit_copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_
  * with n > 0, or a bound that needs 2^32 records or more -> INVALID_ARGUMENT. */
 int mi355_blit_copy_batch_bounded(mi355_blit_t* h, const mi355_blit_desc_t* device_descs, size_t n,
                                   uint64_t max_total_bytes, void* stream);
+
+/* mi355_blit_copy_batch_bounded for callers that cannot allocate: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It
+ * has no counterpart in the reference.  Same arguments, same kernels and same
+ * results, but the prefix sums and chunk records live in a fixed array in the
+ * library's device code (16.25 MiB per GPU, held from the load of the library
+ * to the end of the process) instead of buffers the handle grows on demand,
+ * and the call makes no hipMalloc, hipFree or other allocating call: four
+ * kernel launches on the stream and nothing else.
+ * Limits: n <= MI355_BLIT_NOALLOC_MAX_COPIES, more -> OUT_OF_RESOURCES and
+ * nothing is launched.  The bytes are not limited: the array has room for
+ * 2^19 chunk records (2 GiB of copies) and chunks beyond them are found
+ * through the prefix sums by the copy kernel, as when a bound is exceeded.
+ * The array is one per GPU, shared by every handle and every call on that GPU,
+ * and keeps the last call's contents (each call rewrites all it reads, so
+ * nothing needs clearing): calls that may overlap on one GPU -- on different
+ * streams or handles without an ordering between them -- race and must be
+ * ordered by the caller; calls on one stream are ordered by the stream.  The
+ * engine does not size later batches by this one (nothing is written to host
+ * memory). */
+#define MI355_BLIT_NOALLOC_MAX_COPIES 65536
+int mi355_blit_copy_batch_bounded_noalloc(mi355_blit_t* h, const mi355_blit_desc_t* device_descs, size_t n,
+                                          uint64_t max_total_bytes, void* stream);
 
 /* Pitched 3-D region copy as a shader: range->z layers of range->y rows of
  * range->x bytes, from src at src_offset to dst at dst_offset.  The reference

@@ -18,6 +18,7 @@ KERNEL_COPY_REALIGN = 1
 KERNEL_FILL = 2
 KERNEL_COPY_BATCH = 3
 KERNEL_COPY_RECT = 4
+NOALLOC_MAX_COPIES = 65536
 
 STORE_CACHED = 0
 STORE_NT = 1
@@ -92,6 +93,7 @@ SIGNATURES = {
     "mi355_blit_fill32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t, C.c_void_p]),
     "mi355_blit_copy_batch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]),
     "mi355_blit_copy_batch_bounded": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint64, C.c_void_p]),
+    "mi355_blit_copy_batch_bounded_noalloc": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint64, C.c_void_p]),
     "mi355_blit_copy_rect": (C.c_int, [C.c_void_p, C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
                                        C.POINTER(Dim3), C.POINTER(Dim3), C.c_void_p]),
     "mi355_blit_plan_rect": (C.c_int, [C.POINTER(PitchedPtr), C.POINTER(Dim3), C.POINTER(PitchedPtr),
@@ -199,6 +201,11 @@ class Blit:
         """Device-resident descriptors that together move at most max_total_bytes."""
         addr = device_descs if isinstance(device_descs, int) or device_descs is None else C.cast(device_descs, C.c_void_p)
         return self.lib.mi355_blit_copy_batch_bounded(self.handle, addr, n, max_total_bytes, stream)
+
+    def copy_batch_bounded_noalloc(self, device_descs, n, max_total_bytes, stream=None):
+        """copy_batch_bounded out of the library's fixed scratch array: no allocation."""
+        addr = device_descs if isinstance(device_descs, int) or device_descs is None else C.cast(device_descs, C.c_void_p)
+        return self.lib.mi355_blit_copy_batch_bounded_noalloc(self.handle, addr, n, max_total_bytes, stream)
 
     def copy_rect(self, dst, dst_offset, src, src_offset, extent, stream=None, route=None):
         """dst, src: (base, pitch, slice); offsets and extent: (x bytes, y rows, z layers)."""

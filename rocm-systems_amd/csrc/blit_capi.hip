@@ -40,12 +40,66 @@ struct LedgerSlot {
   bool in_flight = false;
 };
 
+// What the allocation-free batched copy (mi355_blit_copy_batch_bounded_noalloc)
+// may hold: descriptors per call, and chunk records before chunks are looked up
+// in the prefix sums instead.
+constexpr uint64_t kNoAllocMaxCopies = MI355_BLIT_NOALLOC_MAX_COPIES;
+constexpr uint64_t kNoAllocRecords = 1ull << 19;
+// Layout of its scratch memory: the prefix sum within groups of 1024 copies
+// (one word per copy and one for the total), the prefix sum across groups, the
+// chunk records; each part at a multiple of 256 bytes.
+constexpr size_t kScratchChunkStart = 0;
+constexpr size_t kScratchBlockSum = (kScratchChunkStart + (kNoAllocMaxCopies + 1) * sizeof(uint32_t) + 255) / 256 * 256;
+constexpr size_t kScratchRecords = (kScratchBlockSum + (kNoAllocMaxCopies / 1024 + 1) * sizeof(uint32_t) + 255) / 256 * 256;
+constexpr size_t kScratchBytes = kScratchRecords + kNoAllocRecords * sizeof(ChunkRecord);
+static_assert(kScratchBytes <= (17u << 20), "the scratch array is meant to stay modest");
+
+}  // namespace
+
+// Scratch memory of the allocation-free batched copy: 16.25 MiB that every GPU
+// this library runs on holds from the load of the library's code object to the
+// end of the process.  In host code this name is only a stand-in for the
+// symbol, not a device address: host code reaches the memory through the
+// per-device pointer scratch_for_device() keeps (hipGetSymbolAddress), and the
+// kernels take that pointer as an argument.
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+namespace {
+
+// Each GPU holds its own copy of `scratch` at its own address.  Looked up once
+// per device, with that device current, and kept.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+void* g_scratch_ptr[kMaxDevices];
+bool g_scratch_known[kMaxDevices];
+hipError_t g_scratch_err[kMaxDevices];
+
+// The calling thread's current device must be `device`.
+hipError_t scratch_for_device(int device, void** out) {
+  *out = nullptr;
+  if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> g(g_scratch_lock);
+  if (!g_scratch_known[device]) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    g_scratch_err[device] = e;
+    g_scratch_ptr[device] = e == hipSuccess ? p : nullptr;
+    g_scratch_known[device] = true;
+  }
+  *out = g_scratch_ptr[device];
+  return g_scratch_err[device];
+}
+
 }  // namespace
 
 struct mi355_blit {
   int device = 0;
   int num_cus = 0;
   hipStream_t stream = nullptr;
+  // This GPU's copy of `scratch` (a device address), or null with the error
+  // that the lookup gave.
+  unsigned char* scratch_dev = nullptr;
+  hipError_t scratch_err = hipSuccess;
 
   std::mutex lock;  // guards everything below
   mi355_blit_tuning_t tuning{};
@@ -347,6 +401,11 @@ int mi355_blit_create(int device_ordinal, mi355_blit_t** out) {
     return e == hipSuccess ? MI355_BLIT_ERROR : status_of(e);
   }
   h->num_cus = cus;
+  {
+    void* p = nullptr;
+    h->scratch_err = scratch_for_device(device_ordinal, &p);
+    h->scratch_dev = static_cast<unsigned char*>(p);
+  }
   int large_bar = 0;
   if (hipDeviceGetAttribute(&large_bar, hipDeviceAttributeIsLargeBar, device_ordinal) == hipSuccess && large_bar &&
       !std::getenv("MI355_BLIT_HOST_STAGING"))
@@ -483,11 +542,21 @@ int mi355_blit_copy_batch_bounded(mi355_blit_t* h, const mi355_blit_desc_t* devi
 namespace {
 // The two launches of the device-side prefix sum over the copies' chunk
 // counts: chunk_start within groups of 1024 copies, block_sum across groups.
-void launch_scans(mi355_blit* h, hipStream_t s, const BatchDesc* dev_descs, size_t n, BatchDesc* private_copy) {
+// The device memory a batch of device-resident descriptors works in: the
+// handle's own buffers, or the parts of the static scratch array.
+struct BatchDeviceBuffers {
+  uint32_t* chunk_start;
+  uint32_t* block_sum;
+  ChunkRecord* records;
+  uint64_t* seen;  // host memory for the batch's numbers of copies and chunks; may be null
+};
+
+void launch_scans(const BatchDeviceBuffers& b, hipStream_t s, const BatchDesc* dev_descs, size_t n,
+                  BatchDesc* private_copy) {
   const uint32_t n_blocks = static_cast<uint32_t>((n + 1023) / 1024);
-  ScanLocalArgs sl{dev_descs, static_cast<uint64_t>(n), h->chunk_start_dev, h->block_sum_dev, private_copy};
+  ScanLocalArgs sl{dev_descs, static_cast<uint64_t>(n), b.chunk_start, b.block_sum, private_copy};
   hipLaunchKernelGGL(mi355_batch_scan_local, dim3(n_blocks), dim3(1024), 0, s, sl);
-  ScanTopArgs st{h->block_sum_dev, h->chunk_start_dev, static_cast<uint64_t>(n), n_blocks};
+  ScanTopArgs st{b.block_sum, b.chunk_start, static_cast<uint64_t>(n), n_blocks};
   hipLaunchKernelGGL(mi355_batch_scan_top, dim3(1), dim3(1024), 0, s, st);
 }
 
@@ -503,17 +572,30 @@ int launch_records_copy(mi355_blit* h, hipStream_t s, const mi355_blit_plan_t& p
 
 // The same for device-resident descriptors: `records` is what the record
 // buffer has room for, the number of chunks is behind the prefix sums.
-int launch_lookup_copy(mi355_blit* h, hipStream_t s, const mi355_blit_plan_t& p, const BatchLaunch& l,
+int launch_lookup_copy(const BatchDeviceBuffers& b, hipStream_t s, const mi355_blit_plan_t& p, const BatchLaunch& l,
                        uint64_t records, const BatchDesc* dev_descs, size_t n) {
   batch_lookup_kernel_t k = nullptr;
   for (const BatchLookupVariant& v : kBatchLookupVariants)
     if (v.nt_load == p.nt_load && v.store == p.store_policy) k = v.fn;
   if (!k || l.split != 4) return MI355_BLIT_ERROR;
-  BatchLookupArgs a{{h->records_dev, records, h->chunk_start_dev + n, l.waves_per_wg, l.n_waves,
+  BatchLookupArgs a{{b.records, records, b.chunk_start + n, l.waves_per_wg, l.n_waves,
                      make_xcd_runs(p.grid, p.xcd_run)},
-                    dev_descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n), h->batch_seen};
+                    dev_descs, b.chunk_start, b.block_sum, static_cast<uint64_t>(n), b.seen};
   hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
   return MI355_BLIT_SUCCESS;
+}
+
+// Prefix sums, records and the copy for n device-resident descriptors, in the
+// buffers *b: four launches, nothing else.
+int launch_device_batch(const BatchDeviceBuffers& b, hipStream_t s, const mi355_blit_plan_t& p, const BatchLaunch& l,
+                        uint64_t records, const BatchDesc* scanned, const BatchDesc* dev_descs,
+                        BatchDesc* private_copy, size_t n) {
+  launch_scans(b, s, scanned, n, private_copy);
+  EmitRecordsDeviceArgs er{dev_descs, b.chunk_start, b.block_sum, static_cast<uint64_t>(n), b.records, records};
+  hipLaunchKernelGGL(mi355_batch_emit_records_lookup, dim3(static_cast<uint32_t>((records + 255) / 256)),
+                     dim3(256), 0, s, er);
+  BLIT_HIP(hipGetLastError());
+  return launch_lookup_copy(b, s, p, l, records, dev_descs, n);
 }
 
 int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int descs_on_device,
@@ -631,13 +713,8 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
     // leaves a copy of them for the others.
     const BatchDesc* scanned = raw ? h->descs_host[b] : reinterpret_cast<const BatchDesc*>(descs);
     const BatchDesc* dev_descs = raw ? h->descs_private_dev : scanned;
-    launch_scans(h, s, scanned, n, raw ? h->descs_private_dev : nullptr);
-    EmitRecordsDeviceArgs er{dev_descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n),
-                             h->records_dev, sizing.records};
-    hipLaunchKernelGGL(mi355_batch_emit_records_lookup, dim3(static_cast<uint32_t>((sizing.records + 255) / 256)),
-                       dim3(256), 0, s, er);
-    BLIT_HIP(hipGetLastError());
-    rc = launch_lookup_copy(h, s, p, l, sizing.records, dev_descs, n);
+    const BatchDeviceBuffers bufs{h->chunk_start_dev, h->block_sum_dev, h->records_dev, h->batch_seen};
+    rc = launch_device_batch(bufs, s, p, l, sizing.records, scanned, dev_descs, raw ? h->descs_private_dev : nullptr, n);
     if (rc != MI355_BLIT_SUCCESS) return rc;
   }
   BLIT_HIP(hipGetLastError());
@@ -648,6 +725,40 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
   return ledger_record(h, s, shape.total_bytes);
 }
 }  // namespace
+
+int mi355_blit_copy_batch_bounded_noalloc(mi355_blit_t* h, const mi355_blit_desc_t* device_descs, size_t n,
+                                          uint64_t max_total_bytes, void* stream) {
+  if (!h || (!device_descs && n)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (max_total_bytes == 0) return n ? MI355_BLIT_ERROR_INVALID_ARGUMENT : MI355_BLIT_SUCCESS;
+  if (n == 0) return MI355_BLIT_SUCCESS;
+  if (n > kNoAllocMaxCopies) return MI355_BLIT_ERROR_OUT_OF_RESOURCES;
+  std::lock_guard<std::mutex> g(h->lock);
+  DeviceScope scope(h->device);
+  if (scope.err != hipSuccess) return status_of(scope.err);
+  if (!h->scratch_dev) return h->scratch_err != hipSuccess ? status_of(h->scratch_err) : MI355_BLIT_ERROR;
+  hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
+  BatchDeviceSizing sizing = batch_device_sizing(n, max_total_bytes);
+  if (sizing.records == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  // Chunks beyond the records the scratch has room for are looked up in the
+  // prefix sums by the copy kernel: the scratch bounds the number of copies,
+  // not their bytes.
+  if (sizing.records > kNoAllocRecords) sizing.records = kNoAllocRecords;
+  mi355_blit_plan_t p;
+  const BatchLaunch l = plan_batch_records(sizing.grid_chunks, sizing.bytes, true,
+                                           h->has_tuning ? &h->tuning : nullptr, false, &p);
+  // Every word of the scratch that the kernels read was written by a kernel of
+  // this same call before (the prefix sums in full, the records up to the
+  // smaller of the chunk total and the capacity): nothing has to start at zero.
+  const BatchDeviceBuffers bufs{reinterpret_cast<uint32_t*>(h->scratch_dev + kScratchChunkStart),
+                                reinterpret_cast<uint32_t*>(h->scratch_dev + kScratchBlockSum),
+                                reinterpret_cast<ChunkRecord*>(h->scratch_dev + kScratchRecords), nullptr};
+  const BatchDesc* descs = reinterpret_cast<const BatchDesc*>(device_descs);
+  const int rc = launch_device_batch(bufs, s, p, l, sizing.records, descs, descs, nullptr, n);
+  if (rc != MI355_BLIT_SUCCESS) return rc;
+  BLIT_HIP(hipGetLastError());
+  h->last_plan = p;
+  return ledger_record(h, s, sizing.bytes);
+}
 
 int mi355_blit_copy_rect(mi355_blit_t* h, const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
                          const mi355_pitched_ptr_t* src, const mi355_dim3_t* src_offset,

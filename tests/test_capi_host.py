@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol(capi_host):
 
 def test_abi_version_and_status_strings(capi_host):
     lib = capi_host.load()
-    assert lib.mi355_blit_abi_version() == 2
+    assert lib.mi355_blit_abi_version() == 3
     assert lib.mi355_blit_status_string(0) == b"success"
     assert lib.mi355_blit_status_string(capi_host.ERROR_INVALID_ARGUMENT) == b"invalid argument"
     assert lib.mi355_blit_status_string(12345) == b"unknown status"

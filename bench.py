@@ -155,10 +155,14 @@ def make_fill(r, nbytes):
     return fn, verify, nbytes, (dst,)
 
 
-def make_batch(r, n=65536, arena=8 * GIB):
-    """65,536 copies, 64 B .. 256 KiB log-uniform, byte offsets 0..15 on both
-    sides, non-overlapping regions spread over an `arena`-byte source and an
-    `arena`-byte destination (16 GiB in all)."""
+def batch_layout(n=65536, arena=8 * GIB):
+    """Where the batch workload's copies lie: lengths 64 B .. 256 KiB
+    log-uniform, byte offsets 0..15 drawn independently for source and
+    destination, regions carved one behind the other (length rounded up to 256
+    plus a 256-byte guard) with the strides scaled so that the n regions fill
+    an `arena`-byte source and an `arena`-byte destination.  Returns (lens, so,
+    do, offs, stride): copy i moves lens[i] bytes from arena offset offs[i] +
+    so[i] of the source to offs[i] + do[i] of the destination."""
     import numpy as np
     rng = np.random.default_rng(0xB1170005)
     lens = np.floor(64 * 2.0 ** (12 * rng.random(n))).astype(np.int64)
@@ -168,6 +172,14 @@ def make_batch(r, n=65536, arena=8 * GIB):
     scale = (arena - 4096) / float(need.sum())
     stride = (np.floor(need * scale).astype(np.int64) // 256) * 256
     offs = np.concatenate([[0], np.cumsum(stride)[:-1]]) + 256
+    return lens, so, do, offs, stride
+
+
+def make_batch(r, n=65536, arena=8 * GIB):
+    """65,536 copies, 64 B .. 256 KiB log-uniform, byte offsets 0..15 on both
+    sides, non-overlapping regions spread over an `arena`-byte source and an
+    `arena`-byte destination (16 GiB in all)."""
+    lens, so, do, offs, _stride = batch_layout(n, arena)
     src = r.torch.empty(arena + 512, dtype=r.torch.uint8, device="cuda:0")
     dst = r.torch.empty(arena + 512, dtype=r.torch.uint8, device="cuda:0")
     # seeded 64 MiB block repeated: cheap to make, every region still has varied bytes

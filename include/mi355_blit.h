@@ -77,7 +77,34 @@ typedef struct {
                            neighbouring workgroups' tiles, and a cache line two
                            neighbouring tiles share is fetched into one L2 */
   uint32_t route;       /* MI355_BLIT_ROUTE_* the launch was shaped for */
+  uint32_t reference_engine; /* MI355_ENGINE_*: the engine GpuAgent::GetBlitObject
+                           (core/runtime/amd_gpu_agent.cpp:2379-2398) would have
+                           sent the last mi355_hsa_amd_memory_async_copy to;
+                           0 when no such call has been judged.  Reported by
+                           mi355_aql_last_launch_info only */
+  uint32_t reserved;
 } mi355_blit_plan_t;
+
+/* The engine choice of GpuAgent::GetBlitObject for an asynchronous copy within
+ * one GPU's memory (core/runtime/amd_gpu_agent.cpp:2379-2398): below
+ * HSA_FORCE_SDMA_SIZE the SDMA-capable engine of blits_[BlitDevToHost], "to
+ * avoid cache flushing", from there on the blit kernel. */
+enum {
+  MI355_ENGINE_NONE = 0,
+  MI355_ENGINE_BLIT_KERNEL = 1, /* blits_[BlitDevToDev] */
+  MI355_ENGINE_SDMA = 2         /* blits_[BlitDevToHost] */
+};
+
+/* Flag::force_sdma_size() (core/util/flag.h:206-207): HSA_FORCE_SDMA_SIZE read
+ * with atoi, 1 MiB when unset or empty.  Read on every call. */
+uint64_t mi355_policy_force_sdma_size(void);
+
+/* MI355_ENGINE_SDMA when size < force_sdma_size, else MI355_ENGINE_BLIT_KERNEL
+ * (amd_gpu_agent.cpp:2390-2397).  Pure.  With this engine behind BlitDevToDev
+ * the measured crossover against the DMA engine on MI355X is 128 KiB with
+ * system-scope fences and 0 with agent-scope fences: a deployment would set
+ * HSA_FORCE_SDMA_SIZE to that. */
+uint32_t mi355_policy_same_gpu_engine(uint64_t size, uint64_t force_sdma_size);
 
 /* Which memories a linear copy connects.  The reference keeps one blit object
  * per direction (core/inc/amd_gpu_agent.h:588, BlitDevToDev / BlitHostToDev /

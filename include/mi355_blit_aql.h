@@ -12,6 +12,11 @@
  * Signals are passed as hsa_signal_t.handle values (uint64_t), 0 meaning "no
  * signal".  Status values are hsa_status_t values.  Every entry point may be
  * called from any thread.
+ *
+ * MI355_BLIT_LOG_PKTS=1 in the environment of mi355_aql_create[_on] prints one
+ * line per barrier and dispatch packet on stderr, with the fields that
+ * LogPrint(HSA_AMD_LOG_FLAG_BLIT_KERNEL_PKTS, ...) prints in the reference
+ * (core/runtime/amd_blit_kernel.cpp:681-702, 903-923).
  */
 #ifndef MI355_BLIT_AQL_H_
 #define MI355_BLIT_AQL_H_
@@ -36,9 +41,59 @@ typedef struct mi355_aql mi355_aql_t;
  * hsa_iterate_agents order.  Calls hsa_init (reference counted). */
 int mi355_aql_create(int gpu_ordinal, mi355_aql_t** out);
 
+/* The same engine on the caller's agent and the caller's queue: what
+ * BlitKernel::BlitKernel(core::Queue*) + Initialize(const core::Agent&) take
+ * (core/inc/amd_blit_kernel.h:58-66, core/runtime/amd_blit_kernel.cpp:553-591),
+ * the queue being the agent's utility queue that GpuAgent made
+ * (core/runtime/amd_gpu_agent.cpp:692-701: 64 packets, HSA_QUEUE_TYPE_MULTI)
+ * and hands to CreateBlitKernel (:749-759).  hsa_agent_handle is
+ * hsa_agent_t.handle of a GPU agent (core::Agent::public_handle()), hsa_queue
+ * an hsa_queue_t* (core::Queue::public_handle()).  Calls neither hsa_init nor
+ * hsa_shut_down and creates no queue: the runtime must be up, and both it and
+ * the queue stay the caller's and must outlive the engine.  The kernarg ring
+ * and the pending-bytes ledger have queue->size entries, indexed by packet
+ * index like the reference's (amd_blit_kernel.cpp:554-569, 926-941).  Other
+ * producers may use the queue at the same time: slots are reserved with an
+ * atomic add on the write index and nothing else (amd_blit_kernel.cpp:
+ * 844-861), and packets of others are never touched.  Two things follow from
+ * sharing: mi355_aql_wait_idle and mi355_aql_destroy wait, behind a barrier
+ * packet, also for what others queued earlier; and the queue's error callback
+ * is its creator's, who forwards an error with mi355_aql_report_queue_error.
+ * NULL or a queue whose size is not a power of two, or an agent that is not a
+ * GPU -> INVALID_ARGUMENT. */
+int mi355_aql_create_on(uint64_t hsa_agent_handle, void* hsa_queue, mi355_aql_t** out);
+
 /* Replaces BlitKernel::Destroy (amd_blit_kernel.cpp:593-612).  Blocks until
- * every submitted packet has executed. */
+ * every submitted packet has executed (the reference does not wait; its
+ * caller must).  A borrowed queue and a borrowed runtime are left alone. */
 int mi355_aql_destroy(mi355_aql_t* h);
+
+/* Tells the engine that its queue has stopped on an asynchronous error: what
+ * the error callback of a queue the engine created does by itself, and what
+ * the owner of a borrowed queue forwards from its own callback (the role of
+ * core::Queue::DefaultErrorHandler, core/runtime/queue.cpp:52-59).  From then
+ * on submissions answer HSA_STATUS_ERROR and every wait inside the library
+ * ends with HSA_STATUS_ERROR instead of waiting for signals that nobody will
+ * complete.  status == 0 is ignored.  Tests of the error path use it to force
+ * the condition from the host. */
+int mi355_aql_report_queue_error(mi355_aql_t* h, int status);
+
+/* Waits, actively and in slices of about a millisecond, until the signal's
+ * value is below 1: the wait of BlitKernel's blocking calls
+ * (amd_blit_kernel.cpp:632-636, 830-834).  0 -> SUCCESS; a negative value
+ * (a failed command, inc/hsa_ext_amd.h:1735-1739) -> HSA_STATUS_ERROR; a
+ * reported queue error while the value is still 1 or more -> HSA_STATUS_ERROR
+ * where the reference would wait forever. */
+int mi355_aql_wait_signal(mi355_aql_t* h, uint64_t signal);
+
+/* Blocking forms: BlitKernel::SubmitLinearCopyCommand(dst, src, size) and
+ * SubmitLinearFillCommand (amd_blit_kernel.cpp:614-639, 787-837).  They hold
+ * the engine's blocking-call lock, arm its private completion signal with 1,
+ * submit, and wait for that signal only (not for the queue to drain), as
+ * mi355_aql_wait_signal waits.  Argument rules of mi355_aql_copy_route /
+ * mi355_aql_fill32. */
+int mi355_aql_copy_sync(mi355_aql_t* h, void* dst, const void* src, size_t bytes, uint32_t route);
+int mi355_aql_fill32_sync(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dwords);
 
 /* Replaces BlitKernel::SubmitLinearCopyCommand, asynchronous overload
  * (amd_blit_kernel.cpp:641-785): ceil(num_deps / 5) BARRIER_AND packets, then
@@ -132,6 +187,9 @@ int mi355_aql_get_command_time(mi355_aql_t* h, uint64_t completion_signal, uint6
 
 int mi355_aql_set_tuning(mi355_aql_t* h, const mi355_blit_tuning_t* tuning);
 int mi355_aql_last_launch_info(mi355_aql_t* h, mi355_blit_plan_t* out);
+/* Records MI355_ENGINE_* for mi355_aql_last_launch_info to report (the caller
+ * policy does, for every asynchronous copy it judges). */
+int mi355_aql_note_reference_engine(mi355_aql_t* h, uint32_t engine);
 int mi355_aql_num_cus(mi355_aql_t* h);
 
 /* Fence scope of the dispatch packets' acquire and release: 1 = system (the
@@ -184,7 +242,10 @@ int mi355_hsa_amd_memory_fill(mi355_aql_t* h, void* ptr, uint32_t value, size_t 
  * reference learns the direction from the two agents it is handed
  * (GetBlitObject, amd_gpu_agent.cpp:2379-2442); this signature has none, so
  * copies of 1 MiB and more, the sizes whose launch shape depends on it, look
- * the two pointers up (hsa_amd_pointer_info) and take the route they give. */
+ * the two pointers up (hsa_amd_pointer_info) and take the route they give.
+ * The copy always runs on this engine; which engine GetBlitObject would have
+ * picked for it (amd_gpu_agent.cpp:2379-2398, HSA_FORCE_SDMA_SIZE) is left in
+ * mi355_blit_plan_t::reference_engine of mi355_aql_last_launch_info. */
 int mi355_hsa_amd_memory_async_copy(mi355_aql_t* h, void* dst, const void* src, size_t size,
                                     uint32_t num_dep_signals, const uint64_t* dep_signals,
                                     uint64_t completion_signal);

@@ -11,7 +11,13 @@ _U64P = C.POINTER(C.c_uint64)
 
 SIGNATURES = {
     "mi355_aql_create": (C.c_int, [C.c_int, C.POINTER(C.c_void_p)]),
+    "mi355_aql_create_on": (C.c_int, [C.c_uint64, C.c_void_p, C.POINTER(C.c_void_p)]),
     "mi355_aql_destroy": (C.c_int, [C.c_void_p]),
+    "mi355_aql_report_queue_error": (C.c_int, [C.c_void_p, C.c_int]),
+    "mi355_aql_wait_signal": (C.c_int, [C.c_void_p, C.c_uint64]),
+    "mi355_aql_copy_sync": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint32]),
+    "mi355_aql_fill32_sync": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t]),
+    "mi355_aql_note_reference_engine": (C.c_int, [C.c_void_p, C.c_uint32]),
     "mi355_aql_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, _U64P, C.c_uint32, C.c_uint64]),
     "mi355_aql_copy_route": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint32, _U64P, C.c_uint32,
                                        C.c_uint64]),
@@ -84,12 +90,21 @@ class AqlBlit:
 
     backend = "aql"
 
-    def __init__(self, gpu=0):
+    def __init__(self, gpu=0, borrowed=None):
+        """gpu: ordinal among the GPU agents, on a queue of the engine's own.
+        borrowed: a BorrowedQueue instead; the engine then runs on that agent
+        and that queue (mi355_aql_create_on) and leaves both alone on close."""
         self.lib = load()
+        self.borrowed = borrowed
         h = C.c_void_p()
-        st = self.lib.mi355_aql_create(gpu, C.byref(h))
+        if borrowed is not None:
+            st = self.lib.mi355_aql_create_on(borrowed.agent, borrowed.queue, C.byref(h))
+            what = "mi355_aql_create_on"
+        else:
+            st = self.lib.mi355_aql_create(gpu, C.byref(h))
+            what = "mi355_aql_create"
         if st != SUCCESS:
-            raise RuntimeError("mi355_aql_create failed: 0x%x" % st)
+            raise RuntimeError("%s failed: 0x%x" % (what, st))
         self.handle = h
 
     def close(self):
@@ -98,6 +113,18 @@ class AqlBlit:
             self.handle = None
             if st != SUCCESS:
                 raise RuntimeError("mi355_aql_destroy failed: 0x%x" % st)
+
+    def copy_sync(self, dst, src, nbytes, route=0):
+        return self.lib.mi355_aql_copy_sync(self.handle, dst, src, nbytes, route)
+
+    def fill32_sync(self, ptr, value, num_dwords):
+        return self.lib.mi355_aql_fill32_sync(self.handle, ptr, value, num_dwords)
+
+    def wait_signal(self, signal):
+        return self.lib.mi355_aql_wait_signal(self.handle, signal)
+
+    def report_queue_error(self, status=ERROR):
+        return self.lib.mi355_aql_report_queue_error(self.handle, status)
 
     def __enter__(self):
         return self
@@ -240,3 +267,55 @@ class HsaSignals:
         """Blocks until the signal is < 1 (HSA_SIGNAL_CONDITION_LT = 2)."""
         while self.hsa.hsa_signal_wait_scacquire(s, 2, 1, 0xFFFFFFFFFFFFFFFF, 1 if active else 0) >= 1:
             pass
+
+
+class BorrowedQueue:
+    """An HSA queue made by the caller, the way GpuAgent makes its utility
+    queue (hsa_queue_create, 64 packets, HSA_QUEUE_TYPE_MULTI), for an engine to
+    run on (AqlBlit(borrowed=...)).  Holds a reference on the runtime for its
+    lifetime.  `agent` is hsa_agent_t.handle of GPU `gpu`, `queue` the
+    hsa_queue_t* as an int."""
+
+    _AGENT_CB = C.CFUNCTYPE(C.c_int, C.c_uint64, C.c_void_p)
+    _ERROR_CB = C.CFUNCTYPE(None, C.c_int, C.c_void_p, C.c_void_p)
+
+    def __init__(self, gpu=0, packets=64):
+        hsa = C.CDLL("libhsa-runtime64.so.1")
+        self.hsa = hsa
+        hsa.hsa_iterate_agents.argtypes = [self._AGENT_CB, C.c_void_p]
+        hsa.hsa_agent_get_info.argtypes = [C.c_uint64, C.c_int, C.c_void_p]
+        hsa.hsa_queue_create.argtypes = [C.c_uint64, C.c_uint32, C.c_uint32, self._ERROR_CB, C.c_void_p, C.c_uint32,
+                                         C.c_uint32, C.POINTER(C.c_void_p)]
+        hsa.hsa_queue_destroy.argtypes = [C.c_void_p]
+        if hsa.hsa_init() != 0:
+            raise RuntimeError("hsa_init failed")
+        gpus = []
+
+        def visit(agent, _data):
+            kind = C.c_int(-1)
+            hsa.hsa_agent_get_info(agent, 17, C.byref(kind))  # HSA_AGENT_INFO_DEVICE
+            if kind.value == 1:                               # HSA_DEVICE_TYPE_GPU
+                gpus.append(agent)
+            return 0
+
+        self._visit = self._AGENT_CB(visit)
+        hsa.hsa_iterate_agents(self._visit, None)
+        if gpu >= len(gpus):
+            hsa.hsa_shut_down()
+            raise RuntimeError("no GPU agent %d" % gpu)
+        self.agent = gpus[gpu]
+        self.errors = []
+        self._on_error = self._ERROR_CB(lambda status, _queue, _data: self.errors.append(status))
+        q = C.c_void_p()
+        st = hsa.hsa_queue_create(self.agent, packets, 0, self._on_error  # HSA_QUEUE_TYPE_MULTI
+                                  , None, 0xFFFFFFFF, 0xFFFFFFFF, C.byref(q))
+        if st != 0:
+            hsa.hsa_shut_down()
+            raise RuntimeError("hsa_queue_create failed: 0x%x" % st)
+        self.queue = q.value
+
+    def close(self):
+        if self.queue:
+            self.hsa.hsa_queue_destroy(self.queue)
+            self.queue = None
+            self.hsa.hsa_shut_down()

@@ -19,6 +19,9 @@ KERNEL_FILL = 2
 KERNEL_COPY_BATCH = 3
 KERNEL_COPY_RECT = 4
 NOALLOC_MAX_COPIES = 65536
+ENGINE_NONE = 0
+ENGINE_BLIT_KERNEL = 1
+ENGINE_SDMA = 2
 
 STORE_CACHED = 0
 STORE_NT = 1
@@ -36,6 +39,7 @@ class Plan(C.Structure):
         ("byte_shift", C.c_uint32), ("lead_vecs", C.c_uint32),
         ("head_bytes", C.c_uint64), ("body_vecs", C.c_uint64), ("tail_bytes", C.c_uint64),
         ("xcd_run", C.c_uint32), ("route", C.c_uint32),
+        ("reference_engine", C.c_uint32), ("reserved", C.c_uint32),
     ]
 
     def as_dict(self):
@@ -119,6 +123,8 @@ SIGNATURES = {
     "mi355_blit_stream": (C.c_void_p, [C.c_void_p]),
     "mi355_blit_status_string": (C.c_char_p, [C.c_int]),
     "mi355_blit_abi_version": (C.c_int, []),
+    "mi355_policy_force_sdma_size": (C.c_uint64, []),
+    "mi355_policy_same_gpu_engine": (C.c_uint32, [C.c_uint64, C.c_uint64]),
 }
 
 _lib = None

@@ -20,6 +20,7 @@
 #include <string>
 #include <vector>
 
+#include "aql_wait.h"
 #include "blit_args.h"
 #include "blit_kernel_list.h"
 #include "blit_batch_host.h"
@@ -35,9 +36,10 @@ namespace {
 
 using namespace mi355;
 
-// Packets in the queue.  The reference shares the agent's 64-packet utility
-// queue (amd_gpu_agent.h:507-508); a batch here is two packets, so the ring
-// is a little larger.
+// Packets in a queue this library creates for itself (mi355_aql_create).  The
+// reference shares the agent's 64-packet utility queue (amd_gpu_agent.h:
+// 507-508), which mi355_aql_create_on adopts as it is; a batch here is two to
+// four packets, so a queue of the library's own is a little larger.
 constexpr uint32_t kQueuePackets = 256;
 // One kernarg slot per packet slot, as in the reference (amd_blit_kernel.cpp:
 // 565-569): the slot of packet index i is i & mask, so it is free again
@@ -92,6 +94,11 @@ struct mi355_aql {
 
   hsa_queue_t* queue = nullptr;
   uint32_t queue_mask = 0;
+  // mi355_aql_create makes the runtime reference and the queue and gives both
+  // back; mi355_aql_create_on borrows the caller's.
+  bool owns_runtime = false, owns_queue = false;
+  uint64_t wait_slice_ticks = 100000;  // one slice of a bounded wait: about a millisecond
+  bool log_packets = false;            // MI355_BLIT_LOG_PKTS=1
   uint8_t* kernargs = nullptr;
   // The kernarg ring lives in device memory when the host can write there
   // (large BAR): a wave then reads its arguments from HBM instead of from
@@ -112,6 +119,10 @@ struct mi355_aql {
   Kernel scan_local, scan_top, emit_records, emit_records_lookup;
 
   hsa_signal_t idle_signal{};  // completion signal of wait_idle's barrier packet
+  // Completion signal of the blocking calls, guarded by sync_lock
+  // (completion_signal_ and lock_ of the reference, amd_blit_kernel.h:199-204).
+  hsa_signal_t sync_signal{};
+  std::mutex sync_lock;
 
   // Orders packet indices and ledger updates (reservation_lock_ of the
   // reference, amd_blit_kernel.h:209-210).
@@ -129,6 +140,7 @@ struct mi355_aql {
   mi355_blit_tuning_t tuning{};
   bool has_tuning = false;
   mi355_blit_plan_t last_plan{};
+  uint32_t reference_engine = 0;  // MI355_ENGINE_* of the last asynchronous copy the caller policy judged
   uint16_t fence_scope = HSA_FENCE_SCOPE_SYSTEM;
   std::atomic<bool> queue_error{false};
 
@@ -191,7 +203,7 @@ hsa_status_t find_agents_cb(hsa_agent_t agent, void* data) {
   hsa_device_type_t type;
   if (hsa_agent_get_info(agent, HSA_AGENT_INFO_DEVICE, &type) != HSA_STATUS_SUCCESS) return HSA_STATUS_SUCCESS;
   if (type == HSA_DEVICE_TYPE_GPU) {
-    if (h->seen_gpus++ == h->wanted_ordinal) {
+    if (h->wanted_ordinal >= 0 && h->seen_gpus++ == h->wanted_ordinal) {
       h->gpu = agent;
       h->have_gpu = true;
     }
@@ -210,12 +222,68 @@ void queue_error_cb(hsa_status_t status, hsa_queue_t*, void* data) {
   std::fprintf(stderr, "mi355_blit_aql: queue error 0x%x (%s)\n", status, msg ? msg : "?");
 }
 
-// MI355_BLIT_HOST_KERNARGS=1 keeps the kernarg ring in host memory (for
-// measurements and for systems whose BAR writes misbehave).
-bool force_host_kernargs() {
-  const char* v = std::getenv("MI355_BLIT_HOST_KERNARGS");
+// Waits until `signal` drops below 1, in bounded slices, giving up with an
+// error when the queue has reported one (aql_wait.h).
+int wait_signal(mi355_aql* h, hsa_signal_t signal) {
+  return wait_below_one(
+      [signal](uint64_t ticks) {
+        return static_cast<int64_t>(
+            hsa_signal_wait_scacquire(signal, HSA_SIGNAL_CONDITION_LT, 1, ticks, HSA_WAIT_STATE_ACTIVE));
+      },
+      h->queue_error, h->wait_slice_ticks);
+}
+
+bool env_is_one(const char* name) {
+  const char* v = std::getenv(name);
   return v && v[0] == '1';
 }
+
+// What LogPrint(HSA_AMD_LOG_FLAG_BLIT_KERNEL_PKTS, ...) prints for every
+// packet in the reference (amd_blit_kernel.cpp:681-702, 903-923), on stderr
+// when MI355_BLIT_LOG_PKTS=1.
+unsigned header_bits(uint16_t header, unsigned pos, unsigned width) { return (header >> pos) & ((1u << width) - 1); }
+
+void log_barrier_packet(mi355_aql* h, uint16_t header, const hsa_barrier_and_packet_t& pkt, uint64_t index) {
+  std::fprintf(stderr,
+               "HWq=%p, id=%lu, Barrier Header = 0x%x (type=%u, barrier=%u, acquire=%u, release=%u), "
+               "dep_signal=[0x%zx 0x%zx 0x%zx 0x%zx 0x%zx], completion_signal=0x%zx rptr=%lu, wptr=%lu\n",
+               h->queue->base_address, static_cast<unsigned long>(h->queue->id), header,
+               header_bits(header, HSA_PACKET_HEADER_TYPE, HSA_PACKET_HEADER_WIDTH_TYPE),
+               header_bits(header, HSA_PACKET_HEADER_BARRIER, HSA_PACKET_HEADER_WIDTH_BARRIER),
+               header_bits(header, HSA_PACKET_HEADER_SCACQUIRE_FENCE_SCOPE, HSA_PACKET_HEADER_WIDTH_SCACQUIRE_FENCE_SCOPE),
+               header_bits(header, HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE, HSA_PACKET_HEADER_WIDTH_SCRELEASE_FENCE_SCOPE),
+               static_cast<size_t>(pkt.dep_signal[0].handle), static_cast<size_t>(pkt.dep_signal[1].handle),
+               static_cast<size_t>(pkt.dep_signal[2].handle), static_cast<size_t>(pkt.dep_signal[3].handle),
+               static_cast<size_t>(pkt.dep_signal[4].handle), static_cast<size_t>(pkt.completion_signal.handle),
+               static_cast<unsigned long>(hsa_queue_load_read_index_relaxed(h->queue)),
+               static_cast<unsigned long>(index));
+}
+
+void log_dispatch_packet(mi355_aql* h, uint16_t header, uint16_t setup, const hsa_kernel_dispatch_packet_t& pkt,
+                         uint64_t index) {
+  std::fprintf(stderr,
+               "HWq=%p, id=%lu, Dispatch Header = 0x%x (type=%u, barrier=%u, acquire=%u, release=%u), "
+               "setup=%d, grid=[%zu, %zu, %zu], workgroup=[%zu, %zu, %zu], private_seg_size=%zu, "
+               "group_seg_size=%zu, kernel_obj=0x%zx, kernarg_address=0x%zx, completion_signal=0x%zx "
+               "rptr=%lu, wptr=%lu\n",
+               h->queue->base_address, static_cast<unsigned long>(h->queue->id), header,
+               header_bits(header, HSA_PACKET_HEADER_TYPE, HSA_PACKET_HEADER_WIDTH_TYPE),
+               header_bits(header, HSA_PACKET_HEADER_BARRIER, HSA_PACKET_HEADER_WIDTH_BARRIER),
+               header_bits(header, HSA_PACKET_HEADER_SCACQUIRE_FENCE_SCOPE, HSA_PACKET_HEADER_WIDTH_SCACQUIRE_FENCE_SCOPE),
+               header_bits(header, HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE, HSA_PACKET_HEADER_WIDTH_SCRELEASE_FENCE_SCOPE),
+               setup, static_cast<size_t>(pkt.grid_size_x), static_cast<size_t>(pkt.grid_size_y),
+               static_cast<size_t>(pkt.grid_size_z), static_cast<size_t>(pkt.workgroup_size_x),
+               static_cast<size_t>(pkt.workgroup_size_y), static_cast<size_t>(pkt.workgroup_size_z),
+               static_cast<size_t>(pkt.private_segment_size), static_cast<size_t>(pkt.group_segment_size),
+               static_cast<size_t>(pkt.kernel_object), reinterpret_cast<size_t>(pkt.kernarg_address),
+               static_cast<size_t>(pkt.completion_signal.handle),
+               static_cast<unsigned long>(hsa_queue_load_read_index_relaxed(h->queue)),
+               static_cast<unsigned long>(index));
+}
+
+// MI355_BLIT_HOST_KERNARGS=1 keeps the kernarg ring in host memory (for
+// measurements and for systems whose BAR writes misbehave).
+bool force_host_kernargs() { return env_is_one("MI355_BLIT_HOST_KERNARGS"); }
 
 int lookup(mi355_aql* h, const char* name, Kernel* out) {
   const std::string sym = std::string(name) + ".kd";
@@ -265,7 +333,12 @@ int load_code_object(mi355_aql* h) {
 // is full.
 uint64_t acquire_write_index(mi355_aql* h, uint32_t num_packet) {
   const uint64_t index = hsa_queue_add_write_index_scacq_screl(h->queue, num_packet);
-  while (index + num_packet - hsa_queue_load_read_index_relaxed(h->queue) > h->queue->size) sched_yield();
+  // A queue that has stopped on an error never frees a slot: give up waiting
+  // (what is written then is never read, and the waits on its completion end
+  // with an error).
+  while (index + num_packet - hsa_queue_load_read_index_relaxed(h->queue) > h->queue->size &&
+         !h->queue_error.load(std::memory_order_acquire))
+    sched_yield();
   return index;
 }
 
@@ -309,6 +382,7 @@ void write_barriers(mi355_aql* h, uint64_t index, const uint64_t* deps, uint32_t
                       (HSA_FENCE_SCOPE_NONE << HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE);
     if (barrier_bit) header |= 1 << HSA_PACKET_HEADER_BARRIER;
     publish(slot, header, 0);
+    if (h->log_packets) log_barrier_packet(h, header, pkt, index + p);
   }
 }
 
@@ -358,6 +432,7 @@ void write_dispatch(mi355_aql* h, uint64_t index, const Kernel& k, const void* a
                     (release << HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE);
   if (barrier_bit) header |= 1 << HSA_PACKET_HEADER_BARRIER;
   publish(slot, header, 1 << HSA_KERNEL_DISPATCH_PACKET_SETUP_DIMENSIONS);
+  if (h->log_packets) log_dispatch_packet(h, header, 1 << HSA_KERNEL_DISPATCH_PACKET_SETUP_DIMENSIONS, pkt, index);
 }
 
 void tail_waves(const mi355_blit_plan_t& p, uint32_t* partial_wave, uint32_t* edge_wave, uint32_t* waves_per_wg,
@@ -421,9 +496,7 @@ int wait_idle_locked(mi355_aql* h) {
   }
   write_barriers(h, index, nullptr, 0, 1, h->idle_signal.handle, true);
   release_write_index(h, index, 1);
-  while (hsa_signal_wait_scacquire(h->idle_signal, HSA_SIGNAL_CONDITION_LT, 1, UINT64_MAX, HSA_WAIT_STATE_ACTIVE) >= 1) {
-    if (h->queue_error.load()) return MI355_BLIT_ERROR;
-  }
+  if (wait_signal(h, h->idle_signal) != MI355_BLIT_SUCCESS) return MI355_BLIT_ERROR;
   // the barrier had its barrier bit set: everything up to it has completed
   uint64_t seen = h->known_complete.load();
   while (seen < index + 1 && !h->known_complete.compare_exchange_weak(seen, index + 1)) {
@@ -492,35 +565,36 @@ const Kernel* find_batch(mi355_aql* h, const BatchLaunch& l, const mi355_blit_pl
 
 extern "C" {
 
-int mi355_aql_create(int gpu_ordinal, mi355_aql_t** out) {
-  if (!out || gpu_ordinal < 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
-  *out = nullptr;
-  hsa_status_t st = hsa_init();
-  if (st != HSA_STATUS_SUCCESS) return MI355_BLIT_ERROR_NOT_INITIALIZED;
-  mi355_aql* h = new (std::nothrow) mi355_aql;
-  if (!h) {
-    hsa_shut_down();
-    return MI355_BLIT_ERROR_OUT_OF_RESOURCES;
-  }
-  h->wanted_ordinal = gpu_ordinal;
+namespace {
+
+// Everything an engine needs beyond its GPU agent and its queue, which the
+// caller has put into *h: pools, the code object, the kernarg ring and the
+// ledger (both sized by the queue), the signals of its own waits.
+int init_engine(mi355_aql* h) {
   int rc = MI355_BLIT_SUCCESS;
-  auto fail = [&](int code) {
-    mi355_aql_destroy(h);
-    return code;
-  };
-  if (hsa_iterate_agents(find_agents_cb, h) != HSA_STATUS_SUCCESS || !h->have_cpu) return fail(MI355_BLIT_ERROR);
-  if (!h->have_gpu) return fail(MI355_BLIT_ERROR_INVALID_ARGUMENT);
+  if (hsa_iterate_agents(find_agents_cb, h) != HSA_STATUS_SUCCESS || !h->have_cpu) return MI355_BLIT_ERROR;
+  if (!h->have_gpu) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   std::pair<mi355_aql*, bool> ctx{h, false};
   hsa_amd_agent_iterate_memory_pools(h->cpu, find_pools_cb, &ctx);
   ctx.second = true;
   hsa_amd_agent_iterate_memory_pools(h->gpu, find_pools_cb, &ctx);
-  if (!h->have_kernarg || !h->have_host || !h->have_local) return fail(MI355_BLIT_ERROR);
+  if (!h->have_kernarg || !h->have_host || !h->have_local) return MI355_BLIT_ERROR;
   if (hsa_agent_get_info(h->gpu, static_cast<hsa_agent_info_t>(HSA_AMD_AGENT_INFO_COMPUTE_UNIT_COUNT), &h->num_cus) !=
           HSA_STATUS_SUCCESS || h->num_cus == 0)
-    return fail(MI355_BLIT_ERROR);
-  if ((rc = load_code_object(h)) != MI355_BLIT_SUCCESS) return fail(rc);
-  st = hsa_queue_create(h->gpu, kQueuePackets, HSA_QUEUE_TYPE_MULTI, queue_error_cb, h, UINT32_MAX, UINT32_MAX, &h->queue);
-  if (st != HSA_STATUS_SUCCESS) return fail(to_status(st));
+    return MI355_BLIT_ERROR;
+  uint64_t freq = 0;
+  if (hsa_system_get_info(HSA_SYSTEM_INFO_TIMESTAMP_FREQUENCY, &freq) == HSA_STATUS_SUCCESS && freq >= 1000)
+    h->wait_slice_ticks = freq / 1000;
+  h->log_packets = env_is_one("MI355_BLIT_LOG_PKTS");
+  if ((rc = load_code_object(h)) != MI355_BLIT_SUCCESS) return rc;
+  if (!h->queue) {
+    hsa_status_t st = hsa_queue_create(h->gpu, kQueuePackets, HSA_QUEUE_TYPE_MULTI, queue_error_cb, h, UINT32_MAX,
+                                       UINT32_MAX, &h->queue);
+    if (st != HSA_STATUS_SUCCESS) return to_status(st);
+    h->owns_queue = true;
+  }
+  // amd_blit_kernel.cpp:554-569: the ledger and the kernarg ring have one
+  // entry per packet slot of the queue, whoever made it
   h->queue_mask = h->queue->size - 1;
   h->bytes_written.assign(h->queue->size, BytesWritten{~0ull, ~0ull});
   void* ka = nullptr;
@@ -536,11 +610,62 @@ int mi355_aql_create(int gpu_ordinal, mi355_aql_t** out) {
     }
   }
   if (!ka && (rc = alloc(h, h->kernarg_pool, h->queue->size * kKernargSlotBytes, &ka, true)) != MI355_BLIT_SUCCESS)
-    return fail(rc);
+    return rc;
   h->kernargs = static_cast<uint8_t*>(ka);
-  if (hsa_signal_create(1, 0, nullptr, &h->idle_signal) != HSA_STATUS_SUCCESS) return fail(MI355_BLIT_ERROR_OUT_OF_RESOURCES);
+  if (hsa_signal_create(1, 0, nullptr, &h->idle_signal) != HSA_STATUS_SUCCESS) return MI355_BLIT_ERROR_OUT_OF_RESOURCES;
+  if (hsa_signal_create(1, 0, nullptr, &h->sync_signal) != HSA_STATUS_SUCCESS) return MI355_BLIT_ERROR_OUT_OF_RESOURCES;
   for (int i = 0; i < 2; ++i)
-    if (hsa_signal_create(0, 0, nullptr, &h->stage_free[i]) != HSA_STATUS_SUCCESS) return fail(MI355_BLIT_ERROR_OUT_OF_RESOURCES);
+    if (hsa_signal_create(0, 0, nullptr, &h->stage_free[i]) != HSA_STATUS_SUCCESS) return MI355_BLIT_ERROR_OUT_OF_RESOURCES;
+  return MI355_BLIT_SUCCESS;
+}
+
+}  // namespace
+
+int mi355_aql_create(int gpu_ordinal, mi355_aql_t** out) {
+  if (!out || gpu_ordinal < 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  *out = nullptr;
+  hsa_status_t st = hsa_init();
+  if (st != HSA_STATUS_SUCCESS) return MI355_BLIT_ERROR_NOT_INITIALIZED;
+  mi355_aql* h = new (std::nothrow) mi355_aql;
+  if (!h) {
+    hsa_shut_down();
+    return MI355_BLIT_ERROR_OUT_OF_RESOURCES;
+  }
+  h->owns_runtime = true;
+  h->wanted_ordinal = gpu_ordinal;
+  const int rc = init_engine(h);
+  if (rc != MI355_BLIT_SUCCESS) {
+    mi355_aql_destroy(h);
+    return rc;
+  }
+  *out = h;
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_aql_create_on(uint64_t hsa_agent_handle, void* hsa_queue, mi355_aql_t** out) {
+  if (!out) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  *out = nullptr;
+  hsa_queue_t* queue = static_cast<hsa_queue_t*>(hsa_queue);
+  if (!hsa_agent_handle || !queue || !queue->base_address || queue->size == 0 || (queue->size & (queue->size - 1)))
+    return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  hsa_agent_t gpu;
+  gpu.handle = hsa_agent_handle;
+  hsa_device_type_t type;
+  // also what tells a runtime that is not initialised: the caller owns that
+  hsa_status_t st = hsa_agent_get_info(gpu, HSA_AGENT_INFO_DEVICE, &type);
+  if (st != HSA_STATUS_SUCCESS) return to_status(st);
+  if (type != HSA_DEVICE_TYPE_GPU) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  mi355_aql* h = new (std::nothrow) mi355_aql;
+  if (!h) return MI355_BLIT_ERROR_OUT_OF_RESOURCES;
+  h->gpu = gpu;
+  h->have_gpu = true;
+  h->wanted_ordinal = -1;  // the agent walk only looks for the host's agent
+  h->queue = queue;
+  const int rc = init_engine(h);
+  if (rc != MI355_BLIT_SUCCESS) {
+    mi355_aql_destroy(h);
+    return rc;
+  }
   *out = h;
   return MI355_BLIT_SUCCESS;
 }
@@ -548,10 +673,14 @@ int mi355_aql_create(int gpu_ordinal, mi355_aql_t** out) {
 int mi355_aql_destroy(mi355_aql_t* h) {
   if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   int rc = MI355_BLIT_SUCCESS;
+  const bool owns_runtime = h->owns_runtime;
   {
     std::lock_guard<std::mutex> g(h->lock);
+    // The kernarg ring and the batch buffers go away below: everything this
+    // engine has queued must have run.  On a borrowed queue the barrier also
+    // waits for what other producers queued before it.
     if (h->queue && h->idle_signal.handle && !h->queue_error.load()) rc = wait_idle_locked(h);
-    if (h->queue) hsa_queue_destroy(h->queue);
+    if (h->queue && h->owns_queue) hsa_queue_destroy(h->queue);
     h->queue = nullptr;
     free_device(h->kernargs);
     for (int i = 0; i < 2; ++i) {
@@ -566,12 +695,26 @@ int mi355_aql_destroy(mi355_aql_t* h) {
     free_device(h->bounce[0]);
     free_device(h->bounce[1]);
     if (h->idle_signal.handle) hsa_signal_destroy(h->idle_signal);
+    if (h->sync_signal.handle) hsa_signal_destroy(h->sync_signal);
     if (h->have_exe) hsa_executable_destroy(h->exe);
     if (h->have_reader) hsa_code_object_reader_destroy(h->reader);
   }
   delete h;
-  hsa_shut_down();
+  if (owns_runtime) hsa_shut_down();
   return rc;
+}
+
+int mi355_aql_report_queue_error(mi355_aql_t* h, int status) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  if (status != MI355_BLIT_SUCCESS) h->queue_error.store(true, std::memory_order_release);
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_aql_wait_signal(mi355_aql_t* h, uint64_t signal) {
+  if (!h || !signal) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  hsa_signal_t s;
+  s.handle = signal;
+  return wait_signal(h, s);
 }
 
 int mi355_aql_num_cus(mi355_aql_t* h) { return h ? static_cast<int>(h->num_cus) : 0; }
@@ -606,6 +749,14 @@ int mi355_aql_last_launch_info(mi355_aql_t* h, mi355_blit_plan_t* out) {
   if (!h || !out) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   std::lock_guard<std::mutex> g(h->lock);
   *out = h->last_plan;
+  out->reference_engine = h->reference_engine;
+  return MI355_BLIT_SUCCESS;
+}
+
+int mi355_aql_note_reference_engine(mi355_aql_t* h, uint32_t engine) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> g(h->lock);
+  h->reference_engine = engine;
   return MI355_BLIT_SUCCESS;
 }
 
@@ -759,9 +910,7 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
     int rc = ensure_batch_capacity(h, n, 0);
     if (rc != MI355_BLIT_SUCCESS) return rc;
     const unsigned b = h->next_stage;
-    while (hsa_signal_wait_scacquire(h->stage_free[b], HSA_SIGNAL_CONDITION_LT, 1, UINT64_MAX, HSA_WAIT_STATE_ACTIVE) >= 1) {
-      if (h->queue_error.load()) return MI355_BLIT_ERROR;
-    }
+    if (wait_signal(h, h->stage_free[b]) != MI355_BLIT_SUCCESS) return MI355_BLIT_ERROR;
     uint64_t total_bytes = 0;
     rc = batch_stage_raw(descs, n, h->stage[b], &total_bytes);
     if (rc != MI355_BLIT_SUCCESS) return rc;
@@ -797,11 +946,15 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   // 64 chunks, and each piece's first record index (the host, which walks the
   // descriptors anyway, does the prefix sum).  The buffer is free again when
   // the kernel that read it last has finished.
+  // The launch is planned before the staging buffer is armed, so that nothing
+  // can fail between arming it and the packet that frees it again.
+  mi355_blit_plan_t p;
+  const BatchLaunch l = plan_batch_records(total_chunks, total_bytes, total_bytes >= (4ull << 20), t, true, &p);
+  const Kernel* bk = find_batch(h, l, p);
+  if (!bk) return MI355_BLIT_ERROR;
   const unsigned b = h->next_stage;
+  if (wait_signal(h, h->stage_free[b]) != MI355_BLIT_SUCCESS) return MI355_BLIT_ERROR;
   h->next_stage ^= 1;
-  while (hsa_signal_wait_scacquire(h->stage_free[b], HSA_SIGNAL_CONDITION_LT, 1, UINT64_MAX, HSA_WAIT_STATE_ACTIVE) >= 1) {
-    if (h->queue_error.load()) return MI355_BLIT_ERROR;
-  }
   const size_t image_bytes = batch_stage_bytes(shape.pieces);
   batch_stage(h->stage_image, h->stage[b]);
   if (h->stage_in_device_memory[b]) {
@@ -816,10 +969,6 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
                      h->records_dev};
 
   // 2. the copy
-  mi355_blit_plan_t p;
-  const BatchLaunch l = plan_batch_records(total_chunks, total_bytes, total_bytes >= (4ull << 20), t, true, &p);
-  const Kernel* bk = find_batch(h, l, p);
-  if (!bk) return MI355_BLIT_ERROR;
   BatchCopyArgs bc{h->records_dev, total_chunks, nullptr, l.waves_per_wg, l.n_waves, make_xcd_runs(p.grid, p.xcd_run)};
   h->last_plan = p;
 
@@ -986,6 +1135,27 @@ int mi355_aql_copy_rect_route(mi355_aql_t* h, const mi355_pitched_ptr_t* dst, co
   return MI355_BLIT_SUCCESS;
 }
 
+int mi355_aql_copy_sync(mi355_aql_t* h, void* dst, const void* src, size_t bytes, uint32_t route) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  // amd_blit_kernel.cpp:614-639: one blocking command at a time owns the signal
+  std::lock_guard<std::mutex> g(h->sync_lock);
+  hsa_signal_store_relaxed(h->sync_signal, 1);
+  const int rc = mi355_aql_copy_route(h, dst, src, bytes, route, nullptr, 0, h->sync_signal.handle);
+  if (rc != MI355_BLIT_SUCCESS) return rc;
+  // a copy of no bytes completes the signal from a barrier packet
+  return wait_signal(h, h->sync_signal);
+}
+
+int mi355_aql_fill32_sync(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dwords) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  // amd_blit_kernel.cpp:787-837
+  std::lock_guard<std::mutex> g(h->sync_lock);
+  hsa_signal_store_relaxed(h->sync_signal, 1);
+  const int rc = mi355_aql_fill32(h, ptr, value, num_dwords, nullptr, 0, h->sync_signal.handle);
+  if (rc != MI355_BLIT_SUCCESS) return rc;
+  return wait_signal(h, h->sync_signal);
+}
+
 int mi355_aql_wait_idle(mi355_aql_t* h) {
   if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   std::lock_guard<std::mutex> g(h->lock);
@@ -1001,7 +1171,7 @@ uint64_t mi355_aql_pending_bytes(mi355_aql_t* h) {
   const uint64_t known = h->known_complete.load();
   if (known > read) read = known;
   const uint64_t last = h->last_queued;
-  // If the last blit command has been run then the blit is empty.
+  // the queue has consumed the newest command's packet: nothing is pending
   if (read > last) return 0;
   for (uint64_t index = read; index <= last; ++index) {
     const BytesWritten& rec = h->bytes_written[index & h->queue_mask];

@@ -11,6 +11,7 @@
 #include <cstring>
 #include <mutex>
 
+#include "blit_plan.h"
 #include "mi355_blit_aql.h"
 
 namespace {
@@ -113,9 +114,12 @@ int bounced_copy(mi355_aql_t* h, void* dst, const void* src, size_t size, bool t
       if (i) hsa_signal_destroy(done[0]);
       return MI355_BLIT_ERROR_OUT_OF_RESOURCES;
     }
+  // Bounded waits that end with an error when the queue has reported one
+  // (mi355_aql_wait_signal): a piece whose submission failed, or whose queue
+  // died under it, must not leave this call waiting for its signal.
   auto wait = [&](int i) {
-    while (hsa_signal_wait_scacquire(done[i], HSA_SIGNAL_CONDITION_LT, 1, UINT64_MAX, HSA_WAIT_STATE_ACTIVE) >= 1) {
-    }
+    const int w = mi355_aql_wait_signal(h, done[i].handle);
+    if (w != MI355_BLIT_SUCCESS && rc == MI355_BLIT_SUCCESS) rc = w;
   };
   const char* s = static_cast<const char*>(src);
   char* d = static_cast<char*>(dst);
@@ -125,22 +129,31 @@ int bounced_copy(mi355_aql_t* h, void* dst, const void* src, size_t size, bool t
     const int b = piece & 1;
     const size_t len = size - off < half ? size - off : half;
     wait(b);  // the blit that used this half two pieces ago
+    if (rc != MI355_BLIT_SUCCESS) break;
     if (to_device) {
       std::memcpy(buf[b], s + off, len);
       hsa_signal_store_relaxed(done[b], 1);
       rc = mi355_aql_copy_route(h, d + off, buf[b], len, MI355_BLIT_ROUTE_HOST_TO_DEVICE, nullptr, 0, done[b].handle);
+      if (rc != MI355_BLIT_SUCCESS) hsa_signal_store_relaxed(done[b], 0);  // nothing was queued that would
     } else {
       hsa_signal_store_relaxed(done[b], 1);
       rc = mi355_aql_copy_route(h, buf[b], s + off, len, MI355_BLIT_ROUTE_DEVICE_TO_HOST, nullptr, 0, done[b].handle);
+      if (rc != MI355_BLIT_SUCCESS) {
+        hsa_signal_store_relaxed(done[b], 0);
+        break;
+      }
       // drain the previous piece while this one is in flight
       if (piece > 0) {
         wait(b ^ 1);
+        if (rc != MI355_BLIT_SUCCESS) break;
         std::memcpy(d + prev_off, buf[b ^ 1], prev_len);
       }
       prev_off = off;
       prev_len = len;
     }
   }
+  // On an error the signals of pieces still in flight are waited for all the
+  // same (bounded): the buffers are the engine's and the next call reuses them.
   wait(0);
   wait(1);
   if (!to_device && rc == MI355_BLIT_SUCCESS && piece > 0) std::memcpy(d + prev_off, buf[(piece - 1) & 1], prev_len);
@@ -183,9 +196,10 @@ int mi355_hsa_memory_copy(mi355_aql_t* h, void* dst, const void* src, size_t siz
     if (lock_dst.Lock(h, dst, size, &mapped) != MI355_BLIT_SUCCESS) return bounced_copy(h, dst, src, size, false);
     d = mapped;
   }
-  if ((rc = mi355_aql_copy_route(h, d, s, size, route_of(src_sys, dst_sys), nullptr, 0, 0)) != MI355_BLIT_SUCCESS)
-    return rc;
-  return mi355_aql_wait_idle(h);
+  // Waits for this copy's own completion signal, not for the queue to drain:
+  // commands other threads have parked behind unsatisfied dependencies do not
+  // hold it up (amd_blit_kernel.cpp:614-639).
+  return mi355_aql_copy_sync(h, d, s, size, route_of(src_sys, dst_sys));
 }
 
 int mi355_hsa_amd_memory_fill(mi355_aql_t* h, void* ptr, uint32_t value, size_t count) {
@@ -198,8 +212,7 @@ int mi355_hsa_amd_memory_fill(mi355_aql_t* h, void* ptr, uint32_t value, size_t 
   if (rc != MI355_BLIT_SUCCESS) return rc;
   // runtime.cpp:640-655: any GPU that can reach the memory fills it
   if (p.where == Where::kGpu || p.gpu_can_access) {
-    if ((rc = mi355_aql_fill32(h, ptr, value, count, nullptr, 0, 0)) != MI355_BLIT_SUCCESS) return rc;
-    return mi355_aql_wait_idle(h);
+    return mi355_aql_fill32_sync(h, ptr, value, count);
   }
   // host memory: the full pattern, dword by dword
   uint32_t* out = static_cast<uint32_t*>(ptr);
@@ -226,6 +239,14 @@ int mi355_hsa_amd_memory_async_copy(mi355_aql_t* h, void* dst, const void* src, 
     if (classify(h, src, size, &ps) == MI355_BLIT_SUCCESS && classify(h, dst, size, &pd) == MI355_BLIT_SUCCESS)
       route = route_of(ps.where != Where::kGpu, pd.where != Where::kGpu);
   }
+  // GetBlitObject (amd_gpu_agent.cpp:2379-2442): within the GPU the size
+  // decides between the SDMA-capable engine and the blit kernel; across the
+  // host link it is blits_[BlitHostToDev] / [BlitDevToHost], SDMA when the GPU
+  // has such engines.  The copy runs on this engine either way; the choice is
+  // only reported.
+  mi355_aql_note_reference_engine(
+      h, route == MI355_BLIT_ROUTE_DEVICE ? mi355::policy_same_gpu_engine(size, mi355::policy_force_sdma_size())
+                                          : static_cast<uint32_t>(MI355_ENGINE_SDMA));
   return mi355_aql_copy_route(h, dst, src, size, route, dep_signals, num_dep_signals, completion_signal);
 }
 
@@ -316,3 +337,12 @@ int mi355_hsa_amd_memory_async_copy_rect(mi355_aql_t* h, const mi355_pitched_ptr
 }
 
 }  // extern "C"
+
+extern "C" {
+// The engine-choice policy of mi355_blit.h, exported by this library too so
+// that a runtime linking only the AQL engine has it.
+uint64_t mi355_policy_force_sdma_size(void) { return mi355::policy_force_sdma_size(); }
+uint32_t mi355_policy_same_gpu_engine(uint64_t size, uint64_t force_sdma_size) {
+  return mi355::policy_same_gpu_engine(size, force_sdma_size);
+}
+}

@@ -377,6 +377,12 @@ int mi355_blit_plan_fill(uint64_t ptr, uint64_t num_dwords, uint32_t num_cus,
   return plan_fill(ptr, num_dwords, num_cus, tuning, out);
 }
 
+uint64_t mi355_policy_force_sdma_size(void) { return policy_force_sdma_size(); }
+
+uint32_t mi355_policy_same_gpu_engine(uint64_t size, uint64_t force_sdma_size) {
+  return policy_same_gpu_engine(size, force_sdma_size);
+}
+
 int mi355_blit_create(int device_ordinal, mi355_blit_t** out) {
   if (!out) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   *out = nullptr;

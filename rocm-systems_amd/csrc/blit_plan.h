@@ -11,6 +11,7 @@
 #define MI355_BLIT_PLAN_H_
 
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "mi355_blit.h"
 
@@ -106,6 +107,20 @@ constexpr SizeClass kCopyDeviceToHostClasses[] = {
     {0, 256, 1, 0, MI355_BLIT_STORE_SYSTEM_WT, 0},
     {4ull << 20, 256, 1, 1, MI355_BLIT_STORE_SYSTEM_WT, 0},
 };
+
+// The engine GpuAgent::GetBlitObject picks for an asynchronous copy within one
+// GPU (amd_gpu_agent.cpp:2390-2397) and the flag behind it (core/util/flag.h:
+// 206-207: atoi of HSA_FORCE_SDMA_SIZE, 1 MiB when unset or empty; atoi's int
+// becomes the size_t the reference compares with).
+inline uint64_t policy_force_sdma_size() {
+  const char* v = getenv("HSA_FORCE_SDMA_SIZE");
+  if (!v || !v[0]) return 1024 * 1024;
+  return static_cast<uint64_t>(static_cast<size_t>(atoi(v)));
+}
+
+inline uint32_t policy_same_gpu_engine(uint64_t size, uint64_t force_sdma_size) {
+  return size < force_sdma_size ? MI355_ENGINE_SDMA : MI355_ENGINE_BLIT_KERNEL;
+}
 
 inline bool valid_unroll(uint32_t u) { return u == 1 || u == 2 || u == 4; }
 

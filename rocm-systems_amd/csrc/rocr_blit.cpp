@@ -33,9 +33,10 @@ hsa_status_t to_hsa(int st) {
 
 }  // namespace
 
-BlitKernelGfx950::BlitKernelGfx950(core::Queue* queue, Completion completion)
+BlitKernelGfx950::BlitKernelGfx950(core::Queue* queue, Completion completion, int hip_device)
     : core::Blit(),
       queue_(queue),
+      hip_device_(hip_device),
       blit_(nullptr),
       completion_(completion),
       worker_busy_(false),
@@ -50,7 +51,7 @@ BlitKernelGfx950::~BlitKernelGfx950() {}
 hsa_status_t BlitKernelGfx950::Initialize(const core::Agent& agent) {
   hsa_status_t status = hsa_signal_create(1, 0, NULL, &completion_signal_);
   if (status != HSA_STATUS_SUCCESS) return status;
-  int st = mi355_blit_create(agent.gpu_ordinal(), &blit_);
+  int st = mi355_blit_create(hip_device_, &blit_);
   if (st != MI355_BLIT_SUCCESS) return to_hsa(st);
   if (agent.profiling_enabled()) return EnableProfiling(true);
   return HSA_STATUS_SUCCESS;

@@ -8,12 +8,13 @@
 // (core/runtime/amd_gpu_agent.cpp:749-759, 858-863).
 //
 // ROCr's internal headers are not installed with ROCm, so the three internal
-// types the interface mentions are given minimal stand-ins here: core::Agent
-// (only the GPU ordinal and the profiling flag are needed), core::Queue (an
-// opaque pointer, unused: commands go through a HIP stream inside the C ABI)
-// and core::Signal, a thin view of an hsa_signal_t driven through the public
-// hsa_signal_* API.  Inside a ROCr tree the stand-ins are replaced by the real
-// classes; core::Signal::Convert() yields the same hsa_signal_t handle there.
+// types the interface mentions are given minimal stand-ins here, each with
+// only members the real class has under the same name: core::Agent
+// (public_handle(), profiling_enabled(): core/inc/agent.h:310, 320),
+// core::Queue (public_handle(): core/inc/queue.h:373) and core::Signal, a thin
+// view of an hsa_signal_t driven through the public hsa_signal_* API
+// (Convert(): core/inc/signal.h).  Inside a ROCr tree the stand-ins are
+// deleted and the real headers included; nothing else changes.
 #ifndef MI355_ROCR_BLIT_H_
 #define MI355_ROCR_BLIT_H_
 
@@ -36,18 +37,26 @@ namespace core {
 
 class Agent {
  public:
-  explicit Agent(int gpu_ordinal, bool profiling = false)
-      : gpu_ordinal_(gpu_ordinal), profiling_enabled_(profiling) {}
+  explicit Agent(hsa_agent_t public_handle, bool profiling = false)
+      : public_handle_(public_handle), profiling_enabled_(profiling) {}
   virtual ~Agent() {}
-  int gpu_ordinal() const { return gpu_ordinal_; }
+  hsa_agent_t public_handle() const { return public_handle_; }
   bool profiling_enabled() const { return profiling_enabled_; }
 
  private:
-  int gpu_ordinal_;
+  hsa_agent_t public_handle_;
   bool profiling_enabled_;
 };
 
-class Queue;  // opaque
+class Queue {
+ public:
+  explicit Queue(hsa_queue_t* public_handle) : public_handle_(public_handle) {}
+  virtual ~Queue() {}
+  hsa_queue_t* public_handle() const { return public_handle_; }
+
+ private:
+  hsa_queue_t* public_handle_;
+};
 
 class Signal {
  public:
@@ -107,7 +116,11 @@ class BlitKernelGfx950 : public core::Blit {
     kHostCallback,  ///< by hsa_signal_subtract_screlease from a host callback
   };
 
-  explicit BlitKernelGfx950(core::Queue* queue, Completion completion = Completion::kDeviceSignal);
+  /// This engine submits through a HIP stream: it has no use for the queue,
+  /// and it is told which HIP device the agent is (the one thing HIP cannot
+  /// learn from an hsa_agent_t).
+  explicit BlitKernelGfx950(core::Queue* queue, Completion completion = Completion::kDeviceSignal,
+                            int hip_device = 0);
   ~BlitKernelGfx950() override;
 
   /// Binds to the agent's GPU, loads the kernels, creates the completion
@@ -165,6 +178,7 @@ class BlitKernelGfx950 : public core::Blit {
   static void OnComplete(void* user);
 
   core::Queue* queue_;
+  int hip_device_;
   mi355_blit* blit_;
   Completion completion_;
 
@@ -189,7 +203,12 @@ class BlitKernelGfx950 : public core::Blit {
 // dependencies become BARRIER_AND packets, out_signal is the dispatch packet's
 // completion signal and the packet processor decrements it, exactly as in
 // AMD::BlitKernel (core/runtime/amd_blit_kernel.cpp:641-785).  No submission
-// thread, no HIP.  This is the class that replaces AMD::BlitKernel in tree.
+// thread, no HIP.  This is the class that replaces AMD::BlitKernel in tree:
+// like it, the object borrows the queue it is constructed over (the agent's
+// utility queue, which other producers may share: core/inc/amd_blit_kernel.h:
+// 58-66, core/runtime/amd_gpu_agent.cpp:692-701, 749-759) and runs on the
+// agent Initialize() is given; it creates no queue and does not touch the
+// runtime's reference count.
 class BlitKernelGfx950Aql : public core::Blit {
  public:
   /// Which of GpuAgent's blits_ slots the object fills
@@ -227,6 +246,15 @@ class BlitKernelGfx950Aql : public core::Blit {
   uint64_t PendingBytes() override;
   void GangLeader(bool) override {}
   bool GangLeader() const override { return false; }
+
+  /// For the owner of the queue: its error callback forwards an asynchronous
+  /// queue error here (what core::Queue::DefaultErrorHandler stands for,
+  /// core/runtime/queue.cpp:52-59); blocking calls then return
+  /// HSA_STATUS_ERROR instead of waiting for a signal nobody will complete.
+  void ReportQueueError(hsa_status_t status);
+
+  /// The C ABI handle underneath (for the test driver).
+  mi355_aql* c_handle() const { return blit_; }
 
  private:
   core::Queue* queue_;

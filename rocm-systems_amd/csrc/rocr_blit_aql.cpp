@@ -36,7 +36,9 @@ BlitKernelGfx950Aql::~BlitKernelGfx950Aql() {}
 hsa_status_t BlitKernelGfx950Aql::Initialize(const core::Agent& agent) {
   hsa_status_t status = hsa_signal_create(1, 0, NULL, &completion_signal_);
   if (status != HSA_STATUS_SUCCESS) return status;
-  int st = mi355_aql_create(agent.gpu_ordinal(), &blit_);
+  // the queue handed to the constructor and the agent handed here, as they are
+  if (queue_ == nullptr) return HSA_STATUS_ERROR_INVALID_QUEUE;
+  int st = mi355_aql_create_on(agent.public_handle().handle, queue_->public_handle(), &blit_);
   if (st != MI355_BLIT_SUCCESS) return to_hsa(st);
   if (agent.profiling_enabled()) return EnableProfiling(true);
   return HSA_STATUS_SUCCESS;
@@ -64,11 +66,10 @@ hsa_status_t BlitKernelGfx950Aql::SubmitLinearCopyCommand(void* dst, const void*
   int st = mi355_aql_copy_route(blit_, dst, src, size, static_cast<uint32_t>(slot_), nullptr, 0,
                                 completion_signal_.handle);
   if (st != MI355_BLIT_SUCCESS) return to_hsa(st);
-  if (hsa_signal_wait_scacquire(completion_signal_, HSA_SIGNAL_CONDITION_LT, 1, uint64_t(-1),
-                                HSA_WAIT_STATE_ACTIVE) != 0) {
-    return HSA_STATUS_ERROR;
-  }
-  return HSA_STATUS_SUCCESS;
+  // Wait for the packet to finish: 0 is success, anything else (a negative
+  // value, or a queue that has reported an error and will never decrement
+  // the signal) is HSA_STATUS_ERROR (amd_blit_kernel.cpp:632-636).
+  return to_hsa(mi355_aql_wait_signal(blit_, completion_signal_.handle));
 }
 
 hsa_status_t BlitKernelGfx950Aql::SubmitLinearCopyCommand(void* dst, const void* src, size_t size,
@@ -90,11 +91,10 @@ hsa_status_t BlitKernelGfx950Aql::SubmitLinearFillCommand(void* ptr, uint32_t va
   hsa_signal_store_relaxed(completion_signal_, 1);
   int st = mi355_aql_fill32(blit_, ptr, value, count, nullptr, 0, completion_signal_.handle);
   if (st != MI355_BLIT_SUCCESS) return to_hsa(st);
-  if (hsa_signal_wait_scacquire(completion_signal_, HSA_SIGNAL_CONDITION_LT, 1, uint64_t(-1),
-                                HSA_WAIT_STATE_ACTIVE) != 0) {
-    return HSA_STATUS_ERROR;
-  }
-  return HSA_STATUS_SUCCESS;
+  // Wait for the packet to finish: 0 is success, anything else (a negative
+  // value, or a queue that has reported an error and will never decrement
+  // the signal) is HSA_STATUS_ERROR (amd_blit_kernel.cpp:632-636).
+  return to_hsa(mi355_aql_wait_signal(blit_, completion_signal_.handle));
 }
 
 hsa_status_t BlitKernelGfx950Aql::SubmitBatchCopyCommand(const void* descs, size_t n, bool descs_on_device,
@@ -140,6 +140,10 @@ hsa_status_t BlitKernelGfx950Aql::EnableProfiling(bool enable) {
   // amd_blit_kernel.cpp:839-842: the queue's profiling bit
   if (blit_ == nullptr) return HSA_STATUS_ERROR_NOT_INITIALIZED;
   return to_hsa(mi355_aql_enable_profiling(blit_, enable ? 1 : 0));
+}
+
+void BlitKernelGfx950Aql::ReportQueueError(hsa_status_t status) {
+  if (blit_ != nullptr) mi355_aql_report_queue_error(blit_, static_cast<int>(status));
 }
 
 uint64_t BlitKernelGfx950Aql::PendingBytes() { return blit_ ? mi355_aql_pending_bytes(blit_) : 0; }

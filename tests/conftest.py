@@ -150,18 +150,29 @@ def capi(pkg, torch_cuda):
     return pkg.capi
 
 
-@pytest.fixture(scope="session", params=["hip", "aql"])
+@pytest.fixture(scope="session", params=["hip", "aql", "aql_borrowed"])
 def blit(request, capi, pkg):
     """The engine under test, once per submission path: HIP stream launches
-    (mi355_blit.h) and hand-built AQL packets on an HSA queue (mi355_blit_aql.h).
-    Both run the same kernels."""
+    (mi355_blit.h), hand-built AQL packets on an HSA queue of the engine's own
+    (mi355_aql_create), and the same on a 64-packet queue the caller made, the
+    way ROCr hands its utility queue to a blit (mi355_aql_create_on).  All run
+    the same kernels."""
+    queue = None
     if request.param == "hip":
         b = capi.Blit(0)
     else:
         assert os.path.exists(pkg.aql.library_path()), "AQL library missing: no fallback"
-        b = pkg.aql.AqlBlit(0)
+        pkg.aql.load()
+        if request.param == "aql_borrowed":
+            queue = pkg.aql.BorrowedQueue(0, packets=64)
+            b = pkg.aql.AqlBlit(borrowed=queue)
+        else:
+            b = pkg.aql.AqlBlit(0)
     yield b
     b.close()
+    if queue is not None:
+        assert queue.errors == [], "the borrowed queue reported errors: %r" % queue.errors
+        queue.close()
 
 
 @pytest.fixture()

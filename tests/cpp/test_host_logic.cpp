@@ -15,9 +15,13 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
+#include <chrono>
+#include <thread>
 #include <vector>
 
 #include "../../oracle/blit_oracle.h"
+#include "aql_wait.h"
 #include "blit_batch_host.h"
 #include "blit_plan.h"
 #include "blit_rect.h"
@@ -412,9 +416,88 @@ void one_xcd_permutation() {
         "tuning of the run");
 }
 
+// The bounded wait of the AQL engine (csrc/aql_wait.h) without a GPU: the
+// slice is a callable, here a stand-in for hsa_signal_wait_scacquire on a
+// signal that nobody completes (it sleeps the slice out and reports 1).
+void wait_helper_cases() {
+  using clock = std::chrono::steady_clock;
+  int slices = 0;
+  auto never = [&](uint64_t ticks) -> int64_t {
+    ++slices;
+    std::this_thread::sleep_for(std::chrono::microseconds(ticks));
+    return 1;
+  };
+  // 1. the flag set from another thread ends a wait that is in progress
+  {
+    std::atomic<bool> error{false};
+    std::thread setter([&] {
+      std::this_thread::sleep_for(std::chrono::milliseconds(30));
+      error.store(true, std::memory_order_release);
+    });
+    const auto t0 = clock::now();
+    const int rc = wait_below_one(never, error, 1000);
+    const double ms = std::chrono::duration<double, std::milli>(clock::now() - t0).count();
+    setter.join();
+    CHECK(rc == kWaitError, "a wait on a dead queue returned 0x%x", rc);
+    CHECK(ms >= 25.0 && ms < 1000.0 && slices >= 5, "the wait took %.1f ms in %d slices", ms, slices);
+  }
+  // 2. a completed signal wins over the flag: the value is looked at first
+  {
+    std::atomic<bool> error{true};
+    CHECK(wait_below_one([](uint64_t) -> int64_t { return 0; }, error, 1000) == kWaitSuccess, "0 with the flag set");
+  }
+  // 3. a negative value is a failed command, whatever the flag says
+  {
+    std::atomic<bool> error{false};
+    CHECK(wait_below_one([](uint64_t) -> int64_t { return -1; }, error, 1000) == kWaitError, "negative value");
+  }
+  // 4. values above 0 keep the wait going until the signal gets there
+  {
+    std::atomic<bool> error{false};
+    int64_t v = 5;
+    int calls = 0;
+    const int rc = wait_below_one([&](uint64_t) -> int64_t { ++calls; return --v; }, error, 1000);
+    CHECK(rc == kWaitSuccess && calls == 5, "counted down in %d calls, rc 0x%x", calls, rc);
+  }
+  // 5. the flag already set and the signal never completing: one slice, then the error
+  {
+    std::atomic<bool> error{true};
+    slices = 0;
+    CHECK(wait_below_one(never, error, 100) == kWaitError && slices == 1, "%d slices", slices);
+  }
+}
+
+// The engine choice of GetBlitObject restated in csrc/blit_plan.h against the
+// oracle's restatement of the same lines (amd_gpu_agent.cpp:2390-2397).
+void engine_policy_cases() {
+  const uint64_t sizes[] = {0, 1, 4095, 4096, (128u << 10) - 1, 128u << 10, (1u << 20) - 1, 1u << 20, (1u << 20) + 1,
+                            1ull << 30, ~0ull};
+  const uint64_t flags[] = {0, 1, 128u << 10, 1u << 20, 1ull << 40, ~0ull};
+  for (uint64_t size : sizes)
+    for (uint64_t flag : flags) {
+      const bool blit = oracle_ref_same_gpu_uses_blit_kernel(size, flag) != 0;
+      CHECK(policy_same_gpu_engine(size, flag) == (blit ? uint32_t(MI355_ENGINE_BLIT_KERNEL) : uint32_t(MI355_ENGINE_SDMA)),
+            "size %" PRIu64 " flag %" PRIu64, size, flag);
+    }
+  // core/util/flag.h:206-207: unset or empty -> 1 MiB, otherwise atoi
+  unsetenv("HSA_FORCE_SDMA_SIZE");
+  CHECK(policy_force_sdma_size() == 1024 * 1024, "default");
+  setenv("HSA_FORCE_SDMA_SIZE", "", 1);
+  CHECK(policy_force_sdma_size() == 1024 * 1024, "empty");
+  setenv("HSA_FORCE_SDMA_SIZE", "131072", 1);
+  CHECK(policy_force_sdma_size() == 131072, "128 KiB");
+  setenv("HSA_FORCE_SDMA_SIZE", "0", 1);
+  CHECK(policy_force_sdma_size() == 0 && policy_same_gpu_engine(1, 0) == MI355_ENGINE_BLIT_KERNEL, "0: always the blit kernel");
+  setenv("HSA_FORCE_SDMA_SIZE", "-1", 1);  // atoi's int becomes a size_t: every size is below it
+  CHECK(policy_same_gpu_engine(1ull << 40, policy_force_sdma_size()) == MI355_ENGINE_SDMA, "-1");
+  unsetenv("HSA_FORCE_SDMA_SIZE");
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
+  wait_helper_cases();
+  engine_policy_cases();
   const long cases = argc > 1 ? std::atol(argv[1]) : 200000;
   for (long i = 0; i < cases; ++i) {
     one_copy_plan();

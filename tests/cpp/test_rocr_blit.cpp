@@ -21,6 +21,7 @@
 
 #include "../../oracle/blit_oracle.h"
 #include "mi355_blit.h"
+#include "mi355_blit_aql.h"
 #include "rocr_blit.h"
 
 using rocr::AMD::BlitKernelGfx950;
@@ -73,6 +74,27 @@ hsa_signal_t make_signal(hsa_signal_value_t v) {
   if (hsa_signal_create(v, 0, nullptr, &s) != HSA_STATUS_SUCCESS) s.handle = 0;
   return s;
 }
+
+// The agent's utility queue as GpuAgent makes it (amd_gpu_agent.cpp:692-701:
+// minAqlSize_ = 64 packets, HSA_QUEUE_TYPE_MULTI), with an error callback that
+// forwards to whichever engine runs on the queue, as its owner would.
+struct UtilityQueue {
+  hsa_queue_t* q = nullptr;
+  BlitKernelGfx950Aql* engine = nullptr;
+  static void on_error(hsa_status_t status, hsa_queue_t*, void* data) {
+    auto* self = static_cast<UtilityQueue*>(data);
+    std::printf("INFO queue error 0x%x\n", status);
+    if (self->engine) self->engine->ReportQueueError(status);
+  }
+  explicit UtilityQueue(hsa_agent_t gpu, uint32_t packets = 64) {
+    if (hsa_queue_create(gpu, packets, HSA_QUEUE_TYPE_MULTI, on_error, this, UINT32_MAX, UINT32_MAX, &q) !=
+        HSA_STATUS_SUCCESS)
+      q = nullptr;
+  }
+  ~UtilityQueue() {
+    if (q) hsa_queue_destroy(q);
+  }
+};
 
 bool wait_zero(hsa_signal_t s, hsa_wait_state_t state, uint64_t timeout_ms = 20000) {
   // timeout in the system timestamp's units; read its frequency
@@ -385,8 +407,12 @@ void test_host_link_slots(const rocr::core::Agent& agent) {
   REQUIRE(dev.p, "hipMalloc");
   std::vector<uint8_t> want(dev.n, kGuardByte), got;
   REQUIRE(dev.upload(want), "upload");
-  BlitKernelGfx950Aql h2d(nullptr, BlitKernelGfx950Aql::Slot::kHostToDev);
-  BlitKernelGfx950Aql d2h(nullptr, BlitKernelGfx950Aql::Slot::kDevToHost);
+  // both objects on one borrowed queue, as GpuAgent's blit_lambda puts them on queues_[QueueBlitOnly]
+  UtilityQueue uq(agent.public_handle());
+  REQUIRE(uq.q, "hsa_queue_create");
+  rocr::core::Queue queue(uq.q);
+  BlitKernelGfx950Aql h2d(&queue, BlitKernelGfx950Aql::Slot::kHostToDev);
+  BlitKernelGfx950Aql d2h(&queue, BlitKernelGfx950Aql::Slot::kDevToHost);
   REQUIRE(h2d.Initialize(agent) == HSA_STATUS_SUCCESS && d2h.Initialize(agent) == HSA_STATUS_SUCCESS, "Initialize");
   hsa_status_t st = h2d.SubmitLinearCopyCommand(dev.p + kGuard + 5, in + 3, n);
   REQUIRE(st == HSA_STATUS_SUCCESS, "host to device: status 0x%x", st);
@@ -440,6 +466,110 @@ void test_threads(Blit& blit) {
   }
   REQUIRE(dst.download(got), "download");
   REQUIRE(got == want, "bytes differ");
+  std::printf("PASS %s%s\n", name, g_suffix.c_str());
+}
+
+// The engine on a queue it shares with another producer: the driver writes
+// BARRIER_AND packets of its own between the blit's commands, by the same
+// protocol (atomic add on the write index, body, header, doorbell), each with a
+// completion signal of its own.  64 packet slots and some 400 packets: the ring
+// and the engine's kernarg ring, indexed by packet index, wrap several times.
+void write_own_barrier(hsa_queue_t* q, hsa_signal_t completion) {
+  const uint64_t index = hsa_queue_add_write_index_scacq_screl(q, 1);
+  while (index - hsa_queue_load_read_index_relaxed(q) >= q->size) std::this_thread::yield();
+  auto* ring = static_cast<hsa_barrier_and_packet_t*>(q->base_address);
+  hsa_barrier_and_packet_t* slot = &ring[index & (q->size - 1)];
+  hsa_barrier_and_packet_t pkt;
+  std::memset(&pkt, 0, sizeof(pkt));
+  pkt.completion_signal = completion;
+  std::memcpy(reinterpret_cast<uint8_t*>(slot) + 4, reinterpret_cast<uint8_t*>(&pkt) + 4, sizeof(pkt) - 4);
+  const uint16_t header = (HSA_PACKET_TYPE_BARRIER_AND << HSA_PACKET_HEADER_TYPE) |
+                          (HSA_FENCE_SCOPE_NONE << HSA_PACKET_HEADER_SCACQUIRE_FENCE_SCOPE) |
+                          (HSA_FENCE_SCOPE_NONE << HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE);
+  __atomic_store_n(reinterpret_cast<uint32_t*>(slot), static_cast<uint32_t>(header), __ATOMIC_RELEASE);
+  hsa_signal_store_screlease(q->doorbell_signal, static_cast<hsa_signal_value_t>(index));
+}
+
+void test_shared_queue(BlitKernelGfx950Aql& blit, hsa_queue_t* q) {
+  const char* name = "shared_queue_interleaved_packets";
+  REQUIRE(q->size == 64, "the case is meant for the 64-packet utility queue, got %u", q->size);
+  const int kRounds = 96;
+  const size_t n = (96u << 10) + 7, region = ((n + 2 * kGuard + 255) / 256) * 256;
+  std::vector<uint8_t> src_h = seeded(n + 64, 0xB1170088);
+  DeviceBuf src(src_h.size()), dst(region * kRounds);
+  REQUIRE(src.p && dst.p, "hipMalloc");
+  REQUIRE(src.upload(src_h), "upload");
+  std::vector<uint8_t> want(dst.n, kGuardByte), got;
+  REQUIRE(dst.upload(want), "upload");
+  hsa_signal_t mine = make_signal(3 * kRounds), copies = make_signal(kRounds);
+  REQUIRE(mine.handle && copies.handle, "signal");
+  Signal out(copies);
+  std::vector<Signal*> none, gang;
+  for (int i = 0; i < kRounds; ++i) {
+    write_own_barrier(q, mine);
+    uint8_t* d = dst.p + i * region + kGuard;
+    hsa_status_t st;
+    if (i % 3 == 2) {
+      // a blocking fill between the asynchronous copies
+      st = blit.SubmitLinearFillCommand(d, 0x01010101u * (i + 1), n / 4);
+      oracle_fill32(want.data() + i * region + kGuard, 0x01010101u * (i + 1), n / 4);
+      hsa_signal_subtract_screlease(copies, 1);
+    } else {
+      st = blit.SubmitLinearCopyCommand(d + (i & 15), src.p + (i % 7), n, none, out, gang);
+      oracle_copy(want.data() + i * region + kGuard + (i & 15), src_h.data() + (i % 7), n);
+    }
+    REQUIRE(st == HSA_STATUS_SUCCESS, "round %d status 0x%x", i, st);
+    write_own_barrier(q, mine);
+    write_own_barrier(q, mine);
+  }
+  REQUIRE(wait_zero(copies, HSA_WAIT_STATE_ACTIVE), "the blit's commands never completed");
+  REQUIRE(wait_zero(mine, HSA_WAIT_STATE_ACTIVE), "the driver's own packets never completed: %ld left",
+          (long)hsa_signal_load_relaxed(mine));
+  REQUIRE(dst.download(got), "download");
+  REQUIRE(got == want, "bytes differ");
+  uint64_t pending = 1;
+  for (int i = 0; i < 1000 && pending; ++i) {
+    pending = blit.PendingBytes();
+    if (pending) std::this_thread::sleep_for(std::chrono::milliseconds(1));
+  }
+  REQUIRE(pending == 0, "PendingBytes stuck at %llu", (unsigned long long)pending);
+  hsa_signal_destroy(mine);
+  hsa_signal_destroy(copies);
+  std::printf("PASS %s%s\n", name, g_suffix.c_str());
+}
+
+// A queue that has stopped on an error never completes a signal.  The error is
+// forced from the host (the owner's callback forwarding it, without any fault
+// on the GPU): a wait that is already in progress must end with
+// HSA_STATUS_ERROR, and later blocking calls must answer it at once.
+void test_queue_error_ends_waits(const rocr::core::Agent& agent) {
+  const char* name = "queue_error_ends_waits";
+  UtilityQueue uq(agent.public_handle());
+  REQUIRE(uq.q, "hsa_queue_create");
+  rocr::core::Queue queue(uq.q);
+  BlitKernelGfx950Aql blit(&queue);
+  REQUIRE(blit.Initialize(agent) == HSA_STATUS_SUCCESS, "Initialize");
+  DeviceBuf a(4096), b(4096);
+  REQUIRE(a.p && b.p, "hipMalloc");
+  REQUIRE(blit.SubmitLinearCopyCommand(b.p, a.p, 4096) == HSA_STATUS_SUCCESS, "a copy on the healthy queue");
+  hsa_signal_t never = make_signal(1);
+  REQUIRE(never.handle, "signal");
+  std::thread reporter([&] {
+    std::this_thread::sleep_for(std::chrono::milliseconds(50));
+    blit.ReportQueueError(HSA_STATUS_ERROR_EXCEPTION);
+  });
+  const auto t0 = std::chrono::steady_clock::now();
+  const int st = mi355_aql_wait_signal(blit.c_handle(), never.handle);
+  const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+  reporter.join();
+  REQUIRE(st == HSA_STATUS_ERROR, "wait on a signal nobody completes returned 0x%x", st);
+  REQUIRE(ms >= 40.0 && ms < 2000.0, "the wait took %.1f ms", ms);
+  REQUIRE(blit.SubmitLinearCopyCommand(b.p, a.p, 4096) == HSA_STATUS_ERROR, "blocking copy on a failed queue");
+  REQUIRE(blit.SubmitLinearFillCommand(b.p, 1, 16) == HSA_STATUS_ERROR, "blocking fill on a failed queue");
+  hsa_signal_destroy(never);
+  // the queue itself is healthy (the error was only reported): Destroy may
+  // not wait on it, and does not
+  REQUIRE(blit.Destroy(agent) == HSA_STATUS_SUCCESS, "Destroy");
   std::printf("PASS %s%s\n", name, g_suffix.c_str());
 }
 
@@ -512,7 +642,8 @@ int main(int argc, char** argv) {
     for (const char* engine : {"_hip", "_aql"})
       for (const char* c : cases) std::printf("%s%s\n", c, engine);
     std::printf("async_copy_blocked_wait_hip_callback\nchain_a_to_b_to_c_hip_callback\n"
-                "profiling_timestamps_aql\ncopy_rect_with_signal_aql\nhost_link_slots_aql\n");
+                "profiling_timestamps_aql\ncopy_rect_with_signal_aql\nhost_link_slots_aql\n"
+                "shared_queue_interleaved_packets_aql\nqueue_error_ends_waits_aql\n");
     return 0;
   }
   if (hsa_init() != HSA_STATUS_SUCCESS) {
@@ -524,7 +655,20 @@ int main(int argc, char** argv) {
     std::printf("FAIL setup: no HIP device\n");
     return 2;
   }
-  rocr::core::Agent agent(0);
+  hsa_agent_t gpu{0};
+  hsa_iterate_agents(first_gpu_cb, &gpu);
+  if (!gpu.handle) {
+    std::printf("FAIL setup: no GPU agent\n");
+    return 2;
+  }
+  // what GpuAgent hands to CreateBlitKernel: itself and its utility queue
+  rocr::core::Agent agent(gpu);
+  UtilityQueue utility(gpu);
+  if (!utility.q) {
+    std::printf("FAIL setup: hsa_queue_create\n");
+    return 2;
+  }
+  rocr::core::Queue utility_queue(utility.q);
   {
     // the host-callback completion mode of the HIP-stream engine
     g_suffix = "_hip_callback";
@@ -555,7 +699,8 @@ int main(int argc, char** argv) {
       blit = b;
     } else {
       g_suffix = "_aql";
-      auto* b = new BlitKernelGfx950Aql(nullptr);
+      auto* b = new BlitKernelGfx950Aql(&utility_queue);
+      utility.engine = b;
       init = b->Initialize(agent);
       batch = [b](const void* d, size_t n, bool on_device, uint64_t bound, std::vector<Signal*>& deps, Signal& out) {
         return b->SubmitBatchCopyCommand(d, n, on_device, deps, out, bound);
@@ -579,7 +724,9 @@ int main(int argc, char** argv) {
     if (engine == 1) {
       test_profiling_timestamps(*blit);
       test_copy_rect(*static_cast<BlitKernelGfx950Aql*>(blit));
+      test_shared_queue(*static_cast<BlitKernelGfx950Aql*>(blit), utility.q);
       test_host_link_slots(agent);
+      test_queue_error_ends_waits(agent);
     }
     latency_report(*blit, engine == 0 ? "hip_device_signal" : "aql");
     hsa_status_t st = blit->Destroy(agent);
@@ -590,6 +737,7 @@ int main(int argc, char** argv) {
       std::printf("PASS destroy%s\n", g_suffix.c_str());
     }
     delete blit;
+    utility.engine = nullptr;
   }
   hsa_shut_down();
   std::printf("%s (%d failures)\n", g_failures ? "FAILED" : "OK", g_failures);

@@ -24,7 +24,7 @@ def capi_host(pkg):
 
 def test_library_exports_every_declared_symbol(capi_host):
     header = open(os.path.join(ROOT, "include", "mi355_blit.h")).read()
-    declared = set(re.findall(r"\b(mi355_blit_[a-z0-9_]+)\s*\(", header))
+    declared = set(re.findall(r"\b(mi355_(?:blit|policy)_[a-z0-9_]+)\s*\(", header))
     assert declared, "no declarations found"
     lib = C.CDLL(capi_host.library_path())
     for name in sorted(declared):
@@ -42,7 +42,7 @@ def test_abi_version_and_status_strings(capi_host):
 
 
 def test_struct_layouts_match_header(capi_host):
-    assert C.sizeof(capi_host.Plan) == 8 * 4 + 3 * 8 + 2 * 4
+    assert C.sizeof(capi_host.Plan) == 8 * 4 + 3 * 8 + 4 * 4
     assert capi_host.Plan.lead_vecs.offset == 28
     assert C.sizeof(capi_host.Tuning) == 32
     assert C.sizeof(capi_host.Desc) == 24
@@ -228,6 +228,24 @@ def test_aql_library_exports_every_declared_symbol(pkg):
     for name in sorted(declared):
         assert hasattr(lib, name), "library does not export %s" % name
     assert declared == set(pkg.aql.SIGNATURES)
+    # the engine-choice policy of mi355_blit.h is exported by this library too
+    assert hasattr(lib, "mi355_policy_same_gpu_engine") and hasattr(lib, "mi355_policy_force_sdma_size")
+
+
+def test_engine_choice_policy_matches_the_reference(capi_host, oracle, monkeypatch):
+    """GetBlitObject's choice for a copy within one GPU (amd_gpu_agent.cpp:2390-2397)
+    and the flag behind it (flag.h:206-207), against the oracle's restatement."""
+    lib = capi_host.load()
+    for size in (0, 1, 4096, (128 << 10) - 1, 128 << 10, (1 << 20) - 1, 1 << 20, 1 << 30):
+        for flag in (0, 1, 128 << 10, 1 << 20, 1 << 40):
+            want = capi_host.ENGINE_BLIT_KERNEL if oracle.oracle_ref_same_gpu_uses_blit_kernel(size, flag) else capi_host.ENGINE_SDMA
+            assert lib.mi355_policy_same_gpu_engine(size, flag) == want, (size, flag)
+    monkeypatch.delenv("HSA_FORCE_SDMA_SIZE", raising=False)
+    assert lib.mi355_policy_force_sdma_size() == 1 << 20
+    monkeypatch.setenv("HSA_FORCE_SDMA_SIZE", "131072")
+    assert lib.mi355_policy_force_sdma_size() == 131072
+    monkeypatch.setenv("HSA_FORCE_SDMA_SIZE", "")
+    assert lib.mi355_policy_force_sdma_size() == 1 << 20
 
 
 def test_aql_code_object_holds_every_kernel_variant(pkg):

@@ -65,6 +65,119 @@ def test_memory_copy_all_directions(eng, oracle, rand, torch_cuda, n):
     assert np.array_equal(final, want_final)
 
 
+def test_memory_copy_host_to_host_256_mib(eng, oracle, rand):
+    """The reference's own CPU-runnable configuration: 256 MiB of seeded bytes,
+    source and destination 64-byte aligned host memory, through the
+    hsa_memory_copy stand-in (one memcpy on the calling thread,
+    runtime.cpp:507-510); every byte and the guards against the oracle."""
+    n = 256 * MIB
+    raw_src, raw_dst = rand(n + 64, 0xB1170000), _host(n + 2 * GUARD + 64)
+    s_off = (-raw_src.ctypes.data) % 64
+    d_off = (-raw_dst.ctypes.data) % 64 + GUARD
+    assert (raw_src.ctypes.data + s_off) % 64 == 0 and (raw_dst.ctypes.data + d_off) % 64 == 0
+    assert eng.hsa_memory_copy(raw_dst.ctypes.data + d_off, raw_src.ctypes.data + s_off, n) == 0
+    want = _host(n + 2 * GUARD + 64)
+    oracle.oracle_copy(want.ctypes.data + d_off, raw_src.ctypes.data + s_off, n)
+    assert np.array_equal(raw_dst, want)
+
+
+def test_blocking_forms_and_bounded_wait(eng, oracle, rand, signals, torch_cuda):
+    """The blocking copy and fill (their own completion signal, armed and waited
+    for under the engine's blocking-call lock, amd_blit_kernel.cpp:614-639,
+    787-837) and mi355_aql_wait_signal on a command parked behind a dependency
+    that is satisfied later."""
+    torch = torch_cuda
+    n = MIB + 5
+    payload = rand(n, 0xB1170007)
+    src = torch.from_numpy(payload).to("cuda:0")
+    parked = torch.full((n,), 0xEE, dtype=torch.uint8, device="cuda:0")
+    dst = torch.full((n + 2 * GUARD,), 0xEE, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    assert eng.copy_sync(dst.data_ptr() + GUARD, src.data_ptr(), n) == 0
+    assert eng.fill32_sync(dst.data_ptr() + GUARD, 0x01020304, 16) == 0
+    assert eng.copy_sync(dst.data_ptr() + GUARD + 64, src.data_ptr() + 64, 1000) == 0
+    assert eng.copy_sync(dst.data_ptr(), src.data_ptr(), 0) == 0          # nothing to move: still completes
+    assert eng.fill32_sync(dst.data_ptr(), 7, 0) == 0
+    assert eng.copy_sync(None, src.data_ptr(), 8) == 0x1001
+    assert eng.fill32_sync(dst.data_ptr() + 2, 7, 4) == 0x1001
+    want = _host(n + 2 * GUARD)
+    oracle.oracle_copy(want.ctypes.data + GUARD, payload.ctypes.data, n)
+    oracle.oracle_fill32(want.ctypes.data + GUARD, 0x01020304, 16)
+    oracle.oracle_copy(want.ctypes.data + GUARD + 64, payload.ctypes.data + 64, 1000)
+    assert np.array_equal(dst.cpu().numpy(), want)
+    dep, done = signals.create(1), signals.create(1)
+    assert eng.copy(parked.data_ptr(), src.data_ptr(), n, deps=[dep], completion=done) == 0
+    assert signals.load(done) == 1
+    signals.store(dep, 0)
+    assert eng.wait_signal(done) == 0
+    assert np.array_equal(parked.cpu().numpy(), payload)
+    signals.destroy(dep)
+    signals.destroy(done)
+
+
+def test_async_copy_reports_the_reference_engine(eng, pkg, signals, torch_cuda, monkeypatch):
+    """Which engine GetBlitObject would have picked (amd_gpu_agent.cpp:2379-2398)
+    is reported beside the launch: SDMA below HSA_FORCE_SDMA_SIZE, the blit
+    kernel from there on, SDMA across the host link."""
+    torch = torch_cuda
+    capi = pkg.capi
+    a = torch.zeros(4 * MIB, dtype=torch.uint8, device="cuda:0")
+    b = torch.zeros(4 * MIB, dtype=torch.uint8, device="cuda:0")
+    pinned = torch.zeros(4 * MIB, dtype=torch.uint8, pin_memory=True)
+    torch.cuda.synchronize()
+    done = signals.create(1)
+
+    def engine_of(dst, src, n):
+        signals.store(done, 1)
+        assert eng.hsa_amd_memory_async_copy(dst, src, n, completion=done) == 0
+        assert eng.wait_signal(done) == 0
+        return eng.last_plan().reference_engine
+
+    monkeypatch.delenv("HSA_FORCE_SDMA_SIZE", raising=False)
+    assert engine_of(b.data_ptr(), a.data_ptr(), 4096) == capi.ENGINE_SDMA
+    assert engine_of(b.data_ptr(), a.data_ptr(), MIB - 1) == capi.ENGINE_SDMA
+    assert engine_of(b.data_ptr(), a.data_ptr(), MIB) == capi.ENGINE_BLIT_KERNEL
+    assert engine_of(b.data_ptr(), pinned.data_ptr(), 2 * MIB) == capi.ENGINE_SDMA
+    monkeypatch.setenv("HSA_FORCE_SDMA_SIZE", str(128 << 10))
+    assert engine_of(b.data_ptr(), a.data_ptr(), (128 << 10) - 1) == capi.ENGINE_SDMA
+    assert engine_of(b.data_ptr(), a.data_ptr(), 128 << 10) == capi.ENGINE_BLIT_KERNEL
+    monkeypatch.setenv("HSA_FORCE_SDMA_SIZE", "0")
+    assert engine_of(b.data_ptr(), a.data_ptr(), 1) == capi.ENGINE_BLIT_KERNEL
+    signals.destroy(done)
+
+
+def test_packet_log(pkg, signals, torch_cuda, monkeypatch, capfd):
+    """MI355_BLIT_LOG_PKTS=1: one line per barrier and dispatch packet with the
+    fields the reference logs (amd_blit_kernel.cpp:681-702, 903-923)."""
+    import re
+    torch = torch_cuda
+    a = torch.zeros(MIB, dtype=torch.uint8, device="cuda:0")
+    b = torch.zeros(MIB, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    monkeypatch.setenv("MI355_BLIT_LOG_PKTS", "1")
+    e = pkg.aql.AqlBlit(0)
+    try:
+        dep, done = signals.create(0), signals.create(1)
+        capfd.readouterr()
+        assert e.copy(b.data_ptr(), a.data_ptr(), MIB, deps=[dep], completion=done) == 0
+        assert e.wait_signal(done) == 0
+        err = capfd.readouterr().err
+        signals.destroy(dep)
+        signals.destroy(done)
+    finally:
+        e.close()
+    barrier = re.search(r"HWq=0x[0-9a-f]+, id=\d+, Barrier Header = 0x[0-9a-f]+ \(type=3, barrier=0, acquire=0, release=0\), "
+                        r"dep_signal=\[0x%x 0x0 0x0 0x0 0x0\], completion_signal=0x0 rptr=\d+, wptr=(\d+)" % dep, err)
+    assert barrier, err
+    dispatch = re.search(r"Dispatch Header = 0x[0-9a-f]+ \(type=2, barrier=1, acquire=2, release=2\), setup=1, "
+                         r"grid=\[(\d+), 1, 1\], workgroup=\[(\d+), 1, 1\], private_seg_size=0, group_seg_size=0, "
+                         r"kernel_obj=0x[0-9a-f]+, kernarg_address=0x[0-9a-f]+, completion_signal=0x%x rptr=\d+, wptr=(\d+)"
+                         % done, err)
+    assert dispatch, err
+    assert int(dispatch.group(3)) == int(barrier.group(1)) + 1
+    assert int(dispatch.group(1)) % int(dispatch.group(2)) == 0
+
+
 def test_memory_copy_pinned_host(eng, oracle, rand, torch_cuda):
     """Host memory allocated through the runtime (pinned) needs no locking."""
     torch = torch_cuda

@@ -194,19 +194,18 @@ def _log_uniform_lengths(rng, k, max_bytes):
 
 
 def test_misaligned_all_256_offset_pairs(capi, blit, oracle, arenas):
-    """Every (src & 15, dst & 15) pair, 8 log-uniform lengths 1 B .. 64 MiB each
-    (most draws are capped at 4 MiB to keep the host compare short; each pair
-    class still meets lengths up to 64 MiB), guards checked."""
+    """Every (src & 15, dst & 15) pair: 8 lengths drawn log-uniformly from 1 B to
+    64 MiB and used as drawn, and one more drawn log-uniformly from 4 MiB to
+    64 MiB, so that every pair meets the streaming shapes of the heuristics
+    too; destination window and guards compared with the oracle every time."""
     src, src_host, dst = arenas
     rng = np.random.default_rng(0xB1170004)
     for so in range(16):
         for do in range(16):
-            lens = _log_uniform_lengths(rng, 8, 64 * MIB)
-            big_ok = (so * 16 + do) % 37 == 0
+            lens = list(_log_uniform_lengths(rng, 8, 64 * MIB))
+            lens.append(int(4 * MIB * 16.0 ** rng.random()))
             for n in lens:
-                n = int(n)
-                if n > 4 * MIB and not big_ok:
-                    n = int(n % (4 * MIB)) + 1
+                n = min(int(n), 64 * MIB)
                 run_copy_case(capi, blit, oracle, src, src_host, dst, 512 + so, GUARD + 16 + do, n)
                 p = blit.last_plan()
                 assert p.byte_shift == (so - do) % 4
@@ -361,9 +360,9 @@ def test_fill_offsets_and_odd_counts(capi, blit, oracle, arenas):
             run_fill_case(capi, blit, oracle, dst, GUARD + off, count, FILL_VALUE ^ count)
 
 
-def test_fill_1gib_headline(capi, blit, oracle, torch_cuda):
+@pytest.mark.parametrize("count", [1 << 26, 1 << 28])  # 256 MiB (a point of the sweep), 1 GiB (the headline)
+def test_fill_large_full_compare(capi, blit, oracle, torch_cuda, count):
     torch = torch_cuda
-    count = 1 << 28
     dst = Arena(torch, 4 * count + 2 * GUARD, fill=GUARD_BYTE)
     # pre-fill with the complement so that an unwritten dword shows
     dst.view[GUARD:GUARD + 4 * count].view(torch.int32).fill_(~FILL_VALUE & 0x7fffffff)
@@ -854,6 +853,78 @@ def test_batch_65536_copies(capi, blit, oracle, rand, torch_cuda):
         check_ok(capi, submit(), "copy_batch, device-resident descriptors")
         check_ok(capi, blit.synchronize(), "synchronize")
         assert np.array_equal(dst.host(), want)
+
+
+@pytest.fixture(scope="module")
+def batch_arena(capi, oracle, rand, torch_cuda):
+    """The benchmark's batch in its arena: 65,536 copies, 64 B .. 256 KiB
+    log-uniform, byte offsets 0..15 on both sides, regions spread by
+    bench.batch_layout over an 8 GiB source and an 8 GiB destination, so that
+    descriptors lie more than 4 GiB apart and the copies are sparse in memory.
+    Yields the descriptors and the whole destination as the oracle leaves it
+    (every copy by oracle_copy into a buffer of guard bytes), resident on the
+    device for the comparisons."""
+    import bench
+    torch = torch_cuda
+    n, arena = 65536, 8 << 30
+    lens, so, do, offs, stride = bench.batch_layout(n, arena)
+    assert int(offs[-1] + stride[-1]) <= arena and int(offs[-1]) > (7 << 30)
+    block = rand(64 * MIB, 0xB1170005)            # the arena's source bytes: this block, repeated
+    src = torch.empty(arena + 512, dtype=torch.uint8, device="cuda:0")
+    dst = torch.empty(arena + 512, dtype=torch.uint8, device="cuda:0")
+    s_sh, d_sh = (-src.data_ptr()) % 256, (-dst.data_ptr()) % 256
+    block_dev = torch.from_numpy(block).to("cuda:0")
+    for lo in range(0, arena, block.size):
+        src[s_sh + lo:s_sh + lo + block.size].copy_(block_dev)
+    del block_dev
+    # what the oracle leaves in the destination, built and uploaded 1 GiB at a time
+    want_dev = torch.empty(arena, dtype=torch.uint8, device="cuda:0")
+    part = 1 << 30
+    two = np.concatenate([block, block])          # a copy's source bytes may wrap around the block's end
+    begin, end = offs + do, offs + do + lens      # destination ranges, ascending and disjoint
+    for k in range(arena // part):
+        lo, hi = k * part, (k + 1) * part
+        want = np.full(part, GUARD_BYTE, dtype=np.uint8)
+        # the copies that have bytes in [lo, hi); one that straddles a boundary gives each side its share
+        for i in range(int(np.searchsorted(end, lo, side="right")), int(np.searchsorted(begin, hi, side="left"))):
+            a, b = max(int(begin[i]), lo), min(int(end[i]), hi)
+            s_at = (int(offs[i] + so[i]) + a - int(begin[i])) % block.size
+            oracle.oracle_copy(want.ctypes.data + a - lo, two.ctypes.data + s_at, b - a)
+        want_dev[lo:hi].copy_(torch.from_numpy(want))
+    descs = (capi.Desc * n)()
+    for i in range(n):
+        descs[i].dst = dst.data_ptr() + d_sh + int(offs[i] + do[i])
+        descs[i].src = src.data_ptr() + s_sh + int(offs[i] + so[i])
+        descs[i].bytes = int(lens[i])
+    torch.cuda.synchronize()
+    yield descs, n, int(lens.sum()), dst[d_sh:d_sh + arena], want_dev
+    del src, dst, want_dev
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("descriptors", ["host", "device", "device_bounded"])
+def test_batch_65536_copies_in_the_16_gib_arena(capi, blit, batch_arena, torch_cuda, descriptors):
+    """Every byte of the 8 GiB destination -- all 65,536 copies, their guard
+    bands and everything between them -- against what the oracle leaves."""
+    torch = torch_cuda
+    descs, n, total, dst, want = batch_arena
+    dst.fill_(GUARD_BYTE)
+    dev = _to_device(torch, descs) if descriptors != "host" else None
+    torch.cuda.synchronize()
+    if descriptors == "host":
+        st = blit.copy_batch(descs, n)
+    elif descriptors == "device":
+        st = blit.copy_batch(dev.data_ptr(), n, on_device=True)
+    else:
+        st = blit.copy_batch_bounded(dev.data_ptr(), n, total)
+    check_ok(capi, st, "copy_batch")
+    check_ok(capi, blit.synchronize(), "synchronize")
+    if not torch.equal(dst, want):
+        part = 1 << 28
+        for lo in range(0, dst.numel(), part):
+            bad = torch.nonzero(dst[lo:lo + part] != want[lo:lo + part])
+            if bad.numel():
+                raise AssertionError("destination differs from the oracle's, first at byte %d" % (lo + int(bad[0])))
 
 
 def test_batch_back_to_back_reuses_staging(capi, blit, oracle, arenas):

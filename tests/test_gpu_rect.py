@@ -138,6 +138,31 @@ def test_rect_random_narrow_rows(capi, fresh_tuning, oracle, rand, seed):
                   int(rng.integers(0, 256)), int(rng.integers(0, 256)), seed=0x7A220000 + seed)
 
 
+@pytest.mark.parametrize("width", [1101, 1337, 1600, 1999, 2047])
+def test_rect_ragged_rows_wider_than_a_wave(capi, fresh_tuning, oracle, rand, width):
+    """Ragged rows of 1101..2047 bytes go to the slot kernel with up to 128
+    lanes per row, where a wave holds less than a row and a lane's row within
+    the wave is 0 or 1: odd x offsets and pitches, hundreds of rows in 3 layers,
+    single waves and large workgroups, capped grids (waves striding over the
+    slots) and launches permuted in XCD runs."""
+    blit = fresh_tuning
+    rows = 211
+    sshape, dshape = (3, rows + 9, width + 333), (3, rows + 4, 2 * width + 77)
+    ext, so, do = (width, rows, 3), (7 + width % 5, 5, 0), (width - 3, 2, 0)
+    for wg, max_grid, xcd_run in ((64, 0, 1), (256, 0, 1), (1024, 0, 1), (64, 1, 1), (256, 5, 1), (64, 0, 3),
+                                  (256, 0, 2)):
+        blit.set_tuning(wg_size=wg, max_grid=max_grid, xcd_run=xcd_run)
+        p = run_rect_case(capi, blit, oracle, rand, sshape, dshape, ext, so, do, 5, 130 + (width & 15),
+                          seed=0x7A22F000 + width)
+        assert p.kernel == capi.KERNEL_COPY_RECT and p.wg_size == wg
+    st, plan = capi.plan_rect((1 << 40, dshape[2], dshape[1] * dshape[2]), do, (1 << 41, sshape[2], sshape[1] * sshape[2]),
+                              so, ext, None)
+    assert st == capi.SUCCESS
+    if width <= 2000:  # 2047 bytes can touch 129 slots: the first width that goes to the unit kernel
+        assert 64 < plan.lanes_per_row <= 128 and plan.slots == 0, (
+            "the case is meant for the slot kernel with more than a wave per row", plan.lanes_per_row, plan.slots)
+
+
 @pytest.mark.parametrize("xcd_run", [2, 3, 36])
 def test_rect_permuted_launches_are_exact(capi, fresh_tuning, oracle, rand, xcd_run):
     """Both region kernels with their workgroups dealt to the XCDs in runs: a

@@ -139,7 +139,9 @@ typedef struct {
   uint32_t nt_load;
   uint32_t store_policy;
   uint32_t xcd_run;
-  uint32_t reserved[2];
+  uint32_t batch_prefetch; /* batched copies: 0 = heuristic, 1 = no record prefetch,
+                              N > 1 = touch the record N workgroups ahead */
+  uint32_t reserved;
 } mi355_blit_tuning_t;
 
 /* One element of a batched submission.  No counterpart in the reference. */

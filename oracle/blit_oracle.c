@@ -6,6 +6,7 @@
 #include "blit_oracle.h"
 
 #include <pthread.h>
+#include <sched.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -115,6 +116,165 @@ void oracle_copy_mt(void* dst, const void* src, size_t size, int nthreads) {
 
 void oracle_fill32_mt(void* ptr, uint32_t value, size_t count, int nthreads) {
   run_mt((uint8_t*)ptr, NULL, count * 4, value, 1, nthreads);
+}
+
+/* ------------------------------------------------------------------------ */
+/* The host path on T cores, for the benchmark's CPU baseline: worker threads  */
+/* that live as long as the pool, each pinned to one CPU of the process's      */
+/* affinity mask and owning one contiguous slice (a multiple of 64 bytes) of   */
+/* every buffer, which it also touches first, so that its pages sit on its     */
+/* own memory node.                                                            */
+/* ------------------------------------------------------------------------ */
+
+enum { POOL_JOB_NONE = 0, POOL_JOB_COPY, POOL_JOB_FILL, POOL_JOB_TOUCH, POOL_JOB_EXIT };
+
+struct oracle_pool {
+  int nthreads;
+  int pinned; /* threads that could be pinned */
+  pthread_t tid[256];
+  pthread_mutex_t lock;
+  pthread_cond_t go, done;
+  unsigned long generation; /* bumped for every job */
+  int job;
+  int remaining;
+  uint8_t* dst;
+  const uint8_t* src;
+  size_t size;
+  uint32_t value;
+};
+
+typedef struct {
+  struct oracle_pool* pool;
+  int index;
+} pool_arg_t;
+
+/* Slice `index` of `size` bytes cut for n threads. */
+static void pool_slice(size_t size, int n, int index, size_t* off, size_t* len) {
+  size_t per = ((size / (size_t)n) + 63) & ~(size_t)63;
+  size_t lo = per * (size_t)index;
+  if (lo > size) lo = size;
+  size_t hi = (index == n - 1) ? size : lo + per;
+  if (hi > size) hi = size;
+  *off = lo;
+  *len = hi - lo;
+}
+
+static void* pool_worker(void* p) {
+  pool_arg_t* a = (pool_arg_t*)p;
+  struct oracle_pool* pool = a->pool;
+  const int index = a->index;
+  free(a);
+  unsigned long seen = 0;
+  for (;;) {
+    pthread_mutex_lock(&pool->lock);
+    while (pool->generation == seen) pthread_cond_wait(&pool->go, &pool->lock);
+    seen = pool->generation;
+    const int job = pool->job;
+    uint8_t* dst = pool->dst;
+    const uint8_t* src = pool->src;
+    const size_t size = pool->size;
+    const uint32_t value = pool->value;
+    pthread_mutex_unlock(&pool->lock);
+    if (job == POOL_JOB_EXIT) return NULL;
+    size_t off, len;
+    pool_slice(size, pool->nthreads, index, &off, &len);
+    if (len) {
+      if (job == POOL_JOB_COPY) oracle_copy(dst + off, src + off, len);
+      else if (job == POOL_JOB_FILL) oracle_fill32(dst + off, value, len / 4);
+      else if (job == POOL_JOB_TOUCH) memset(dst + off, 0, len);
+    }
+    pthread_mutex_lock(&pool->lock);
+    if (--pool->remaining == 0) pthread_cond_signal(&pool->done);
+    pthread_mutex_unlock(&pool->lock);
+  }
+}
+
+static void pool_run(struct oracle_pool* pool, int job, void* dst, const void* src, size_t size, uint32_t value) {
+  pthread_mutex_lock(&pool->lock);
+  pool->job = job;
+  pool->dst = (uint8_t*)dst;
+  pool->src = (const uint8_t*)src;
+  pool->size = size;
+  pool->value = value;
+  pool->remaining = pool->nthreads;
+  ++pool->generation;
+  pthread_cond_broadcast(&pool->go);
+  while (pool->remaining) pthread_cond_wait(&pool->done, &pool->lock);
+  pthread_mutex_unlock(&pool->lock);
+}
+
+oracle_pool_t* oracle_pool_create(int nthreads) {
+  if (nthreads < 1) nthreads = 1;
+  if (nthreads > 256) nthreads = 256;
+  struct oracle_pool* pool = (struct oracle_pool*)calloc(1, sizeof(*pool));
+  if (!pool) return NULL;
+  pool->nthreads = nthreads;
+  pthread_mutex_init(&pool->lock, NULL);
+  pthread_cond_init(&pool->go, NULL);
+  pthread_cond_init(&pool->done, NULL);
+  cpu_set_t allowed;
+  CPU_ZERO(&allowed);
+  const int have_mask = sched_getaffinity(0, sizeof(allowed), &allowed) == 0;
+  int next_cpu = 0;
+  for (int t = 0; t < nthreads; ++t) {
+    pool_arg_t* a = (pool_arg_t*)malloc(sizeof(*a));
+    if (!a || (a->pool = pool, a->index = t, pthread_create(&pool->tid[t], NULL, pool_worker, a) != 0)) {
+      free(a);
+      pool->nthreads = t;
+      break;
+    }
+    if (have_mask) {
+      /* the t-th allowed CPU, wrapping when there are more threads than CPUs */
+      int cpu = -1;
+      for (int tries = 0; tries < 2 * CPU_SETSIZE; ++tries) {
+        const int c = next_cpu++ % CPU_SETSIZE;
+        if (CPU_ISSET(c, &allowed)) {
+          cpu = c;
+          break;
+        }
+      }
+      if (cpu >= 0) {
+        cpu_set_t one;
+        CPU_ZERO(&one);
+        CPU_SET(cpu, &one);
+        if (pthread_setaffinity_np(pool->tid[t], sizeof(one), &one) == 0) ++pool->pinned;
+      }
+    }
+  }
+  if (pool->nthreads == 0) {
+    free(pool);
+    return NULL;
+  }
+  return pool;
+}
+
+void oracle_pool_destroy(oracle_pool_t* pool) {
+  if (!pool) return;
+  pthread_mutex_lock(&pool->lock);
+  pool->job = POOL_JOB_EXIT;
+  ++pool->generation;
+  pthread_cond_broadcast(&pool->go);
+  pthread_mutex_unlock(&pool->lock);
+  for (int t = 0; t < pool->nthreads; ++t) pthread_join(pool->tid[t], NULL);
+  pthread_mutex_destroy(&pool->lock);
+  pthread_cond_destroy(&pool->go);
+  pthread_cond_destroy(&pool->done);
+  free(pool);
+}
+
+int oracle_pool_threads(const oracle_pool_t* pool) { return pool ? pool->nthreads : 0; }
+int oracle_pool_pinned(const oracle_pool_t* pool) { return pool ? pool->pinned : 0; }
+
+void oracle_pool_first_touch(oracle_pool_t* pool, void* buf, size_t size) {
+  pool_run(pool, POOL_JOB_TOUCH, buf, NULL, size, 0);
+}
+
+void oracle_pool_copy(oracle_pool_t* pool, void* dst, const void* src, size_t size) {
+  pool_run(pool, POOL_JOB_COPY, dst, src, size, 0);
+}
+
+void oracle_pool_fill32(oracle_pool_t* pool, void* ptr, uint32_t value, size_t count) {
+  pool_run(pool, POOL_JOB_FILL, ptr, NULL, count * 4, value);
 }
 
 /* ------------------------------------------------------------------------ */

@@ -123,6 +123,24 @@ void oracle_ref_host_fill(void* ptr, uint32_t value, size_t count);
 void oracle_copy_mt(void* dst, const void* src, size_t size, int nthreads);
 void oracle_fill32_mt(void* ptr, uint32_t value, size_t count, int nthreads);
 
+/* The same host path on a pool of worker threads that outlive the call, for
+ * the benchmark's CPU baseline: `nthreads` threads, each pinned to one CPU of
+ * the process's affinity mask (where the system allows it) and owning one
+ * contiguous slice, a multiple of 64 bytes, of every buffer.
+ * oracle_pool_first_touch makes every thread write zeros over its own slice,
+ * so that a freshly allocated buffer's pages are placed by their owner;
+ * oracle_pool_copy and oracle_pool_fill32 are memcpy / the dword loop on the
+ * same slices.  Pinned by: output equal to oracle_copy / oracle_fill32 for
+ * thread counts 1..33 and sizes that do not divide evenly (tests/test_oracle.py). */
+typedef struct oracle_pool oracle_pool_t;
+oracle_pool_t* oracle_pool_create(int nthreads);
+void oracle_pool_destroy(oracle_pool_t* pool);
+int oracle_pool_threads(const oracle_pool_t* pool);
+int oracle_pool_pinned(const oracle_pool_t* pool); /* threads that could be pinned */
+void oracle_pool_first_touch(oracle_pool_t* pool, void* buf, size_t size);
+void oracle_pool_copy(oracle_pool_t* pool, void* dst, const void* src, size_t size);
+void oracle_pool_fill32(oracle_pool_t* pool, void* ptr, uint32_t value, size_t count);
+
 /* --- argument validation at the API edge -------------------------------- */
 /* Status codes follow inc/hsa.h: SUCCESS 0, ERROR 0x1000, INVALID_ARGUMENT 0x1001. */
 enum { ORACLE_STATUS_SUCCESS = 0, ORACLE_STATUS_ERROR = 0x1000, ORACLE_STATUS_INVALID_ARGUMENT = 0x1001 };

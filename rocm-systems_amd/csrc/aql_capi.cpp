@@ -969,7 +969,8 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
                      h->records_dev};
 
   // 2. the copy
-  BatchCopyArgs bc{h->records_dev, total_chunks, nullptr, l.waves_per_wg, l.n_waves, make_xcd_runs(p.grid, p.xcd_run)};
+  BatchCopyArgs bc{h->records_dev, total_chunks, nullptr, l.waves_per_wg, l.n_waves, make_xcd_runs(p.grid, p.xcd_run),
+                   l.prefetch_waves, 0};
   h->last_plan = p;
 
   const uint32_t nb = barrier_packets(num_deps);
@@ -1033,7 +1034,7 @@ int copy_batch_device_locked(mi355_aql_t* h, const BatchDesc* scanned, size_t n,
     if (v.nt_load == p.nt_load && v.store == p.store_policy) bk = &v.k;
   if (!bk || l.split != 4) return MI355_BLIT_ERROR;
   BatchLookupArgs bc{{h->records_dev, sizing.records, h->chunk_start_dev + n, l.waves_per_wg, l.n_waves,
-                      make_xcd_runs(p.grid, p.xcd_run)},
+                      make_xcd_runs(p.grid, p.xcd_run), l.prefetch_waves, 0},
                      descs, h->chunk_start_dev, h->block_sum_dev, static_cast<uint64_t>(n), h->batch_seen};
   h->last_plan = p;
 

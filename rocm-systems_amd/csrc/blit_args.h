@@ -166,6 +166,12 @@ struct BatchCopyArgs {
   uint32_t waves_per_wg;
   uint32_t n_waves;
   XcdRuns xcd;
+  // Not 0: the first wave of a chunk also touches the record of the chunk this
+  // many waves ahead of it, which the same XCD gets to a few microseconds later
+  // (one round of XCD runs on; in launch order a multiple of 8 workgroups), so
+  // that the record is in that XCD's L2 when its own waves ask for it.
+  uint32_t prefetch_waves;
+  uint32_t pad;
 };
 
 // The copy over records for device-resident descriptors, whose number of

@@ -571,7 +571,8 @@ int launch_records_copy(mi355_blit* h, hipStream_t s, const mi355_blit_plan_t& p
                         uint64_t total_chunks) {
   batch_kernel_t k = select_batch_kernel(l.split, p.nt_load != 0, p.store_policy);
   if (!k) return MI355_BLIT_ERROR;
-  BatchCopyArgs bc{h->records_dev, total_chunks, nullptr, l.waves_per_wg, l.n_waves, make_xcd_runs(p.grid, p.xcd_run)};
+  BatchCopyArgs bc{h->records_dev, total_chunks, nullptr, l.waves_per_wg, l.n_waves, make_xcd_runs(p.grid, p.xcd_run),
+                   l.prefetch_waves, 0};
   hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, bc);
   return MI355_BLIT_SUCCESS;
 }
@@ -585,7 +586,7 @@ int launch_lookup_copy(const BatchDeviceBuffers& b, hipStream_t s, const mi355_b
     if (v.nt_load == p.nt_load && v.store == p.store_policy) k = v.fn;
   if (!k || l.split != 4) return MI355_BLIT_ERROR;
   BatchLookupArgs a{{b.records, records, b.chunk_start + n, l.waves_per_wg, l.n_waves,
-                     make_xcd_runs(p.grid, p.xcd_run)},
+                     make_xcd_runs(p.grid, p.xcd_run), l.prefetch_waves, 0},
                     dev_descs, b.chunk_start, b.block_sum, static_cast<uint64_t>(n), b.seen};
   hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
   return MI355_BLIT_SUCCESS;

@@ -605,6 +605,26 @@ __device__ __forceinline__ BatchDesc load_desc(const BatchDesc* p) {
   return d;
 }
 
+// A wave's record is a dependent load in front of everything else it does, and
+// the records of chunks that run at the same time miss L2 together: every wave
+// would wait for memory twice, once for its record and once for its data.  So
+// the first wave of a chunk also reads one word of the record that the same
+// XCD will need `ahead` waves later, with an ordinary vector load that returns
+// before the data loads behind it: the line (four records) is then in that
+// XCD's L2 when its time comes.  The value is not used; keep_alive() only keeps
+// the compiler from dropping the load.
+__device__ __forceinline__ unsigned touch_record_ahead(const ChunkRecord* records, uint64_t w, unsigned q,
+                                                       unsigned ahead, unsigned split, uint64_t total_chunks,
+                                                       unsigned lane) {
+  unsigned v = 0;
+  if (ahead && q == 0 && lane == 0) {
+    const uint64_t c = (w + ahead) / split;
+    if (c < total_chunks) v = ld_u32<false>(reinterpret_cast<const unsigned*>(records + c));
+  }
+  return v;
+}
+__device__ __forceinline__ void keep_alive(unsigned v) { asm volatile("" ::"v"(v)); }
+
 // SPLIT waves per 4 KiB chunk, chunks in global order and waves in address
 // order within a chunk: the dispatcher then walks memory densely, the shape
 // that streams best for a single large copy.  Each wave reads its chunk's
@@ -618,14 +638,16 @@ __device__ __forceinline__ void batch_copy_records_body(const BatchCopyArgs& a) 
   const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd);
   const uint64_t n_waves = a.n_waves;
   for (uint64_t w = wave; w < total_chunks * SPLIT; w += n_waves) {
-    const ChunkRecord rec = load_record(records + w / SPLIT);
     const unsigned q = static_cast<unsigned>(w % SPLIT);
+    const unsigned touched = touch_record_ahead(records, w, q, a.prefetch_waves, SPLIT, total_chunks, lane);
+    const ChunkRecord rec = load_record(records + w / SPLIT);
     const unsigned v0 = q * (kChunkVecs / SPLIT);
     v4u x[U];
     unsigned e;
     record_load<U, NTL>(rec, v0, lane, x, e);
     record_store<U, NTS>(rec, v0, lane, x, e);
     record_edges(rec, q == 0, q == SPLIT - 1, lane);
+    keep_alive(touched);
   }
 }
 
@@ -711,16 +733,19 @@ __device__ __forceinline__ void batch_copy_lookup_body(const BatchLookupArgs& a)
   const uint64_t n_waves = a.copy.n_waves;
   if (wave == 0 && lane == 0 && a.seen)
     __hip_atomic_store(a.seen, a.n << 32 | total_chunks, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  const uint64_t have = total_chunks < capacity ? total_chunks : capacity;  // chunks with a record
   for (uint64_t w = wave; w < total_chunks * SPLIT; w += n_waves) {
     const uint64_t c = w / SPLIT;
-    const ChunkRecord rec = c < capacity ? load_record(records + c) : lookup_record(a, static_cast<uint32_t>(c));
     const unsigned q = static_cast<unsigned>(w % SPLIT);
+    const unsigned touched = touch_record_ahead(records, w, q, a.copy.prefetch_waves, SPLIT, have, lane);
+    const ChunkRecord rec = c < capacity ? load_record(records + c) : lookup_record(a, static_cast<uint32_t>(c));
     const unsigned v0 = q * (kChunkVecs / SPLIT);
     v4u x[U];
     unsigned e;
     record_load<U, NTL>(rec, v0, lane, x, e);
     record_store<U, NTS>(rec, v0, lane, x, e);
     record_edges(rec, q == 0, q == SPLIT - 1, lane);
+    keep_alive(touched);
   }
 }
 

@@ -156,6 +156,7 @@ struct BatchLaunch {
   uint32_t split;         // waves per chunk
   uint32_t waves_per_wg;
   uint32_t n_waves;
+  uint32_t prefetch_waves;  // BatchCopyArgs::prefetch_waves
 };
 
 // total_chunks: the number of records, or a bound on it.  streaming: whether
@@ -172,7 +173,11 @@ inline BatchLaunch plan_batch_records(uint64_t total_chunks, uint64_t total_byte
   p->store_policy = streaming ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED;
   if (t && t->store_policy >= 1 && t->store_policy <= 4) p->store_policy = t->store_policy - 1;
   BatchLaunch l;
-  p->wg_size = 256;
+  // Single-wave workgroups, four to a chunk: a wave starts as soon as one wave
+  // slot is free instead of waiting for four on one CU (65,536 copies, 4.1 GB:
+  // 698 us against 700 us spread over two 8 GiB arenas, 663 against 670 packed
+  // densely).
+  p->wg_size = 64;
   l.split = 4;
   if (t && shape_tunable) {
     if (t->wg_size >= 64 && t->wg_size <= 1024 && t->wg_size % 64 == 0) p->wg_size = t->wg_size;
@@ -186,6 +191,15 @@ inline BatchLaunch plan_batch_records(uint64_t total_chunks, uint64_t total_byte
   p->grid = static_cast<uint32_t>(wgs);
   l.n_waves = static_cast<uint32_t>(wgs * l.waves_per_wg);
   p->xcd_run = batch_xcd_run(total_bytes, l.split, l.waves_per_wg, t);
+  // The record a wave needs is touched one round of XCD runs earlier (in launch
+  // order: 4096 workgroups earlier, a multiple of 8 and so on the same XCD).
+  // Measured with 65,536 copies (4.1 GB): 700 us against 705 us without spread
+  // over two 8 GiB arenas, 670 against 690 packed densely; a distance of half a
+  // round or less (528 .. 2112 workgroups of 256) gains nothing, the touched
+  // line then sits in another XCD's L2.
+  uint32_t ahead_wgs = p->xcd_run > 1 ? 8 * p->xcd_run : 4096;
+  if (t && t->batch_prefetch) ahead_wgs = t->batch_prefetch > 1 ? t->batch_prefetch : 0;
+  l.prefetch_waves = ahead_wgs * l.waves_per_wg;
   return l;
 }
 

@@ -62,6 +62,8 @@ mi355_blit_tuning_t random_tuning() {
   t.max_grid = below(3) ? 0 : static_cast<uint32_t>(below(5000));
   t.nt_load = static_cast<uint32_t>(below(3));
   t.store_policy = static_cast<uint32_t>(below(6));
+  const uint32_t prefetch[] = {0, 0, 1, 4224};
+  t.batch_prefetch = prefetch[below(4)];
   return t;
 }
 
@@ -381,11 +383,15 @@ void one_batch_launch() {
   const bool capped = tuned && t.max_grid && t.max_grid < (chunks * l.split + l.waves_per_wg - 1) / l.waves_per_wg;
   if (capped) CHECK(p.grid == t.max_grid, "grid cap");
   else CHECK(l.n_waves >= chunks * l.split && l.n_waves < chunks * l.split + l.waves_per_wg, "one wave per part of a chunk");
-  if (!tuned || !tunable) CHECK(p.wg_size == 256 && l.split == 4, "fixed shape");
+  if (!tuned || !tunable) CHECK(p.wg_size == 64 && l.split == 4, "fixed shape");
+  // the record touched ahead belongs to the same XCD: whole rounds of 8 workgroups away
+  const bool no_prefetch = tuned && t.batch_prefetch == 1;
+  CHECK(no_prefetch ? l.prefetch_waves == 0 : (l.prefetch_waves % (8 * l.waves_per_wg) == 0 || (tuned && t.batch_prefetch > 1)),
+        "prefetch distance %u", l.prefetch_waves);
   if (!tuned) {
     CHECK(p.nt_load == (bytes >= (4ull << 20)) && p.store_policy == (p.nt_load ? MI355_BLIT_STORE_NT : MI355_BLIT_STORE_CACHED),
           "cache policy by size");
-    CHECK(p.xcd_run == (bytes >= (64ull << 20) ? 528u : 0u), "XCD runs by size: %u", p.xcd_run);
+    CHECK(p.xcd_run == (bytes >= (64ull << 20) ? 4 * 528u : 0u), "XCD runs by size: %u", p.xcd_run);
   }
 }
 
@@ -411,7 +417,7 @@ void one_xcd_permutation() {
     if (b >= 8) CHECK(w == last[b & 7] + 1 || w == last[b & 7] + 1 + 7 * run, "XCD %u jumps from %u to %u", b & 7, last[b & 7], w);
     last[b & 7] = w;
   }
-  const mi355_blit_tuning_t linear{0, 0, 0, 0, 0, 1, {0, 0}}, forced{0, 0, 0, 0, 0, 99, {0, 0}};
+  const mi355_blit_tuning_t linear{0, 0, 0, 0, 0, 1, 0, 0}, forced{0, 0, 0, 0, 0, 99, 0, 0};
   CHECK(plan_xcd_run(288, nullptr) == 288 && plan_xcd_run(288, &linear) == 0 && plan_xcd_run(0, &forced) == 99,
         "tuning of the run");
 }

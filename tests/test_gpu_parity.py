@@ -495,6 +495,11 @@ def _make_batch(capi, rng, src, dst, n, min_len=64, max_len=256 << 10):
     return descs, lens, offs, so, do, total
 
 
+def _grid_chunks(p):
+    """Chunks a batch launch has waves for: four waves to a 4 KiB chunk."""
+    return p.grid * (p.wg_size // 64) // (4 // p.unroll)
+
+
 def _expect_batch(oracle, src_host, total, lens, offs, so, do):
     want = np.full(total, GUARD_BYTE, dtype=np.uint8)
     for i in range(len(lens)):
@@ -713,7 +718,7 @@ def test_batch_bound_exceeded_costs_speed_not_bytes(capi, blit, oracle, arenas, 
     check_ok(capi, blit.copy_batch_bounded(descs_dev.data_ptr(), n, bound), "copy_batch_bounded")
     check_ok(capi, blit.synchronize(), "synchronize")
     p = blit.last_plan()
-    assert p.grid < int((lens // 4096).sum()), "the case is meant to leave chunks without a wave of their own"
+    assert _grid_chunks(p) < int((lens // 4096).sum()), "the case is meant to leave chunks without a wave of their own"
     assert np.array_equal(dst.host(0, total), _expect_batch(oracle, src_host, total, lens, offs, so, do))
 
 
@@ -735,7 +740,7 @@ def test_batch_unbounded_beyond_what_the_library_assumes(capi, blit, oracle, ran
     torch.cuda.synchronize()
     check_ok(capi, blit.copy_batch(descs_dev.data_ptr(), n, on_device=True), "copy_batch")
     check_ok(capi, blit.synchronize(), "synchronize")
-    assert blit.last_plan().grid * 2 < int((lens // 4096).sum())
+    assert _grid_chunks(blit.last_plan()) * 2 < int((lens // 4096).sum())
     got = dst.host(0, total)
     want = _expect_batch(oracle, src_host, total, lens, offs, so, do)
     assert np.array_equal(got, want)
@@ -763,7 +768,7 @@ def test_batch_unbounded_sizes_itself_by_the_batch_before(capi, pkg, oracle, are
             torch.cuda.synchronize()
             check_ok(capi, eng.copy_batch(dev.data_ptr(), n, on_device=True), "copy_batch")
             check_ok(capi, eng.synchronize(), "synchronize")
-            grids.append(eng.last_plan().grid)
+            grids.append(_grid_chunks(eng.last_plan()))
             assert np.array_equal(dst.host(0, total), want), "call %d" % call
         assert grids[0] == 8 * n
         # 16 or 17 chunks a copy: the second and third launches follow what the first one counted
@@ -778,7 +783,7 @@ def test_batch_unbounded_sizes_itself_by_the_batch_before(capi, pkg, oracle, are
             torch.cuda.synchronize()
             check_ok(capi, eng.copy_batch(dev2.data_ptr(), n2, on_device=True), "copy_batch")
             check_ok(capi, eng.synchronize(), "synchronize")
-            grids.append(eng.last_plan().grid)
+            grids.append(_grid_chunks(eng.last_plan()))
             assert np.array_equal(dst.host(0, total2), want2), "short copies, call %d" % call
         assert grids[3] > 10 * n2 and grids[4] <= 2 * n2 + 32, grids
     finally:
@@ -803,7 +808,7 @@ def test_batch_of_many_short_copies_is_staged_as_it_is(capi, blit, oracle, arena
         check_ok(capi, blit.copy_batch(descs, n), "copy_batch")
         check_ok(capi, blit.synchronize(), "synchronize")
         p = blit.last_plan()
-        assert p.kernel == capi.KERNEL_COPY_BATCH and p.grid == int(lens.sum()) // 4096 + n, p.as_dict()
+        assert p.kernel == capi.KERNEL_COPY_BATCH and _grid_chunks(p) == int(lens.sum()) // 4096 + n, p.as_dict()
         assert np.array_equal(dst.host(0, total), _expect_batch(oracle, src_host, total, lens, offs, so, do)), seed
     # a copy of bytes without a source: refused before anything is launched
     descs[n // 2].src = None

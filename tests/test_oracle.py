@@ -133,6 +133,41 @@ def test_mt_variants_equal_single_thread(oracle, rand):
         assert np.array_equal(a, b)
 
 
+def test_thread_pool_equals_single_thread(oracle, rand):
+    """The pooled host path of the CPU baseline (persistent pinned workers, one
+    contiguous slice each) against the single-thread oracle: thread counts that
+    do and do not divide the size, more threads than 64-byte blocks, guards."""
+    import ctypes
+    for name, res, args in (("oracle_pool_create", ctypes.c_void_p, [ctypes.c_int]),
+                            ("oracle_pool_destroy", None, [ctypes.c_void_p]),
+                            ("oracle_pool_threads", ctypes.c_int, [ctypes.c_void_p]),
+                            ("oracle_pool_pinned", ctypes.c_int, [ctypes.c_void_p]),
+                            ("oracle_pool_first_touch", None, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]),
+                            ("oracle_pool_copy", None, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]),
+                            ("oracle_pool_fill32", None, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_size_t])):
+        fn = getattr(oracle, name)
+        fn.restype, fn.argtypes = res, args
+    guard = 128
+    for threads in (1, 2, 7, 16, 33):
+        pool = oracle.oracle_pool_create(threads)
+        assert pool and oracle.oracle_pool_threads(pool) == threads
+        assert 0 <= oracle.oracle_pool_pinned(pool) <= threads
+        for n in (0, 1, 63, 64, 65, 1000, (3 << 20) + 13, 1 << 22):
+            src = rand(n + 1, 11 + threads)
+            got = np.full(n + 2 * guard, 0xEE, dtype=np.uint8)
+            want = got.copy()
+            oracle.oracle_pool_first_touch(pool, got.ctypes.data + guard, n)
+            assert (got[guard:guard + n] == 0).all() and (got[:guard] == 0xEE).all() and (got[guard + n:] == 0xEE).all()
+            oracle.oracle_pool_copy(pool, got.ctypes.data + guard, src.ctypes.data, n)
+            oracle.oracle_copy(want.ctypes.data + guard, src.ctypes.data, n)
+            assert np.array_equal(got, want), (threads, n)
+            cnt = n // 4
+            oracle.oracle_pool_fill32(pool, got.ctypes.data + guard, 0xA5C30F1E, cnt)
+            oracle.oracle_fill32(want.ctypes.data + guard, 0xA5C30F1E, cnt)
+            assert np.array_equal(got, want), (threads, n)
+        oracle.oracle_pool_destroy(pool)
+
+
 # ---- API-edge validation -----------------------------------------------------
 
 def test_validate_copy(oracle):

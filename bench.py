@@ -396,20 +396,25 @@ def aql_path(r, pkg):
         do = (-dst.data_ptr()) % 256 + 9
         assert r.torch.equal(dst[do:do + GIB - 64], src[so:so + GIB - 64]), "AQL copy result differs"
         eng.enable_profiling(False)
-        lat = {}
         c = sig.create(1)
-        for n in (4096, 65536, MIB):
-            ts = []
-            for i in range(220):
-                sig.store(c, 1)
-                t0 = time.perf_counter()
-                r.check(eng.copy(D, S, n, completion=c), "copy")
-                sig.wait_below_one(c)
-                ts.append(time.perf_counter() - t0)
-            ts = sorted(ts[20:])
-            lat[str(n)] = round(ts[len(ts) // 2] * 1e6, 2)
+        for key, system_scope in (("small_copy_us", True), ("small_copy_us_agent_scope", False)):
+            # system scope: the reference's fences (amd_blit_kernel.cpp:870-873); agent scope: for
+            # callers whose consumers are kernels on this GPU
+            eng.set_system_scope_fences(system_scope)
+            lat = {}
+            for n in (4096, 65536, MIB):
+                ts = []
+                for i in range(220):
+                    sig.store(c, 1)
+                    t0 = time.perf_counter()
+                    r.check(eng.copy(D, S, n, completion=c), "copy")
+                    sig.wait_below_one(c)
+                    ts.append(time.perf_counter() - t0)
+                ts = sorted(ts[20:])
+                lat[str(n)] = round(ts[len(ts) // 2] * 1e6, 2)
+            out[key] = lat
+        eng.set_system_scope_fences(True)
         sig.destroy(c)
-        out["small_copy_us"] = lat
         del src, dst
         r.torch.cuda.empty_cache()
         # the batch, whole submission by the host clock
@@ -429,7 +434,9 @@ def aql_path(r, pkg):
         out["batch_65536"] = {"gbs": round(algo / us / 1e3, 1), "frac_of_peak": round(algo / us / 1e3 / HBM_PEAK_GBS, 4),
                               "us_per_launch": round(us, 2)}
         out["how"] = ("AQL packets on an HSA queue; 1 GiB cases: packet-processor timestamps of 20 commands; "
-                      "batch: host clock over 20 submissions; small copies: host clock, median of 200")
+                      "batch: host clock over 20 submissions; small copies: blocking copy by the host clock through the "
+                      "Python binding, submit to completion signal seen, median of 200 (the native driver's figures, "
+                      "cut at the packet processor's timestamps, are in profiles/small_copy_latency.md)")
         del keep, hip_blit
     finally:
         eng.close()

@@ -631,6 +631,68 @@ void latency_report(Blit& blit, const char* mode) {
   }
 }
 
+// Where the time of a small blocking copy goes on the AQL path, the way
+// rocrtst times one (memory_async_copy.cc:396-405: submit, then spin on the
+// completion signal), cut at the packet processor's own timestamps: host
+// submit call | doorbell to start of the kernel | kernel | end of the kernel
+// to the host seeing the signal.  The signal's stamps are in the system
+// timestamp domain (the runtime translates them), like the host's readings.
+uint64_t now_ticks() {
+  uint64_t t = 0;
+  hsa_system_get_info(HSA_SYSTEM_INFO_TIMESTAMP, &t);
+  return t;
+}
+
+double median_of(std::vector<double>& v) {
+  std::sort(v.begin(), v.end());
+  return v[v.size() / 2];
+}
+
+void latency_breakdown(bool system_scope, const char* kernargs, const mi355_blit_tuning_t* tuning = nullptr,
+                       const char* shape = "heuristic") {
+  mi355_aql_t* h = nullptr;
+  if (mi355_aql_create(0, &h) != MI355_BLIT_SUCCESS) {
+    std::printf("FAIL latency_breakdown: mi355_aql_create\n");
+    ++g_failures;
+    return;
+  }
+  mi355_aql_set_tuning(h, tuning);
+  mi355_aql_set_system_scope_fences(h, system_scope ? 1 : 0);
+  mi355_aql_enable_profiling(h, 1);
+  uint64_t freq = 0;
+  hsa_system_get_info(HSA_SYSTEM_INFO_TIMESTAMP_FREQUENCY, &freq);
+  const double us_per_tick = 1e6 / double(freq);
+  DeviceBuf a(1 << 20), b(1 << 20);
+  hsa_signal_t done = make_signal(1);
+  if (!a.p || !b.p || !done.handle) return;
+  for (size_t n : {size_t(4096), size_t(65536), size_t(1 << 20)}) {
+    std::vector<double> submit, to_start, kernel, to_host, total;
+    for (int i = 0; i < 320; ++i) {
+      hsa_signal_store_relaxed(done, 1);
+      const uint64_t t0 = now_ticks();
+      if (mi355_aql_copy(h, b.p, a.p, n, nullptr, 0, done.handle) != MI355_BLIT_SUCCESS) return;
+      const uint64_t t1 = now_ticks();
+      while (hsa_signal_wait_scacquire(done, HSA_SIGNAL_CONDITION_LT, 1, UINT64_MAX, HSA_WAIT_STATE_ACTIVE) >= 1) {
+      }
+      const uint64_t t2 = now_ticks();
+      uint64_t start = 0, end = 0;
+      if (mi355_aql_get_command_time(h, done.handle, &start, &end, nullptr) != MI355_BLIT_SUCCESS) return;
+      if (i < 20) continue;
+      submit.push_back(double(t1 - t0) * us_per_tick);
+      to_start.push_back((double(start) - double(t1)) * us_per_tick);
+      kernel.push_back(double(end - start) * us_per_tick);
+      to_host.push_back((double(t2) - double(end)) * us_per_tick);
+      total.push_back(double(t2 - t0) * us_per_tick);
+    }
+    std::printf("INFO latency_breakdown fences=%s kernargs=%s shape=%s bytes=%zu total=%.2f submit_call=%.2f doorbell_to_start=%.2f "
+                "kernel=%.2f end_to_host=%.2f (medians of %zu, us)\n",
+                system_scope ? "system" : "agent", kernargs, shape, n, median_of(total), median_of(submit), median_of(to_start),
+                median_of(kernel), median_of(to_host), total.size());
+  }
+  hsa_signal_destroy(done);
+  mi355_aql_destroy(h);
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
@@ -649,6 +711,33 @@ int main(int argc, char** argv) {
   if (hsa_init() != HSA_STATUS_SUCCESS) {
     std::printf("FAIL setup: hsa_init failed (no GPU?)\n");
     return 2;
+  }
+  if (argc > 1 && std::string(argv[1]) == "--latency") {
+    // test_rocr_blit --latency: the breakdown only, for the placement of the
+    // kernarg ring the environment asks for (MI355_BLIT_HOST_KERNARGS=1: host memory)
+    const char* env = std::getenv("MI355_BLIT_HOST_KERNARGS");
+    const char* where = env && env[0] == '1' ? "host" : "device";
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count < 1) return 2;
+    latency_breakdown(true, where);
+    latency_breakdown(false, where);
+    if (argc > 2 && std::string(argv[2]) == "shapes") {
+      // what the launch shape and the store policy of a small copy are worth under system-scope fences
+      mi355_blit_tuning_t t{};
+      t.store_policy = MI355_BLIT_STORE_AGENT_WT + 1;
+      latency_breakdown(true, where, &t, "stores_sc1");
+      t.store_policy = MI355_BLIT_STORE_SYSTEM_WT + 1;
+      latency_breakdown(true, where, &t, "stores_sc0_sc1");
+      t.store_policy = MI355_BLIT_STORE_NT + 1;
+      latency_breakdown(true, where, &t, "stores_nt");
+      t = mi355_blit_tuning_t{};
+      t.wg_size = 1024;
+      latency_breakdown(true, where, &t, "wg1024");
+      t.wg_size = 64;
+      latency_breakdown(true, where, &t, "wg64");
+    }
+    hsa_shut_down();
+    return g_failures ? 1 : 0;
   }
   int count = 0;
   if (hipGetDeviceCount(&count) != hipSuccess || count < 1) {

@@ -46,11 +46,15 @@ def parse_args():
     # that peaks around the tenth launch and is gone by the fiftieth, whatever the kernel): the
     # default warm-up covers it.
     ap.add_argument("--warmup", type=int, default=WARMUP_AFTER_IDLE)
-    ap.add_argument("--workload", default="copy", choices=["copy", "fill", "misaligned", "batch", "rect", "calib"])
+    ap.add_argument("--workload", default="copy",
+                    choices=["copy", "fill", "misaligned", "batch", "rect", "calib", "idle_series"])
     ap.add_argument("--bytes", type=int, default=GIB, help="transfer size of the copy/fill workloads")
     ap.add_argument("--rect", default="8192,131072,262144,0,0",
                     help="shape of the rect workload: rows,width,pitch[,source x,destination x] in bytes")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-verify", action="store_true",
+                    help="skip the check of the timed workload's result (for runs under a profiler, whose trace "
+                         "would otherwise record the check's own kernels: 200,000 of them for the batch)")
     ap.add_argument("--no-also", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget")
     return ap.parse_args()
@@ -581,6 +585,82 @@ def reference_rect(r, hsa, S, D):
     return round(2 * rows * width / best / 1e9, 1) if best else None
 
 
+def idle_series(pkg, torch, nbytes, launches, idle_s):
+    """How a burst of back-to-back copies of nbytes settles after idle_s seconds
+    without work: the pace of every launch (end of command i minus end of
+    command i-1, from the packet processor's timestamps in the completion
+    signals, AQL path) next to the clocks and the power the driver reports in
+    sysfs, sampled every millisecond by a host thread while the burst runs."""
+    import glob
+    import threading
+    aql = pkg.aql
+    paths = {}
+    for card in sorted(glob.glob("/sys/class/drm/card*/device")):
+        if os.path.exists(card + "/pp_dpm_sclk"):
+            paths = {"sclk": card + "/pp_dpm_sclk", "mclk": card + "/pp_dpm_mclk"}
+            power = glob.glob(card + "/hwmon/hwmon*/power1_input") + glob.glob(card + "/hwmon/hwmon*/power1_average")
+            if power:
+                paths["power_uW"] = power[0]
+            break
+
+    def current(path):
+        try:
+            text = open(path).read()
+        except OSError:
+            return None
+        for line in text.splitlines():
+            if line.strip().endswith("*"):
+                return line.split(":")[1].strip().rstrip("*").strip()
+        return text.strip()[:32]
+
+    eng = aql.AqlBlit(0)
+    sig = aql.HsaSignals()
+    a = torch.empty(nbytes + 512, dtype=torch.uint8, device="cuda:0").fill_(3)
+    b = torch.empty(nbytes + 512, dtype=torch.uint8, device="cuda:0").fill_(5)
+    A, B = aligned_ptr(a), aligned_ptr(b)
+    torch.cuda.synchronize()
+    eng.enable_profiling(True)
+    sigs = [sig.create(1) for _ in range(launches)]
+    samples, stop = [], []
+
+    def sampler():
+        while not stop:
+            samples.append((time.perf_counter(),) + tuple(current(paths[k]) for k in sorted(paths)))
+            time.sleep(0.001)
+
+    time.sleep(idle_s)
+    th = threading.Thread(target=sampler)
+    th.start()
+    time.sleep(0.005)
+    t0 = time.perf_counter()
+    for c in sigs:
+        assert eng.copy(B, A, nbytes, completion=c) == 0
+    sig.wait_below_one(sigs[-1])
+    time.sleep(0.005)
+    stop.append(1)
+    th.join()
+    ends = []
+    first_start = None
+    for c in sigs:
+        x, y, f = C.c_uint64(), C.c_uint64(), C.c_uint64()
+        assert eng.lib.mi355_aql_get_command_time(eng.handle, c, C.byref(x), C.byref(y), C.byref(f)) == 0
+        if first_start is None:
+            first_start = x.value * 1e6 / f.value
+        ends.append(y.value * 1e6 / f.value)
+        sig.destroy(c)
+    eng.close()
+    pace = [round(ends[0] - first_start, 1)] + [round(ends[i] - ends[i - 1], 1) for i in range(1, launches)]
+    # the samples that differ from the one before
+    changes, last = [], None
+    for smp in samples:
+        if smp[1:] != last:
+            changes.append([round((smp[0] - t0) * 1e3, 1)] + list(smp[1:]))
+            last = smp[1:]
+    return {"metric": "pace of back-to-back %d MiB copies after %.1f s idle" % (nbytes // MIB, idle_s),
+            "unit": "us per launch", "launches": launches, "pace_us": pace,
+            "sysfs_columns": ["ms since first submit"] + sorted(paths), "sysfs_changes": changes}
+
+
 def cpu_model():
     try:
         with open("/proc/cpuinfo") as f:
@@ -679,6 +759,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     pkg = entry.load_package()
+    if args.workload == "idle_series":
+        print(json.dumps(idle_series(pkg, torch, args.bytes, max(args.steps, 10), 3.0)))
+        return
     r = Runner(torch, pkg)
     nbytes = args.bytes
 
@@ -711,7 +794,8 @@ def main():
         traffic_key = "batch_65536"
 
     wall, dev_us = r.time_launches(fn, args.steps, args.warmup)
-    verify()
+    if not args.no_verify:
+        verify()
     plan = r.blit.last_plan().as_dict()
     value = algo * args.steps / wall / 1e9
     achieved = algo / dev_us / 1e3

@@ -3,6 +3,9 @@
  * blit-kernel data path.  Paths cited are relative to
  * projects/rocr-runtime/runtime/hsa-runtime/ in the reference tree.
  */
+#ifndef _GNU_SOURCE
+#define _GNU_SOURCE /* CPU_SET, sched_getaffinity, pthread_setaffinity_np */
+#endif
 #include "blit_oracle.h"
 
 #include <pthread.h>

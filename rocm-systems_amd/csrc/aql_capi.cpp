@@ -460,6 +460,18 @@ void tail_waves(const mi355_blit_plan_t& p, uint32_t* partial_wave, uint32_t* ed
 
 uint32_t barrier_packets(uint32_t num_deps) { return (num_deps + 4) / 5; }
 
+// Whether a transfer's dispatch packet carries the barrier bit although no
+// dependency asks for it.  The reference leaves the bit clear on every blit
+// (amd_blit_kernel.cpp:870-882): consecutive blits may overlap, which hides
+// the launch latency of small ones.  Large ones lose by it: while one transfer
+// drains, the next one's waves start on another stretch of memory and the two
+// streams disturb each other in DRAM (back-to-back 1 GiB copies: 334 us apiece
+// overlapping, 317 us one after the other, the gap between them included).  So
+// transfers that stream past the caches wait for the queue to drain; that is a
+// stronger order than the interface promises, never a weaker one.
+constexpr uint64_t kSerialiseMinBytes = 4ull << 20;
+bool serialise(uint64_t bytes) { return bytes >= kSerialiseMinBytes; }
+
 void free_device(void* p) {
   if (p) (void)hsa_amd_memory_pool_free(p);
 }
@@ -861,7 +873,7 @@ int mi355_aql_copy_route(mi355_aql_t* h, void* dst, const void* src, size_t byte
   // Barrier bit clear, as in the reference: consecutive blits may overlap
   // unless linked by signals.  After dependency barriers the bit is set so
   // that the copy cannot start before them.
-  write_dispatch(h, index + nb, *k, &a, sizeof(a), p.grid, p.wg_size, completion_signal, nb != 0);
+  write_dispatch(h, index + nb, *k, &a, sizeof(a), p.grid, p.wg_size, completion_signal, nb != 0 || serialise(bytes));
   release_write_index(h, index, total);
   return MI355_BLIT_SUCCESS;
 }
@@ -904,7 +916,7 @@ int mi355_aql_fill32(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dword
     record_blit_history(h, num_dwords * 4, index + total - 1);
   }
   write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
-  write_dispatch(h, index + nb, *k, &a, sizeof(a), p.grid, p.wg_size, completion_signal, nb != 0);
+  write_dispatch(h, index + nb, *k, &a, sizeof(a), p.grid, p.wg_size, completion_signal, nb != 0 || serialise(num_dwords * 4));
   release_write_index(h, index, total);
   return MI355_BLIT_SUCCESS;
 }
@@ -1146,9 +1158,11 @@ int mi355_aql_copy_rect_route(mi355_aql_t* h, const mi355_pitched_ptr_t* dst, co
   }
   write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
   if (rp.narrow)
-    write_dispatch(h, index + nb, *k, &rp.nargs, sizeof(rp.nargs), rp.grid, rp.wg_size, completion_signal, nb != 0);
+    write_dispatch(h, index + nb, *k, &rp.nargs, sizeof(rp.nargs), rp.grid, rp.wg_size, completion_signal,
+                   nb != 0 || serialise(rp.total_bytes));
   else
-    write_dispatch(h, index + nb, *k, &rp.args, sizeof(rp.args), rp.grid, rp.wg_size, completion_signal, nb != 0);
+    write_dispatch(h, index + nb, *k, &rp.args, sizeof(rp.args), rp.grid, rp.wg_size, completion_signal,
+                   nb != 0 || serialise(rp.total_bytes));
   release_write_index(h, index, total);
   return MI355_BLIT_SUCCESS;
 }

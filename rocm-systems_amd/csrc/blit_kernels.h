@@ -764,111 +764,141 @@ __device__ __forceinline__ uint64_t row_units(uint64_t n_virtual, unsigned unit)
   return n_virtual > kRowOverflowVecs + unit ? (n_virtual - kRowOverflowVecs + unit - 1) / unit : 1;
 }
 
+// One unit slot of a region whose rows are tiled like a linear copy
+// (RectArgs::plain_rows): U loads and U stores per lane and nothing else.  A
+// row's last unit may be a partial one, whose lanes beyond the row's end have
+// nothing to do, or have up to kRowOverflowVecs vectors more than a unit, which
+// its first lanes take.
 template <int U, bool NTL, int NTS>
-__device__ __forceinline__ void rect_copy_body(const RectArgs& a) {
+__device__ __forceinline__ void rect_plain_unit(const RectArgs& a, uint32_t slot, unsigned lane) {
   constexpr unsigned kUnit = kWave * U;
-  const unsigned lane = threadIdx.x & (kWave - 1);
-  const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd);
-  const uint64_t n_waves = a.n_waves;
-  if (a.plain_rows) {
-    // Rows of whole vectors, aligned like a linear copy's tiles: a unit is U
-    // loads and U stores per lane and nothing else.  A row's last unit may be
-    // a partial one, whose lanes beyond the row's end have nothing to do, or
-    // have up to kRowOverflowVecs vectors more than a unit, which its first
-    // lanes take.
-    for (uint64_t w = wave; w < a.total_slots; w += n_waves) {
-      const uint32_t slot = static_cast<uint32_t>(w);
-      const uint32_t line = div_magic(slot, a.magic_slots);
-      const uint32_t kq = slot - line * a.slots;
-      const uint32_t layer = div_magic(line, a.magic_rows);
-      const uint32_t y = line - layer * a.rows;
-      const uint64_t in_row = static_cast<uint64_t>(kq) * (kUnit * 16) + lane * 16;
-      const v4u_a4* sv = reinterpret_cast<const v4u_a4*>(a.src + layer * a.src_slice + y * a.src_pitch + in_row);
-      v4u* dv = reinterpret_cast<v4u*>(a.dst + layer * a.dst_slice + y * a.dst_pitch + in_row);
-      const bool over = kq + 1 == a.slots && in_row + U * (kWave * 16) < a.width;
-      v4u x[U + 1];
+  const uint32_t line = div_magic(slot, a.magic_slots);
+  const uint32_t kq = slot - line * a.slots;
+  const uint32_t layer = div_magic(line, a.magic_rows);
+  const uint32_t y = line - layer * a.rows;
+  const uint64_t in_row = static_cast<uint64_t>(kq) * (kUnit * 16) + lane * 16;
+  const v4u_a4* sv = reinterpret_cast<const v4u_a4*>(a.src + layer * a.src_slice + y * a.src_pitch + in_row);
+  v4u* dv = reinterpret_cast<v4u*>(a.dst + layer * a.dst_slice + y * a.dst_pitch + in_row);
+  const bool over = kq + 1 == a.slots && in_row + U * (kWave * 16) < a.width;
+  v4u x[U + 1];
 #pragma unroll
-      for (int u = 0; u < U; ++u)
-        if (in_row + u * (kWave * 16) < a.width) x[u] = ld_v4<NTL>(sv + u * kWave);
-      if (over) x[U] = ld_v4<NTL>(sv + U * kWave);
+  for (int u = 0; u < U; ++u)
+    if (in_row + u * (kWave * 16) < a.width) x[u] = ld_v4<NTL>(sv + u * kWave);
+  if (over) x[U] = ld_v4<NTL>(sv + U * kWave);
 #pragma unroll
-      for (int u = 0; u < U; ++u)
-        if (in_row + u * (kWave * 16) < a.width) st_v4<NTS>(dv + u * kWave, x[u]);
-      if (over) st_v4<NTS>(dv + U * kWave, x[U]);
+  for (int u = 0; u < U; ++u)
+    if (in_row + u * (kWave * 16) < a.width) st_v4<NTS>(dv + u * kWave, x[u]);
+  if (over) st_v4<NTS>(dv + U * kWave, x[U]);
+}
+
+// One unit slot of a region with rows of any alignment.  Most units of a wide
+// row lie inside it (neither its first nor its last): those are found with as
+// little arithmetic as possible and moved like a tile of the linear copy, the
+// others take the general path behind.  (Every instruction in front of a
+// wave's first load counts: with 32 waves on a CU sharing its issue slots, a
+// hundred scalar instructions are a fifth of a wave's life.)
+template <int U, bool NTL, int NTS>
+__device__ __forceinline__ void rect_unit(const RectArgs& a, uint32_t slot, unsigned lane) {
+  constexpr unsigned kUnit = kWave * U;
+  const uint32_t line = div_magic(slot, a.magic_slots);  // row index through all layers
+  const uint32_t kq = slot - line * a.slots;
+  uint8_t* drow = a.dst + line * a.dst_pitch;
+  const uint8_t* srow = a.src + line * a.src_pitch;
+  if (a.total_slots > a.slots * a.rows) {  // more than one layer
+    const uint32_t layer = div_magic(line, a.magic_rows);
+    const uint32_t y = line - layer * a.rows;
+    drow = a.dst + layer * a.dst_slice + y * a.dst_pitch;
+    srow = a.src + layer * a.src_slice + y * a.src_pitch;
+  }
+  // Rows of this kernel are wider than 64 slots, so a row's head (the bytes in
+  // front of its first 16-byte aligned destination address) is never cut.
+  const unsigned head = (0u - static_cast<unsigned>(reinterpret_cast<uintptr_t>(drow))) & 15;
+  const unsigned lead = (static_cast<unsigned>(reinterpret_cast<uintptr_t>(drow)) + head) & 255;  // bytes below the body in its first unit
+  // merged rows can be longer than 2^32 vectors: 64-bit counts
+  const uint64_t n_virtual = (lead + (a.width - head)) >> 4;
+  const uint64_t units = row_units(n_virtual, kUnit);
+  if (kq != 0 && kq + 1 < units) {
+    // destination of the unit's lane 0: 256-byte aligned, kq units above the row's anchor
+    uint8_t* const d = drow + head - lead + static_cast<uint64_t>(kq) * (kUnit * 16);
+    const uint8_t* const sb = srow + (d - drow);
+    const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(sb)) & 3;
+    const v4u_a4* sv = reinterpret_cast<const v4u_a4*>(sb - r) + lane;
+    v4u* dv = reinterpret_cast<v4u*>(d) + lane;
+    v4u x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) x[u] = ld_v4<NTL>(sv + u * kWave);
+    // lane 0 fetches the dword behind the unit: with r != 0 it holds the
+    // last r bytes the unit needs, and the row goes on behind it
+    unsigned e = 0;
+    if (r && lane == 0) e = ld_u32<NTL>(reinterpret_cast<const unsigned*>(sv + kUnit));
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const unsigned nxt = (u + 1 < U) ? x[u + 1 < U ? u + 1 : u].x : e;
+      const unsigned w4 = wave_rotate_down1(lane == 0 ? nxt : x[u].x);
+      st_v4<NTS>(dv + u * kWave, realign(x[u], w4, r));
     }
     return;
   }
-  for (uint64_t w = wave; w < a.total_slots; w += n_waves) {
-    const uint32_t slot = static_cast<uint32_t>(w);
-    const uint32_t line = div_magic(slot, a.magic_slots);  // row index through all layers
-    const uint32_t kq = slot - line * a.slots;
-    const uint32_t layer = div_magic(line, a.magic_rows);
-    const uint32_t y = line - layer * a.rows;
-    BatchDesc row;
-    row.dst = a.dst + layer * a.dst_slice + y * a.dst_pitch;
-    row.src = a.src + layer * a.src_slice + y * a.src_pitch;
-    row.bytes = a.width;
-    const DescShape sh = desc_shape(row);
-    // merged rows can be longer than 2^32 vectors: 64-bit indices
-    const uint64_t n_virtual = sh.n_vec + sh.lead;
-    const uint64_t units = row_units(n_virtual, kUnit);
-    if (kq >= units) continue;
-    const bool last = kq + 1 == units;
-    const uint64_t v0 = static_cast<uint64_t>(kq) * kUnit;
-    const uint64_t lo = v0 > sh.lead ? v0 : sh.lead;
-    const uint64_t end = last ? n_virtual : v0 + kUnit;
-    const uint8_t* sb = row.src + sh.head;
-    const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(sb)) & 3;
-    const v4u_a4* sv = reinterpret_cast<const v4u_a4*>(sb - r) - sh.lead;
-    v4u* dv = reinterpret_cast<v4u*>(row.dst + sh.head) - sh.lead;
-    if (kq != 0 && !last) {
-      // A unit inside its row (most are, in a wide row): it lies above the
-      // row's lead and head, every lane has its U vectors, and it is moved
-      // like a tile of the linear copy.
-      const uint64_t base = v0 + lane;
-      v4u x[U];
+  if (kq >= units) return;  // the row has fewer units than the widest one
+  // The row's first or last unit (or its only one): a cut range of vectors,
+  // the head and tail bytes, one more predicated vector per lane for the
+  // overflow of a last unit.
+  const bool last = kq + 1 == units;
+  const unsigned lead_vecs = lead >> 4;
+  const uint64_t v0 = static_cast<uint64_t>(kq) * kUnit;
+  const uint64_t lo = v0 > lead_vecs ? v0 : lead_vecs;
+  const uint64_t end = last ? n_virtual : v0 + kUnit;
+  const uint8_t* sb = srow + head;
+  const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(sb)) & 3;
+  const v4u_a4* sv = reinterpret_cast<const v4u_a4*>(sb - r) - lead_vecs;
+  v4u* dv = reinterpret_cast<v4u*>(drow + head) - lead_vecs;
+  v4u x[U + 1];
 #pragma unroll
-      for (int u = 0; u < U; ++u) x[u] = ld_v4<NTL>(sv + base + u * kWave);
-      // lane 0 fetches the dword behind the unit: with r != 0 it holds the
-      // last r bytes the unit needs, and the row goes on behind it
-      unsigned e = 0;
-      if (r && lane == 0) e = ld_u32<NTL>(reinterpret_cast<const unsigned*>(sv + v0 + kUnit));
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const unsigned nxt = (u + 1 < U) ? x[u + 1 < U ? u + 1 : u].x : e;
-        const unsigned w4 = wave_rotate_down1(lane == 0 ? nxt : x[u].x);
-        st_v4<NTS>(dv + base + u * kWave, realign(x[u], w4, r));
-      }
-      continue;
-    }
-    // U vectors per lane, and one more for the overflow of a row's last unit
-    v4u x[U + 1];
-#pragma unroll
-    for (int u = 0; u <= U; ++u) {
-      const uint64_t idx = v0 + lane + u * kWave;
-      if (idx >= lo && idx < end) x[u] = ld_v4<NTL>(sv + idx);
-    }
-    // the dword behind the unit's last vector: with r != 0 it holds that
-    // vector's last r bytes
-    unsigned e = 0;
-    if (r && end > lo) e = ld_u32<NTL>(reinterpret_cast<const unsigned*>(sv + end));
-#pragma unroll
-    for (int u = 0; u <= U; ++u) {
-      const uint64_t idx = v0 + lane + u * kWave;
-      const unsigned nxt = x[u < U ? u + 1 : u].x;  // lane 0's copy is what lane 63 needs
-      unsigned w4 = wave_rotate_down1(lane == 0 ? nxt : x[u].x);
-      if (idx + 1 == end) w4 = e;
-      if (idx >= lo && idx < end) st_v4<NTS>(dv + idx, realign(x[u], w4, r));
-    }
-    // bytes in front of the first vector and behind the last
-    const unsigned tail = static_cast<unsigned>(row.bytes - sh.head - 16 * sh.n_vec);
-    if (kq == 0 && lane < sh.head) {
-      row.dst[lane] = row.src[lane];
-    } else if (last && lane >= 16 && lane - 16 < tail) {
-      const uint64_t off = sh.head + 16 * sh.n_vec + lane - 16;
-      row.dst[off] = row.src[off];
-    }
+  for (int u = 0; u <= U; ++u) {
+    const uint64_t idx = v0 + lane + u * kWave;
+    if (idx >= lo && idx < end) x[u] = ld_v4<NTL>(sv + idx);
   }
+  // the dword behind the unit's last vector: with r != 0 it holds that
+  // vector's last r bytes
+  unsigned e = 0;
+  if (r && end > lo) e = ld_u32<NTL>(reinterpret_cast<const unsigned*>(sv + end));
+#pragma unroll
+  for (int u = 0; u <= U; ++u) {
+    const uint64_t idx = v0 + lane + u * kWave;
+    const unsigned nxt = x[u < U ? u + 1 : u].x;  // lane 0's copy is what lane 63 needs
+    unsigned w4 = wave_rotate_down1(lane == 0 ? nxt : x[u].x);
+    if (idx + 1 == end) w4 = e;
+    if (idx >= lo && idx < end) st_v4<NTS>(dv + idx, realign(x[u], w4, r));
+  }
+  // bytes in front of the first vector and behind the last
+  const uint64_t body_end = head + 16 * (n_virtual - lead_vecs);
+  const unsigned tail = static_cast<unsigned>(a.width - body_end);
+  if (kq == 0 && lane < head) {
+    drow[lane] = srow[lane];
+  } else if (last && lane >= 16 && lane - 16 < tail) {
+    const uint64_t off = body_end + lane - 16;
+    drow[off] = srow[off];
+  }
+}
+
+template <int U, bool NTL, int NTS>
+__device__ __forceinline__ void rect_copy_body(const RectArgs& a) {
+  const unsigned lane = threadIdx.x & (kWave - 1);
+  uint64_t w = global_wave_xcd(a.waves_per_wg, a.xcd);
+  if (w >= a.total_slots) return;
+  // A grid with a wave for every unit slot (the usual case) goes through the
+  // body once; waves of a capped grid stride over the slots.
+  if (a.plain_rows) {
+    do {
+      rect_plain_unit<U, NTL, NTS>(a, static_cast<uint32_t>(w), lane);
+      w += a.n_waves;
+    } while (w < a.total_slots);
+    return;
+  }
+  do {
+    rect_unit<U, NTL, NTS>(a, static_cast<uint32_t>(w), lane);
+    w += a.n_waves;
+  } while (w < a.total_slots);
 }
 
 // Moves bytes [off, end) of the 16-byte aligned destination slot `slot`, not

@@ -132,22 +132,6 @@ class Runner:
         self.tstream.synchronize()
         return [ev[i].elapsed_time(ev[i + 1]) * 1e3 for i in range(steps)]
 
-    def time_groups(self, fn, groups, per_group, idle_s):
-        """Mean microseconds per launch of consecutive groups of launches,
-        starting after `idle_s` seconds without work: how a burst of launches
-        settles after an idle period."""
-        torch = self.torch
-        self.tstream.synchronize()
-        time.sleep(idle_s)
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(groups + 1)]
-        ev[0].record(self.tstream)
-        for g in range(groups):
-            for _ in range(per_group):
-                fn()
-            ev[g + 1].record(self.tstream)
-        self.tstream.synchronize()
-        return [round(ev[g].elapsed_time(ev[g + 1]) * 1e3 / per_group, 2) for g in range(groups)]
-
     def check(self, st, what):
         self.capi.check(st, what)
 
@@ -801,8 +785,12 @@ def main():
     achieved = algo / dev_us / 1e3
     # the same launches one by one (median, best), right behind the timed region
     each = sorted(r.time_each(fn, max(args.steps, 5), 0))
-    # and how a burst settles after an idle period: mean per launch of 8 groups of 10
-    hump = r.time_groups(fn, 8, 10, 2.0) if not args.no_also else None
+    # and how a burst of launches runs after an idle period: 60 launches one by one after 2 s without work
+    hump = None
+    if not args.no_also:
+        r.tstream.synchronize()
+        time.sleep(2.0)
+        hump = [round(u, 1) for u in r.time_each(fn, 60, 0)]
 
     also = {}
     if not args.no_also:
@@ -846,12 +834,13 @@ def main():
                                         "an event between every two (each figure includes the event's few "
                                         "microseconds of queue time; kernel_us, the mean, does not)" % len(each)},
         "idle_hump": None if hump is None else {
-            "us_per_launch_in_groups_of_10": hump,
-            "what": "80 back-to-back launches of the headline workload after 2 s without work, mean per launch of "
-                    "each group of 10: the first launches after an idle period run fastest and the pace then "
-                    "settles 3-5 % lower while the clocks the driver reports stay where they are "
-                    "(profiles/copy_after_idle.md); the timed region above is whatever the requested warm-up "
-                    "puts it on"},
+            "us_per_launch": hump,
+            "what": "60 back-to-back launches of the headline workload after 2 s without work, timed one by one "
+                    "(an event between every two).  On this GPU a burst that follows an idle period often runs "
+                    "about 4 % slow for some 3 ms, from about 3.5 ms in (launches 11-20 of 1 GiB copies), in some "
+                    "bursts and not in others, while the clocks the driver reports stay where they are "
+                    "(profiles/copy_after_idle.md).  A timed region of 20 steps behind 5 warm-up launches lies "
+                    "across that window; the default warm-up of 60 launches lies behind it"},
         "also": also,
     }
     if not args.no_cpu_baseline:

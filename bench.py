@@ -51,6 +51,8 @@ def parse_args():
     ap.add_argument("--bytes", type=int, default=GIB, help="transfer size of the copy/fill workloads")
     ap.add_argument("--rect", default="8192,131072,262144,0,0",
                     help="shape of the rect workload: rows,width,pitch[,source x,destination x] in bytes")
+    ap.add_argument("--path", default="aql", choices=["aql", "hip"],
+                    help="submission path of the idle_series workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true",
                     help="skip the check of the timed workload's result (for runs under a profiler, whose trace "
@@ -724,6 +726,23 @@ def cpu_baseline(ora, budget_s):
     return out
 
 
+def idle_series_hip(pkg, torch, nbytes, launches, idle_s, bursts=3):
+    """The HIP path's counterpart of idle_series: `bursts` bursts of back-to-back
+    copies of nbytes, each after idle_s seconds without work, every launch
+    timed by an event recorded behind it (so each figure includes what an event
+    costs the queue).  Under `rocprofv3 --kernel-trace` the trace holds the
+    kernels' own durations for the same launches."""
+    r = Runner(torch, pkg)
+    fn, _, _, keep = make_copy(r, nbytes)
+    series = []
+    for _ in range(bursts):
+        r.tstream.synchronize()
+        time.sleep(idle_s)
+        series.append([round(x, 1) for x in r.time_each(fn, launches, 0)])
+    return {"metric": "pace of back-to-back %d MiB copies after %.1f s idle, HIP path" % (nbytes // MIB, idle_s),
+            "unit": "us per launch", "launches": launches, "pace_us": series}
+
+
 def load_traffic(kernel_key):
     """HBM bytes per launch from committed rocprofv3 --pmc runs (FETCH_SIZE +
     WRITE_SIZE, scaled by a plain copy kernel of known size), if recorded."""
@@ -744,7 +763,8 @@ def main():
         sys.exit("bench.py needs a GPU")
     pkg = entry.load_package()
     if args.workload == "idle_series":
-        print(json.dumps(idle_series(pkg, torch, args.bytes, max(args.steps, 10), 3.0)))
+        series = idle_series if args.path == "aql" else idle_series_hip
+        print(json.dumps(series(pkg, torch, args.bytes, max(args.steps, 10), 3.0)))
         return
     r = Runner(torch, pkg)
     nbytes = args.bytes

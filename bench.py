@@ -296,9 +296,14 @@ def rect_shapes(r):
         fn, verify, algo, keep = make_rect(r, rows, width, pitch, sx, dx)
         _, us = r.time_launches(fn, 20, WARMUP_AFTER_IDLE)
         verify()
-        out["%dx%d/%d+%d,%d" % (rows, width, pitch, sx, dx)] = {
-            "gbs": round(algo / us / 1e3, 1), "us_per_launch": round(us, 2),
-            "unroll": r.blit.last_plan().unroll}
+        rec = {"gbs": round(algo / us / 1e3, 1), "us_per_launch": round(us, 2),
+               "unroll": r.blit.last_plan().unroll}
+        # HBM bytes per launch from the committed counter runs, where this shape has one: rows that
+        # use part of every 128-byte line they touch move more bytes than they copy
+        traffic = load_traffic("rect_%dx%d_%d" % (rows, width, pitch)) if (sx, dx) == (0, 0) else None
+        if traffic:
+            rec["hbm_traffic_gbs"] = round(traffic / us / 1e3, 1)
+        out["%dx%d/%d+%d,%d" % (rows, width, pitch, sx, dx)] = rec
         del fn, verify, keep
         r.torch.cuda.empty_cache()
     return out

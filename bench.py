@@ -47,7 +47,7 @@ def parse_args():
     # default warm-up covers it.
     ap.add_argument("--warmup", type=int, default=WARMUP_AFTER_IDLE)
     ap.add_argument("--workload", default="copy",
-                    choices=["copy", "fill", "misaligned", "batch", "rect", "calib", "idle_series"])
+                    choices=["copy", "fill", "misaligned", "batch", "rect", "calib", "idle_series", "batch_layouts"])
     ap.add_argument("--bytes", type=int, default=GIB, help="transfer size of the copy/fill workloads")
     ap.add_argument("--rect", default="8192,131072,262144,0,0",
                     help="shape of the rect workload: rows,width,pitch[,source x,destination x] in bytes")
@@ -235,6 +235,83 @@ def make_batch(r, n=65536, arena=8 * GIB):
         # nothing was written between the regions: the bytes that are not zero are at most the copies' own
         assert int((dst != 0).sum().item()) <= int(lens.sum()), "bytes written outside the copies"
     return fn, verify, int(2 * lens.sum()), (src, dst, descs)
+
+
+def batch_layouts(r, n=65536, arena=8 * GIB):
+    """Where a batch's time goes, from the product path alone: the benchmark's
+    65,536 copies laid out in other ways, and other batches of the same size,
+    each timed like the headline (20 back-to-back submissions behind the
+    warm-up) and checked on a sample of 512 copies.  The arenas are the
+    benchmark's: 8 GiB of source, 8 GiB of destination."""
+    import numpy as np
+    lens, so, do, offs, _stride = batch_layout(n, arena)
+    src = r.torch.empty(arena + 512, dtype=r.torch.uint8, device="cuda:0")
+    dst = r.torch.empty(arena + 512, dtype=r.torch.uint8, device="cuda:0")
+    blk_d = r.torch.from_numpy(seeded_bytes(64 * MIB, 0xB1170005)).to("cuda:0")
+    for lo in range(0, arena, 64 * MIB):
+        src[lo:lo + 64 * MIB].copy_(blk_d[:min(64 * MIB, arena - lo)])
+    r.torch.cuda.synchronize()
+    S, D = aligned_ptr(src), aligned_ptr(dst)
+    sh, dh = S - src.data_ptr(), D - dst.data_ptr()
+    need = ((lens + 255) // 256) * 256 + 256
+    packed = np.concatenate([[0], np.cumsum(need)[:-1]]) + 256
+
+    def clustered(cluster_bytes):
+        """Dense clusters of about cluster_bytes, the clusters spread evenly over the arena."""
+        out = np.empty(n, dtype=np.int64)
+        gap_ratio = (arena - 4096) / float(need.sum())
+        at, start, filled = 256, 0, 0
+        for i in range(n):
+            if filled >= cluster_bytes:
+                start = start + int(filled * gap_ratio) // 4096 * 4096
+                at, filled = start + 256, 0
+            out[i] = at
+            at += int(need[i])
+            filled += int(need[i])
+        assert at < arena
+        return out
+
+    zero = so * 0
+    whole = (lens // 4096 + 1) * 4096
+    even = np.full(n, 32 * 1024, dtype=np.int64)
+    layouts = [
+        ("benchmark: spread over the arenas, byte offsets 0..15", offs, so, do, lens),
+        ("the same copies packed, 256-byte gaps", packed, so, do, lens),
+        ("the same copies in dense clusters of 2 MiB spread over the arenas", clustered(2 * MIB), so, do, lens),
+        ("the same copies in dense clusters of 512 KiB spread over the arenas", clustered(512 * 1024), so, do, lens),
+        ("benchmark placement, source and destination 256-byte aligned", offs, zero, zero, lens),
+        ("benchmark placement, aligned, lengths rounded up to whole 4 KiB chunks", offs, zero, zero, whole),
+        ("65,536 copies of 32 KiB, contiguous", np.arange(n, dtype=np.int64) * 32768, zero, zero, even),
+        ("8,192 copies of 256 KiB, contiguous", np.arange(8192, dtype=np.int64) * 262144, zero[:8192], zero[:8192],
+         np.full(8192, 262144, dtype=np.int64)),
+        ("1 copy of 2 GiB", np.zeros(1, dtype=np.int64), zero[:1], zero[:1], np.full(1, 2 * GIB, dtype=np.int64)),
+    ]
+    rng = np.random.default_rng(0xB1170105)
+    out = {}
+    for name, at, s_off, d_off, ln in layouts:
+        m = len(ln)
+        descs = (r.capi.Desc * m)()
+        for i in range(m):
+            descs[i].dst = D + int(at[i] + d_off[i])
+            descs[i].src = S + int(at[i] + s_off[i])
+            descs[i].bytes = int(ln[i])
+        fn = lambda: r.check(r.blit.copy_batch(descs, m, False, r.stream), "copy_batch")
+        dst.zero_()
+        r.torch.cuda.synchronize()
+        _, us = r.time_launches(fn, 20, WARMUP_AFTER_IDLE)
+        for i in (range(m) if m <= 512 else rng.integers(0, m, 512)):
+            a = dst[dh + int(at[i] + d_off[i]):dh + int(at[i] + d_off[i] + ln[i])]
+            b = src[sh + int(at[i] + s_off[i]):sh + int(at[i] + s_off[i] + ln[i])]
+            assert r.torch.equal(a, b), "%s: copy %d differs" % (name, i)
+        algo = 2 * int(ln.sum())
+        out[name] = {"us_per_batch": round(us, 1), "bytes": algo, "gbs": round(algo / us / 1e3, 1),
+                     "frac_of_peak": round(algo / us / 1e3 / HBM_PEAK_GBS, 4)}
+    fn = lambda: r.check(r.blit.copy(D, S, 2 * GIB, r.stream), "copy")
+    _, us = r.time_launches(fn, 20, WARMUP_AFTER_IDLE)
+    out["for comparison: linear copy of 2 GiB"] = {"us_per_launch": round(us, 1), "bytes": 4 * GIB,
+                                                  "gbs": round(4 * GIB / us / 1e3, 1),
+                                                  "frac_of_peak": round(4 * GIB / us / 1e3 / HBM_PEAK_GBS, 4)}
+    return out
 
 
 def make_batch_device(r):
@@ -773,6 +850,11 @@ def main():
         return
     r = Runner(torch, pkg)
     nbytes = args.bytes
+    if args.workload == "batch_layouts":
+        print(json.dumps({"metric": "batched copy on several layouts", "unit": "us per batch",
+                          "layouts": batch_layouts(r)}))
+        r.blit.close()
+        return
 
     if args.workload == "copy":
         fn, verify, algo, keep = make_copy(r, nbytes)

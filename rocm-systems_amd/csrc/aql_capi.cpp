@@ -993,7 +993,7 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   }
   hsa_signal_store_relaxed(h->stage_free[b], 1);
 
-  // 1. one lane per piece writes the piece's chunk records
+  // 1. the chunk records, kEmitPiecesPerWave pieces to a wave
   EmitRecordsArgs er{h->stage[b], reinterpret_cast<const uint32_t*>(h->stage[b] + shape.pieces), shape.pieces,
                      h->records_dev};
 
@@ -1015,7 +1015,7 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   // Both packets wait for everything before them (barrier bit): the first for
   // whatever still reads the shared record buffer; it frees the staging buffer
   // when it is done with it.
-  write_dispatch(h, i++, h->emit_records, &er, sizeof(er), static_cast<uint32_t>((shape.pieces + 255) / 256), 256,
+  write_dispatch(h, i++, h->emit_records, &er, sizeof(er), emit_records_grid(shape.pieces), 256,
                  h->stage_free[b].handle, true, Chain::kFirst);
   write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true, Chain::kLast);
   release_write_index(h, index, total);

@@ -137,7 +137,15 @@ struct ScanTopArgs {
 };
 
 // Host-resident descriptors: the host has cut them into pieces and summed
-// their chunk counts; one lane per piece writes the piece's records.
+// their chunk counts.  A wave of the record kernel takes kEmitPiecesPerWave
+// pieces, one in each of its first lanes, and all of its 64 lanes write their
+// records; emit_records_grid is the number of 256-lane workgroups n pieces need.
+constexpr unsigned kEmitPiecesPerWave = 8;
+inline uint32_t emit_records_grid(uint64_t n) {
+  const uint64_t per_wg = 4 * kEmitPiecesPerWave;
+  return static_cast<uint32_t>((n + per_wg - 1) / per_wg);
+}
+
 struct EmitRecordsArgs {
   const BatchDesc* descs;       // staged by the host
   const uint32_t* first_record; // index of each piece's first record

@@ -700,11 +700,10 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
   if (walk) {
     // The image the host staged (the descriptors, cut into pieces of at most 64
     // chunks, and each piece's first record index) is all the GPU needs to
-    // write the records, a wave for 64 pieces.
+    // write the records, a wave for kEmitPiecesPerWave pieces.
     const BatchDesc* staged = h->descs_host[b];
     EmitRecordsArgs er{staged, reinterpret_cast<const uint32_t*>(staged + shape.pieces), shape.pieces, h->records_dev};
-    hipLaunchKernelGGL(mi355_batch_emit_records, dim3(static_cast<uint32_t>((shape.pieces + 255) / 256)), dim3(256),
-                       0, s, er);
+    hipLaunchKernelGGL(mi355_batch_emit_records, dim3(emit_records_grid(shape.pieces)), dim3(256), 0, s, er);
     BLIT_HIP(hipGetLastError());
 
     rc = launch_records_copy(h, s, p, l, shape.total_chunks);

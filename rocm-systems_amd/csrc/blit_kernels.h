@@ -453,18 +453,22 @@ __device__ __forceinline__ ChunkRecord make_record(const BatchDesc& d, uint32_t 
   return r;
 }
 
-// Launched with workgroups of 256, one lane per (piece of a) copy.  A wave
-// writes the records of its 64 copies together: their chunk counts are summed
-// across the wave, and lane l writes records l, l + 64, ... of the wave's
-// combined list, finding each record's copy by bisecting the running sum with
-// lane shuffles.  The work is balanced whatever the mix of lengths, and
-// consecutive lanes write consecutive records (whole cache lines); one lane
-// writing all records of its own copy took 22 us for the benchmark's 542,613
-// records, this takes 11.  The descriptors and the record indices were written
+// Launched with workgroups of 256 (emit_records_grid).  A wave takes
+// kEmitPiecesPerWave (pieces of) copies, one in each of its first lanes, and
+// writes their records together: the chunk counts are summed across the wave,
+// and lane l writes records l, l + 64, ... of the wave's combined list, finding
+// each record's copy by bisecting the running sum with lane shuffles.  The
+// work is balanced whatever the mix of lengths, and consecutive lanes write
+// consecutive records (whole cache lines).  One lane writing all records of
+// its own copy took 22 us for the benchmark's 542,613 records and 64 copies to
+// a wave 11 us; but 64 copies to a wave is 64 rounds for a wave whose pieces
+// are all 64 chunks long, and few waves: one copy of 2 GiB (8,192 pieces) took
+// 37 us.  The descriptors and the record indices were written
 // by the host, into host memory or across the bus into device memory, behind
 // the GPU's caches: they are read at system scope.
-// Writes the records of one wave's 64 copies: lane l holds copy (dst, src,
-// bytes) with `chunks` records, the wave's records start at out[0].
+// Writes the records of one wave's copies: lane l holds copy (dst, src,
+// bytes) with `chunks` records (none in a lane without a copy), the wave's
+// records start at out[0].
 __device__ __forceinline__ void emit_wave_records(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t chunks,
                                                   ChunkRecord* out, unsigned lane) {
   // exclusive running sum of the chunk counts over the wave's lanes
@@ -504,8 +508,9 @@ __device__ __forceinline__ void emit_wave_records(uint64_t dst, uint64_t src, ui
 
 __device__ __forceinline__ void emit_records_body(const EmitRecordsArgs& a) {
   const unsigned lane = threadIdx.x & (kWave - 1);
-  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
-  const bool valid = i < a.n;
+  const uint64_t wave = static_cast<uint64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
+  const uint64_t i = wave * kEmitPiecesPerWave + lane;
+  const bool valid = lane < kEmitPiecesPerWave && i < a.n;
   uint64_t dst = 0, src = 0, bytes = 0;
   uint32_t first = 0;
   if (valid) {

@@ -53,6 +53,8 @@ def parse_args():
                     help="shape of the rect workload: rows,width,pitch[,source x,destination x] in bytes")
     ap.add_argument("--path", default="aql", choices=["aql", "hip"],
                     help="submission path of the idle_series workload")
+    ap.add_argument("--constant-bytes", action="store_true",
+                    help="idle_series: copy a source of constant bytes instead of the workload's seeded random ones")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true",
                     help="skip the check of the timed workload's result (for runs under a profiler, whose trace "
@@ -72,6 +74,22 @@ def seeded_bytes(n, seed):
     return np.random.default_rng(seed).integers(0, 256, n, dtype=np.uint8)
 
 
+def device_bytes(torch, n, seed=None):
+    """n + 512 bytes of device memory; with a seed, n seeded bytes from the
+    first 256-byte boundary on."""
+    t = torch.empty(n + 512, dtype=torch.uint8, device="cuda:0")
+    if seed is not None:
+        # seeded on the host, in 64 MiB pieces
+        step = 64 * MIB
+        off = (-t.data_ptr()) % 256
+        for lo in range(0, n, step):
+            m = min(step, n - lo)
+            host = seeded_bytes(m, seed + lo // step)
+            t[off + lo:off + lo + m].copy_(torch.from_numpy(host))
+    torch.cuda.synchronize()
+    return t
+
+
 class Runner:
     def __init__(self, torch, pkg):
         self.torch = torch
@@ -84,18 +102,7 @@ class Runner:
         assert self.stream, "need a non-null stream"
 
     def device_bytes(self, n, seed=None):
-        import numpy as np
-        t = self.torch.empty(n + 512, dtype=self.torch.uint8, device="cuda:0")
-        if seed is not None:
-            # seeded on the host, in 64 MiB pieces
-            step = 64 * MIB
-            off = (-t.data_ptr()) % 256
-            for lo in range(0, n, step):
-                m = min(step, n - lo)
-                host = seeded_bytes(m, seed + lo // step)
-                t[off + lo:off + lo + m].copy_(self.torch.from_numpy(host))
-        self.torch.cuda.synchronize()
-        return t
+        return device_bytes(self.torch, n, seed)
 
     def time_launches(self, fn, steps, warmup):
         """W untimed + K timed back-to-back launches.  Returns (wall seconds for
@@ -653,12 +660,15 @@ def reference_rect(r, hsa, S, D):
     return round(2 * rows * width / best / 1e9, 1) if best else None
 
 
-def idle_series(pkg, torch, nbytes, launches, idle_s):
+def idle_series(pkg, torch, nbytes, launches, idle_s, constant_bytes=False):
     """How a burst of back-to-back copies of nbytes settles after idle_s seconds
     without work: the pace of every launch (end of command i minus end of
     command i-1, from the packet processor's timestamps in the completion
     signals, AQL path) next to the clocks and the power the driver reports in
-    sysfs, sampled every millisecond by a host thread while the burst runs."""
+    sysfs, sampled every millisecond by a host thread while the burst runs.
+    The source holds the headline workload's seeded bytes or, as a control,
+    the same byte everywhere: what the device's power management does to a
+    burst depends on how much the data toggles."""
     import glob
     import threading
     aql = pkg.aql
@@ -683,7 +693,9 @@ def idle_series(pkg, torch, nbytes, launches, idle_s):
 
     eng = aql.AqlBlit(0)
     sig = aql.HsaSignals()
-    a = torch.empty(nbytes + 512, dtype=torch.uint8, device="cuda:0").fill_(3)
+    a = device_bytes(torch, nbytes, None if constant_bytes else 0xB1170003)
+    if constant_bytes:
+        a.fill_(3)
     b = torch.empty(nbytes + 512, dtype=torch.uint8, device="cuda:0").fill_(5)
     A, B = aligned_ptr(a), aligned_ptr(b)
     torch.cuda.synchronize()
@@ -724,7 +736,8 @@ def idle_series(pkg, torch, nbytes, launches, idle_s):
         if smp[1:] != last:
             changes.append([round((smp[0] - t0) * 1e3, 1)] + list(smp[1:]))
             last = smp[1:]
-    return {"metric": "pace of back-to-back %d MiB copies after %.1f s idle" % (nbytes // MIB, idle_s),
+    return {"metric": "pace of back-to-back %d MiB copies of %s bytes after %.1f s idle, AQL path" % (
+                nbytes // MIB, "constant" if constant_bytes else "seeded random", idle_s),
             "unit": "us per launch", "launches": launches, "pace_us": pace,
             "sysfs_columns": ["ms since first submit"] + sorted(paths), "sysfs_changes": changes}
 
@@ -808,7 +821,7 @@ def cpu_baseline(ora, budget_s):
     return out
 
 
-def idle_series_hip(pkg, torch, nbytes, launches, idle_s, bursts=3):
+def idle_series_hip(pkg, torch, nbytes, launches, idle_s, constant_bytes=False, bursts=3):
     """The HIP path's counterpart of idle_series: `bursts` bursts of back-to-back
     copies of nbytes, each after idle_s seconds without work, every launch
     timed by an event recorded behind it (so each figure includes what an event
@@ -816,12 +829,17 @@ def idle_series_hip(pkg, torch, nbytes, launches, idle_s, bursts=3):
     kernels' own durations for the same launches."""
     r = Runner(torch, pkg)
     fn, _, _, keep = make_copy(r, nbytes)
+    if constant_bytes:
+        keep[0].fill_(3)
+        fn()
     series = []
     for _ in range(bursts):
         r.tstream.synchronize()
+        torch.cuda.synchronize()
         time.sleep(idle_s)
         series.append([round(x, 1) for x in r.time_each(fn, launches, 0)])
-    return {"metric": "pace of back-to-back %d MiB copies after %.1f s idle, HIP path" % (nbytes // MIB, idle_s),
+    return {"metric": "pace of back-to-back %d MiB copies of %s bytes after %.1f s idle, HIP path" % (
+                nbytes // MIB, "constant" if constant_bytes else "seeded random", idle_s),
             "unit": "us per launch", "launches": launches, "pace_us": series}
 
 
@@ -846,7 +864,7 @@ def main():
     pkg = entry.load_package()
     if args.workload == "idle_series":
         series = idle_series if args.path == "aql" else idle_series_hip
-        print(json.dumps(series(pkg, torch, args.bytes, max(args.steps, 10), 3.0)))
+        print(json.dumps(series(pkg, torch, args.bytes, max(args.steps, 10), 3.0, args.constant_bytes)))
         return
     r = Runner(torch, pkg)
     nbytes = args.bytes
@@ -893,11 +911,24 @@ def main():
     # the same launches one by one (median, best), right behind the timed region
     each = sorted(r.time_each(fn, max(args.steps, 5), 0))
     # and how a burst of launches runs after an idle period: 60 launches one by one after 2 s without work
-    hump = None
+    hump = hump_constant = None
     if not args.no_also:
         r.tstream.synchronize()
         time.sleep(2.0)
         hump = [round(u, 1) for u in r.time_each(fn, 60, 0)]
+        hump_constant = None
+        if args.workload == "copy":
+            # the control: the same burst with a source of constant bytes
+            const_src = r.device_bytes(nbytes + 64)
+            const_src.fill_(3)
+            D = aligned_ptr(keep[1])
+            fn_const = lambda: r.check(r.blit.copy(D, aligned_ptr(const_src), nbytes, r.stream), "copy")
+            fn_const()
+            r.tstream.synchronize()
+            torch.cuda.synchronize()
+            time.sleep(2.0)
+            hump_constant = [round(u, 1) for u in r.time_each(fn_const, 40, 0)]
+            del const_src
 
     also = {}
     if not args.no_also:
@@ -942,12 +973,16 @@ def main():
                                         "microseconds of queue time; kernel_us, the mean, does not)" % len(each)},
         "idle_hump": None if hump is None else {
             "us_per_launch": hump,
+            "us_per_launch_constant_bytes": hump_constant,
             "what": "60 back-to-back launches of the headline workload after 2 s without work, timed one by one "
-                    "(an event between every two).  On this GPU a burst that follows an idle period often runs "
-                    "about 4 % slow for some 3 ms, from about 3.5 ms in (launches 11-20 of 1 GiB copies), in some "
-                    "bursts and not in others, while the clocks the driver reports stay where they are "
-                    "(profiles/copy_after_idle.md).  A timed region of 20 steps behind 5 warm-up launches lies "
-                    "across that window; the default warm-up of 60 launches lies behind it"},
+                    "(an event between every two), and as a control 40 launches of the same copy from a source "
+                    "of constant bytes (every byte 3), also after 2 s without work.  With the workload's random "
+                    "bytes a burst that follows an idle period runs 4-10 % slow for some 3 ms, from about 3.5 ms "
+                    "in (launches 11-20 of 1 GiB copies), on either submission path and whatever the host does "
+                    "meanwhile; with constant bytes it does not, and the clocks the driver reports stay where "
+                    "they are: the device's power management answering the current that toggling data draws, "
+                    "not the kernel (profiles/copy_after_idle.md).  A timed region of 20 steps behind 5 warm-up "
+                    "launches lies across that window; the default warm-up of 60 launches lies behind it"},
         "also": also,
     }
     if not args.no_cpu_baseline:

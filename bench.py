@@ -364,9 +364,11 @@ def make_rect(r, rows=8192, width=128 * 1024, pitch=256 * 1024, s_x=0, d_x=0):
 
 
 RECT_SHAPES = (
-    # rows, width, pitch, src x, dst x: 1 GiB moved each (the last two 256 MiB)
+    # rows, width, pitch, src x, dst x: 1 GiB moved each (the last two 256 MiB); the third has a pitch that is
+    # not a power of two
     (8192, 128 * 1024, 256 * 1024, 0, 0),
     (8192, 128 * 1024 - 7, 256 * 1024 + 4, 3, 9),
+    (8192, 128 * 1024, 260 * 1024, 0, 0),
     (262144, 4096, 8192, 0, 0),
     (1048576, 1024, 2048, 0, 0),
     (1048576, 256, 512, 0, 0),

@@ -62,6 +62,32 @@ inline uint64_t rect_gcd(uint64_t a, uint64_t b) {
   return a;
 }
 
+// Whether rows of whole cache lines are better written through L2 (sc1, the
+// linear copy's stores) than with non-temporal stores.  Measured on MI355X
+// over some 90 shapes of 0.125 to 1 GiB, rows of 128 bytes to 128 KiB at
+// pitches of 1.002 to 8 times the width, GB/s of bytes moved, sc1 against nt:
+//  * rows under 1 KiB (a wave stores pieces of several rows): sc1 wins at
+//    every pitch, by 1 to 18 % (512-byte rows at a 2176-byte pitch 6956 against
+//    5891, 128-byte rows at 384 bytes 6812 against 5867);
+//  * rows of 1 KiB and more (every wave stores one contiguous KiB): sc1 wins by
+//    3 to 9 % when the pitch is a power of two (4 KiB rows at 8 KiB 6648 against
+//    6141) or a multiple of 128 KiB (128 KiB rows at 384 KiB 6572 against 6351),
+//    is level at multiples of 64 KiB, and loses by 4 to 20 % at any other pitch
+//    (2 KiB rows at 4352 bytes 5330 against 6384, 16 KiB rows at 68 KiB 5493
+//    against 6074, 128 KiB rows at 260 KiB 5775 against 6419), unless the rows
+//    nearly abut (a gap of up to 3 % of the pitch: 16 KiB rows at 16,640 bytes
+//    6531 against 6382).
+// The batched copy, whose chunks lie at arbitrary 256-byte boundaries, shows
+// the same preference for nt.  What the pitch changes is the order in which
+// the rows' lines reach the memory channels; the rule is what the measurements
+// say, not a model of them.
+inline bool rect_whole_lines_write_through(uint64_t width, uint64_t dst_pitch) {
+  if (width < 1024) return true;
+  const uint64_t pow2_divisor = dst_pitch & (~dst_pitch + 1);
+  if (pow2_divisor == dst_pitch || pow2_divisor >= (64u << 10)) return true;
+  return dst_pitch >= width && (dst_pitch - width) * 32 <= dst_pitch;
+}
+
 inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset, const mi355_pitched_ptr_t* src,
                      const mi355_dim3_t* src_offset, const mi355_dim3_t* range, const mi355_blit_tuning_t* t,
                      RectPlan* out, uint32_t route = MI355_BLIT_ROUTE_DEVICE) {
@@ -168,13 +194,15 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
     n.magic64 = magic_divisor(n.lanes_per_row);
     out->unroll = 1;
     // Measured on MI355X with 2^20 rows.  When every store is a whole cache
-    // line, single-wave workgroups and written-through stores are best (1 KiB
-    // rows 312 us against 349 us, 512 B rows 167 against 177).  Waves that share
+    // line, single-wave workgroups and, at the pitches named above
+    // (rect_whole_lines_write_through), written-through stores are best (1 KiB
+    // rows at 2 KiB 312 us against 349 us, 512 B rows at 1 KiB 167 against 177).  Waves that share
     // cache lines with their neighbours want to be in one workgroup, hence on
     // one CU (520 B rows at a 1 KiB pitch, 33 lanes a row: 241 us with workgroups
     // of 256, 283 us with single waves, whose neighbours run on other XCDs), and
     // non-temporal stores.
-    if (whole_lines && streaming && !store_tuned && !to_host) out->store_policy = MI355_BLIT_STORE_AGENT_WT;
+    if (whole_lines && streaming && !store_tuned && !to_host && rect_whole_lines_write_through(width, dp))
+      out->store_policy = MI355_BLIT_STORE_AGENT_WT;
     // No two waves touch the same destination line when rows are whole lines,
     // or when waves hold whole rows and neighbouring rows are a line apart.
     const bool rows_apart = dp >= width + 127 && (layers == 1 || ds >= (rows - 1) * dp + width + 127);
@@ -211,7 +239,8 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
   // Measured on MI355X, 1 GiB moved in rows of 4 KiB and of 128 KiB.  Rows whose
   // every store is a whole cache line (first row, pitches and width multiples
   // of 128 bytes): one vector per lane, workgroups of 256 (of 64 for plain
-  // rows, below), stores written through L2 like the linear copy's, 320-326 us
+  // rows, below), stores written through L2 like the linear copy's at the
+  // pitches that suit them (rect_whole_lines_write_through), 320-326 us
   // (6.6-6.7 TB/s) against 333-341 us with the shape below.  Any other rows: two vectors per lane,
   // workgroups of 128, non-temporal stores (written-through stores lose 8-15 %
   // there: the rows' cut ends are partial lines).
@@ -230,7 +259,8 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
     unroll = 1;
     default_wg = 256;
   }
-  if (whole_lines && streaming && !store_tuned && !to_host) out->store_policy = MI355_BLIT_STORE_AGENT_WT;
+  if (whole_lines && streaming && !store_tuned && !to_host && rect_whole_lines_write_through(width, dp))
+    out->store_policy = MI355_BLIT_STORE_AGENT_WT;
   if (t && (t->unroll == 1 || t->unroll == 2 || t->unroll == 4)) unroll = t->unroll;
   out->unroll = unroll;
   // Row destinations differ by multiples of g modulo 256: the largest unit

@@ -343,6 +343,45 @@ def test_plan_rect_slots_follow_row_alignment(capi_host):
     assert st == SUCCESS and (p.lanes_per_row, p.wg_size, p.xcd_run) == (33, 256, 144)        # 4 waves x 1 KiB
 
 
+def test_plan_rect_whole_line_rows_store_policy_follows_the_pitch(capi_host):
+    """Rows of whole cache lines are written through L2 when they are under
+    1 KiB, or when the destination pitch is a power of two, a multiple of
+    64 KiB or within 3 % of the width; at any other pitch their stores are
+    non-temporal (rect_whole_lines_write_through)."""
+    base_d, base_s = 0x7f0000000000, 0x7f1000000000
+    K = 1024
+    WT, NT = capi_host.STORE_AGENT_WT, capi_host.STORE_NT
+    cases = [
+        # width, destination pitch, rows, expected
+        (128 * K, 256 * K, 8192, WT), (128 * K, 260 * K, 8192, NT), (128 * K, 384 * K, 8192, WT),
+        (128 * K, 192 * K, 8192, WT), (128 * K, 160 * K, 8192, NT), (128 * K, 132 * K, 8192, WT),
+        (128 * K, 136 * K + 128, 8192, NT),
+        (16 * K, 16 * K + 256, 65536, WT), (16 * K, 20 * K, 65536, NT), (16 * K, 32 * K, 65536, WT),
+        (2 * K, 4 * K, 262144, WT), (2 * K, 4352, 262144, NT), (2 * K, 2304, 262144, NT),
+        (1 * K, 2 * K, 524288, WT), (1 * K, 2304, 524288, NT),              # the slot kernel, one row a wave
+        (512, 2176, 524288, WT), (256, 640, 1 << 20, WT), (128, 384, 1 << 20, WT),
+    ]
+    for width, pitch, rows, want in cases:
+        st, p = capi_host.plan_rect((base_d, pitch, 0), (0, 0, 0), (base_s, pitch, 0), (0, 0, 0), (width, rows, 1))
+        assert st == SUCCESS and p.nt_load == 1 and p.store_policy == want, (width, pitch, p.store_policy)
+        # the source's pitch plays no part
+        st, p = capi_host.plan_rect((base_d, pitch, 0), (0, 0, 0), (base_s, 2 * pitch + 128, 0), (0, 0, 0), (width, rows, 1))
+        assert st == SUCCESS and p.store_policy == want, (width, pitch)
+    # with bytes to realign the rule is the same; rows that are not whole lines keep non-temporal stores
+    st, p = capi_host.plan_rect((base_d, 8448, 0), (0, 0, 0), (base_s, 8448, 0), (1, 0, 0), (4096, 262144, 1))
+    assert st == SUCCESS and p.store_policy == NT
+    st, p = capi_host.plan_rect((base_d, 8192, 0), (0, 0, 0), (base_s, 8192, 0), (1, 0, 0), (4096, 262144, 1))
+    assert st == SUCCESS and p.store_policy == WT
+    st, p = capi_host.plan_rect((base_d, 8192, 0), (16, 0, 0), (base_s, 8192, 0), (0, 0, 0), (4096, 262144, 1))
+    assert st == SUCCESS and p.store_policy == NT
+    # below 4 MiB nothing bypasses the caches, and tuning overrides the rule
+    st, p = capi_host.plan_rect((base_d, 4352, 0), (0, 0, 0), (base_s, 4352, 0), (0, 0, 0), (2048, 64, 1))
+    assert st == SUCCESS and p.store_policy == capi_host.STORE_CACHED
+    st, p = capi_host.plan_rect((base_d, 4352, 0), (0, 0, 0), (base_s, 4352, 0), (0, 0, 0), (2048, 262144, 1),
+                                capi_host.Tuning(store_policy=3))
+    assert st == SUCCESS and p.store_policy == WT
+
+
 def test_plan_rect_routes_across_the_host_link(capi_host):
     """A region one side of which is host memory: the same rows, slots and
     merging, launched as at most 128 workgroups of 256 in launch order, stores

@@ -141,7 +141,9 @@ typedef struct {
   uint32_t xcd_run;
   uint32_t batch_prefetch; /* batched copies: 0 = heuristic, 1 = no record prefetch,
                               N > 1 = touch the record N workgroups ahead */
-  uint32_t reserved;
+  uint32_t batch_staging;  /* batches of host-resident descriptors: 0 = heuristic, 1 = the host
+                              walks the descriptors, 2 = they are staged as they are and the
+                              GPU does the prefix sum */
 } mi355_blit_tuning_t;
 
 /* One element of a batched submission.  No counterpart in the reference. */
@@ -210,7 +212,11 @@ int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwo
  * descs may live in host memory (descs_on_device == 0: the library checks and
  * stages them before it returns, so the array may be reused at once) or be
  * device-resident (descs_on_device != 0: read in place, must stay
- * valid until completion).  The host cannot see the lengths of
+ * valid until completion).  Host-resident descriptors are either walked by the
+ * host (their chunks counted and summed: one small kernel before the copy) or,
+ * from 4096 copies on, staged as they are for the GPU's own prefix sum when
+ * the copies are short or no batch is running that would hide the walk
+ * (mi355_blit_tuning_t::batch_staging overrides the choice).  The host cannot see the lengths of
  * device-resident descriptors: it sizes the launch by the bytes per copy of
  * the last such batch on the handle (which the copy kernel leaves in host
  * memory; 32 KiB a copy before any has run), the kernels read the real chunk

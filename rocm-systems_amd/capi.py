@@ -50,7 +50,7 @@ class Tuning(C.Structure):
     _fields_ = [
         ("wg_size", C.c_uint32), ("unroll", C.c_uint32), ("max_grid", C.c_uint32),
         ("nt_load", C.c_uint32), ("store_policy", C.c_uint32), ("xcd_run", C.c_uint32),
-        ("batch_prefetch", C.c_uint32), ("reserved", C.c_uint32),
+        ("batch_prefetch", C.c_uint32), ("batch_staging", C.c_uint32),
     ]
 
 

@@ -170,6 +170,10 @@ struct mi355_aql {
   ChunkRecord* records_dev = nullptr;
   size_t batch_capacity = 0, records_capacity = 0;
   uint64_t* batch_seen = nullptr;  // host memory: copies << 32 | chunks of the last device-resident batch
+  // Index of the last packet of the latest batch; the engine is taken to be
+  // idle, as far as batches go, once the queue's read index has passed it.
+  uint64_t last_batch_index = 0;
+  bool any_batch = false;
 
   // bounce buffers of host<->device copies (mi355_aql_staging)
   void* bounce[2] = {nullptr, nullptr};
@@ -933,7 +937,12 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   if (n > 0xffffffffull) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   if (h->queue_error.load()) return MI355_BLIT_ERROR;
   std::unique_lock<std::mutex> g(h->lock);
-  if (batch_prefers_raw_staging(descs, n)) {
+  // The packet processor publishes the read index with a delay: a batch that
+  // has just finished may still count as running, which only means that the
+  // host walks the descriptors as it would have anyway.
+  const bool engine_idle = !h->any_batch || hsa_queue_load_read_index_scacquire(h->queue) > h->last_batch_index ||
+                           h->known_complete.load() > h->last_batch_index;
+  if (batch_prefers_raw_staging(descs, n, engine_idle, h->has_tuning ? &h->tuning : nullptr)) {
     // The walk below would take longer than the copies: stage the descriptors
     // as they are and take them from there like device-resident ones.
     int rc = ensure_batch_capacity(h, n, 0);
@@ -1019,6 +1028,8 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
                  h->stage_free[b].handle, true, Chain::kFirst);
   write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true, Chain::kLast);
   release_write_index(h, index, total);
+  h->last_batch_index = index + total - 1;
+  h->any_batch = true;
   return MI355_BLIT_SUCCESS;
 }
 
@@ -1085,6 +1096,8 @@ int copy_batch_device_locked(mi355_aql_t* h, const BatchDesc* scanned, size_t n,
                  static_cast<uint32_t>((sizing.records + 255) / 256), 256, 0, true, Chain::kMiddle);
   write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true, Chain::kLast);
   release_write_index(h, index, total);
+  h->last_batch_index = index + total - 1;
+  h->any_batch = true;
   return MI355_BLIT_SUCCESS;
 }
 

@@ -205,8 +205,19 @@ inline int batch_build(const mi355_blit_desc_t* descs, size_t n, BatchImage* ima
 constexpr size_t kBatchRawMinCopies = 4096;
 constexpr uint64_t kBatchRawMaxMeanBytes = 8192;
 
-inline bool batch_prefers_raw_staging(const mi355_blit_desc_t* descs, size_t n) {
+// engine_idle: no batch of this engine is still running, so nothing hides the
+// walk: a batch submitted to an idle engine starts as late as the host
+// finishes with it.  Staged as they are the descriptors cost the host 1 ns
+// each instead of 3.6 and the GPU two small launches more: 65,536 copies of
+// 64 B .. 256 KiB, one batch at a time, take 927 us from submission to
+// completion through the walk and 720 us as device-resident descriptors;
+// submitted back to back the walk is hidden behind the batch before and wins
+// (693 against 705 us a batch).  t->batch_staging overrides the choice.
+inline bool batch_prefers_raw_staging(const mi355_blit_desc_t* descs, size_t n, bool engine_idle,
+                                      const mi355_blit_tuning_t* t) {
+  if (t && t->batch_staging) return t->batch_staging == 2;
   if (n < kBatchRawMinCopies) return false;
+  if (engine_idle) return true;
   uint64_t sum = 0;
   const size_t step = n / 64;
   for (size_t k = 0; k < 64; ++k) sum += descs[k * step].bytes;

@@ -841,12 +841,20 @@ def test_batch_65536_copies(capi, blit, oracle, rand, torch_cuda):
     rng = np.random.default_rng(0xB1170005)
     descs, lens, offs, so, do, total2 = _make_batch(capi, rng, src, dst, n)
     assert total2 <= total
-    check_ok(capi, blit.copy_batch(descs, n), "copy_batch")
-    check_ok(capi, blit.synchronize(), "synchronize")
-    got = dst.host()
     want = np.full(total, GUARD_BYTE, dtype=np.uint8)
     want[:total2] = _expect_batch(oracle, src_host, total2, lens, offs, so, do)
-    assert np.array_equal(got, want)
+    # host-resident descriptors both ways -- walked by the host, and staged as
+    # they are for the GPU's own prefix sum -- and then as the library chooses
+    # (an idle engine gets them as they are)
+    for staging in (1, 2, 0):
+        blit.set_tuning(**({"batch_staging": staging} if staging else {}))
+        dst.fill(0, total, GUARD_BYTE)
+        torch.cuda.synchronize()
+        check_ok(capi, blit.copy_batch(descs, n), "copy_batch")
+        check_ok(capi, blit.synchronize(), "synchronize")
+        assert blit.last_plan().kernel == capi.KERNEL_COPY_BATCH
+        assert np.array_equal(dst.host(), want), "staging %d" % staging
+    blit.set_tuning()
     # the same descriptors resident in device memory: sized by the library's
     # assumption, by the batch before, and by the caller's bound
     descs_dev = _to_device(torch, descs)
@@ -907,17 +915,19 @@ def batch_arena(capi, oracle, rand, torch_cuda):
     torch.cuda.empty_cache()
 
 
-@pytest.mark.parametrize("descriptors", ["host", "device", "device_bounded"])
+@pytest.mark.parametrize("descriptors", ["host_walked", "host_as_they_are", "device", "device_bounded"])
 def test_batch_65536_copies_in_the_16_gib_arena(capi, blit, batch_arena, torch_cuda, descriptors):
     """Every byte of the 8 GiB destination -- all 65,536 copies, their guard
     bands and everything between them -- against what the oracle leaves."""
     torch = torch_cuda
     descs, n, total, dst, want = batch_arena
     dst.fill_(GUARD_BYTE)
-    dev = _to_device(torch, descs) if descriptors != "host" else None
+    dev = _to_device(torch, descs) if descriptors.startswith("device") else None
     torch.cuda.synchronize()
-    if descriptors == "host":
+    if descriptors.startswith("host"):
+        blit.set_tuning(batch_staging=1 if descriptors == "host_walked" else 2)
         st = blit.copy_batch(descs, n)
+        blit.set_tuning()
     elif descriptors == "device":
         st = blit.copy_batch(dev.data_ptr(), n, on_device=True)
     else:

@@ -940,8 +940,10 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   // The packet processor publishes the read index with a delay: a batch that
   // has just finished may still count as running, which only means that the
   // host walks the descriptors as it would have anyway.
-  const bool engine_idle = !h->any_batch || hsa_queue_load_read_index_scacquire(h->queue) > h->last_batch_index ||
-                           h->known_complete.load() > h->last_batch_index;
+  auto engine_idle = [h]() {
+    return !h->any_batch || hsa_queue_load_read_index_scacquire(h->queue) > h->last_batch_index ||
+           h->known_complete.load() > h->last_batch_index;
+  };
   if (batch_prefers_raw_staging(descs, n, engine_idle, h->has_tuning ? &h->tuning : nullptr)) {
     // The walk below would take longer than the copies: stage the descriptors
     // as they are and take them from there like device-resident ones.

@@ -213,15 +213,16 @@ constexpr uint64_t kBatchRawMaxMeanBytes = 8192;
 // completion through the walk and 720 us as device-resident descriptors;
 // submitted back to back the walk is hidden behind the batch before and wins
 // (693 against 705 us a batch).  t->batch_staging overrides the choice.
-inline bool batch_prefers_raw_staging(const mi355_blit_desc_t* descs, size_t n, bool engine_idle,
+// engine_idle is only asked when the answer depends on it.
+template <typename IdleFn>
+inline bool batch_prefers_raw_staging(const mi355_blit_desc_t* descs, size_t n, IdleFn engine_idle,
                                       const mi355_blit_tuning_t* t) {
   if (t && t->batch_staging) return t->batch_staging == 2;
   if (n < kBatchRawMinCopies) return false;
-  if (engine_idle) return true;
   uint64_t sum = 0;
   const size_t step = n / 64;
   for (size_t k = 0; k < 64; ++k) sum += descs[k * step].bytes;
-  return sum <= 64 * kBatchRawMaxMeanBytes;
+  return sum <= 64 * kBatchRawMaxMeanBytes || engine_idle();
 }
 
 // Copies the descriptors as they are to where the GPU reads them, checking

@@ -627,9 +627,11 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
   // and taken from there like device-resident ones.
   // Whether the batch before has finished: its event is the last thing it left
   // in its stream.
-  const unsigned before = h->next_host ^ 1;
-  if (h->batch_busy[before] && hipEventQuery(h->batch_done[before]) == hipSuccess) h->batch_busy[before] = false;
-  const bool engine_idle = !h->batch_busy[before];
+  auto engine_idle = [h]() {
+    const unsigned before = h->next_host ^ 1;
+    if (h->batch_busy[before] && hipEventQuery(h->batch_done[before]) == hipSuccess) h->batch_busy[before] = false;
+    return !h->batch_busy[before];
+  };
   const bool raw = !descs_on_device &&
                    batch_prefers_raw_staging(descs, n, engine_idle, h->has_tuning ? &h->tuning : nullptr);
   const bool walk = !descs_on_device && !raw;

@@ -53,6 +53,9 @@ def parse_args():
                     help="shape of the rect workload: rows,width,pitch[,source x,destination x] in bytes")
     ap.add_argument("--path", default="aql", choices=["aql", "hip"],
                     help="submission path of the idle_series workload")
+    ap.add_argument("--tune", default="",
+                    help="overrides of the launch heuristics for the timed workload, as field=value pairs of "
+                         "mi355_blit_tuning_t separated by commas (e.g. store_policy=2,xcd_run=1)")
     ap.add_argument("--constant-bytes", action="store_true",
                     help="idle_series: copy a source of constant bytes instead of the workload's seeded random ones")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -910,6 +913,9 @@ def main():
         name = "65536 batched D2D copies, 64 B..256 KiB log-uniform, offsets 0..15, 16 GiB arena"
         traffic_key = "batch_65536"
 
+    if args.tune:
+        r.check(r.blit.set_tuning(**{k: int(v) for k, v in (kv.split("=") for kv in args.tune.split(","))}), "set_tuning")
+        name += " [tuning: %s]" % args.tune
     wall, dev_us = r.time_launches(fn, args.steps, args.warmup)
     if not args.no_verify:
         verify()
@@ -918,6 +924,8 @@ def main():
     achieved = algo / dev_us / 1e3
     # the same launches one by one (median, best), right behind the timed region
     each = sorted(r.time_each(fn, max(args.steps, 5), 0))
+    if args.tune:
+        r.blit.set_tuning()
     # and how a burst of launches runs after an idle period: 60 launches one by one after 2 s without work
     hump = hump_constant = None
     if not args.no_also:

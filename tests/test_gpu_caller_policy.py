@@ -178,6 +178,58 @@ def test_packet_log(pkg, signals, torch_cuda, monkeypatch, capfd):
     assert int(dispatch.group(1)) % int(dispatch.group(2)) == 0
 
 
+def test_kernarg_ring_in_host_memory(pkg, capi, oracle, rand, torch_cuda, monkeypatch):
+    """MI355_BLIT_HOST_KERNARGS=1 keeps every kernarg slot in host memory, as the
+    reference does (amd_blit_kernel.cpp:565-569): a small copy, a copy of many
+    workgroups, a fill and a batch against the oracle."""
+    torch = torch_cuda
+    monkeypatch.setenv("MI355_BLIT_HOST_KERNARGS", "1")
+    e = pkg.aql.AqlBlit(0)
+    try:
+        n = 24 * MIB + 13
+        payload = rand(n + 64, 0xB1170009)
+        src = torch.from_numpy(payload).to("cuda:0")
+        dst = torch.full((n + 2 * GUARD,), 0xEE, dtype=torch.uint8, device="cuda:0")
+        torch.cuda.synchronize()
+        for size, s_off, d_off in ((4099, 3, 9), (n, 5, 2)):
+            dst.fill_(0xEE)
+            torch.cuda.synchronize()
+            assert e.copy(dst.data_ptr() + GUARD + d_off, src.data_ptr() + s_off, size) == 0
+            assert e.synchronize() == 0
+            want = _host(n + 2 * GUARD)
+            oracle.oracle_copy(want.ctypes.data + GUARD + d_off, payload.ctypes.data + s_off, size)
+            assert np.array_equal(dst.cpu().numpy(), want), size
+        dst.fill_(0xEE)
+        torch.cuda.synchronize()
+        assert e.fill32(dst.data_ptr() + GUARD + 4, 0xabcdef12, (n - 8) // 4) == 0
+        assert e.synchronize() == 0
+        want = _host(n + 2 * GUARD)
+        oracle.oracle_fill32(want.ctypes.data + GUARD + 4, 0xabcdef12, (n - 8) // 4)
+        assert np.array_equal(dst.cpu().numpy(), want)
+        # a batch: 300 copies of 1 .. 200,000 bytes at byte offsets
+        rng = np.random.default_rng(99)
+        m = 300
+        descs = (capi.Desc * m)()
+        dst.fill_(0xEE)
+        torch.cuda.synchronize()
+        want = _host(n + 2 * GUARD)
+        at = GUARD
+        for i in range(m):
+            ln = int(rng.integers(1, 80000))
+            so, do = int(rng.integers(0, 16)), int(rng.integers(0, 16))
+            descs[i].dst = dst.data_ptr() + at + do
+            descs[i].src = src.data_ptr() + at + so
+            descs[i].bytes = ln
+            oracle.oracle_copy(want.ctypes.data + at + do, payload.ctypes.data + at + so, ln)
+            at += (ln + 15 + 255) // 256 * 256 + 256
+        assert at < n
+        assert e.copy_batch(descs, m) == 0
+        assert e.synchronize() == 0
+        assert np.array_equal(dst.cpu().numpy(), want)
+    finally:
+        e.close()
+
+
 def test_memory_copy_pinned_host(eng, oracle, rand, torch_cuda):
     """Host memory allocated through the runtime (pinned) needs no locking."""
     torch = torch_cuda

@@ -1,8 +1,10 @@
 """Copy, fill and region copy of the HIP-stream path recorded into a HIP graph:
 each is one kernel launch with its arguments by value and no allocation, so a
-captured sequence must replay exactly.  The graph is replayed several times
-with the program's own eager work and synchronisations in between, new source
-bytes before every replay, and every replay is checked against the CPU oracle."""
+captured sequence must replay exactly; so must the allocation-free batched
+copy, whose four launches take their scratch memory from a static array.  The
+graph is replayed several times with the program's own eager work and
+synchronisations in between, new source bytes before every replay, and every
+replay is checked against the CPU oracle."""
 import numpy as np
 import pytest
 
@@ -92,4 +94,55 @@ def test_batches_refuse_a_capturing_stream(capi, torch_cuda):
         assert blit.copy_batch(descs, 2, False, None) == capi.SUCCESS
         assert blit.synchronize() == capi.SUCCESS
         assert torch.equal(dst[:4000], src[:4000]) and torch.equal(dst[4096:8096], src[4096:8096])
+        del graph
+
+
+def test_allocation_free_batch_replays_with_new_descriptors(capi, oracle, rand, torch_cuda):
+    """mi355_blit_copy_batch_bounded_noalloc is the batched copy for callers
+    that cannot allocate, a capturing stream among them: recorded once, the
+    graph reads the device-resident descriptors anew at every replay.  Four
+    replays with different descriptors and source bytes each, eager work on the
+    engine in between, every replay against the oracle."""
+    torch = torch_cuda
+    n, room = 700, 24 << 20
+    src = torch.empty(room, dtype=torch.uint8, device="cuda:0")
+    dst = torch.empty(room, dtype=torch.uint8, device="cuda:0")
+    dev = torch.zeros(n * 24, dtype=torch.uint8, device="cuda:0")
+    bound = 20 << 20
+    with capi.Blit(0) as blit:
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            s = torch.cuda.current_stream().cuda_stream
+            assert blit.copy_batch_bounded_noalloc(dev.data_ptr(), n, bound, s) == capi.SUCCESS
+        assert blit.pending_bytes() == 0
+        for replay in range(4):
+            rng = np.random.default_rng(0x6EA92000 + replay)
+            src_h = rand(room, 0x6EA93000 + replay)
+            lens = np.floor(2.0 ** (17 * rng.random(n))).astype(np.int64)     # 1 B .. 128 KiB
+            lens[rng.integers(0, n, 20)] = 0
+            stride = ((lens + 255) // 256) * 256 + 512
+            offs = np.concatenate([[0], np.cumsum(stride)[:-1]]) + 256
+            assert int(offs[-1] + stride[-1]) <= room and int(lens.sum()) <= bound
+            so, do = rng.integers(0, 16, n), rng.integers(0, 256, n)
+            descs = (capi.Desc * n)()
+            want = np.full(room, GUARD_BYTE, dtype=np.uint8)
+            for i in range(n):
+                descs[i].dst = dst.data_ptr() + int(offs[i] + do[i])
+                descs[i].src = src.data_ptr() + int(offs[i] + so[i])
+                descs[i].bytes = int(lens[i])
+                oracle.oracle_copy(want.ctypes.data + int(offs[i] + do[i]), src_h.ctypes.data + int(offs[i] + so[i]),
+                                   int(lens[i]))
+            dev.copy_(torch.from_numpy(np.frombuffer(bytes(descs), dtype=np.uint8).copy()))
+            src.copy_(torch.from_numpy(src_h))
+            dst.fill_(GUARD_BYTE)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert np.array_equal(dst.cpu().numpy(), want), "replay %d" % replay
+            # eager work between replays: a batch through the allocating entry point and a copy
+            assert blit.copy_batch(descs, n) == capi.SUCCESS
+            assert blit.copy(dst.data_ptr(), src.data_ptr(), 4096) == capi.SUCCESS
+            assert blit.synchronize() == capi.SUCCESS
         del graph

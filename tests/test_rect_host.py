@@ -382,6 +382,40 @@ def test_plan_rect_whole_line_rows_store_policy_follows_the_pitch(capi_host):
     assert st == SUCCESS and p.store_policy == WT
 
 
+def test_plan_rect_plain_rows_order_follows_the_pitches(capi_host):
+    """Plain rows of a large region run in XCD runs of 576 units, except in the
+    narrow window where launch order was measured to win: both pitches powers of
+    two, rows of 4 KiB or a multiple of 8 KiB up to 48 KiB that take up three
+    eighths of a pitch or less (but at least an eighth), one layer
+    (rect_plain_rows_in_launch_order)."""
+    base_d, base_s = 0x7f0000000000, 0x7f1000000000
+    K = 1024
+    GIB = 1 << 30
+    cases = [
+        # width, destination pitch, source pitch, launch order?
+        (32 * K, 128 * K, 128 * K, True), (32 * K, 256 * K, 256 * K, True), (32 * K, 64 * K, 64 * K, False),
+        (32 * K, 512 * K, 512 * K, False), (32 * K, 128 * K, 256 * K, True), (32 * K, 32 * K, 128 * K, True),
+        (32 * K, 128 * K, 32 * K, True), (32 * K, 128 * K + 256, 128 * K, False), (32 * K, 128 * K, 128 * K + 256, False),
+        (4 * K, 16 * K, 16 * K, True), (4 * K, 8 * K, 8 * K, False), (8 * K, 32 * K, 32 * K, True),
+        (12 * K, 64 * K, 64 * K, False), (24 * K, 64 * K, 64 * K, True), (48 * K, 128 * K, 128 * K, True),
+        (64 * K, 256 * K, 256 * K, False), (2 * K, 8 * K, 8 * K, False), (128 * K, 512 * K, 512 * K, False),
+    ]
+    for width, dp, sp, order in cases:
+        rows = GIB // width
+        st, p = capi_host.plan_rect((base_d, dp, 0), (0, 0, 0), (base_s, sp, 0), (0, 0, 0), (width, rows, 1))
+        assert st == SUCCESS and p.plain_rows == 1 and p.wg_size == 64, (width, dp, sp)
+        assert p.xcd_run == (0 if order else 576), (width, dp, sp, p.xcd_run)
+    # x offsets change nothing; several layers, a small region and tuning do
+    st, p = capi_host.plan_rect((base_d, 128 * K, 0), (4096, 0, 0), (base_s, 128 * K, 0), (8192, 0, 0), (32 * K, 32768, 1))
+    assert st == SUCCESS and (p.plain_rows, p.xcd_run) == (1, 0)
+    st, p = capi_host.plan_rect((base_d, 128 * K, 1 << 30), (0, 0, 0), (base_s, 128 * K, 1 << 30), (0, 0, 0),
+                                (32 * K, 4096, 4))
+    assert st == SUCCESS and (p.plain_rows, p.xcd_run) == (1, 576)
+    st, p = capi_host.plan_rect((base_d, 128 * K, 0), (0, 0, 0), (base_s, 128 * K, 0), (0, 0, 0), (32 * K, 32768, 1),
+                                capi_host.Tuning(xcd_run=288))
+    assert st == SUCCESS and p.xcd_run == 288
+
+
 def test_plan_rect_routes_across_the_host_link(capi_host):
     """A region one side of which is host memory: the same rows, slots and
     merging, launched as at most 128 workgroups of 256 in launch order, stores

@@ -927,8 +927,8 @@ int mi355_aql_fill32(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dword
 
 namespace {
 int copy_batch_device_locked(mi355_aql_t* h, const BatchDesc* scanned, size_t n, uint64_t max_total_bytes,
-                             uint64_t staged_free, const uint64_t* dep_signals, uint32_t num_deps,
-                             uint64_t completion_signal);
+                             uint64_t likely_chunks, uint64_t staged_free, const uint64_t* dep_signals,
+                             uint32_t num_deps, uint64_t completion_signal);
 }
 
 int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t n, const uint64_t* dep_signals,
@@ -951,8 +951,8 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
     if (rc != MI355_BLIT_SUCCESS) return rc;
     const unsigned b = h->next_stage;
     if (wait_signal(h, h->stage_free[b]) != MI355_BLIT_SUCCESS) return MI355_BLIT_ERROR;
-    uint64_t total_bytes = 0;
-    rc = batch_stage_raw(descs, n, h->stage[b], &total_bytes);
+    uint64_t total_bytes = 0, likely_chunks = 0;
+    rc = batch_stage_raw(descs, n, h->stage[b], &total_bytes, &likely_chunks);
     if (rc != MI355_BLIT_SUCCESS) return rc;
     if (total_bytes == 0) {
       g.unlock();
@@ -965,8 +965,8 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
     h->next_stage ^= 1;
     hsa_signal_store_relaxed(h->stage_free[b], 1);
     // the bytes are known exactly: they size the launch as a caller's bound would
-    rc = copy_batch_device_locked(h, h->stage[b], n, total_bytes, h->stage_free[b].handle, dep_signals, num_deps,
-                                  completion_signal);
+    rc = copy_batch_device_locked(h, h->stage[b], n, total_bytes, likely_chunks, h->stage_free[b].handle, dep_signals,
+                                  num_deps, completion_signal);
     if (rc != MI355_BLIT_SUCCESS) hsa_signal_store_relaxed(h->stage_free[b], 0);
     return rc;
   }
@@ -1045,8 +1045,8 @@ namespace {
 // staged; the first kernel, their only reader, leaves a copy for the others
 // and sets that signal to 0 when it is done.
 int copy_batch_device_locked(mi355_aql_t* h, const BatchDesc* scanned, size_t n, uint64_t max_total_bytes,
-                             uint64_t staged_free, const uint64_t* dep_signals, uint32_t num_deps,
-                             uint64_t completion_signal) {
+                             uint64_t likely_chunks, uint64_t staged_free, const uint64_t* dep_signals,
+                             uint32_t num_deps, uint64_t completion_signal) {
   int rc;
   if (!h->batch_seen) {
     // where the copy kernel leaves its numbers of copies and chunks (batch_device_sizing)
@@ -1055,7 +1055,7 @@ int copy_batch_device_locked(mi355_aql_t* h, const BatchDesc* scanned, size_t n,
     *h->batch_seen = 0;
   }
   const BatchDeviceSizing sizing =
-      batch_device_sizing(n, max_total_bytes, *static_cast<volatile uint64_t*>(h->batch_seen));
+      batch_device_sizing(n, max_total_bytes, *static_cast<volatile uint64_t*>(h->batch_seen), likely_chunks);
   if (sizing.records == 0) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   rc = ensure_batch_capacity(h, n, sizing.records);
   if (rc != MI355_BLIT_SUCCESS) return rc;
@@ -1110,7 +1110,7 @@ int copy_batch_device(mi355_aql_t* h, const mi355_blit_desc_t* device_descs, siz
   if (h->queue_error.load()) return MI355_BLIT_ERROR;
   if (n == 0) return mi355_aql_copy(h, h, h, 0, dep_signals, num_deps, completion_signal);
   std::lock_guard<std::mutex> g(h->lock);
-  return copy_batch_device_locked(h, reinterpret_cast<const BatchDesc*>(device_descs), n, max_total_bytes, 0,
+  return copy_batch_device_locked(h, reinterpret_cast<const BatchDesc*>(device_descs), n, max_total_bytes, 0, 0,
                                   dep_signals, num_deps, completion_signal);
 }
 }  // namespace

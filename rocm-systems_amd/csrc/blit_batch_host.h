@@ -61,8 +61,8 @@ inline uint64_t batch_bound_chunks(uint64_t n, uint64_t max_total_bytes) {
 // without knowing the lengths.  With a bound from the caller both follow the
 // bound.  Without one the library goes by the last such batch on the engine,
 // whose copy kernel left its numbers of copies and chunks in host memory
-// (`seen`, copies << 32 | chunks; 0 = none yet): the same chunks per copy plus
-// 3 %, and before any batch has reported, 8 chunks (32 KiB) a copy.  The grid
+// (`seen`, copies << 32 | chunks; 0 = none yet): the same chunks per copy less
+// 1.5 %, and before any batch has reported, 8 chunks (32 KiB) a copy.  The grid
 // has one 4-wave workgroup per chunk; waves beyond the real total end at once
 // (0.2 ns of dispatch each: 65,536 copies of 256 bytes take 64 us on a grid of
 // 65,536 workgroups and 160 us on one of 524,288), waves stride when there are
@@ -81,7 +81,10 @@ struct BatchDeviceSizing {
   uint64_t bytes;        // what the launch heuristics take the batch's size to be
 };
 
-inline BatchDeviceSizing batch_device_sizing(uint64_t n, uint64_t max_total_bytes, uint64_t seen = 0) {
+// likely_chunks: the host's own estimate of the chunk count (batch_stage_raw),
+// 0 for none; the grid then follows it instead of the bytes.
+inline BatchDeviceSizing batch_device_sizing(uint64_t n, uint64_t max_total_bytes, uint64_t seen = 0,
+                                             uint64_t likely_chunks = 0) {
   BatchDeviceSizing z;
   if (max_total_bytes) {
     // 0: a bound beyond what 32-bit record indices can count, which no batch
@@ -90,10 +93,15 @@ inline BatchDeviceSizing batch_device_sizing(uint64_t n, uint64_t max_total_byte
     if (c > kBatchMaxDeviceRecords) c = kBatchMaxDeviceRecords;
     z.records = c;
     // Room for the most chunks the bound allows (two more than bytes / 4096
-    // per copy), a grid for what is likely (one more): waves without a chunk
-    // cost their dispatch (65,536 copies of 2 GB: 715 us with a workgroup for
-    // every possible chunk, 698 us with 4 % fewer workgroups than chunks).
-    z.grid_chunks = max_total_bytes / (16 * kBatchChunkVecs) + n;
+    // per copy), a grid for a little less than is likely (half a chunk more
+    // per copy than bytes / 4096).  A wave without a chunk is not free -- it
+    // takes a slot until it has read the chunk count -- while waves that stride
+    // to a second chunk cost next to nothing: 65,536 copies of 2 GB
+    // (542,613 chunks) take 712 us on a grid for 559,585 chunks, 700 us on one
+    // for 542,613, 535,000 or 524,288, 705 us on one for 500,000.
+    z.grid_chunks = max_total_bytes / (16 * kBatchChunkVecs) + n / 2 + 1;
+    if (z.grid_chunks < n) z.grid_chunks = n;  // short copies: a chunk each
+    if (likely_chunks) z.grid_chunks = likely_chunks - likely_chunks / 64 + 1;
     if (z.grid_chunks > c) z.grid_chunks = c;
     z.bytes = max_total_bytes;
   } else {
@@ -101,11 +109,11 @@ inline BatchDeviceSizing batch_device_sizing(uint64_t n, uint64_t max_total_byte
     if (seen_copies && seen_chunks) {
       // both below 2^32: the product fits
       const uint64_t likely = (seen_chunks * n + seen_copies - 1) / seen_copies;
-      z.grid_chunks = likely + likely / 32 + 16;
+      z.grid_chunks = likely - likely / 64 + 1;
     } else {
       z.grid_chunks = kBatchAssumedChunksPerCopy * n;
     }
-    z.records = 2 * z.grid_chunks;
+    z.records = 2 * z.grid_chunks + 32;
     if (z.records < kBatchMinDeviceRecords) z.records = kBatchMinDeviceRecords;
     if (z.records > kBatchMaxDeviceRecords) z.records = kBatchMaxDeviceRecords;
     if (z.grid_chunks > z.records) z.grid_chunks = z.records;
@@ -227,8 +235,15 @@ inline bool batch_prefers_raw_staging(const mi355_blit_desc_t* descs, size_t n, 
 
 // Copies the descriptors as they are to where the GPU reads them, checking
 // them on the way (a copy of bytes needs both pointers) and adding up their
-// bytes.
-inline int batch_stage_raw(const mi355_blit_desc_t* descs, size_t n, void* stage, uint64_t* total_bytes) {
+// bytes.  *likely_chunks gets an estimate of the batch's chunk count for the
+// grid: the bytes' share is exact, bytes / 4096, and what the copies' ends add
+// to it -- between nothing and a chunk a copy, depending on where the copies
+// start and end within their chunks -- is taken from about a thousand
+// descriptors spread over the batch (65,536 copies of 4000 bytes have 65,536
+// chunks, not the 96,769 that half a chunk a copy would make of them:
+// 123 against 142 us).
+inline int batch_stage_raw(const mi355_blit_desc_t* descs, size_t n, void* stage, uint64_t* total_bytes,
+                           uint64_t* likely_chunks) {
   BatchDesc* out = static_cast<BatchDesc*>(stage);
   uint64_t bytes = 0;
   bool bad = false;
@@ -241,6 +256,20 @@ inline int batch_stage_raw(const mi355_blit_desc_t* descs, size_t n, void* stage
     out[i].bytes = d.bytes;
   }
   *total_bytes = bytes;
+  // every descriptor of a small batch; of a large one 1024 at golden-ratio
+  // steps, which no period in the batch's make-up can fall in with
+  const uint64_t samples = n > 1024 ? 1024 : n;
+  uint64_t sample_chunks = 0, sample_bytes = 0;
+  for (uint64_t k = 0; k < samples; ++k) {
+    const size_t i = n > 1024 ? static_cast<size_t>(k * 0x9e3779b97f4a7c15ull % n) : static_cast<size_t>(k);
+    sample_chunks += batch_desc_chunks(reinterpret_cast<uintptr_t>(descs[i].dst), descs[i].bytes);
+    sample_bytes += descs[i].bytes;
+  }
+  const uint64_t chunk_bytes = 16 * kBatchChunkVecs;
+  const uint64_t ends = sample_chunks * chunk_bytes > sample_bytes ? sample_chunks * chunk_bytes - sample_bytes : 0;
+  *likely_chunks = bytes / chunk_bytes +
+                   static_cast<uint64_t>(static_cast<double>(ends) / static_cast<double>(chunk_bytes * samples) *
+                                         static_cast<double>(n));
   return bad ? MI355_BLIT_ERROR_INVALID_ARGUMENT : MI355_BLIT_SUCCESS;
 }
 

@@ -663,12 +663,14 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
     batch_stage(h->stage_image, h->descs_host[b]);
   } else if (raw) {
     uint64_t total_bytes = 0;
-    rc = batch_stage_raw(descs, n, h->descs_host[b], &total_bytes);
+    uint64_t likely_chunks = 0;
+    rc = batch_stage_raw(descs, n, h->descs_host[b], &total_bytes, &likely_chunks);
     if (rc != MI355_BLIT_SUCCESS) return rc;
     if (total_bytes == 0) return MI355_BLIT_SUCCESS;
     staged_bytes = n * sizeof(BatchDesc);
-    // the bytes are known exactly: they size the launch as a caller's bound would
-    sizing = batch_device_sizing(n, total_bytes);
+    // the bytes are known exactly: they size the record buffer as a caller's
+    // bound would, and the grid follows the host's estimate of the chunk count
+    sizing = batch_device_sizing(n, total_bytes, 0, likely_chunks);
   } else {
     // lengths are only known on the device
     if (!h->batch_seen) {

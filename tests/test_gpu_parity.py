@@ -751,7 +751,7 @@ def test_batch_unbounded_sizes_itself_by_the_batch_before(capi, pkg, oracle, are
     """Without a bound the first device-resident batch on an engine is launched
     for 8 chunks a copy; its copy kernel leaves the numbers of copies and chunks
     in host memory and the next batch is launched for the same chunks per copy
-    plus 3 %.  Bytes are the oracle's whatever the guess."""
+    less 1.5 %.  Bytes are the oracle's whatever the guess."""
     torch = torch_cuda
     src, src_host, dst = arenas
     eng = capi.Blit(0) if path == "hip" else pkg.aql.AqlBlit(0)
@@ -772,7 +772,7 @@ def test_batch_unbounded_sizes_itself_by_the_batch_before(capi, pkg, oracle, are
             assert np.array_equal(dst.host(0, total), want), "call %d" % call
         assert grids[0] == 8 * n
         # 16 or 17 chunks a copy: the second and third launches follow what the first one counted
-        assert grids[1] == grids[2] and abs(grids[1] - chunks * 33 // 32 - 16) <= n // 4, (grids, chunks)
+        assert grids[1] == grids[2] and abs(grids[1] - chunks * 63 // 64 - 1) <= n // 4, (grids, chunks)
         # a batch of short copies next: sized by the long ones once, by itself afterwards
         n2 = 300
         descs2, lens2, offs2, so2, do2, total2 = _make_batch(capi, rng, src, dst, n2, min_len=64, max_len=512)
@@ -808,7 +808,10 @@ def test_batch_of_many_short_copies_is_staged_as_it_is(capi, blit, oracle, arena
         check_ok(capi, blit.copy_batch(descs, n), "copy_batch")
         check_ok(capi, blit.synchronize(), "synchronize")
         p = blit.last_plan()
-        assert p.kernel == capi.KERNEL_COPY_BATCH and _grid_chunks(p) == int(lens.sum()) // 4096 + n, p.as_dict()
+        # the grid follows the host's estimate of the chunk count: a little under it, never far off
+        chunks = sum((int(d.dst) % 256 // 16 * 16 + int(d.bytes) + 4095) // 4096 for d in descs if d.bytes)
+        assert p.kernel == capi.KERNEL_COPY_BATCH and 0.93 * chunks <= _grid_chunks(p) <= 1.01 * chunks + 2, \
+            (p.as_dict(), chunks, int(lens.sum()), n, seed)
         assert np.array_equal(dst.host(0, total), _expect_batch(oracle, src_host, total, lens, offs, so, do)), seed
     # a copy of bytes without a source: refused before anything is launched
     descs[n // 2].src = None

@@ -18,6 +18,7 @@ ROCR_LIB = os.path.join(LIB_DIR, "libmi355blit_rocr.so")
 ROCR_TEST = os.path.join(LIB_DIR, "test_rocr_blit")
 ORACLE_LIB = os.path.join(ORACLE_DIR, "libblit_oracle.so")
 HOST_LOGIC_TEST = os.path.join(LIB_DIR, "test_host_logic")
+KERNELS_ON_CPU_TEST = os.path.join(LIB_DIR, "test_kernels_on_cpu")
 
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
@@ -117,6 +118,20 @@ def build_host_logic_test():
     return HOST_LOGIC_TEST
 
 
+def build_kernels_on_cpu_test():
+    """The blit kernels compiled for the host over tests/cpp/lane_emulation.h
+    (lanes in lock step, every access checked), under AddressSanitizer and
+    UBSan."""
+    test_src = os.path.join(ROOT, "tests", "cpp", "test_kernels_on_cpu.cpp")
+    if not os.path.exists(test_src):
+        return None
+    os.makedirs(LIB_DIR, exist_ok=True)
+    _run(["g++", "-O1", "-g", "-std=c++17", "-Wall", "-Wno-unknown-pragmas", "-fsanitize=address,undefined",
+          "-fno-sanitize-recover=all", "-static-libasan", "-static-libubsan", "-I", INCLUDE, "-I", CSRC,
+          "-I", os.path.join(ROOT, "tests", "cpp"), "-o", KERNELS_ON_CPU_TEST, test_src])
+    return KERNELS_ON_CPU_TEST
+
+
 def build_oracle():
     """CPU oracle (test infrastructure) -> oracle/libblit_oracle.so"""
     _run(["make", "-C", ORACLE_DIR, "-B", "libblit_oracle.so"])
@@ -129,7 +144,7 @@ def build_all():
     if r:
         out.append(r)
     out.append(build_oracle())
-    for t in (build_rocr_test(), build_host_logic_test()):
+    for t in (build_rocr_test(), build_host_logic_test(), build_kernels_on_cpu_test()):
         if t:
             out.append(t)
     return out

@@ -450,18 +450,6 @@ void write_dispatch(mi355_aql* h, uint64_t index, const Kernel& k, const void* a
   if (h->log_packets) log_dispatch_packet(h, header, 1 << HSA_KERNEL_DISPATCH_PACKET_SETUP_DIMENSIONS, pkt, index);
 }
 
-void tail_waves(const mi355_blit_plan_t& p, uint32_t* partial_wave, uint32_t* edge_wave, uint32_t* waves_per_wg,
-                uint32_t* n_waves_out) {
-  const uint64_t n_waves = static_cast<uint64_t>(p.grid) * (p.wg_size / 64);
-  const uint64_t first_full = p.lead_vecs ? 1 : 0;
-  const uint64_t end_full = (p.body_vecs + p.lead_vecs) / (64ull * p.unroll);
-  const uint64_t n_full = end_full > first_full ? end_full - first_full : 0;
-  *waves_per_wg = p.wg_size / 64;
-  *n_waves_out = static_cast<uint32_t>(n_waves);
-  *partial_wave = static_cast<uint32_t>(n_full % n_waves);
-  *edge_wave = static_cast<uint32_t>((n_full + 1) % n_waves);
-}
-
 uint32_t barrier_packets(uint32_t num_deps) { return (num_deps + 4) / 5; }
 
 // Whether a transfer's dispatch packet carries the barrier bit although no
@@ -858,14 +846,7 @@ int mi355_aql_copy_route(mi355_aql_t* h, void* dst, const void* src, size_t byte
     release_write_index(h, index, n);
     return MI355_BLIT_SUCCESS;
   }
-  a.dst = static_cast<uint8_t*>(dst);
-  a.src = static_cast<const uint8_t*>(src);
-  a.bytes = bytes;
-  a.n_vec = p.body_vecs;
-  a.head = static_cast<uint32_t>(p.head_bytes);
-  a.lead = p.lead_vecs;
-  tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
-  a.xcd = make_xcd_runs(p.grid, p.xcd_run);
+  a = make_copy_args(p, dst, src, bytes);
   const uint32_t total = nb + 1;
   uint64_t index;
   {
@@ -902,15 +883,7 @@ int mi355_aql_fill32(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dword
     if (!k) return MI355_BLIT_ERROR;
     h->last_plan = p;
   }
-  FillArgs a{};
-  a.dst = static_cast<uint32_t*>(ptr);
-  a.n_dwords = num_dwords;
-  a.n_vec = p.body_vecs;
-  a.head = static_cast<uint32_t>(p.head_bytes / 4);
-  a.lead = p.lead_vecs;
-  a.value = value;
-  tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
-  a.xcd = make_xcd_runs(p.grid, p.xcd_run);
+  const FillArgs a = make_fill_args(p, ptr, value, num_dwords);
   const uint32_t nb = barrier_packets(num_deps);
   const uint32_t total = nb + 1;
   uint64_t index;

@@ -229,20 +229,6 @@ rect_kernel_t select_rect_kernel(unsigned unroll, bool ntl, unsigned policy) {
   return nullptr;
 }
 
-// Which waves of the launch take the partial last tile and the edges.
-void set_tail_waves(const mi355_blit_plan_t& p, uint32_t* partial_wave, uint32_t* edge_wave,
-                    uint32_t* waves_per_wg, uint32_t* n_waves_out) {
-  const uint64_t n_waves = static_cast<uint64_t>(p.grid) * (p.wg_size / 64);
-  *waves_per_wg = p.wg_size / 64;
-  *n_waves_out = static_cast<uint32_t>(n_waves);
-  // full tiles, as tile_range() counts them on the device
-  const uint64_t first_full = p.lead_vecs ? 1 : 0;
-  const uint64_t end_full = (p.body_vecs + p.lead_vecs) / (64ull * p.unroll);
-  const uint64_t n_full = end_full > first_full ? end_full - first_full : 0;
-  *partial_wave = static_cast<uint32_t>(n_full % n_waves);
-  *edge_wave = static_cast<uint32_t>((n_full + 1) % n_waves);
-}
-
 // Puts a marker behind everything submitted so far.  Caller holds h->lock.
 // When the ledger is full the oldest marker is waited for, the back-pressure
 // ROCr applies when its AQL ring is full (amd_blit_kernel.cpp:844-854).
@@ -485,15 +471,7 @@ int mi355_blit_copy_route(mi355_blit_t* h, void* dst, const void* src, size_t by
   if (rc != MI355_BLIT_SUCCESS) return rc;
   copy_kernel_t k = select_copy_kernel(p);
   if (!k) return MI355_BLIT_ERROR;
-  CopyArgs a;
-  a.dst = static_cast<uint8_t*>(dst);
-  a.src = static_cast<const uint8_t*>(src);
-  a.bytes = bytes;
-  a.n_vec = p.body_vecs;
-  a.head = static_cast<uint32_t>(p.head_bytes);
-  a.lead = p.lead_vecs;
-  set_tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
-  a.xcd = make_xcd_runs(p.grid, p.xcd_run);
+  const CopyArgs a = make_copy_args(p, dst, src, bytes);
   hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
   hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
   BLIT_HIP(hipGetLastError());
@@ -513,15 +491,7 @@ int mi355_blit_fill32(mi355_blit_t* h, void* ptr, uint32_t value, size_t num_dwo
   if (rc != MI355_BLIT_SUCCESS) return rc;
   fill_kernel_t k = select_fill_kernel(p);
   if (!k) return MI355_BLIT_ERROR;
-  FillArgs a;
-  a.dst = static_cast<uint32_t*>(ptr);
-  a.n_dwords = num_dwords;
-  a.n_vec = p.body_vecs;
-  a.head = static_cast<uint32_t>(p.head_bytes / 4);
-  a.lead = p.lead_vecs;
-  a.value = value;
-  set_tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
-  a.xcd = make_xcd_runs(p.grid, p.xcd_run);
+  const FillArgs a = make_fill_args(p, ptr, value, num_dwords);
   hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
   hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
   BLIT_HIP(hipGetLastError());

@@ -36,116 +36,21 @@
 #ifndef MI355_BLIT_KERNELS_H_
 #define MI355_BLIT_KERNELS_H_
 
-#include <hip/hip_runtime.h>
 #include <stdint.h>
+
+// The device primitives (memory accessors, moves between lanes, ids).  A host
+// build that executes these kernels lane by lane names its own header here.
+#ifdef MI355_BLIT_DEVICE_HEADER
+#include MI355_BLIT_DEVICE_HEADER
+#else
+#include "blit_device.h"
+#endif
 
 #include "blit_args.h"
 
 namespace mi355 {
 
-typedef unsigned v4u __attribute__((ext_vector_type(4)));
-// Same vector with only dword alignment promised: the compiler still emits one
-// global_load_dwordx4, which the memory pipeline accepts at any dword address.
-typedef v4u v4u_a4 __attribute__((aligned(4)));
-
-
-// Every pointer these kernels dereference points into global memory, but one
-// that was itself loaded from memory (the chunk records of a batch) reaches the
-// compiler as a generic pointer and would be accessed with flat_* instructions,
-// which go through the aperture check and count against both memory counters.
-// The accessors below therefore state the address space.
-#define MI355_GLOBAL __attribute__((address_space(1)))
-
-template <typename T>
-__device__ __forceinline__ const T MI355_GLOBAL* as_global(const T* p) {
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Wold-style-cast"
-  return (const T MI355_GLOBAL*)(p);
-#pragma clang diagnostic pop
-}
-template <typename T>
-__device__ __forceinline__ T MI355_GLOBAL* as_global(T* p) {
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Wold-style-cast"
-  return (T MI355_GLOBAL*)(p);
-#pragma clang diagnostic pop
-}
-
-template <bool NT>
-__device__ __forceinline__ v4u ld_v4(const v4u_a4* p) {
-  if constexpr (NT) return __builtin_nontemporal_load(as_global(p));
-  else return *as_global(p);
-}
-template <bool NT>
-__device__ __forceinline__ unsigned ld_u32(const unsigned* p) {
-  if constexpr (NT) return __builtin_nontemporal_load(as_global(p));
-  else return *as_global(p);
-}
-__device__ __forceinline__ uint8_t ld_u8(const uint8_t* p) { return *as_global(p); }
-__device__ __forceinline__ void st_u8(uint8_t* p, uint8_t v) { *as_global(p) = v; }
-__device__ __forceinline__ void st_u32(unsigned* p, unsigned v) { *as_global(p) = v; }
-
-// Store cache policies (values of mi355_blit_plan_t::store_policy).
-constexpr int kStoreCached = 0;   // plain write-back L2
-constexpr int kStoreNt = 1;       // non-temporal hint
-constexpr int kStoreAgentWt = 2;  // sc1: written through L2 at agent scope
-constexpr int kStoreSystemWt = 3; // sc0 sc1: written through at system scope
-
-// The policies are spelled out in asm: the write-through forms have no builtin
-// for a 16-byte store, and the non-temporal builtin's hint was seen to get lost
-// on the way through the optimizer (the body store of one realigning variant
-// came out as a plain store).  A store needs no wait of its own, and on gfx9
-// the extra outstanding store only makes a compiler-placed s_waitcnt vmcnt(n)
-// wait longer, never shorter.  A store of more than 8 bytes reads its data
-// registers after issue: a VALU write to them within the next 2 wait states
-// (gfx940 and later) corrupts the data.  The compiler pads its own stores but
-// cannot see into the asm, so the s_nop is part of it.  The asm forms take any
-// byte address.
-template <int POLICY>
-__device__ __forceinline__ void st_v4_at(uintptr_t p, v4u v) {
-  if constexpr (POLICY == kStoreNt) {
-    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
-  } else if constexpr (POLICY == kStoreAgentWt) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
-  } else if constexpr (POLICY == kStoreSystemWt) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
-  } else {
-    typedef v4u v4u_any __attribute__((aligned(1)));
-    *as_global(reinterpret_cast<v4u_any*>(p)) = v;
-  }
-}
-template <int POLICY>
-__device__ __forceinline__ void st_v4(v4u* p, v4u v) {
-  if constexpr (POLICY == kStoreCached) *as_global(p) = v;
-  else st_v4_at<POLICY>(reinterpret_cast<uintptr_t>(p), v);
-}
-
-// 16-byte accesses at any byte address: gfx950 under HSA runs with unaligned
-// global access enabled, and the compiler emits one dwordx4 for these too.
-typedef v4u v4u_a1 __attribute__((aligned(1)));
-
-template <bool NT>
-__device__ __forceinline__ v4u ld_v4_any(const uint8_t* p) {
-  if constexpr (NT) return __builtin_nontemporal_load(as_global(reinterpret_cast<const v4u_a1*>(p)));
-  else return *as_global(reinterpret_cast<const v4u_a1*>(p));
-}
-
-template <int POLICY>
-__device__ __forceinline__ void st_v4_any(uintptr_t p, v4u v) {
-  st_v4_at<POLICY>(p, v);
-}
-
-// Lane i receives the value lane (i + 1) % 64 passed in (DPP wave_rol:1).
-__device__ __forceinline__ unsigned wave_rotate_down1(unsigned v) {
-  return __builtin_amdgcn_update_dpp(0u, v, 0x134, 0xf, 0xf, false);
-}
-
-// Bytes r..r+3 of the little-endian pair {hi:lo}, r in 0..3.
-__device__ __forceinline__ unsigned shift_bytes(unsigned hi, unsigned lo, unsigned r) {
-  return __builtin_amdgcn_alignbyte(hi, lo, r);
-}
-
-__device__ __forceinline__ v4u realign(v4u x, unsigned w4, unsigned r) {
+MI355_DEVICE v4u realign(v4u x, unsigned w4, unsigned r) {
   v4u o;
   o.x = shift_bytes(x.y, x.x, r);
   o.y = shift_bytes(x.z, x.y, r);
@@ -172,7 +77,7 @@ struct TileRange {
 };
 
 template <int U>
-__device__ __forceinline__ TileRange tile_range(uint64_t n_vec, unsigned lead) {
+MI355_DEVICE TileRange tile_range(uint64_t n_vec, unsigned lead) {
   constexpr uint64_t kTile = kWave * U;
   TileRange t;
   t.n_virtual = n_vec + lead;
@@ -186,7 +91,7 @@ __device__ __forceinline__ TileRange tile_range(uint64_t n_vec, unsigned lead) {
 // whole waves: wave w of n_waves takes full tiles first_full + w, + n_waves,
 // ...; wave partial_wave takes the cut tiles at either end.
 template <int U, bool NTL, int NTS, bool SHIFT>
-__device__ __forceinline__ void copy_vectors(v4u* __restrict__ d, const v4u_a4* __restrict__ s,
+MI355_DEVICE void copy_vectors(v4u* __restrict__ d, const v4u_a4* __restrict__ s,
                                              unsigned r, uint64_t n_vec, unsigned lead,
                                              uint64_t wave, uint64_t n_waves,
                                              uint64_t partial_wave, unsigned lane) {
@@ -246,34 +151,34 @@ __device__ __forceinline__ void copy_vectors(v4u* __restrict__ d, const v4u_a4* 
 
 // Head (< 16 bytes in front of the first aligned vector) and tail (< 16 bytes
 // after the last one), one byte per lane: lanes 0..15 head, 16..31 tail.
-__device__ __forceinline__ void copy_edges(uint8_t* dst, const uint8_t* src, uint64_t bytes,
+MI355_DEVICE void copy_edges(uint8_t* dst, const uint8_t* src, uint64_t bytes,
                                            unsigned head, uint64_t n_vec, unsigned lane) {
   const uint64_t tail_off = head + 16 * n_vec;
   const unsigned tail = static_cast<unsigned>(bytes - tail_off);
   if (lane < head) {
-    dst[lane] = src[lane];
+    st_u8(dst + lane, ld_u8(src + lane));
   } else if (lane >= 16 && lane - 16 < tail) {
-    dst[tail_off + lane - 16] = src[tail_off + lane - 16];
+    st_u8(dst + tail_off + lane - 16, ld_u8(src + tail_off + lane - 16));
   }
 }
 
 // Index of the calling wave among all waves of the launch (wave-uniform).
-__device__ __forceinline__ uint64_t global_wave(unsigned waves_per_wg) {
-  return __builtin_amdgcn_readfirstlane(blockIdx.x * waves_per_wg + threadIdx.x / kWave);
+MI355_DEVICE uint64_t global_wave(unsigned waves_per_wg) {
+  return wave_uniform(workgroup_index() * waves_per_wg + thread_in_workgroup() / kWave);
 }
 
 // global_wave() of a launch whose workgroups take their work in runs per XCD
 // (xcd_workgroup): workgroups below x.full swap places among themselves, the
 // others keep theirs.  x.full == 0: launch order.
-__device__ __forceinline__ uint64_t global_wave_xcd(unsigned waves_per_wg, const XcdRuns& x) {
-  uint32_t wg = blockIdx.x;
+MI355_DEVICE uint64_t global_wave_xcd(unsigned waves_per_wg, const XcdRuns& x) {
+  uint32_t wg = workgroup_index();
   if (wg < x.full) wg = xcd_workgroup(wg, x);
-  return __builtin_amdgcn_readfirstlane(wg * waves_per_wg + threadIdx.x / kWave);
+  return wave_uniform(wg * waves_per_wg + thread_in_workgroup() / kWave);
 }
 
 template <int U, bool NTL, int NTS, bool SHIFT>
-__device__ __forceinline__ void copy_body(const CopyArgs& a) {
-  const unsigned lane = threadIdx.x & (kWave - 1);
+MI355_DEVICE void copy_body(const CopyArgs& a) {
+  const unsigned lane = thread_in_workgroup() & (kWave - 1);
   const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd);
   const uint64_t n_waves = a.n_waves;
   const uint8_t* sb = a.src + a.head;
@@ -285,8 +190,8 @@ __device__ __forceinline__ void copy_body(const CopyArgs& a) {
 }
 
 template <int U, int NTS>
-__device__ __forceinline__ void fill_body(const FillArgs& a) {
-  const unsigned lane = threadIdx.x & (kWave - 1);
+MI355_DEVICE void fill_body(const FillArgs& a) {
+  const unsigned lane = thread_in_workgroup() & (kWave - 1);
   const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd);
   const uint64_t n_waves = a.n_waves;
   const v4u val = {a.value, a.value, a.value, a.value};
@@ -312,8 +217,8 @@ __device__ __forceinline__ void fill_body(const FillArgs& a) {
     // whole dwords outside the vector body: lanes 0..3 head, 4..7 tail
     const uint64_t tail_off = a.head + 4 * a.n_vec;
     const unsigned tail = static_cast<unsigned>(a.n_dwords - tail_off);
-    if (lane < a.head) a.dst[lane] = a.value;
-    else if (lane >= 4 && lane - 4 < tail) a.dst[tail_off + lane - 4] = a.value;
+    if (lane < a.head) st_u32(a.dst + lane, a.value);
+    else if (lane >= 4 && lane - 4 < tail) st_u32(a.dst + tail_off + lane - 4, a.value);
   }
 }
 
@@ -334,7 +239,7 @@ struct DescShape {
   uint64_t n_vec;   // body vectors
 };
 
-__device__ __forceinline__ DescShape desc_shape(const BatchDesc& d) {
+MI355_DEVICE DescShape desc_shape(const BatchDesc& d) {
   DescShape sh;
   const unsigned a = static_cast<unsigned>(reinterpret_cast<uintptr_t>(d.dst));
   const unsigned h = (16 - (a & 15)) & 15;
@@ -344,7 +249,7 @@ __device__ __forceinline__ DescShape desc_shape(const BatchDesc& d) {
   return sh;
 }
 
-__device__ __forceinline__ unsigned desc_chunks(const BatchDesc& d) {
+MI355_DEVICE unsigned desc_chunks(const BatchDesc& d) {
   if (d.bytes == 0) return 0;
   const DescShape sh = desc_shape(d);
   const uint64_t c = (sh.n_vec + sh.lead + kChunkVecs - 1) / kChunkVecs;
@@ -353,27 +258,27 @@ __device__ __forceinline__ unsigned desc_chunks(const BatchDesc& d) {
 
 // Exclusive prefix sum over the 1024 lanes of a workgroup; *total gets the sum.
 // lds holds 16 words.
-__device__ __forceinline__ uint32_t block_scan_1024(uint32_t v, uint32_t* lds, uint32_t* total) {
-  const unsigned lane = threadIdx.x & (kWave - 1);
-  const unsigned w = threadIdx.x / kWave;
+MI355_DEVICE uint32_t block_scan_1024(uint32_t v, uint32_t* lds, uint32_t* total) {
+  const unsigned lane = thread_in_workgroup() & (kWave - 1);
+  const unsigned w = thread_in_workgroup() / kWave;
   uint32_t incl = v;
 #pragma unroll
   for (unsigned off = 1; off < kWave; off <<= 1) {
-    const uint32_t x = __shfl_up(incl, off, kWave);
+    const uint32_t x = lane_read_up(incl, off);
     if (lane >= off) incl += x;
   }
   if (lane == kWave - 1) lds[w] = incl;
-  __syncthreads();
+  workgroup_barrier();
   if (w == 0) {
     uint32_t s = lane < 16 ? lds[lane] : 0;
 #pragma unroll
     for (unsigned off = 1; off < 16; off <<= 1) {
-      const uint32_t x = __shfl_up(s, off, kWave);
+      const uint32_t x = lane_read_up(s, off);
       if (lane >= off) s += x;
     }
     if (lane < 16) lds[lane] = s;
   }
-  __syncthreads();
+  workgroup_barrier();
   *total = lds[15];
   return (w ? lds[w - 1] : 0) + incl - v;
 }
@@ -388,53 +293,53 @@ __device__ __forceinline__ uint32_t block_scan_1024(uint32_t v, uint32_t* lds, u
 // A copy's first chunk is block_sum[i / 1024] + chunk_start[i].  This is the
 // path of device-resident descriptors; for host-resident ones the host does
 // the sum (mi355_batch_emit_records).
-__device__ __forceinline__ void scan_local_body(const ScanLocalArgs& a) {
+MI355_DEVICE void scan_local_body(const ScanLocalArgs& a) {
   const BatchDesc* __restrict__ descs = a.descs;
   const uint64_t n = a.n;
   uint32_t* __restrict__ chunk_start = a.chunk_start;
   uint32_t* __restrict__ block_sum = a.block_sum;
-  __shared__ uint32_t lds[16];
-  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 1024 + threadIdx.x;
+  MI355_LDS uint32_t lds[16];
+  const uint64_t i = static_cast<uint64_t>(workgroup_index()) * 1024 + thread_in_workgroup();
   BatchDesc d{nullptr, nullptr, 0};
   if (i < n) {
     if (a.private_copy) {
       const uint64_t* w = reinterpret_cast<const uint64_t*>(descs + i);
-      d.dst = reinterpret_cast<uint8_t*>(__hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM));
-      d.src = reinterpret_cast<const uint8_t*>(__hip_atomic_load(w + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM));
-      d.bytes = __hip_atomic_load(w + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-      a.private_copy[i] = d;
+      d.dst = reinterpret_cast<uint8_t*>(ld_system_u64(w));
+      d.src = reinterpret_cast<const uint8_t*>(ld_system_u64(w + 1));
+      d.bytes = ld_system_u64(w + 2);
+      st_obj(a.private_copy + i, d);
     } else {
-      d = descs[i];
+      d = ld_obj(descs + i);
     }
   }
   const uint32_t c = i < n ? desc_chunks(d) : 0;
   uint32_t total;
   const uint32_t excl = block_scan_1024(c, lds, &total);
-  if (i < n) chunk_start[i] = excl;
-  if (threadIdx.x == 0) block_sum[blockIdx.x] = total;
+  if (i < n) st_u32(chunk_start + i, excl);
+  if (thread_in_workgroup() == 0) st_u32(block_sum + workgroup_index(), total);
 }
 
-__device__ __forceinline__ void scan_top_body(const ScanTopArgs& a) {
+MI355_DEVICE void scan_top_body(const ScanTopArgs& a) {
   uint32_t* __restrict__ block_sum = a.block_sum;
   uint32_t* __restrict__ chunk_start = a.chunk_start;
   const uint64_t n = a.n;
   const uint32_t n_blocks = a.n_blocks;
-  __shared__ uint32_t lds[16];
+  MI355_LDS uint32_t lds[16];
   uint32_t carry = 0;
   for (uint32_t base = 0; base < n_blocks; base += 1024) {
-    const uint32_t j = base + threadIdx.x;
-    const uint32_t v = j < n_blocks ? block_sum[j] : 0;
+    const uint32_t j = base + thread_in_workgroup();
+    const uint32_t v = j < n_blocks ? ld_u32<false>(block_sum + j) : 0;
     uint32_t total;
     const uint32_t excl = block_scan_1024(v, lds, &total);
-    if (j < n_blocks) block_sum[j] = carry + excl;
+    if (j < n_blocks) st_u32(block_sum + j, carry + excl);
     carry += total;
-    __syncthreads();  // lds is reused by the next round
+    workgroup_barrier();  // lds is reused by the next round
   }
-  if (threadIdx.x == 0) chunk_start[n] = carry;
+  if (thread_in_workgroup() == 0) st_u32(chunk_start + n, carry);
 }
 
 // Chunk k of a copy.
-__device__ __forceinline__ ChunkRecord make_record(const BatchDesc& d, uint32_t k) {
+MI355_DEVICE ChunkRecord make_record(const BatchDesc& d, uint32_t k) {
   const DescShape sh = desc_shape(d);
   const uint64_t n_virtual = sh.n_vec + sh.lead;
   uint64_t lo = static_cast<uint64_t>(k) * kChunkVecs;
@@ -469,17 +374,17 @@ __device__ __forceinline__ ChunkRecord make_record(const BatchDesc& d, uint32_t 
 // Writes the records of one wave's copies: lane l holds copy (dst, src,
 // bytes) with `chunks` records (none in a lane without a copy), the wave's
 // records start at out[0].
-__device__ __forceinline__ void emit_wave_records(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t chunks,
+MI355_DEVICE void emit_wave_records(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t chunks,
                                                   ChunkRecord* out, unsigned lane) {
   // exclusive running sum of the chunk counts over the wave's lanes
   uint32_t incl = chunks;
 #pragma unroll
   for (unsigned off = 1; off < kWave; off <<= 1) {
-    const uint32_t x = __shfl_up(incl, off, kWave);
+    const uint32_t x = lane_read_up(incl, off);
     if (lane >= off) incl += x;
   }
   const uint32_t excl = incl - chunks;
-  const uint32_t total = __shfl(incl, kWave - 1, kWave);
+  const uint32_t total = lane_read(incl, kWave - 1);
   const uint32_t dst_lo = static_cast<uint32_t>(dst), dst_hi = static_cast<uint32_t>(dst >> 32);
   const uint32_t src_lo = static_cast<uint32_t>(src), src_hi = static_cast<uint32_t>(src >> 32);
   const uint32_t len_lo = static_cast<uint32_t>(bytes), len_hi = static_cast<uint32_t>(bytes >> 32);
@@ -492,33 +397,33 @@ __device__ __forceinline__ void emit_wave_records(uint64_t dst, uint64_t src, ui
     unsigned owner = 0;
 #pragma unroll
     for (unsigned step = kWave / 2; step >= 1; step >>= 1) {
-      const uint32_t e = __shfl(excl, owner + step, kWave);
+      const uint32_t e = lane_read(excl, owner + step);
       if (e <= j) owner += step;
     }
     BatchDesc d;
-    d.dst = reinterpret_cast<uint8_t*>(static_cast<uint64_t>(__shfl(dst_hi, owner, kWave)) << 32 |
-                                       __shfl(dst_lo, owner, kWave));
-    d.src = reinterpret_cast<const uint8_t*>(static_cast<uint64_t>(__shfl(src_hi, owner, kWave)) << 32 |
-                                             __shfl(src_lo, owner, kWave));
-    d.bytes = static_cast<uint64_t>(__shfl(len_hi, owner, kWave)) << 32 | __shfl(len_lo, owner, kWave);
-    const uint32_t k = j - __shfl(excl, owner, kWave);
-    if (j < total) out[j] = make_record(d, k);
+    d.dst = reinterpret_cast<uint8_t*>(static_cast<uint64_t>(lane_read(dst_hi, owner)) << 32 |
+                                       lane_read(dst_lo, owner));
+    d.src = reinterpret_cast<const uint8_t*>(static_cast<uint64_t>(lane_read(src_hi, owner)) << 32 |
+                                             lane_read(src_lo, owner));
+    d.bytes = static_cast<uint64_t>(lane_read(len_hi, owner)) << 32 | lane_read(len_lo, owner);
+    const uint32_t k = j - lane_read(excl, owner);
+    if (j < total) st_obj(out + j, make_record(d, k));
   }
 }
 
-__device__ __forceinline__ void emit_records_body(const EmitRecordsArgs& a) {
-  const unsigned lane = threadIdx.x & (kWave - 1);
-  const uint64_t wave = static_cast<uint64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
+MI355_DEVICE void emit_records_body(const EmitRecordsArgs& a) {
+  const unsigned lane = thread_in_workgroup() & (kWave - 1);
+  const uint64_t wave = static_cast<uint64_t>(workgroup_index()) * 4 + thread_in_workgroup() / kWave;
   const uint64_t i = wave * kEmitPiecesPerWave + lane;
   const bool valid = lane < kEmitPiecesPerWave && i < a.n;
   uint64_t dst = 0, src = 0, bytes = 0;
   uint32_t first = 0;
   if (valid) {
     const uint64_t* w = reinterpret_cast<const uint64_t*>(a.descs + i);
-    dst = __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    src = __hip_atomic_load(w + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    bytes = __hip_atomic_load(w + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    first = __hip_atomic_load(a.first_record + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    dst = ld_system_u64(w);
+    src = ld_system_u64(w + 1);
+    bytes = ld_system_u64(w + 2);
+    first = ld_system_u32(a.first_record + i);
   }
   BatchDesc mine;
   mine.dst = reinterpret_cast<uint8_t*>(dst);
@@ -526,14 +431,14 @@ __device__ __forceinline__ void emit_records_body(const EmitRecordsArgs& a) {
   mine.bytes = bytes;
   const uint32_t chunks = valid ? desc_chunks(mine) : 0;
   // the wave's records are consecutive: lane 0's first record starts them
-  emit_wave_records(dst, src, bytes, chunks, a.records + __shfl(first, 0, kWave), lane);
+  emit_wave_records(dst, src, bytes, chunks, a.records + lane_read(first, 0), lane);
 }
 
 // Loads of one wave's share of a chunk: virtual vector indices [v0, v0 + 64 U)
 // cut to [lead, lead + n_vec); up to U vectors per lane and, when the source
 // is not dword aligned, the dword behind the share's last vector.
 template <int U, bool NTL>
-__device__ __forceinline__ void record_load(const ChunkRecord& rec, unsigned v0, unsigned lane,
+MI355_DEVICE void record_load(const ChunkRecord& rec, unsigned v0, unsigned lane,
                                             v4u (&x)[U], unsigned& e) {
   const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(rec.src)) & 3;
   const v4u_a4* sv = reinterpret_cast<const v4u_a4*>(rec.src - r) - rec.lead;
@@ -551,7 +456,7 @@ __device__ __forceinline__ void record_load(const ChunkRecord& rec, unsigned v0,
 // Realign and store what record_load fetched.  With a dword-aligned source
 // the realignment is the identity (shift 0).
 template <int U, int NTS>
-__device__ __forceinline__ void record_store(const ChunkRecord& rec, unsigned v0, unsigned lane,
+MI355_DEVICE void record_store(const ChunkRecord& rec, unsigned v0, unsigned lane,
                                              const v4u (&x)[U], unsigned e) {
   const unsigned r = static_cast<unsigned>(reinterpret_cast<uintptr_t>(rec.src)) & 3;
   v4u* dv = reinterpret_cast<v4u*>(rec.dst) - rec.lead;
@@ -568,7 +473,7 @@ __device__ __forceinline__ void record_store(const ChunkRecord& rec, unsigned v0
 }
 
 // Head bytes in front of the chunk's first vector, tail bytes behind its last.
-__device__ __forceinline__ void record_edges(const ChunkRecord& rec, bool do_head, bool do_tail,
+MI355_DEVICE void record_edges(const ChunkRecord& rec, bool do_head, bool do_tail,
                                              unsigned lane) {
   if (do_head && lane < rec.head) {
     st_u8(rec.dst - rec.head + lane, ld_u8(rec.src - rec.head + lane));
@@ -576,38 +481,6 @@ __device__ __forceinline__ void record_edges(const ChunkRecord& rec, bool do_hea
     const uint64_t off = 16ull * rec.n_vec + lane - 16;
     st_u8(rec.dst + off, ld_u8(rec.src + off));
   }
-}
-
-// One record, fetched with a scalar load.  The records were written by an
-// earlier launch and are only read here; reading them through the constant
-// address space tells the compiler so (a pointer taken out of the argument
-// struct carries no such promise, and the record would otherwise be fetched by
-// all 64 lanes with vector loads).
-__device__ __forceinline__ ChunkRecord load_record(const ChunkRecord* p) {
-  typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
-  typedef const u32x8 __attribute__((address_space(4))) * ConstPtr;
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Wold-style-cast"
-  const u32x8 v = *(ConstPtr)(p);
-#pragma clang diagnostic pop
-  ChunkRecord r;
-  __builtin_memcpy(&r, &v, sizeof(r));
-  return r;
-}
-
-// A descriptor at an address that is the same for every lane, through the
-// constant address space like a record.
-__device__ __forceinline__ BatchDesc load_desc(const BatchDesc* p) {
-  typedef const uint64_t __attribute__((address_space(4))) * ConstPtr;
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Wold-style-cast"
-  ConstPtr q = (ConstPtr)(p);
-#pragma clang diagnostic pop
-  BatchDesc d;
-  d.dst = reinterpret_cast<uint8_t*>(q[0]);
-  d.src = reinterpret_cast<const uint8_t*>(q[1]);
-  d.bytes = q[2];
-  return d;
 }
 
 // A wave's record is a dependent load in front of everything else it does, and
@@ -618,7 +491,7 @@ __device__ __forceinline__ BatchDesc load_desc(const BatchDesc* p) {
 // before the data loads behind it: the line (four records) is then in that
 // XCD's L2 when its time comes.  The value is not used; keep_alive() only keeps
 // the compiler from dropping the load.
-__device__ __forceinline__ unsigned touch_record_ahead(const ChunkRecord* records, uint64_t w, unsigned q,
+MI355_DEVICE unsigned touch_record_ahead(const ChunkRecord* records, uint64_t w, unsigned q,
                                                        unsigned ahead, unsigned split, uint64_t total_chunks,
                                                        unsigned lane) {
   unsigned v = 0;
@@ -628,24 +501,23 @@ __device__ __forceinline__ unsigned touch_record_ahead(const ChunkRecord* record
   }
   return v;
 }
-__device__ __forceinline__ void keep_alive(unsigned v) { asm volatile("" ::"v"(v)); }
 
 // SPLIT waves per 4 KiB chunk, chunks in global order and waves in address
 // order within a chunk: the dispatcher then walks memory densely, the shape
 // that streams best for a single large copy.  Each wave reads its chunk's
 // record (one 32-byte scalar load) and then moves 256 / SPLIT vectors.
 template <int SPLIT, bool NTL, int NTS>
-__device__ __forceinline__ void batch_copy_records_body(const BatchCopyArgs& a) {
+MI355_DEVICE void batch_copy_records_body(const BatchCopyArgs& a) {
   constexpr int U = kChunkVecs / kWave / SPLIT;
   const ChunkRecord* __restrict__ records = a.records;
   const uint64_t total_chunks = a.total_chunks;
-  const unsigned lane = threadIdx.x & (kWave - 1);
+  const unsigned lane = thread_in_workgroup() & (kWave - 1);
   const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd);
   const uint64_t n_waves = a.n_waves;
   for (uint64_t w = wave; w < total_chunks * SPLIT; w += n_waves) {
     const unsigned q = static_cast<unsigned>(w % SPLIT);
     const unsigned touched = touch_record_ahead(records, w, q, a.prefetch_waves, SPLIT, total_chunks, lane);
-    const ChunkRecord rec = load_record(records + w / SPLIT);
+    const ChunkRecord rec = ld_uniform_record(records + w / SPLIT);
     const unsigned v0 = q * (kChunkVecs / SPLIT);
     v4u x[U];
     unsigned e;
@@ -662,22 +534,15 @@ __device__ __forceinline__ void batch_copy_records_body(const BatchCopyArgs& a) 
 // chunks share their start with their successor and lose to it).  c is below
 // the batch's chunk total; *k is the chunk's index within its copy.
 // UNIFORM: c is the same for every lane of the wave, and the prefix sums come
-// in through scalar loads (the constant address space, as for a record).
+// in through scalar loads, as a record does.
 template <bool UNIFORM>
-__device__ __forceinline__ uint32_t ld_prefix(const uint32_t* p) {
-  if constexpr (UNIFORM) {
-    typedef const uint32_t __attribute__((address_space(4))) * ConstPtr;
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Wold-style-cast"
-    return *(ConstPtr)(p);
-#pragma clang diagnostic pop
-  } else {
-    return ld_u32<false>(p);
-  }
+MI355_DEVICE uint32_t ld_prefix(const uint32_t* p) {
+  if constexpr (UNIFORM) return ld_uniform_u32(p);
+  else return ld_u32<false>(p);
 }
 
 template <bool UNIFORM>
-__device__ __forceinline__ uint64_t find_copy_of_chunk(const uint32_t* __restrict__ block_sum,
+MI355_DEVICE uint64_t find_copy_of_chunk(const uint32_t* __restrict__ block_sum,
                                                        const uint32_t* __restrict__ chunk_start, uint64_t n,
                                                        uint32_t c, uint32_t* k) {
   uint64_t lo = 0, hi = (n + 1023) / 1024 - 1;
@@ -697,14 +562,14 @@ __device__ __forceinline__ uint64_t find_copy_of_chunk(const uint32_t* __restric
 }
 
 // The record of chunk c, the same for every lane of the wave.
-__device__ __forceinline__ ChunkRecord lookup_record(const BatchLookupArgs& a, uint32_t c) {
+MI355_DEVICE ChunkRecord lookup_record(const BatchLookupArgs& a, uint32_t c) {
   uint32_t k;
   const uint64_t found = find_copy_of_chunk<true>(a.block_sum, a.chunk_start, a.n,
-                                                  __builtin_amdgcn_readfirstlane(c), &k);
+                                                  wave_uniform(c), &k);
   // Every lane has found the same copy: say so, and its descriptor comes in
   // through scalar loads like a record.
-  const uint32_t i = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(found));
-  return make_record(load_desc(a.descs + i), __builtin_amdgcn_readfirstlane(k));
+  const uint32_t i = wave_uniform(static_cast<uint32_t>(found));
+  return make_record(ld_uniform_desc(a.descs + i), wave_uniform(k));
 }
 
 // Records for device-resident descriptors, one lane per record: the lane finds
@@ -713,13 +578,13 @@ __device__ __forceinline__ ChunkRecord lookup_record(const BatchLookupArgs& a, u
 // to do.  Costs the same whatever the copies' lengths (a wave writing the
 // records of its own 64 copies stalls on a long copy: 100 copies of 4 MiB took
 // 300 us that way).
-__device__ __forceinline__ void emit_records_lookup_body(const EmitRecordsDeviceArgs& a) {
-  const uint64_t j = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+MI355_DEVICE void emit_records_lookup_body(const EmitRecordsDeviceArgs& a) {
+  const uint64_t j = static_cast<uint64_t>(workgroup_index()) * 256 + thread_in_workgroup();
   const uint64_t total = ld_u32<false>(a.chunk_start + a.n);
   if (j >= total || j >= a.capacity) return;
   uint32_t k;
   const uint64_t i = find_copy_of_chunk<false>(a.block_sum, a.chunk_start, a.n, static_cast<uint32_t>(j), &k);
-  a.records[j] = make_record(a.descs[i], k);
+  st_obj(a.records + j, make_record(ld_obj(a.descs + i), k));
 }
 
 // The copy over records when only the device knows how many chunks there are:
@@ -727,23 +592,23 @@ __device__ __forceinline__ void emit_records_lookup_body(const EmitRecordsDevice
 // end at once, and waves stride when there are more chunks than waves.  One
 // 4 KiB chunk per four waves, as above.
 template <bool NTL, int NTS>
-__device__ __forceinline__ void batch_copy_lookup_body(const BatchLookupArgs& a) {
+MI355_DEVICE void batch_copy_lookup_body(const BatchLookupArgs& a) {
   constexpr int SPLIT = 4;
   constexpr int U = kChunkVecs / kWave / SPLIT;
   const ChunkRecord* __restrict__ records = a.copy.records;
   const uint64_t capacity = a.copy.total_chunks;
-  const uint64_t total_chunks = *a.copy.total;
-  const unsigned lane = threadIdx.x & (kWave - 1);
+  const uint64_t total_chunks = ld_u32<false>(a.copy.total);
+  const unsigned lane = thread_in_workgroup() & (kWave - 1);
   const uint64_t wave = global_wave_xcd(a.copy.waves_per_wg, a.copy.xcd);
   const uint64_t n_waves = a.copy.n_waves;
   if (wave == 0 && lane == 0 && a.seen)
-    __hip_atomic_store(a.seen, a.n << 32 | total_chunks, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    st_system_u64(a.seen, a.n << 32 | total_chunks);
   const uint64_t have = total_chunks < capacity ? total_chunks : capacity;  // chunks with a record
   for (uint64_t w = wave; w < total_chunks * SPLIT; w += n_waves) {
     const uint64_t c = w / SPLIT;
     const unsigned q = static_cast<unsigned>(w % SPLIT);
     const unsigned touched = touch_record_ahead(records, w, q, a.copy.prefetch_waves, SPLIT, have, lane);
-    const ChunkRecord rec = c < capacity ? load_record(records + c) : lookup_record(a, static_cast<uint32_t>(c));
+    const ChunkRecord rec = c < capacity ? ld_uniform_record(records + c) : lookup_record(a, static_cast<uint32_t>(c));
     const unsigned v0 = q * (kChunkVecs / SPLIT);
     v4u x[U];
     unsigned e;
@@ -765,7 +630,7 @@ __device__ __forceinline__ void batch_copy_lookup_body(const BatchLookupArgs& a)
 // fewer skip the rest.  No memory beyond the two regions, one launch.
 constexpr unsigned kRowOverflowVecs = 15;
 
-__device__ __forceinline__ uint64_t row_units(uint64_t n_virtual, unsigned unit) {
+MI355_DEVICE uint64_t row_units(uint64_t n_virtual, unsigned unit) {
   return n_virtual > kRowOverflowVecs + unit ? (n_virtual - kRowOverflowVecs + unit - 1) / unit : 1;
 }
 
@@ -775,7 +640,7 @@ __device__ __forceinline__ uint64_t row_units(uint64_t n_virtual, unsigned unit)
 // nothing to do, or have up to kRowOverflowVecs vectors more than a unit, which
 // its first lanes take.
 template <int U, bool NTL, int NTS>
-__device__ __forceinline__ void rect_plain_unit(const RectArgs& a, uint32_t slot, unsigned lane) {
+MI355_DEVICE void rect_plain_unit(const RectArgs& a, uint32_t slot, unsigned lane) {
   constexpr unsigned kUnit = kWave * U;
   const uint32_t line = div_magic(slot, a.magic_slots);
   const uint32_t kq = slot - line * a.slots;
@@ -803,7 +668,7 @@ __device__ __forceinline__ void rect_plain_unit(const RectArgs& a, uint32_t slot
 // wave's first load counts: with 32 waves on a CU sharing its issue slots, a
 // hundred scalar instructions are a fifth of a wave's life.)
 template <int U, bool NTL, int NTS>
-__device__ __forceinline__ void rect_unit(const RectArgs& a, uint32_t slot, unsigned lane) {
+MI355_DEVICE void rect_unit(const RectArgs& a, uint32_t slot, unsigned lane) {
   constexpr unsigned kUnit = kWave * U;
   const uint32_t line = div_magic(slot, a.magic_slots);  // row index through all layers
   const uint32_t kq = slot - line * a.slots;
@@ -879,16 +744,16 @@ __device__ __forceinline__ void rect_unit(const RectArgs& a, uint32_t slot, unsi
   const uint64_t body_end = head + 16 * (n_virtual - lead_vecs);
   const unsigned tail = static_cast<unsigned>(a.width - body_end);
   if (kq == 0 && lane < head) {
-    drow[lane] = srow[lane];
+    st_u8(drow + lane, ld_u8(srow + lane));
   } else if (last && lane >= 16 && lane - 16 < tail) {
     const uint64_t off = body_end + lane - 16;
-    drow[off] = srow[off];
+    st_u8(drow + off, ld_u8(srow + off));
   }
 }
 
 template <int U, bool NTL, int NTS>
-__device__ __forceinline__ void rect_copy_body(const RectArgs& a) {
-  const unsigned lane = threadIdx.x & (kWave - 1);
+MI355_DEVICE void rect_copy_body(const RectArgs& a) {
+  const unsigned lane = thread_in_workgroup() & (kWave - 1);
   uint64_t w = global_wave_xcd(a.waves_per_wg, a.xcd);
   if (w >= a.total_slots) return;
   // A grid with a wave for every unit slot (the usual case) goes through the
@@ -911,7 +776,7 @@ __device__ __forceinline__ void rect_copy_body(const RectArgs& a) {
 // has them, single bytes at its ragged ends; the source is read in the aligned
 // dwords that hold at least one wanted byte, all loads before the first store.
 template <bool NTL>
-__device__ __forceinline__ void copy_partial_slot(uintptr_t slot, unsigned off, unsigned end,
+MI355_DEVICE void copy_partial_slot(uintptr_t slot, unsigned off, unsigned end,
                                                   const uint8_t* sa) {
   const uintptr_t ss = reinterpret_cast<uintptr_t>(sa) - off;  // source of the slot's byte 0
   const unsigned r = static_cast<unsigned>(ss) & 3;
@@ -954,8 +819,8 @@ __device__ __forceinline__ void copy_partial_slot(uintptr_t slot, unsigned off, 
 // same values: no byte loop and no divergence.  Only rows under 16 bytes go
 // through copy_partial_slot.
 template <bool NTL, int NTS>
-__device__ __forceinline__ void rect_narrow_body(const RectNarrowArgs& a) {
-  const unsigned lane = threadIdx.x & (kWave - 1);
+MI355_DEVICE void rect_narrow_body(const RectNarrowArgs& a) {
+  const unsigned lane = thread_in_workgroup() & (kWave - 1);
   const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd);
   const uint32_t lpr = a.lanes_per_row;
   const uint64_t total = static_cast<uint64_t>(a.lines) * lpr;
@@ -963,7 +828,7 @@ __device__ __forceinline__ void rect_narrow_body(const RectNarrowArgs& a) {
   for (uint64_t w = wave; w < n_groups; w += a.n_waves) {
     // row and slot of this lane's number 64 w + lane
     const uint64_t first = w * kWave;
-    const uint64_t line0 = lpr == 1 ? first : __umul64hi(first, a.magic64);  // first / lpr
+    const uint64_t line0 = lpr == 1 ? first : mul_hi_u64(first, a.magic64);  // first / lpr
     const unsigned t = static_cast<unsigned>(first - line0 * lpr) + lane;    // < lpr + 64
     const unsigned g = div_magic(t, a.magic64);                              // t / lpr
     const unsigned j = t - g * lpr;
@@ -1003,18 +868,15 @@ __device__ __forceinline__ void rect_narrow_body(const RectNarrowArgs& a) {
 // and raise the interrupt that wakes waiters sleeping in the kernel driver.
 // ---------------------------------------------------------------------------
 
-__device__ __forceinline__ void signal_complete_body(const SignalArgs& a) {
+MI355_DEVICE void signal_complete_body(const SignalArgs& a) {
   HsaSignalAbi* sig = a.sig;
-  if (threadIdx.x != 0) return;
-  __hip_atomic_fetch_sub(&sig->value, static_cast<int64_t>(1), __ATOMIC_RELEASE,
-                         __HIP_MEMORY_SCOPE_SYSTEM);
+  if (thread_in_workgroup() != 0) return;
+  signal_decrement_system(&sig->value);
   uint64_t* mailbox = reinterpret_cast<uint64_t*>(sig->event_mailbox_ptr);
   if (mailbox) {
     const uint32_t id = sig->event_id;
-    __hip_atomic_store(mailbox, static_cast<uint64_t>(id), __ATOMIC_RELEASE,
-                       __HIP_MEMORY_SCOPE_SYSTEM);
-    // MSG_INTERRUPT with the event id's low byte in m0
-    __builtin_amdgcn_s_sendmsg(1, __builtin_amdgcn_readfirstlane(id) & 0xff);
+    st_system_release_u64(mailbox, static_cast<uint64_t>(id));
+    send_interrupt(id);
   }
 }
 
@@ -1035,59 +897,59 @@ __device__ __forceinline__ void signal_complete_body(const SignalArgs& a) {
 #include "blit_kernel_list.h"
 
 #define MI355_DEFINE_COPY(U, L, S, R)                                                  \
-  extern "C" __global__ void __launch_bounds__(1024)                                   \
+  MI355_KERNEL(1024) void                                   \
       mi355_copy_u##U##_l##L##_s##S##_r##R(mi355::CopyArgs a) {                        \
     mi355::copy_body<U, L != 0, S, R != 0>(a);                                         \
   }
 MI355_FOR_EACH_COPY_KERNEL(MI355_DEFINE_COPY)
 
 #define MI355_DEFINE_FILL(U, S)                                                        \
-  extern "C" __global__ void __launch_bounds__(1024) mi355_fill_u##U##_s##S(mi355::FillArgs a) { \
+  MI355_KERNEL(1024) void mi355_fill_u##U##_s##S(mi355::FillArgs a) { \
     mi355::fill_body<U, S>(a);                                                         \
   }
 MI355_FOR_EACH_FILL_KERNEL(MI355_DEFINE_FILL)
 
 #define MI355_DEFINE_BATCH_RECORDS(P, L, S)                                            \
-  extern "C" __global__ void __launch_bounds__(1024)                                   \
+  MI355_KERNEL(1024) void                                   \
       mi355_batch_records_p##P##_l##L##_s##S(mi355::BatchCopyArgs a) {                 \
     mi355::batch_copy_records_body<P, L != 0, S>(a);                                   \
   }
 MI355_FOR_EACH_BATCH_RECORDS_KERNEL(MI355_DEFINE_BATCH_RECORDS)
 
 #define MI355_DEFINE_RECT(U, L, S)                                                     \
-  extern "C" __global__ void __launch_bounds__(1024)                                   \
+  MI355_KERNEL(1024) void                                   \
       mi355_rect_u##U##_l##L##_s##S(mi355::RectArgs a) {                               \
     mi355::rect_copy_body<U, L != 0, S>(a);                                            \
   }
 MI355_FOR_EACH_RECT_KERNEL(MI355_DEFINE_RECT)
 
 #define MI355_DEFINE_RECT_NARROW(L, S)                                                 \
-  extern "C" __global__ void __launch_bounds__(1024)                                   \
+  MI355_KERNEL(1024) void                                   \
       mi355_rect_narrow_l##L##_s##S(mi355::RectNarrowArgs a) {                         \
     mi355::rect_narrow_body<L != 0, S>(a);                                             \
   }
 MI355_FOR_EACH_RECT_NARROW_KERNEL(MI355_DEFINE_RECT_NARROW)
 
 #define MI355_DEFINE_BATCH_LOOKUP(L, S)                                                \
-  extern "C" __global__ void __launch_bounds__(1024)                                   \
+  MI355_KERNEL(1024) void                                   \
       mi355_batch_lookup_l##L##_s##S(mi355::BatchLookupArgs a) {                       \
     mi355::batch_copy_lookup_body<L != 0, S>(a);                                       \
   }
 MI355_FOR_EACH_BATCH_LOOKUP_KERNEL(MI355_DEFINE_BATCH_LOOKUP)
 
-extern "C" __global__ void __launch_bounds__(1024) mi355_batch_scan_local(mi355::ScanLocalArgs a) {
+MI355_KERNEL(1024) void mi355_batch_scan_local(mi355::ScanLocalArgs a) {
   mi355::scan_local_body(a);
 }
-extern "C" __global__ void __launch_bounds__(1024) mi355_batch_scan_top(mi355::ScanTopArgs a) {
+MI355_KERNEL(1024) void mi355_batch_scan_top(mi355::ScanTopArgs a) {
   mi355::scan_top_body(a);
 }
-extern "C" __global__ void __launch_bounds__(256) mi355_batch_emit_records(mi355::EmitRecordsArgs a) {
+MI355_KERNEL(256) void mi355_batch_emit_records(mi355::EmitRecordsArgs a) {
   mi355::emit_records_body(a);
 }
-extern "C" __global__ void __launch_bounds__(256) mi355_batch_emit_records_lookup(mi355::EmitRecordsDeviceArgs a) {
+MI355_KERNEL(256) void mi355_batch_emit_records_lookup(mi355::EmitRecordsDeviceArgs a) {
   mi355::emit_records_lookup_body(a);
 }
-extern "C" __global__ void __launch_bounds__(64) mi355_signal_complete(mi355::SignalArgs a) {
+MI355_KERNEL(64) void mi355_signal_complete(mi355::SignalArgs a) {
   mi355::signal_complete_body(a);
 }
 

@@ -13,6 +13,7 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include "blit_args.h"
 #include "mi355_blit.h"
 
 namespace mi355 {
@@ -276,6 +277,49 @@ inline int plan_fill(uint64_t ptr, uint64_t num_dwords, uint32_t num_cus,
   apply_launch_shape(p, pick_class(kFillClasses, bytes), num_cus, t);
   p->nt_load = 0;
   return MI355_BLIT_SUCCESS;
+}
+
+// Which waves of a launch take the cut tiles at both ends and the head / tail
+// bytes: the two after the wave of the last full tile.
+inline void plan_tail_waves(const mi355_blit_plan_t& p, uint32_t* partial_wave, uint32_t* edge_wave,
+                            uint32_t* waves_per_wg, uint32_t* n_waves_out) {
+  const uint64_t n_waves = static_cast<uint64_t>(p.grid) * (p.wg_size / 64);
+  *waves_per_wg = p.wg_size / 64;
+  *n_waves_out = static_cast<uint32_t>(n_waves);
+  // full tiles, as tile_range() counts them on the device
+  const uint64_t first_full = p.lead_vecs ? 1 : 0;
+  const uint64_t end_full = (p.body_vecs + p.lead_vecs) / (64ull * p.unroll);
+  const uint64_t n_full = end_full > first_full ? end_full - first_full : 0;
+  *partial_wave = static_cast<uint32_t>(n_full % n_waves);
+  *edge_wave = static_cast<uint32_t>((n_full + 1) % n_waves);
+}
+
+// The kernel argument block of a planned copy / fill: what either submission
+// path hands to the kernel (p.grid workgroups of p.wg_size).
+inline CopyArgs make_copy_args(const mi355_blit_plan_t& p, void* dst, const void* src, uint64_t bytes) {
+  CopyArgs a{};
+  a.dst = static_cast<uint8_t*>(dst);
+  a.src = static_cast<const uint8_t*>(src);
+  a.bytes = bytes;
+  a.n_vec = p.body_vecs;
+  a.head = static_cast<uint32_t>(p.head_bytes);
+  a.lead = p.lead_vecs;
+  plan_tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
+  a.xcd = make_xcd_runs(p.grid, p.xcd_run);
+  return a;
+}
+
+inline FillArgs make_fill_args(const mi355_blit_plan_t& p, void* ptr, uint32_t value, uint64_t num_dwords) {
+  FillArgs a{};
+  a.dst = static_cast<uint32_t*>(ptr);
+  a.n_dwords = num_dwords;
+  a.n_vec = p.body_vecs;
+  a.head = static_cast<uint32_t>(p.head_bytes / 4);
+  a.lead = p.lead_vecs;
+  a.value = value;
+  plan_tail_waves(p, &a.partial_wave, &a.edge_wave, &a.waves_per_wg, &a.n_waves);
+  a.xcd = make_xcd_runs(p.grid, p.xcd_run);
+  return a;
 }
 
 }  // namespace mi355

@@ -47,7 +47,8 @@ def parse_args():
     # default warm-up covers it.
     ap.add_argument("--warmup", type=int, default=WARMUP_AFTER_IDLE)
     ap.add_argument("--workload", default="copy",
-                    choices=["copy", "fill", "misaligned", "batch", "rect", "calib", "idle_series", "batch_layouts"])
+                    choices=["copy", "fill", "misaligned", "batch", "rect", "calib", "idle_series", "batch_layouts",
+                             "sustain"])
     ap.add_argument("--bytes", type=int, default=GIB, help="transfer size of the copy/fill workloads")
     ap.add_argument("--rect", default="8192,131072,262144,0,0",
                     help="shape of the rect workload: rows,width,pitch[,source x,destination x] in bytes")
@@ -58,6 +59,10 @@ def parse_args():
                          "mi355_blit_tuning_t separated by commas (e.g. store_policy=2,xcd_run=1)")
     ap.add_argument("--constant-bytes", action="store_true",
                     help="idle_series: copy a source of constant bytes instead of the workload's seeded random ones")
+    ap.add_argument("--settle-ms", type=float, default=60.0,
+                    help="milliseconds of back-to-back launches of the workload in front of the warm-up, which bring "
+                         "the device from idle to its sustained clocks (reported in the line; 0 = none)")
+    ap.add_argument("--no-sample", action="store_true", help="do not sample the clocks from sysfs around the timed region")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true",
                     help="skip the check of the timed workload's result (for runs under a profiler, whose trace "
@@ -78,19 +83,97 @@ def seeded_bytes(n, seed):
 
 
 def device_bytes(torch, n, seed=None):
-    """n + 512 bytes of device memory; with a seed, n seeded bytes from the
-    first 256-byte boundary on."""
+    """n + 512 bytes of device memory; with a seed, n seeded uniform random
+    bytes from the first 256-byte boundary on, drawn on the device (a seeded
+    generator of the device's own: the host stays out of it, and the GPU is not
+    left idle for the seconds a host-side draw and upload of a GiB take)."""
     t = torch.empty(n + 512, dtype=torch.uint8, device="cuda:0")
     if seed is not None:
-        # seeded on the host, in 64 MiB pieces
-        step = 64 * MIB
+        g = torch.Generator(device="cuda:0")
+        g.manual_seed(seed)
         off = (-t.data_ptr()) % 256
-        for lo in range(0, n, step):
-            m = min(step, n - lo)
-            host = seeded_bytes(m, seed + lo // step)
-            t[off + lo:off + lo + m].copy_(torch.from_numpy(host))
+        t[off:off + n].random_(0, 256, generator=g)
     torch.cuda.synchronize()
     return t
+
+
+SAMPLER_SOURCE = r"""
+import glob, os, sys, time, json, signal
+period = float(sys.argv[1])
+paths = {}
+for card in sorted(glob.glob('/sys/class/drm/card*/device')):
+    if os.path.exists(card + '/pp_dpm_sclk'):
+        paths = {'sclk': card + '/pp_dpm_sclk', 'mclk': card + '/pp_dpm_mclk'}
+        power = glob.glob(card + '/hwmon/hwmon*/power1_input') + glob.glob(card + '/hwmon/hwmon*/power1_average')
+        if power:
+            paths['power_uW'] = power[0]
+        break
+cols = sorted(paths)
+def current(path):
+    try:
+        text = open(path).read()
+    except OSError:
+        return None
+    for line in text.splitlines():
+        if line.strip().endswith('*'):
+            return line.split(':')[1].strip().rstrip('*').strip()
+    return text.strip()[:32]
+stop = []
+signal.signal(signal.SIGTERM, lambda *a: stop.append(1))
+samples = []
+while not stop and len(samples) < 400000:
+    samples.append([time.perf_counter()] + [current(paths[k]) for k in cols])
+    time.sleep(period)
+json.dump({'columns': cols, 'samples': samples}, sys.stdout)
+"""
+
+
+class SysfsSampler:
+    """The clocks and the power the driver reports for the first GPU, read from
+    sysfs every `period` seconds while a measurement runs -- by a process of
+    its own, which never touches the GPU: a sampling thread in this process
+    would take the interpreter lock from the thread that launches and waits
+    (measured: 1.5 us per step of a 20-step timed region).  Its clock,
+    time.perf_counter, is the system's monotonic clock and so the same as this
+    process's."""
+
+    def __init__(self, period=0.002):
+        self.period = period
+        self.proc = None
+        self.cols, self.samples = [], []
+
+    def columns(self):
+        return self.cols
+
+    def start(self):
+        import subprocess
+        self.proc = subprocess.Popen([sys.executable, "-c", SAMPLER_SOURCE, str(self.period)], stdout=subprocess.PIPE,
+                                     stderr=subprocess.DEVNULL, text=True)
+        return self
+
+    def stop(self):
+        if self.proc:
+            self.proc.terminate()
+            try:
+                out, _ = self.proc.communicate(timeout=20)
+                got = json.loads(out)
+                self.cols, self.samples = got["columns"], [tuple(x) for x in got["samples"]]
+            except Exception:  # a sampler that fails costs the line its clock columns, nothing else
+                self.proc.kill()
+            self.proc = None
+        return self
+
+    def changes(self, t0, t1=None):
+        """The samples between t0 and t1 that differ from the one before, as
+        [ms since t0, columns...]."""
+        out, last = [], None
+        for smp in self.samples:
+            if smp[0] < t0 - 0.003 or (t1 is not None and smp[0] > t1 + 0.003):
+                continue
+            if smp[1:] != last:
+                out.append([round((smp[0] - t0) * 1e3, 1)] + list(smp[1:]))
+                last = smp[1:]
+        return out
 
 
 class Runner:
@@ -123,10 +206,32 @@ class Runner:
         for _ in range(steps):
             fn()
         e1.record(self.tstream)
+        # the host watches for the closing event instead of sleeping on it: a blocked wait's wake-up is a few
+        # tens of microseconds of a 6 ms region; the synchronisation behind it then returns at once
+        while not e1.query():
+            pass
         self.tstream.synchronize()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
         return t1 - t0, e0.elapsed_time(e1) * 1e3 / steps
+
+    def settle(self, fn, min_ms):
+        """Back-to-back launches of the workload until min_ms of them have run:
+        brings the device from idle to its sustained state (clocks, power) before
+        anything is timed.  Returns (launches, milliseconds)."""
+        t0 = time.perf_counter()
+        n = 0
+        while (time.perf_counter() - t0) * 1e3 < min_ms:
+            for _ in range(8):
+                fn()
+            n += 8
+            self.tstream.synchronize()
+        return n, (time.perf_counter() - t0) * 1e3
+
+    def time_settled(self, fn, steps, settle_ms=40.0, warmup=5):
+        """time_launches behind a settle burst: what the secondary figures use."""
+        self.settle(fn, settle_ms)
+        return self.time_launches(fn, steps, warmup)
 
     def time_each(self, fn, steps, warmup):
         """Durations of `steps` consecutive launches, one by one: an event is
@@ -308,7 +413,7 @@ def batch_layouts(r, n=65536, arena=8 * GIB):
         fn = lambda: r.check(r.blit.copy_batch(descs, m, False, r.stream), "copy_batch")
         dst.zero_()
         r.torch.cuda.synchronize()
-        _, us = r.time_launches(fn, 20, WARMUP_AFTER_IDLE)
+        _, us = r.time_settled(fn, 20)
         for i in (range(m) if m <= 512 else rng.integers(0, m, 512)):
             a = dst[dh + int(at[i] + d_off[i]):dh + int(at[i] + d_off[i] + ln[i])]
             b = src[sh + int(at[i] + s_off[i]):sh + int(at[i] + s_off[i] + ln[i])]
@@ -317,7 +422,7 @@ def batch_layouts(r, n=65536, arena=8 * GIB):
         out[name] = {"us_per_batch": round(us, 1), "bytes": algo, "gbs": round(algo / us / 1e3, 1),
                      "frac_of_peak": round(algo / us / 1e3 / HBM_PEAK_GBS, 4)}
     fn = lambda: r.check(r.blit.copy(D, S, 2 * GIB, r.stream), "copy")
-    _, us = r.time_launches(fn, 20, WARMUP_AFTER_IDLE)
+    _, us = r.time_settled(fn, 20)
     out["for comparison: linear copy of 2 GiB"] = {"us_per_launch": round(us, 1), "bytes": 4 * GIB,
                                                   "gbs": round(4 * GIB / us / 1e3, 1),
                                                   "frac_of_peak": round(4 * GIB / us / 1e3 / HBM_PEAK_GBS, 4)}
@@ -383,7 +488,7 @@ def rect_shapes(r):
     out = {}
     for rows, width, pitch, sx, dx in RECT_SHAPES:
         fn, verify, algo, keep = make_rect(r, rows, width, pitch, sx, dx)
-        _, us = r.time_launches(fn, 20, WARMUP_AFTER_IDLE)
+        _, us = r.time_settled(fn, 20)
         verify()
         rec = {"gbs": round(algo / us / 1e3, 1), "us_per_launch": round(us, 2),
                "unroll": r.blit.last_plan().unroll}
@@ -412,14 +517,123 @@ def size_sweep(r):
     for k in range(11):
         n = 4096 * 4 ** k
         iters = 100 if n <= MIB else (30 if n <= 256 * MIB else 8)
-        _, us = r.time_launches(lambda: r.check(r.blit.copy(D, S, n, r.stream), "copy"), iters, WARMUP_AFTER_IDLE)
+        _, us = r.time_settled(lambda: r.check(r.blit.copy(D, S, n, r.stream), "copy"), iters)
         out["copy"][str(n)] = {"us": round(us, 2), "gbs": round(2 * n / us / 1e3, 1)}
-        _, us = r.time_launches(lambda: r.check(r.blit.fill32(D, FILL_VALUE, n // 4, r.stream), "fill32"), iters, WARMUP_AFTER_IDLE)
+        _, us = r.time_settled(lambda: r.check(r.blit.fill32(D, FILL_VALUE, n // 4, r.stream), "fill32"), iters)
         out["fill"][str(n)] = {"us": round(us, 2), "gbs": round(n / us / 1e3, 1)}
     so, do = (-src.data_ptr()) % 256, (-dst.data_ptr()) % 256
     r.check(r.blit.copy(D, S, top, r.stream), "copy")
     r.tstream.synchronize()
     assert r.torch.equal(dst[do:do + top], src[so:so + top]), "4 GiB copy differs"
+    return out
+
+
+def misaligned_figures(r, pkg):
+    """BASELINE's misaligned configuration in full: a 1 GiB - 64 B copy for one
+    offset pair of every class the kernels distinguish -- (src - dst) & 3 picks
+    the kernel (0: dword-aligned loads, else realignment), (src - dst) & 12
+    where the source sits in its 16 bytes -- plus the headline pair (3, 9); a
+    length sweep 1 B .. 64 MiB at (3, 9), back-to-back launches; and the
+    blocking 4 KiB copy at (3, 9) on both submission paths.  Every copy is
+    compared with its source."""
+    torch = r.torch
+    n = GIB - 64
+    src = r.device_bytes(GIB + 64, seed=0xB1170004)
+    dst = r.device_bytes(GIB + 64)
+    S, D = aligned_ptr(src), aligned_ptr(dst)
+    sh, dh = S - src.data_ptr(), D - dst.data_ptr()
+
+    def same(so, do, m):
+        return torch.equal(dst[dh + do:dh + do + m], src[sh + so:sh + so + m])
+
+    out = {"classes_1GiB": {}, "length_sweep_3_9": {}, "blocking_4KiB_us": {}}
+    pairs = [((9 + c) & 15, 9) for c in range(8)] + [(3, 9)]
+    for so, do in pairs:
+        fn = lambda: r.check(r.blit.copy(D + do, S + so, n, r.stream), "copy")
+        _, us = r.time_settled(fn, 20)
+        assert same(so, do, n), "misaligned copy (%d, %d) differs" % (so, do)
+        out["classes_1GiB"]["src&15=%d,dst&15=%d" % (so, do)] = {
+            "shift": (so - do) & 3, "src_slot": (so - do) & 12, "us_per_launch": round(us, 2),
+            "gbs": round(2 * n / us / 1e3, 1), "frac_of_peak": round(2 * n / us / 1e3 / HBM_PEAK_GBS, 4)}
+    for m in (1, 64, 1024, 16 * 1024, 256 * 1024, 4 * MIB, 64 * MIB):
+        dst[dh:dh + m + 64].zero_()
+        fn = lambda: r.check(r.blit.copy(D + 9, S + 3, m, r.stream), "copy")
+        _, us = r.time_settled(fn, 100 if m <= 4 * MIB else 30)
+        assert same(3, 9, m) and int(dst[dh + 9 + m]) == 0 and int(dst[dh + 8]) == 0, "misaligned copy of %d bytes differs" % m
+        out["length_sweep_3_9"][str(m)] = {"us_per_launch": round(us, 2), "gbs": round(2 * m / us / 1e3, 2)}
+    ts = []
+    for i in range(220):
+        t0 = time.perf_counter()
+        r.check(r.blit.copy(D + 9, S + 3, 4096), "copy")
+        r.check(r.blit.synchronize(), "synchronize")
+        ts.append(time.perf_counter() - t0)
+    ts = sorted(ts[20:])
+    out["blocking_4KiB_us"]["hip"] = round(ts[len(ts) // 2] * 1e6, 2)
+    eng = pkg.aql.AqlBlit(0)
+    sig = pkg.aql.HsaSignals()
+    try:
+        c = sig.create(1)
+        ts = []
+        for i in range(220):
+            sig.store(c, 1)
+            t0 = time.perf_counter()
+            r.check(eng.copy(D + 9, S + 3, 4096, completion=c), "copy")
+            sig.wait_below_one(c)
+            ts.append(time.perf_counter() - t0)
+        ts = sorted(ts[20:])
+        out["blocking_4KiB_us"]["aql"] = round(ts[len(ts) // 2] * 1e6, 2)
+        sig.destroy(c)
+    finally:
+        eng.close()
+    assert same(3, 9, 4096)
+    out["how"] = ("1 GiB - 64 B per class: HIP events around 20 back-to-back launches behind a settle burst; length sweep: "
+                  "the same with 100 launches (30 at 64 MiB), launch-bound below a few MiB; blocking: submit to completion "
+                  "seen by the host, median of 200, through the Python binding")
+    return out
+
+
+def sustain_series(r):
+    """Whether a long transfer is slower per byte than a short one, and why: in
+    one process, back-to-back aligned copies of 1 GiB (272 launches), of 4 GiB
+    (68 launches: the same bytes, the same ~86 ms of load) and of 1 GiB again,
+    each series after a second without work, every launch timed by an event
+    behind it, with the clocks the driver reports sampled every millisecond.
+    Under `rocprofv3 --kernel-trace` the trace holds the kernels' own durations
+    for the same launches."""
+    torch = r.torch
+    top = 4 * GIB
+    src = r.device_bytes(top + 64, seed=0xB1170003)
+    dst = r.device_bytes(top + 64)
+    S, D = aligned_ptr(src), aligned_ptr(dst)
+    out = {"metric": "pace of back-to-back aligned copies, 1 GiB against 4 GiB", "unit": "us per GiB", "series": []}
+    sampler = SysfsSampler(0.001).start()
+    windows = []
+    for gib, launches in ((1, 272), (4, 68), (1, 272)):
+        n = gib * GIB
+        fn = lambda: r.check(r.blit.copy(D, S, n, r.stream), "copy")
+        r.tstream.synchronize()
+        torch.cuda.synchronize()
+        time.sleep(1.0)
+        t0 = time.perf_counter()
+        us = r.time_each(fn, launches, 0)
+        windows.append((t0, time.perf_counter()))
+        per_gib = [u / gib for u in us]
+        k = launches // 4
+
+        def mean(v):
+            return round(sum(v) / len(v), 2)
+        out["series"].append({
+            "copy_GiB": gib, "launches": launches,
+            "us_per_GiB_by_quarter_of_the_series": [mean(per_gib[i * k:(i + 1) * k]) for i in range(4)],
+            "us_per_GiB_last_half": mean(per_gib[launches // 2:]),
+            "us_per_GiB_min": round(min(per_gib), 2),
+            "us_per_launch": [round(u, 1) for u in us]})
+    sampler.stop()
+    for series, (t0, t1) in zip(out["series"], windows):
+        series["sysfs_columns"] = ["ms since first launch"] + sampler.columns()
+        series["sysfs_changes"] = sampler.changes(t0, t1)
+    so, do = (-src.data_ptr()) % 256, (-dst.data_ptr()) % 256
+    assert torch.equal(dst[do:do + top], src[so:so + top]), "4 GiB copy differs"
     return out
 
 
@@ -680,28 +894,7 @@ def idle_series(pkg, torch, nbytes, launches, idle_s, constant_bytes=False):
     The source holds the headline workload's seeded bytes or, as a control,
     the same byte everywhere: what the device's power management does to a
     burst depends on how much the data toggles."""
-    import glob
-    import threading
     aql = pkg.aql
-    paths = {}
-    for card in sorted(glob.glob("/sys/class/drm/card*/device")):
-        if os.path.exists(card + "/pp_dpm_sclk"):
-            paths = {"sclk": card + "/pp_dpm_sclk", "mclk": card + "/pp_dpm_mclk"}
-            power = glob.glob(card + "/hwmon/hwmon*/power1_input") + glob.glob(card + "/hwmon/hwmon*/power1_average")
-            if power:
-                paths["power_uW"] = power[0]
-            break
-
-    def current(path):
-        try:
-            text = open(path).read()
-        except OSError:
-            return None
-        for line in text.splitlines():
-            if line.strip().endswith("*"):
-                return line.split(":")[1].strip().rstrip("*").strip()
-        return text.strip()[:32]
-
     eng = aql.AqlBlit(0)
     sig = aql.HsaSignals()
     a = device_bytes(torch, nbytes, None if constant_bytes else 0xB1170003)
@@ -712,24 +905,15 @@ def idle_series(pkg, torch, nbytes, launches, idle_s, constant_bytes=False):
     torch.cuda.synchronize()
     eng.enable_profiling(True)
     sigs = [sig.create(1) for _ in range(launches)]
-    samples, stop = [], []
-
-    def sampler():
-        while not stop:
-            samples.append((time.perf_counter(),) + tuple(current(paths[k]) for k in sorted(paths)))
-            time.sleep(0.001)
-
+    sampler = SysfsSampler(0.001).start()
     time.sleep(idle_s)
-    th = threading.Thread(target=sampler)
-    th.start()
-    time.sleep(0.005)
     t0 = time.perf_counter()
     for c in sigs:
         assert eng.copy(B, A, nbytes, completion=c) == 0
     sig.wait_below_one(sigs[-1])
+    t1 = time.perf_counter()
     time.sleep(0.005)
-    stop.append(1)
-    th.join()
+    sampler.stop()
     ends = []
     first_start = None
     for c in sigs:
@@ -741,16 +925,10 @@ def idle_series(pkg, torch, nbytes, launches, idle_s, constant_bytes=False):
         sig.destroy(c)
     eng.close()
     pace = [round(ends[0] - first_start, 1)] + [round(ends[i] - ends[i - 1], 1) for i in range(1, launches)]
-    # the samples that differ from the one before
-    changes, last = [], None
-    for smp in samples:
-        if smp[1:] != last:
-            changes.append([round((smp[0] - t0) * 1e3, 1)] + list(smp[1:]))
-            last = smp[1:]
     return {"metric": "pace of back-to-back %d MiB copies of %s bytes after %.1f s idle, AQL path" % (
                 nbytes // MIB, "constant" if constant_bytes else "seeded random", idle_s),
             "unit": "us per launch", "launches": launches, "pace_us": pace,
-            "sysfs_columns": ["ms since first submit"] + sorted(paths), "sysfs_changes": changes}
+            "sysfs_columns": ["ms since first submit"] + sampler.columns(), "sysfs_changes": sampler.changes(t0, t1)}
 
 
 def cpu_model():
@@ -854,20 +1032,44 @@ def idle_series_hip(pkg, torch, nbytes, launches, idle_s, constant_bytes=False, 
             "unit": "us per launch", "launches": launches, "pace_us": series}
 
 
+# The sources that decide what the kernels do and how they are launched: the
+# counter figures in profiles/hbm_traffic.json hold for one state of these.
+KERNEL_SOURCES = ("blit_kernels.h", "blit_device.h", "blit_args.h", "blit_plan.h", "blit_rect.h", "blit_batch_host.h",
+                  "blit_kernel_list.h")
+
+
+def kernel_sources_sha256():
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "rocm-systems_amd", "csrc", name), "rb") as f:
+            h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()
+
+
 def load_traffic(kernel_key):
     """HBM bytes per launch from committed rocprofv3 --pmc runs (FETCH_SIZE +
-    WRITE_SIZE, scaled by a plain copy kernel of known size), if recorded."""
+    WRITE_SIZE, scaled by a plain copy kernel of known size), if recorded --
+    and only if they were taken from the kernels as they are now: the file
+    carries the hash of the kernel and plan sources it was measured on, and
+    figures from another state of them are not reported."""
     path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if not os.path.exists(path):
         return None
     with open(path) as f:
-        return json.load(f).get(kernel_key, {}).get("bytes_per_launch")
+        recorded = json.load(f)
+    if recorded.get("kernel_sources_sha256") != kernel_sources_sha256():
+        return None
+    return recorded.get(kernel_key, {}).get("bytes_per_launch")
 
 
 def main():
     args = parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus)
+    # the clock sampler is a process of its own and is started before this one touches the GPU
+    main_flow = args.workload not in ("idle_series", "sustain", "batch_layouts")
+    sampler = SysfsSampler(0.002).start() if main_flow and not args.no_sample else None
     import torch
     import __graft_entry__ as entry
     if not torch.cuda.is_available():
@@ -879,6 +1081,10 @@ def main():
         return
     r = Runner(torch, pkg)
     nbytes = args.bytes
+    if args.workload == "sustain":
+        print(json.dumps(sustain_series(r)))
+        r.blit.close()
+        return
     if args.workload == "batch_layouts":
         print(json.dumps({"metric": "batched copy on several layouts", "unit": "us per batch",
                           "layouts": batch_layouts(r)}))
@@ -916,14 +1122,44 @@ def main():
     if args.tune:
         r.check(r.blit.set_tuning(**{k: int(v) for k, v in (kv.split("=") for kv in args.tune.split(","))}), "set_tuning")
         name += " [tuning: %s]" % args.tune
+    # The timed region: [settle burst] [W warm-up launches] [K timed launches], back to back, and right behind
+    # them the same K launches once more with an event between every two, so that the line shows launch by launch
+    # what the device did around the timed region; the clocks the driver reports are sampled over all of it.
+    r.tstream.synchronize()
+    torch.cuda.synchronize()
+    t_ready = time.perf_counter()
+    t_first = time.perf_counter()
+    settle_launches, settle_ms = r.settle(fn, args.settle_ms) if args.settle_ms > 0 else (0, 0.0)
+    t_timed = time.perf_counter()
     wall, dev_us = r.time_launches(fn, args.steps, args.warmup)
+    t_replica = time.perf_counter()
+    replica = r.time_each(fn, max(args.steps, 5), 0)
+    t_end = time.perf_counter()
+    if sampler:
+        sampler.stop()
+    timed_region = {
+        "settle_ms": round(settle_ms, 1), "settle_launches": settle_launches,
+        "host_idle_before_first_launch_ms": round((t_first - t_ready) * 1e3, 2),
+        "phases_ms_since_first_launch": {"settle": [0.0, round((t_timed - t_first) * 1e3, 1)],
+                                         "warmup_and_timed": [round((t_timed - t_first) * 1e3, 1),
+                                                              round((t_replica - t_first) * 1e3, 1)],
+                                         "one_by_one": [round((t_replica - t_first) * 1e3, 1),
+                                                        round((t_end - t_first) * 1e3, 1)]},
+        "us_per_launch_one_by_one": [round(u, 1) for u in replica],
+        "sysfs_columns": (["ms since first launch"] + sampler.columns()) if sampler else None,
+        "sysfs_changes": sampler.changes(t_first, t_end) if sampler else None,
+        "what": "the device is brought to its sustained state by settle_ms of back-to-back launches of the workload "
+                "itself (BASELINE asks for the rate a transfer sustains), then W warm-up and K timed launches follow "
+                "without a gap: `value` is bytes over the host's wall clock around the K launches, roofline.kernel_us "
+                "the HIP events around the same K launches.  us_per_launch_one_by_one are the next K launches, an "
+                "event between every two (each figure includes the event's few microseconds of queue time)",
+    }
     if not args.no_verify:
         verify()
     plan = r.blit.last_plan().as_dict()
     value = algo * args.steps / wall / 1e9
     achieved = algo / dev_us / 1e3
-    # the same launches one by one (median, best), right behind the timed region
-    each = sorted(r.time_each(fn, max(args.steps, 5), 0))
+    each = sorted(replica)
     if args.tune:
         r.blit.set_tuning()
     # and how a burst of launches runs after an idle period: 60 launches one by one after 2 s without work
@@ -957,7 +1193,7 @@ def main():
                            ("batch_65536_device_descriptors", lambda: make_batch_device(r)),
                            ("rect_8192x131072_262144", lambda: make_rect(r))):
             f2, v2, a2, k2 = maker()
-            w2, us2 = r.time_launches(f2, 30, max(args.warmup, WARMUP_AFTER_IDLE))
+            w2, us2 = r.time_settled(f2, 30)
             v2()
             also[key] = {"gbs": round(a2 / us2 / 1e3, 1), "frac_of_peak": round(a2 / us2 / 1e3 / HBM_PEAK_GBS, 4),
                          "us_per_launch": round(us2, 2)}
@@ -973,6 +1209,8 @@ def main():
                 also[key]["blocking_us_median"] = round(sorted(lat)[len(lat) // 2], 1)
             del f2, v2, k2
             torch.cuda.empty_cache()
+        also["misaligned"] = misaligned_figures(r, pkg)
+        r.torch.cuda.empty_cache()
         also["small_copy_us"] = small_copy_latency(r)
         also["size_sweep"] = size_sweep(r)
         also["rect_shapes"] = rect_shapes(r)
@@ -994,9 +1232,11 @@ def main():
                      "traffic": load_traffic(traffic_key) if traffic_key else None,
                      "kernel_us": round(dev_us, 2), "algorithmic_bytes_per_launch": algo,
                      "kernel_us_median": round(each[len(each) // 2], 2), "kernel_us_best": round(each[0], 2),
-                     "per_launch_note": "median and best of %d launches timed one by one behind the timed region, "
-                                        "an event between every two (each figure includes the event's few "
-                                        "microseconds of queue time; kernel_us, the mean, does not)" % len(each)},
+                     "per_launch_note": "median and best of the %d launches timed one by one right behind the timed "
+                                        "region (timed_region.us_per_launch_one_by_one; each figure includes an "
+                                        "event's few microseconds of queue time; kernel_us, the mean over the "
+                                        "timed region, does not)" % len(each)},
+        "timed_region": timed_region,
         "idle_hump": None if hump is None else {
             "us_per_launch": hump,
             "us_per_launch_constant_bytes": hump_constant,
@@ -1007,8 +1247,8 @@ def main():
                     "in (launches 11-20 of 1 GiB copies), on either submission path and whatever the host does "
                     "meanwhile; with constant bytes it does not, and the clocks the driver reports stay where "
                     "they are: the device's power management answering the current that toggling data draws, "
-                    "not the kernel (profiles/copy_after_idle.md).  A timed region of 20 steps behind 5 warm-up "
-                    "launches lies across that window; the default warm-up of 60 launches lies behind it"},
+                    "not the kernel (profiles/copy_after_idle.md).  The timed region above is kept clear of that "
+                    "window by its settle burst"},
         "also": also,
     }
     if not args.no_cpu_baseline:

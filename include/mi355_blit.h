@@ -248,7 +248,11 @@ int mi355_blit_copy_batch_bounded(mi355_blit_t* h, const mi355_blit_desc_t* devi
  * library's device code (16.25 MiB per GPU, held from the load of the library
  * to the end of the process) instead of buffers the handle grows on demand,
  * and the call makes no hipMalloc, hipFree or other allocating call: four
- * kernel launches on the stream and nothing else.
+ * kernel launches on the stream and nothing else -- no event, no wait, no
+ * write to host memory (and a hipSetDevice pair only when the calling thread's
+ * current device is not the handle's).  For the same reason the command is not
+ * entered in the pending-bytes ledger: mi355_blit_pending_bytes does not see
+ * it, and the caller, who owns the stream, waits on the stream.
  * Limits: n <= MI355_BLIT_NOALLOC_MAX_COPIES, more -> OUT_OF_RESOURCES and
  * nothing is launched.  The bytes are not limited: the array has room for
  * 2^19 chunk records (2 GiB of copies) and chunks beyond them are found
@@ -338,6 +342,20 @@ int mi355_blit_plan_rect_route(const mi355_pitched_ptr_t* dst, const mi355_dim3_
  * of a signal created by hsa_signal_create / hsa_amd_signal_create (its memory
  * is visible to every GPU); it must stay alive until it has been decremented. */
 int mi355_blit_signal_complete(mi355_blit_t* h, uint64_t hsa_signal_handle, void* stream);
+
+/* Timestamps for a command on a stream, in the signal's start_ts / end_ts:
+ * replaces what the packet processor writes into the completion signal of a
+ * dispatch on a queue whose profiling bit BlitKernel::EnableProfiling has set
+ * (amd_blit_kernel.cpp:839-842; read by hsa_amd_profiling_get_async_copy_time,
+ * hsa_ext_amd.cpp:474-502).  A HIP stream has no such bit, so a one-lane kernel
+ * queued in front of the command stamps start_ts and the completion kernel
+ * behind it stamps end_ts before it decrements the signal.  The stamps are
+ * ticks of the GPU's own clock, as the packet processor's are;
+ * hsa_amd_profiling_convert_tick_to_system_domain converts them. */
+#define MI355_BLIT_STAMP_START 1u            /* start_ts = now */
+#define MI355_BLIT_STAMP_END_AND_COMPLETE 2u /* end_ts = now, then as mi355_blit_signal_complete */
+#define MI355_BLIT_STAMP_END 3u              /* end_ts = now; the signal's value is left alone */
+int mi355_blit_signal_stamp(mi355_blit_t* h, uint64_t hsa_signal_handle, uint32_t which, void* stream);
 
 /* Runs fn(user) on a host thread once every command submitted before it on the
  * stream has completed: the host-side alternative to

@@ -68,6 +68,24 @@ int mi355_aql_create_on(uint64_t hsa_agent_handle, void* hsa_queue, mi355_aql_t*
  * caller must).  A borrowed queue and a borrowed runtime are left alone. */
 int mi355_aql_destroy(mi355_aql_t* h);
 
+/* The kernels of one GPU agent.  The reference's agent owns the blit shaders:
+ * GpuAgent::AssembleShader makes the code once and every BlitKernel of the
+ * agent's blits_[] slots runs it, GpuAgent::ReleaseShader frees it
+ * (core/runtime/amd_gpu_agent.cpp:251-428, core/runtime/amd_blit_kernel.cpp:
+ * 574-590, 600-604).  Here the gfx950 code object is loaded once per agent and
+ * process: every engine created on the agent (mi355_aql_create,
+ * mi355_aql_create_on) takes a reference to the same executable and gives it
+ * back in mi355_aql_destroy, and the last reference unloads it, whatever the
+ * order.  An owner that wants the executable to outlive its engines -- the
+ * agent itself, which creates its blits lazily and drops them at will -- holds
+ * a reference of its own with _acquire / _release; the runtime must be up for
+ * both.  _info tells which executable (hsa_executable_t.handle) an engine runs
+ * and how many references it has at the moment. */
+typedef struct mi355_aql_code_object mi355_aql_code_object_t;
+int mi355_aql_code_object_acquire(uint64_t hsa_agent_handle, mi355_aql_code_object_t** out);
+int mi355_aql_code_object_release(mi355_aql_code_object_t* code);
+int mi355_aql_code_object_info(mi355_aql_t* h, uint64_t* executable_handle, uint32_t* users);
+
 /* Tells the engine that its queue has stopped on an asynchronous error: what
  * the error callback of a queue the engine created does by itself, and what
  * the owner of a borrowed queue forwards from its own callback (the role of
@@ -100,7 +118,15 @@ int mi355_aql_fill32_sync(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_
  * one KERNEL_DISPATCH packet whose completion_signal is `completion_signal`
  * (decremented once by the packet processor when the copy is done).
  * dst or src NULL -> INVALID_ARGUMENT.  bytes == 0: a barrier packet carries
- * the dependencies and the completion signal, nothing is copied. */
+ * the dependencies and the completion signal, nothing is copied.
+ * The dispatch packet's barrier bit: set behind dependency barriers (the copy
+ * must not start before them); otherwise clear, as in the reference
+ * (amd_blit_kernel.cpp:870-882: consecutive blits may overlap), with one
+ * exception on an engine that runs on a queue of its own (mi355_aql_create):
+ * there a copy, fill or region copy of 4 MiB or more carries the bit, because
+ * two large transfers that overlap slow each other down
+ * (mi355_aql_set_large_transfer_barrier).  An engine on a borrowed queue
+ * (mi355_aql_create_on) keeps the reference's packets. */
 int mi355_aql_copy(mi355_aql_t* h, void* dst, const void* src, size_t bytes,
                    const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal);
 
@@ -119,8 +145,12 @@ int mi355_aql_fill32(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dword
                      const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal);
 
 /* Batched small copies (no counterpart in the reference): n host-resident
- * descriptors, one submission of two packets, the last one carrying the
- * completion signal. */
+ * descriptors in one submission, the last packet carrying the completion
+ * signal: two dispatch packets when the host walks the descriptors (record
+ * kernel, copy), four when it stages them as they are for the GPU to do the
+ * prefix sum (chosen for thousands of short copies, and whenever no batch is
+ * running on the engine), behind ceil(num_deps / 5) barrier packets -- all with
+ * the barrier bit set.  That matters on a borrowed 64-packet queue. */
 int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t n,
                          const uint64_t* dep_signals, uint32_t num_deps, uint64_t completion_signal);
 
@@ -197,6 +227,18 @@ int mi355_aql_num_cus(mi355_aql_t* h);
  * enough when no other device or the host reads the result without a later
  * system-scope release. */
 int mi355_aql_set_system_scope_fences(mi355_aql_t* h, int enable);
+
+/* Whether a copy, fill or region copy of 4 MiB or more carries the barrier bit
+ * although no dependency asks for it (1) or is queued like the reference's
+ * blits, bit clear (0).  With the bit clear the packet processor starts a
+ * transfer while the one before still drains; the two then work on stretches
+ * of memory far apart and both slow down (back-to-back 1 GiB copies: 334 us
+ * apiece overlapping, 317 us one after the other).  With the bit set a transfer
+ * waits for every earlier packet on the queue, other producers' included,
+ * which is why the default is 1 on a queue of the engine's own
+ * (mi355_aql_create) and 0 on a borrowed one (mi355_aql_create_on).  A
+ * stronger order than core::Blit promises, never a weaker one. */
+int mi355_aql_set_large_transfer_barrier(mi355_aql_t* h, int enable);
 
 /* hsa_agent_t.handle of the engine's GPU. */
 uint64_t mi355_aql_gpu_agent(mi355_aql_t* h);

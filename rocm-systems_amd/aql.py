@@ -14,6 +14,10 @@ SIGNATURES = {
     "mi355_aql_create_on": (C.c_int, [C.c_uint64, C.c_void_p, C.POINTER(C.c_void_p)]),
     "mi355_aql_destroy": (C.c_int, [C.c_void_p]),
     "mi355_aql_report_queue_error": (C.c_int, [C.c_void_p, C.c_int]),
+    "mi355_aql_set_large_transfer_barrier": (C.c_int, [C.c_void_p, C.c_int]),
+    "mi355_aql_code_object_acquire": (C.c_int, [C.c_uint64, C.POINTER(C.c_void_p)]),
+    "mi355_aql_code_object_release": (C.c_int, [C.c_void_p]),
+    "mi355_aql_code_object_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32)]),
     "mi355_aql_wait_signal": (C.c_int, [C.c_void_p, C.c_uint64]),
     "mi355_aql_copy_sync": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint32]),
     "mi355_aql_fill32_sync": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_size_t]),
@@ -122,6 +126,17 @@ class AqlBlit:
 
     def wait_signal(self, signal):
         return self.lib.mi355_aql_wait_signal(self.handle, signal)
+
+    def set_large_transfer_barrier(self, enable):
+        return self.lib.mi355_aql_set_large_transfer_barrier(self.handle, 1 if enable else 0)
+
+    def code_object_info(self):
+        """(hsa_executable_t.handle the engine's kernels come from, references to it)."""
+        exe, users = C.c_uint64(), C.c_uint32()
+        st = self.lib.mi355_aql_code_object_info(self.handle, C.byref(exe), C.byref(users))
+        if st != SUCCESS:
+            raise RuntimeError("mi355_aql_code_object_info failed: 0x%x" % st)
+        return exe.value, users.value
 
     def report_queue_error(self, status=ERROR):
         return self.lib.mi355_aql_report_queue_error(self.handle, status)

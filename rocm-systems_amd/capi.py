@@ -108,6 +108,7 @@ SIGNATURES = {
                                              C.POINTER(Dim3), C.POINTER(Dim3), C.POINTER(Tuning), C.c_uint32,
                                              C.POINTER(RectPlan)]),
     "mi355_blit_signal_complete": (C.c_int, [C.c_void_p, C.c_uint64, C.c_void_p]),
+    "mi355_blit_signal_stamp": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint32, C.c_void_p]),
     "mi355_blit_add_callback": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "mi355_blit_synchronize": (C.c_int, [C.c_void_p]),
     "mi355_blit_pending_bytes": (C.c_uint64, [C.c_void_p]),

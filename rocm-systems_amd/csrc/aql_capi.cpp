@@ -12,6 +12,7 @@
 #include <xmmintrin.h>
 
 #include <atomic>
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -83,6 +84,31 @@ int to_status(hsa_status_t s) { return static_cast<int>(s); }
 
 }  // namespace
 
+// The kernels of one GPU agent: one loaded executable and the kernel objects
+// found in it, shared by every engine on that agent and released with the last
+// reference.  In the reference the agent owns the blit shaders
+// (GpuAgent::AssembleShader / ReleaseShader, core/runtime/amd_gpu_agent.cpp:
+// 251-428) and hands the same code to each of its blits_[] slots.
+struct mi355_aql_code_object {
+  hsa_agent_t gpu{};
+  hsa_executable_t exe{};
+  hsa_code_object_reader_t reader{};
+  bool have_exe = false, have_reader = false;
+  std::vector<CopyKernel> copy_kernels{MI355_FOR_EACH_COPY_KERNEL(MI355_COPY_NAME)};
+  std::vector<FillKernel> fill_kernels{MI355_FOR_EACH_FILL_KERNEL(MI355_FILL_NAME)};
+  std::vector<BatchKernel> batch_kernels{MI355_FOR_EACH_BATCH_RECORDS_KERNEL(MI355_BATCH_NAME)};
+  std::vector<RectKernel> rect_kernels{MI355_FOR_EACH_RECT_KERNEL(MI355_RECT_NAME)};
+  std::vector<RectKernel> rect_narrow_kernels{MI355_FOR_EACH_RECT_NARROW_KERNEL(MI355_RECT_NARROW_NAME)};
+  std::vector<RectKernel> batch_lookup_kernels{MI355_FOR_EACH_BATCH_LOOKUP_KERNEL(MI355_BATCH_LOOKUP_NAME)};
+  Kernel scan_local, scan_top, emit_records, emit_records_lookup;
+  uint32_t users = 0;  // guarded by g_code_objects_lock
+
+  ~mi355_aql_code_object() {
+    if (have_exe) hsa_executable_destroy(exe);
+    if (have_reader) hsa_code_object_reader_destroy(reader);
+  }
+};
+
 struct mi355_aql {
   hsa_agent_t gpu{};
   hsa_agent_t cpu{};
@@ -117,16 +143,8 @@ struct mi355_aql {
   // in host memory; 64 KiB: equal; 1 MiB: 10.9 against 21.4 us).
   uint8_t* kernargs_host = nullptr;
 
-  hsa_executable_t exe{};
-  hsa_code_object_reader_t reader{};
-  bool have_exe = false, have_reader = false;
-  std::vector<CopyKernel> copy_kernels{MI355_FOR_EACH_COPY_KERNEL(MI355_COPY_NAME)};
-  std::vector<FillKernel> fill_kernels{MI355_FOR_EACH_FILL_KERNEL(MI355_FILL_NAME)};
-  std::vector<BatchKernel> batch_kernels{MI355_FOR_EACH_BATCH_RECORDS_KERNEL(MI355_BATCH_NAME)};
-  std::vector<RectKernel> rect_kernels{MI355_FOR_EACH_RECT_KERNEL(MI355_RECT_NAME)};
-  std::vector<RectKernel> rect_narrow_kernels{MI355_FOR_EACH_RECT_NARROW_KERNEL(MI355_RECT_NARROW_NAME)};
-  std::vector<RectKernel> batch_lookup_kernels{MI355_FOR_EACH_BATCH_LOOKUP_KERNEL(MI355_BATCH_LOOKUP_NAME)};
-  Kernel scan_local, scan_top, emit_records, emit_records_lookup;
+  // the agent's kernels: a reference taken at creation, given back by destroy
+  mi355_aql_code_object* code = nullptr;
 
   hsa_signal_t idle_signal{};  // completion signal of wait_idle's barrier packet
   // Completion signal of the blocking calls, guarded by sync_lock
@@ -152,6 +170,9 @@ struct mi355_aql {
   mi355_blit_plan_t last_plan{};
   uint32_t reference_engine = 0;  // MI355_ENGINE_* of the last asynchronous copy the caller policy judged
   uint16_t fence_scope = HSA_FENCE_SCOPE_SYSTEM;
+  // Transfers of 4 MiB and more carry the barrier bit (serialise()): set for an
+  // engine on a queue of its own, clear on a borrowed queue.
+  std::atomic<bool> serialise_large{false};
   std::atomic<bool> queue_error{false};
 
   // batched path: two staging buffers used alternately, device buffers.  The
@@ -299,10 +320,10 @@ void log_dispatch_packet(mi355_aql* h, uint16_t header, uint16_t setup, const hs
 // measurements and for systems whose BAR writes misbehave).
 bool force_host_kernargs() { return env_is_one("MI355_BLIT_HOST_KERNARGS"); }
 
-int lookup(mi355_aql* h, const char* name, Kernel* out) {
+int lookup(mi355_aql_code_object* c, const char* name, Kernel* out) {
   const std::string sym = std::string(name) + ".kd";
   hsa_executable_symbol_t s;
-  AQL_HSA(hsa_executable_get_symbol_by_name(h->exe, sym.c_str(), &h->gpu, &s));
+  AQL_HSA(hsa_executable_get_symbol_by_name(c->exe, sym.c_str(), &c->gpu, &s));
   AQL_HSA(hsa_executable_symbol_get_info(s, HSA_EXECUTABLE_SYMBOL_INFO_KERNEL_OBJECT, &out->object));
   AQL_HSA(hsa_executable_symbol_get_info(s, HSA_EXECUTABLE_SYMBOL_INFO_KERNEL_KERNARG_SEGMENT_SIZE,
                                          &out->kernarg_size));
@@ -315,45 +336,102 @@ int lookup(mi355_aql* h, const char* name, Kernel* out) {
 }
 
 // What AssembleShader does for the reference, with a real code object.
-int load_code_object(mi355_aql* h) {
+int load_code_object(mi355_aql_code_object* c) {
   const size_t size = static_cast<size_t>(mi355_blit_hsaco_end - mi355_blit_hsaco);
-  AQL_HSA(hsa_code_object_reader_create_from_memory(mi355_blit_hsaco, size, &h->reader));
-  h->have_reader = true;
-  AQL_HSA(hsa_executable_create_alt(HSA_PROFILE_FULL, HSA_DEFAULT_FLOAT_ROUNDING_MODE_DEFAULT, nullptr, &h->exe));
-  h->have_exe = true;
-  AQL_HSA(hsa_executable_load_agent_code_object(h->exe, h->gpu, h->reader, nullptr, nullptr));
-  AQL_HSA(hsa_executable_freeze(h->exe, nullptr));
+  AQL_HSA(hsa_code_object_reader_create_from_memory(mi355_blit_hsaco, size, &c->reader));
+  c->have_reader = true;
+  AQL_HSA(hsa_executable_create_alt(HSA_PROFILE_FULL, HSA_DEFAULT_FLOAT_ROUNDING_MODE_DEFAULT, nullptr, &c->exe));
+  c->have_exe = true;
+  AQL_HSA(hsa_executable_load_agent_code_object(c->exe, c->gpu, c->reader, nullptr, nullptr));
+  AQL_HSA(hsa_executable_freeze(c->exe, nullptr));
   int rc;
-  for (auto& k : h->copy_kernels)
-    if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
-  for (auto& k : h->fill_kernels)
-    if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
-  for (auto& k : h->batch_kernels)
-    if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
-  for (auto& k : h->rect_kernels)
-    if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
-  for (auto& k : h->rect_narrow_kernels)
-    if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
-  if ((rc = lookup(h, "mi355_batch_scan_local", &h->scan_local)) != MI355_BLIT_SUCCESS) return rc;
-  if ((rc = lookup(h, "mi355_batch_scan_top", &h->scan_top)) != MI355_BLIT_SUCCESS) return rc;
-  if ((rc = lookup(h, "mi355_batch_emit_records", &h->emit_records)) != MI355_BLIT_SUCCESS) return rc;
-  if ((rc = lookup(h, "mi355_batch_emit_records_lookup", &h->emit_records_lookup)) != MI355_BLIT_SUCCESS) return rc;
-  for (auto& k : h->batch_lookup_kernels)
-    if ((rc = lookup(h, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
+  for (auto& k : c->copy_kernels)
+    if ((rc = lookup(c, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
+  for (auto& k : c->fill_kernels)
+    if ((rc = lookup(c, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
+  for (auto& k : c->batch_kernels)
+    if ((rc = lookup(c, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
+  for (auto& k : c->rect_kernels)
+    if ((rc = lookup(c, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
+  for (auto& k : c->rect_narrow_kernels)
+    if ((rc = lookup(c, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
+  if ((rc = lookup(c, "mi355_batch_scan_local", &c->scan_local)) != MI355_BLIT_SUCCESS) return rc;
+  if ((rc = lookup(c, "mi355_batch_scan_top", &c->scan_top)) != MI355_BLIT_SUCCESS) return rc;
+  if ((rc = lookup(c, "mi355_batch_emit_records", &c->emit_records)) != MI355_BLIT_SUCCESS) return rc;
+  if ((rc = lookup(c, "mi355_batch_emit_records_lookup", &c->emit_records_lookup)) != MI355_BLIT_SUCCESS) return rc;
+  for (auto& k : c->batch_lookup_kernels)
+    if ((rc = lookup(c, k.name, &k.k)) != MI355_BLIT_SUCCESS) return rc;
   return MI355_BLIT_SUCCESS;
 }
 
+// One code object per agent in this process, found by the agent's handle.
+std::mutex g_code_objects_lock;
+std::vector<mi355_aql_code_object*> g_code_objects;
+
+int code_object_acquire(hsa_agent_t gpu, mi355_aql_code_object** out) {
+  std::lock_guard<std::mutex> g(g_code_objects_lock);
+  for (mi355_aql_code_object* c : g_code_objects)
+    if (c->gpu.handle == gpu.handle) {
+      ++c->users;
+      *out = c;
+      return MI355_BLIT_SUCCESS;
+    }
+  mi355_aql_code_object* c = new (std::nothrow) mi355_aql_code_object;
+  if (!c) return MI355_BLIT_ERROR_OUT_OF_RESOURCES;
+  c->gpu = gpu;
+  const int rc = load_code_object(c);
+  if (rc != MI355_BLIT_SUCCESS) {
+    delete c;
+    return rc;
+  }
+  c->users = 1;
+  g_code_objects.push_back(c);
+  *out = c;
+  return MI355_BLIT_SUCCESS;
+}
+
+int code_object_release(mi355_aql_code_object* c) {
+  std::lock_guard<std::mutex> g(g_code_objects_lock);
+  for (size_t i = 0; i < g_code_objects.size(); ++i)
+    if (g_code_objects[i] == c) {
+      if (--c->users == 0) {
+        g_code_objects.erase(g_code_objects.begin() + static_cast<long>(i));
+        delete c;  // destroys the executable
+      }
+      return MI355_BLIT_SUCCESS;
+    }
+  return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+}
+
+
 // amd_blit_kernel.cpp:844-854: reserve num_packet slots; yield while the ring
-// is full.
-uint64_t acquire_write_index(mi355_aql* h, uint32_t num_packet) {
+// is full.  False when the queue has reported an error: before the write index
+// was touched, or, if the report came while waiting for room, once the read
+// index has stood still for two milliseconds more -- a queue that has stopped
+// never frees a slot.  The caller then writes no packet and rings no doorbell:
+// slots that were never freed may hold packets of other producers.  (While the
+// read index still moves the wait goes on: on a queue that works, a reserved
+// slot left unwritten would stop the packet processor for everybody.)
+bool acquire_write_index(mi355_aql* h, uint32_t num_packet, uint64_t* out) {
+  if (h->queue_error.load(std::memory_order_acquire)) return false;
   const uint64_t index = hsa_queue_add_write_index_scacq_screl(h->queue, num_packet);
-  // A queue that has stopped on an error never frees a slot: give up waiting
-  // (what is written then is never read, and the waits on its completion end
-  // with an error).
-  while (index + num_packet - hsa_queue_load_read_index_relaxed(h->queue) > h->queue->size &&
-         !h->queue_error.load(std::memory_order_acquire))
+  *out = index;
+  uint64_t last_read = hsa_queue_load_read_index_relaxed(h->queue);
+  auto last_progress = std::chrono::steady_clock::now();
+  while (index + num_packet - hsa_queue_load_read_index_relaxed(h->queue) > h->queue->size) {
+    if (h->queue_error.load(std::memory_order_acquire)) {
+      const uint64_t rd = hsa_queue_load_read_index_relaxed(h->queue);
+      const auto now = std::chrono::steady_clock::now();
+      if (rd != last_read) {
+        last_read = rd;
+        last_progress = now;
+      } else if (now - last_progress > std::chrono::milliseconds(2)) {
+        return false;
+      }
+    }
     sched_yield();
-  return index;
+  }
+  return true;
 }
 
 // amd_blit_kernel.cpp:935-941
@@ -461,8 +539,12 @@ uint32_t barrier_packets(uint32_t num_deps) { return (num_deps + 4) / 5; }
 // overlapping, 317 us one after the other, the gap between them included).  So
 // transfers that stream past the caches wait for the queue to drain; that is a
 // stronger order than the interface promises, never a weaker one.
+// On a queue the engine borrowed the reference's packet format is kept (bit
+// clear): with the bit set a large blit would also wait for every earlier
+// packet of the queue's other producers.  mi355_aql_set_large_transfer_barrier
+// overrides either default.
 constexpr uint64_t kSerialiseMinBytes = 4ull << 20;
-bool serialise(uint64_t bytes) { return bytes >= kSerialiseMinBytes; }
+bool serialise(const mi355_aql* h, uint64_t bytes) { return h->serialise_large.load() && bytes >= kSerialiseMinBytes; }
 
 void free_device(void* p) {
   if (p) (void)hsa_amd_memory_pool_free(p);
@@ -506,7 +588,10 @@ int wait_idle_locked(mi355_aql* h) {
   uint64_t index;
   {
     std::lock_guard<std::mutex> r(h->reservation_lock);
-    index = acquire_write_index(h, 1);
+    if (!acquire_write_index(h, 1, &index)) {
+      hsa_signal_store_relaxed(h->idle_signal, 0);
+      return MI355_BLIT_ERROR;
+    }
     record_blit_history(h, 0, index);
   }
   write_barriers(h, index, nullptr, 0, 1, h->idle_signal.handle, true);
@@ -563,7 +648,7 @@ int ensure_batch_capacity(mi355_aql* h, size_t n, size_t n_records) {
 }
 
 const Kernel* find_copy(mi355_aql* h, const mi355_blit_plan_t& p) {
-  for (const auto& v : h->copy_kernels)
+  for (const auto& v : h->code->copy_kernels)
     if (v.unroll == p.unroll && v.nt_load == p.nt_load && v.store == p.store_policy &&
         v.realign == (p.byte_shift ? 1u : 0u))
       return &v.k;
@@ -571,7 +656,7 @@ const Kernel* find_copy(mi355_aql* h, const mi355_blit_plan_t& p) {
 }
 
 const Kernel* find_batch(mi355_aql* h, const BatchLaunch& l, const mi355_blit_plan_t& p) {
-  for (const auto& v : h->batch_kernels)
+  for (const auto& v : h->code->batch_kernels)
     if (v.split == l.split && v.nt_load == p.nt_load && v.store == p.store_policy) return &v.k;
   return nullptr;
 }
@@ -601,12 +686,13 @@ int init_engine(mi355_aql* h) {
   if (hsa_system_get_info(HSA_SYSTEM_INFO_TIMESTAMP_FREQUENCY, &freq) == HSA_STATUS_SUCCESS && freq >= 1000)
     h->wait_slice_ticks = freq / 1000;
   h->log_packets = env_is_one("MI355_BLIT_LOG_PKTS");
-  if ((rc = load_code_object(h)) != MI355_BLIT_SUCCESS) return rc;
+  if ((rc = code_object_acquire(h->gpu, &h->code)) != MI355_BLIT_SUCCESS) return rc;
   if (!h->queue) {
     hsa_status_t st = hsa_queue_create(h->gpu, kQueuePackets, HSA_QUEUE_TYPE_MULTI, queue_error_cb, h, UINT32_MAX,
                                        UINT32_MAX, &h->queue);
     if (st != HSA_STATUS_SUCCESS) return to_status(st);
     h->owns_queue = true;
+    h->serialise_large.store(true);
   }
   // amd_blit_kernel.cpp:554-569: the ledger and the kernarg ring have one
   // entry per packet slot of the queue, whoever made it
@@ -717,12 +803,37 @@ int mi355_aql_destroy(mi355_aql_t* h) {
     free_device(h->bounce[1]);
     if (h->idle_signal.handle) hsa_signal_destroy(h->idle_signal);
     if (h->sync_signal.handle) hsa_signal_destroy(h->sync_signal);
-    if (h->have_exe) hsa_executable_destroy(h->exe);
-    if (h->have_reader) hsa_code_object_reader_destroy(h->reader);
+    if (h->code) code_object_release(h->code);
+    h->code = nullptr;
   }
   delete h;
   if (owns_runtime) hsa_shut_down();
   return rc;
+}
+
+int mi355_aql_code_object_acquire(uint64_t hsa_agent_handle, mi355_aql_code_object_t** out) {
+  if (!out || !hsa_agent_handle) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  *out = nullptr;
+  hsa_agent_t gpu;
+  gpu.handle = hsa_agent_handle;
+  hsa_device_type_t type;
+  hsa_status_t st = hsa_agent_get_info(gpu, HSA_AGENT_INFO_DEVICE, &type);
+  if (st != HSA_STATUS_SUCCESS) return to_status(st);
+  if (type != HSA_DEVICE_TYPE_GPU) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  return code_object_acquire(gpu, out);
+}
+
+int mi355_aql_code_object_release(mi355_aql_code_object_t* code) {
+  if (!code) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  return code_object_release(code);
+}
+
+int mi355_aql_code_object_info(mi355_aql_t* h, uint64_t* executable_handle, uint32_t* users) {
+  if (!h || !h->code) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> g(g_code_objects_lock);
+  if (executable_handle) *executable_handle = h->code->exe.handle;
+  if (users) *users = h->code->users;
+  return MI355_BLIT_SUCCESS;
 }
 
 int mi355_aql_report_queue_error(mi355_aql_t* h, int status) {
@@ -788,6 +899,12 @@ int mi355_aql_set_system_scope_fences(mi355_aql_t* h, int enable) {
   return MI355_BLIT_SUCCESS;
 }
 
+int mi355_aql_set_large_transfer_barrier(mi355_aql_t* h, int enable) {
+  if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  h->serialise_large.store(enable != 0);
+  return MI355_BLIT_SUCCESS;
+}
+
 int mi355_aql_enable_profiling(mi355_aql_t* h, int enable) {
   if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   AQL_HSA(hsa_amd_profiling_set_profiler_enabled(h->queue, enable ? 1 : 0));
@@ -839,7 +956,7 @@ int mi355_aql_copy_route(mi355_aql_t* h, void* dst, const void* src, size_t byte
     uint64_t index;
     {
       std::lock_guard<std::mutex> r(h->reservation_lock);
-      index = acquire_write_index(h, n);
+      if (!acquire_write_index(h, n, &index)) return MI355_BLIT_ERROR;
       record_blit_history(h, 0, index + n - 1);
     }
     write_barriers(h, index, dep_signals, num_deps, n, completion_signal, false);
@@ -851,14 +968,14 @@ int mi355_aql_copy_route(mi355_aql_t* h, void* dst, const void* src, size_t byte
   uint64_t index;
   {
     std::lock_guard<std::mutex> r(h->reservation_lock);
-    index = acquire_write_index(h, total);
+    if (!acquire_write_index(h, total, &index)) return MI355_BLIT_ERROR;
     record_blit_history(h, bytes, index + total - 1);
   }
   write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
   // Barrier bit clear, as in the reference: consecutive blits may overlap
   // unless linked by signals.  After dependency barriers the bit is set so
   // that the copy cannot start before them.
-  write_dispatch(h, index + nb, *k, &a, sizeof(a), p.grid, p.wg_size, completion_signal, nb != 0 || serialise(bytes));
+  write_dispatch(h, index + nb, *k, &a, sizeof(a), p.grid, p.wg_size, completion_signal, nb != 0 || serialise(h, bytes));
   release_write_index(h, index, total);
   return MI355_BLIT_SUCCESS;
 }
@@ -878,7 +995,7 @@ int mi355_aql_fill32(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dword
     std::lock_guard<std::mutex> g(h->lock);
     int rc = plan_fill(reinterpret_cast<uint64_t>(ptr), num_dwords, h->num_cus, h->has_tuning ? &h->tuning : nullptr, &p);
     if (rc != MI355_BLIT_SUCCESS) return rc;
-    for (const auto& v : h->fill_kernels)
+    for (const auto& v : h->code->fill_kernels)
       if (v.unroll == p.unroll && v.store == p.store_policy) k = &v.k;
     if (!k) return MI355_BLIT_ERROR;
     h->last_plan = p;
@@ -889,11 +1006,11 @@ int mi355_aql_fill32(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_dword
   uint64_t index;
   {
     std::lock_guard<std::mutex> r(h->reservation_lock);
-    index = acquire_write_index(h, total);
+    if (!acquire_write_index(h, total, &index)) return MI355_BLIT_ERROR;
     record_blit_history(h, num_dwords * 4, index + total - 1);
   }
   write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
-  write_dispatch(h, index + nb, *k, &a, sizeof(a), p.grid, p.wg_size, completion_signal, nb != 0 || serialise(num_dwords * 4));
+  write_dispatch(h, index + nb, *k, &a, sizeof(a), p.grid, p.wg_size, completion_signal, nb != 0 || serialise(h, num_dwords * 4));
   release_write_index(h, index, total);
   return MI355_BLIT_SUCCESS;
 }
@@ -913,9 +1030,16 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   // The packet processor publishes the read index with a delay: a batch that
   // has just finished may still count as running, which only means that the
   // host walks the descriptors as it would have anyway.
+  // Idle means nothing of this engine is in flight, batch or not: behind a
+  // running 1 GiB copy the walk is hidden just as it is behind a batch.
   auto engine_idle = [h]() {
-    return !h->any_batch || hsa_queue_load_read_index_scacquire(h->queue) > h->last_batch_index ||
-           h->known_complete.load() > h->last_batch_index;
+    uint64_t last;
+    {
+      std::lock_guard<std::mutex> r(h->reservation_lock);
+      if (!h->anything_queued) return true;
+      last = h->last_queued;
+    }
+    return hsa_queue_load_read_index_scacquire(h->queue) > last || h->known_complete.load() > last;
   };
   if (batch_prefers_raw_staging(descs, n, engine_idle, h->has_tuning ? &h->tuning : nullptr)) {
     // The walk below would take longer than the copies: stage the descriptors
@@ -991,7 +1115,10 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   uint64_t index;
   {
     std::lock_guard<std::mutex> r(h->reservation_lock);
-    index = acquire_write_index(h, total);
+    if (!acquire_write_index(h, total, &index)) {
+      hsa_signal_store_relaxed(h->stage_free[b], 0);  // armed above; nothing will read the staging buffer
+      return MI355_BLIT_ERROR;
+    }
     record_blit_history(h, total_bytes, index + total - 1);
   }
   write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
@@ -999,7 +1126,7 @@ int mi355_aql_copy_batch(mi355_aql_t* h, const mi355_blit_desc_t* descs, size_t 
   // Both packets wait for everything before them (barrier bit): the first for
   // whatever still reads the shared record buffer; it frees the staging buffer
   // when it is done with it.
-  write_dispatch(h, i++, h->emit_records, &er, sizeof(er), emit_records_grid(shape.pieces), 256,
+  write_dispatch(h, i++, h->code->emit_records, &er, sizeof(er), emit_records_grid(shape.pieces), 256,
                  h->stage_free[b].handle, true, Chain::kFirst);
   write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true, Chain::kLast);
   release_write_index(h, index, total);
@@ -1045,7 +1172,7 @@ int copy_batch_device_locked(mi355_aql_t* h, const BatchDesc* scanned, size_t n,
   mi355_blit_plan_t p;
   const BatchLaunch l = plan_batch_records(sizing.grid_chunks, sizing.bytes, true, t, false, &p);
   const Kernel* bk = nullptr;
-  for (const auto& v : h->batch_lookup_kernels)
+  for (const auto& v : h->code->batch_lookup_kernels)
     if (v.nt_load == p.nt_load && v.store == p.store_policy) bk = &v.k;
   if (!bk || l.split != 4) return MI355_BLIT_ERROR;
   BatchLookupArgs bc{{h->records_dev, sizing.records, h->chunk_start_dev + n, l.waves_per_wg, l.n_waves,
@@ -1058,16 +1185,17 @@ int copy_batch_device_locked(mi355_aql_t* h, const BatchDesc* scanned, size_t n,
   uint64_t index;
   {
     std::lock_guard<std::mutex> r(h->reservation_lock);
-    index = acquire_write_index(h, total);
+    // (a caller that armed staged_free takes it back when this fails)
+    if (!acquire_write_index(h, total, &index)) return MI355_BLIT_ERROR;
     // without a bound the lengths are unknown here: keep the record non-zero
     record_blit_history(h, max_total_bytes ? max_total_bytes : n, index + total - 1);
   }
   write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
   uint64_t i = index + nb;
   // every packet waits for the one before; the first also for whatever still uses the shared buffers
-  write_dispatch(h, i++, h->scan_local, &sl, sizeof(sl), n_blocks, 1024, staged_free, true, Chain::kFirst);
-  write_dispatch(h, i++, h->scan_top, &stp, sizeof(stp), 1, 1024, 0, true, Chain::kMiddle);
-  write_dispatch(h, i++, h->emit_records_lookup, &er, sizeof(er),
+  write_dispatch(h, i++, h->code->scan_local, &sl, sizeof(sl), n_blocks, 1024, staged_free, true, Chain::kFirst);
+  write_dispatch(h, i++, h->code->scan_top, &stp, sizeof(stp), 1, 1024, 0, true, Chain::kMiddle);
+  write_dispatch(h, i++, h->code->emit_records_lookup, &er, sizeof(er),
                  static_cast<uint32_t>((sizing.records + 255) / 256), 256, 0, true, Chain::kMiddle);
   write_dispatch(h, i++, *bk, &bc, sizeof(bc), p.grid, p.wg_size, completion_signal, true, Chain::kLast);
   release_write_index(h, index, total);
@@ -1122,10 +1250,10 @@ int mi355_aql_copy_rect_route(mi355_aql_t* h, const mi355_pitched_ptr_t* dst, co
     if (rc != MI355_BLIT_SUCCESS) return rc;
     if (!rp.empty && !rp.linear) {
       if (rp.narrow) {
-        for (const auto& v : h->rect_narrow_kernels)
+        for (const auto& v : h->code->rect_narrow_kernels)
           if (v.nt_load == rp.streaming && v.store == rp.store_policy) k = &v.k;
       } else {
-        for (const auto& v : h->rect_kernels)
+        for (const auto& v : h->code->rect_kernels)
           if (v.unroll == rp.unroll && v.nt_load == rp.streaming && v.store == rp.store_policy) k = &v.k;
       }
       if (!k) return MI355_BLIT_ERROR;
@@ -1141,16 +1269,16 @@ int mi355_aql_copy_rect_route(mi355_aql_t* h, const mi355_pitched_ptr_t* dst, co
   uint64_t index;
   {
     std::lock_guard<std::mutex> r(h->reservation_lock);
-    index = acquire_write_index(h, total);
+    if (!acquire_write_index(h, total, &index)) return MI355_BLIT_ERROR;
     record_blit_history(h, rp.total_bytes, index + total - 1);
   }
   write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
   if (rp.narrow)
     write_dispatch(h, index + nb, *k, &rp.nargs, sizeof(rp.nargs), rp.grid, rp.wg_size, completion_signal,
-                   nb != 0 || serialise(rp.total_bytes));
+                   nb != 0 || serialise(h, rp.total_bytes));
   else
     write_dispatch(h, index + nb, *k, &rp.args, sizeof(rp.args), rp.grid, rp.wg_size, completion_signal,
-                   nb != 0 || serialise(rp.total_bytes));
+                   nb != 0 || serialise(h, rp.total_bytes));
   release_write_index(h, index, total);
   return MI355_BLIT_SUCCESS;
 }
@@ -1161,7 +1289,10 @@ int mi355_aql_copy_sync(mi355_aql_t* h, void* dst, const void* src, size_t bytes
   std::lock_guard<std::mutex> g(h->sync_lock);
   hsa_signal_store_relaxed(h->sync_signal, 1);
   const int rc = mi355_aql_copy_route(h, dst, src, bytes, route, nullptr, 0, h->sync_signal.handle);
-  if (rc != MI355_BLIT_SUCCESS) return rc;
+  if (rc != MI355_BLIT_SUCCESS) {
+    hsa_signal_store_relaxed(h->sync_signal, 0);  // nothing was queued that would complete it
+    return rc;
+  }
   // a copy of no bytes completes the signal from a barrier packet
   return wait_signal(h, h->sync_signal);
 }
@@ -1172,7 +1303,10 @@ int mi355_aql_fill32_sync(mi355_aql_t* h, void* ptr, uint32_t value, size_t num_
   std::lock_guard<std::mutex> g(h->sync_lock);
   hsa_signal_store_relaxed(h->sync_signal, 1);
   const int rc = mi355_aql_fill32(h, ptr, value, num_dwords, nullptr, 0, h->sync_signal.handle);
-  if (rc != MI355_BLIT_SUCCESS) return rc;
+  if (rc != MI355_BLIT_SUCCESS) {
+    hsa_signal_store_relaxed(h->sync_signal, 0);
+    return rc;
+  }
   return wait_signal(h, h->sync_signal);
 }
 

@@ -196,9 +196,11 @@ int mi355_hsa_memory_copy(mi355_aql_t* h, void* dst, const void* src, size_t siz
     if (lock_dst.Lock(h, dst, size, &mapped) != MI355_BLIT_SUCCESS) return bounced_copy(h, dst, src, size, false);
     d = mapped;
   }
-  // Waits for this copy's own completion signal, not for the queue to drain:
-  // commands other threads have parked behind unsatisfied dependencies do not
-  // hold it up (amd_blit_kernel.cpp:614-639).
+  // Waits for this copy's own completion signal, not for the queue to drain
+  // (amd_blit_kernel.cpp:614-639).  With the barrier bit clear, commands other
+  // threads have parked behind unsatisfied dependencies do not hold the copy
+  // up either; a copy of 4 MiB or more on an engine's own queue carries the
+  // bit (mi355_aql_set_large_transfer_barrier) and does wait for them.
   return mi355_aql_copy_sync(h, d, s, size, route_of(src_sys, dst_sys));
 }
 

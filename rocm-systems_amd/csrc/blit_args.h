@@ -264,8 +264,21 @@ struct HsaSignalAbi {
 };
 static_assert(sizeof(HsaSignalAbi) == 64, "amd_signal_t is 64 bytes");
 
+// What mi355_signal_complete does to the signal.  The stamps are the signal's
+// start_ts / end_ts, which the packet processor writes for a dispatch on a
+// queue with the profiling bit set (amd_blit_kernel.cpp:839-842) and
+// hsa_amd_profiling_get_async_copy_time reads (hsa_ext_amd.cpp:474-502); on a
+// HIP stream there is no such bit and one-lane kernels in front of and behind
+// the command write them.
+constexpr uint32_t kSignalComplete = 0;             // decrement, wake waiters
+constexpr uint32_t kSignalStampStart = 1;           // start_ts = now, nothing else
+constexpr uint32_t kSignalStampEndAndComplete = 2;  // end_ts = now, then complete
+constexpr uint32_t kSignalStampEnd = 3;             // end_ts = now, nothing else
+
 struct SignalArgs {
   HsaSignalAbi* sig;
+  uint32_t mode;
+  uint32_t pad;
 };
 
 }  // namespace mi355

@@ -213,8 +213,8 @@ inline int batch_build(const mi355_blit_desc_t* descs, size_t n, BatchImage* ima
 constexpr size_t kBatchRawMinCopies = 4096;
 constexpr uint64_t kBatchRawMaxMeanBytes = 8192;
 
-// engine_idle: no batch of this engine is still running, so nothing hides the
-// walk: a batch submitted to an idle engine starts as late as the host
+// engine_idle: nothing of this engine is still running (no batch, no other
+// command), so nothing hides the walk: a batch submitted to an idle engine starts as late as the host
 // finishes with it.  Staged as they are the descriptors cost the host 1 ns
 // each instead of 3.6 and the GPU two small launches more: 65,536 copies of
 // 64 B .. 256 KiB, one batch at a time, take 927 us from submission to

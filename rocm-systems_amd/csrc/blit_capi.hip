@@ -595,12 +595,15 @@ int copy_batch(mi355_blit_t* h, const mi355_blit_desc_t* descs, size_t n, int de
   // exact chunk total, one small kernel before the copy), or, when the walk
   // would take longer than the copies themselves, they are staged as they are
   // and taken from there like device-resident ones.
-  // Whether the batch before has finished: its event is the last thing it left
-  // in its stream.
+  // Idle means nothing of this engine is in flight: the batch before has
+  // finished (its event is the last thing it left in its stream) and so has
+  // whatever was submitted since (a 1 GiB copy hides the walk as well as a
+  // batch does).
   auto engine_idle = [h]() {
     const unsigned before = h->next_host ^ 1;
     if (h->batch_busy[before] && hipEventQuery(h->batch_done[before]) == hipSuccess) h->batch_busy[before] = false;
-    return !h->batch_busy[before];
+    if (h->batch_busy[before]) return false;
+    return !h->unmarked || hipStreamQuery(h->last_stream) == hipSuccess;
   };
   const bool raw = !descs_on_device &&
                    batch_prefers_raw_staging(descs, n, engine_idle, h->has_tuning ? &h->tuning : nullptr);
@@ -743,7 +746,10 @@ int mi355_blit_copy_batch_bounded_noalloc(mi355_blit_t* h, const mi355_blit_desc
   if (rc != MI355_BLIT_SUCCESS) return rc;
   BLIT_HIP(hipGetLastError());
   h->last_plan = p;
-  return ledger_record(h, s, sizing.bytes);
+  // No entry in the pending-bytes ledger: a command on another stream than the
+  // last one makes the ledger record an event there, and a full ledger waits
+  // for its oldest one -- neither belongs in a call that is four launches.
+  return MI355_BLIT_SUCCESS;
 }
 
 int mi355_blit_copy_rect(mi355_blit_t* h, const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset,
@@ -830,16 +836,28 @@ int mi355_blit_plan_rect_route(const mi355_pitched_ptr_t* dst, const mi355_dim3_
   return MI355_BLIT_SUCCESS;
 }
 
-int mi355_blit_signal_complete(mi355_blit_t* h, uint64_t hsa_signal_handle, void* stream) {
+namespace {
+int launch_signal_kernel(mi355_blit_t* h, uint64_t hsa_signal_handle, uint32_t mode, void* stream) {
   if (!h || !hsa_signal_handle || (hsa_signal_handle & 63)) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   std::lock_guard<std::mutex> g(h->lock);
   DeviceScope scope(h->device);
   if (scope.err != hipSuccess) return status_of(scope.err);
   hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
-  SignalArgs sa{reinterpret_cast<HsaSignalAbi*>(hsa_signal_handle)};
+  SignalArgs sa{reinterpret_cast<HsaSignalAbi*>(hsa_signal_handle), mode, 0};
   hipLaunchKernelGGL(mi355_signal_complete, dim3(1), dim3(64), 0, s, sa);
   BLIT_HIP(hipGetLastError());
   return MI355_BLIT_SUCCESS;
+}
+}  // namespace
+
+int mi355_blit_signal_complete(mi355_blit_t* h, uint64_t hsa_signal_handle, void* stream) {
+  return launch_signal_kernel(h, hsa_signal_handle, kSignalComplete, stream);
+}
+
+int mi355_blit_signal_stamp(mi355_blit_t* h, uint64_t hsa_signal_handle, uint32_t which, void* stream) {
+  if (which != MI355_BLIT_STAMP_START && which != MI355_BLIT_STAMP_END && which != MI355_BLIT_STAMP_END_AND_COMPLETE)
+    return MI355_BLIT_ERROR_INVALID_ARGUMENT;
+  return launch_signal_kernel(h, hsa_signal_handle, which, stream);
 }
 
 int mi355_blit_add_callback(mi355_blit_t* h, mi355_blit_callback_t fn, void* user, void* stream) {

@@ -206,6 +206,10 @@ MI355_DEVICE unsigned thread_in_workgroup() { return threadIdx.x; }
 MI355_DEVICE unsigned workgroup_index() { return blockIdx.x; }
 MI355_DEVICE void workgroup_barrier() { __syncthreads(); }
 
+// The GPU's free-running 100 MHz counter (s_memrealtime): the clock the packet
+// processor stamps completion signals with.
+MI355_DEVICE uint64_t realtime_ticks() { return __builtin_amdgcn_s_memrealtime(); }
+
 // MSG_INTERRUPT with an event id's low byte in m0.
 MI355_DEVICE void send_interrupt(uint32_t event_id) {
   __builtin_amdgcn_s_sendmsg(1, __builtin_amdgcn_readfirstlane(event_id) & 0xff);

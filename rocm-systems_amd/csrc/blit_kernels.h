@@ -871,6 +871,14 @@ MI355_DEVICE void rect_narrow_body(const RectNarrowArgs& a) {
 MI355_DEVICE void signal_complete_body(const SignalArgs& a) {
   HsaSignalAbi* sig = a.sig;
   if (thread_in_workgroup() != 0) return;
+  if (a.mode == kSignalStampStart) {
+    st_system_release_u64(&sig->start_ts, realtime_ticks());
+    return;
+  }
+  if (a.mode == kSignalStampEndAndComplete || a.mode == kSignalStampEnd) {
+    st_system_release_u64(&sig->end_ts, realtime_ticks());
+    if (a.mode == kSignalStampEnd) return;
+  }
   signal_decrement_system(&sig->value);
   uint64_t* mailbox = reinterpret_cast<uint64_t*>(sig->event_mailbox_ptr);
   if (mailbox) {

@@ -100,6 +100,14 @@ bool BlitKernelGfx950::DepsSatisfied(const std::vector<hsa_signal_t>& deps) {
 
 hsa_status_t BlitKernelGfx950::Launch(const Command& cmd) {
   int st;
+  // With profiling on, the command's signal gets the timestamps the packet
+  // processor would give it on a profiled queue: a stamp kernel in front, the
+  // end stamp in (or, with host-callback completion, in front of) the completion.
+  const bool stamp = profiling_.load() && cmd.out.handle != 0;
+  if (stamp) {
+    st = mi355_blit_signal_stamp(blit_, cmd.out.handle, MI355_BLIT_STAMP_START, nullptr);
+    if (st != MI355_BLIT_SUCCESS) return to_hsa(st);
+  }
   switch (cmd.op) {
     case Op::Copy: st = mi355_blit_copy(blit_, cmd.dst, cmd.src, cmd.size, nullptr); break;
     case Op::Fill: st = mi355_blit_fill32(blit_, cmd.dst, cmd.value, cmd.size, nullptr); break;
@@ -114,8 +122,13 @@ hsa_status_t BlitKernelGfx950::Launch(const Command& cmd) {
   }
   if (st != MI355_BLIT_SUCCESS) return to_hsa(st);
   if (completion_ == Completion::kDeviceSignal) {
-    st = mi355_blit_signal_complete(blit_, cmd.out.handle, nullptr);
+    st = stamp ? mi355_blit_signal_stamp(blit_, cmd.out.handle, MI355_BLIT_STAMP_END_AND_COMPLETE, nullptr)
+               : mi355_blit_signal_complete(blit_, cmd.out.handle, nullptr);
   } else {
+    if (stamp) {
+      st = mi355_blit_signal_stamp(blit_, cmd.out.handle, MI355_BLIT_STAMP_END, nullptr);
+      if (st != MI355_BLIT_SUCCESS) return to_hsa(st);
+    }
     st = mi355_blit_add_callback(blit_, &BlitKernelGfx950::OnComplete,
                                  reinterpret_cast<void*>(cmd.out.handle), nullptr);
   }
@@ -247,8 +260,8 @@ hsa_status_t BlitKernelGfx950::SubmitBatchCopyCommand(const void* descs, size_t 
 hsa_status_t BlitKernelGfx950::EnableProfiling(bool enable) {
   // The reference flips the AQL queue's profiling bit so that the packet
   // processor stamps the completion signal (amd_blit_kernel.cpp:839-842).
-  // A HIP stream has no such bit: the request is recorded, timestamps are
-  // not written.
+  // A HIP stream has no such bit: while profiling is on, Launch() queues
+  // one-lane kernels that write start_ts and end_ts from the GPU's clock.
   profiling_.store(enable);
   return HSA_STATUS_SUCCESS;
 }

@@ -13,13 +13,23 @@
 // (public_handle(), profiling_enabled(): core/inc/agent.h:310, 320),
 // core::Queue (public_handle(): core/inc/queue.h:373) and core::Signal, a thin
 // view of an hsa_signal_t driven through the public hsa_signal_* API
-// (Convert(): core/inc/signal.h).  Inside a ROCr tree the stand-ins are
-// deleted and the real headers included; nothing else changes.
+// (Convert(): core/inc/signal.h:285-297).  Inside a ROCr tree
+// MI355_ROCR_IN_TREE is defined: the stand-ins and the repeated core::Blit go
+// away, the real core/inc/blit.h, agent.h, queue.h and signal.h come in, and
+// nothing else changes (tests/test_rocr_in_tree.py compiles
+// rocr_blit_aql.cpp that way against the reference's headers).
 #ifndef MI355_ROCR_BLIT_H_
 #define MI355_ROCR_BLIT_H_
 
+#ifdef MI355_ROCR_IN_TREE
+#include "core/inc/agent.h"
+#include "core/inc/blit.h"
+#include "core/inc/queue.h"
+#include "core/inc/signal.h"
+#else
 #include <hsa/hsa.h>
 #include <hsa/hsa_ext_amd.h>
+#endif
 #include <stdint.h>
 
 #include <atomic>
@@ -33,6 +43,7 @@ struct mi355_blit;
 struct mi355_aql;
 
 namespace rocr {
+#ifndef MI355_ROCR_IN_TREE
 namespace core {
 
 class Agent {
@@ -105,6 +116,7 @@ class Blit {
 };
 
 }  // namespace core
+#endif  // MI355_ROCR_IN_TREE
 
 namespace AMD {
 

@@ -470,6 +470,7 @@ MI355_DEVICE unsigned workgroup_index() { return lane_emu::g_m.workgroup; }
 MI355_DEVICE void workgroup_barrier() { lane_emu::barrier_arrive(); }
 
 // The completion of an HSA signal is not part of what runs here.
+MI355_DEVICE uint64_t realtime_ticks() { return 0; }
 MI355_DEVICE void send_interrupt(uint32_t) {}
 MI355_DEVICE void signal_decrement_system(int64_t* value) { --*value; }
 MI355_DEVICE void st_system_release_u64(uint64_t* p, uint64_t v) { *p = v; }

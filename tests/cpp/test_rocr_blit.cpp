@@ -20,6 +20,7 @@
 #include <vector>
 
 #include "../../oracle/blit_oracle.h"
+#include "blit_args.h"
 #include "mi355_blit.h"
 #include "mi355_blit_aql.h"
 #include "rocr_blit.h"
@@ -613,6 +614,63 @@ void test_profiling_timestamps(Blit& blit) {
   std::printf("PASS %s%s\n", name, g_suffix.c_str());
 }
 
+// The HIP-stream engine has no queue bit to flip: with profiling on it stamps
+// the command's signal from the device (one-lane kernels in front of and behind
+// the command).  The stamps are raw ticks of the GPU's clock, like the packet
+// processor's; converted to the system domain with the public HSA call they
+// must lie between the host's own readings of that clock around the copy.
+void test_profiling_stamps_from_device(Blit& blit) {
+  const char* name = "profiling_timestamps";
+  hsa_agent_t gpu{0};
+  hsa_iterate_agents(first_gpu_cb, &gpu);
+  REQUIRE(gpu.handle, "no GPU agent");
+  const size_t n = 64u << 20;
+  DeviceBuf a(n), b(n);
+  REQUIRE(a.p && b.p, "hipMalloc");
+  REQUIRE(blit.EnableProfiling(true) == HSA_STATUS_SUCCESS, "EnableProfiling(true)");
+  uint64_t freq = 0;
+  hsa_system_get_info(HSA_SYSTEM_INFO_TIMESTAMP_FREQUENCY, &freq);
+  REQUIRE(freq, "no timestamp frequency");
+  for (int round = 0; round < 3; ++round) {
+    hsa_signal_t s = make_signal(1);
+    Signal sig(s);
+    std::vector<Signal*> none, gang;
+    uint64_t before = 0, after = 0;
+    hsa_system_get_info(HSA_SYSTEM_INFO_TIMESTAMP, &before);
+    REQUIRE(blit.SubmitLinearCopyCommand(b.p, a.p, n, none, sig, gang) == HSA_STATUS_SUCCESS, "submit");
+    REQUIRE(wait_zero(s, HSA_WAIT_STATE_BLOCKED), "copy never completed");
+    hsa_system_get_info(HSA_SYSTEM_INFO_TIMESTAMP, &after);
+    const mi355::HsaSignalAbi* raw = reinterpret_cast<const mi355::HsaSignalAbi*>(s.handle);
+    const uint64_t start_raw = raw->start_ts, end_raw = raw->end_ts;
+    REQUIRE(start_raw != 0 && end_raw > start_raw, "stamps not written: start %llu end %llu",
+            (unsigned long long)start_raw, (unsigned long long)end_raw);
+    uint64_t start = 0, end = 0;
+    REQUIRE(hsa_amd_profiling_convert_tick_to_system_domain(gpu, start_raw, &start) == HSA_STATUS_SUCCESS, "convert");
+    REQUIRE(hsa_amd_profiling_convert_tick_to_system_domain(gpu, end_raw, &end) == HSA_STATUS_SUCCESS, "convert");
+    const double us = double(end - start) * 1e6 / double(freq);
+    // the conversion interpolates between two readings of both clocks: allow it a few microseconds
+    const uint64_t slack = freq / 20000;  // 50 us
+    std::printf("INFO profiling_copy_64MiB_us%s %.1f (submit to start %.1f us, end to seen %.1f us)\n", g_suffix.c_str(), us,
+                (double(start) - double(before)) * 1e6 / double(freq), (double(after) - double(end)) * 1e6 / double(freq));
+    REQUIRE(us > 5.0 && us < 5000.0, "implausible copy time %.1f us", us);
+    REQUIRE(start + slack >= before && end <= after + slack,
+            "stamps outside the host's window: before %llu start %llu end %llu after %llu", (unsigned long long)before,
+            (unsigned long long)start, (unsigned long long)end, (unsigned long long)after);
+    hsa_signal_destroy(s);
+  }
+  REQUIRE(blit.EnableProfiling(false) == HSA_STATUS_SUCCESS, "EnableProfiling(false)");
+  // off again: the signal of the next command keeps its zeros
+  hsa_signal_t s = make_signal(1);
+  Signal sig(s);
+  std::vector<Signal*> none, gang;
+  REQUIRE(blit.SubmitLinearCopyCommand(b.p, a.p, n, none, sig, gang) == HSA_STATUS_SUCCESS, "submit");
+  REQUIRE(wait_zero(s, HSA_WAIT_STATE_BLOCKED), "copy never completed");
+  const mi355::HsaSignalAbi* raw = reinterpret_cast<const mi355::HsaSignalAbi*>(s.handle);
+  REQUIRE(raw->start_ts == 0 && raw->end_ts == 0, "stamps written with profiling off");
+  hsa_signal_destroy(s);
+  std::printf("PASS %s%s\n", name, g_suffix.c_str());
+}
+
 void latency_report(Blit& blit, const char* mode) {
   // host-observed time per blocking call, submit -> completion seen
   // (the way memory_async_copy.cc:396-405 times a copy)
@@ -704,7 +762,7 @@ int main(int argc, char** argv) {
     for (const char* engine : {"_hip", "_aql"})
       for (const char* c : cases) std::printf("%s%s\n", c, engine);
     std::printf("async_copy_blocked_wait_hip_callback\nchain_a_to_b_to_c_hip_callback\n"
-                "profiling_timestamps_aql\ncopy_rect_with_signal_aql\nhost_link_slots_aql\n"
+                "profiling_timestamps_hip_callback\nprofiling_timestamps_hip\nprofiling_timestamps_aql\ncopy_rect_with_signal_aql\nhost_link_slots_aql\n"
                 "shared_queue_interleaved_packets_aql\nqueue_error_ends_waits_aql\n");
     return 0;
   }
@@ -768,6 +826,7 @@ int main(int argc, char** argv) {
     }
     test_async_copy_signal(cb, HSA_WAIT_STATE_BLOCKED, "async_copy_blocked_wait");
     test_chain(cb);
+    test_profiling_stamps_from_device(cb);
     latency_report(cb, "hip_host_callback");
     if (cb.Destroy(agent) != HSA_STATUS_SUCCESS) {
       std::printf("FAIL destroy (host callback)\n");
@@ -810,6 +869,7 @@ int main(int argc, char** argv) {
     test_zero_size_and_bad_args(*blit);
     test_batch(*blit, batch);
     test_threads(*blit);
+    if (engine == 0) test_profiling_stamps_from_device(*blit);
     if (engine == 1) {
       test_profiling_timestamps(*blit);
       test_copy_rect(*static_cast<BlitKernelGfx950Aql*>(blit));

@@ -178,6 +178,54 @@ def test_packet_log(pkg, signals, torch_cuda, monkeypatch, capfd):
     assert int(dispatch.group(1)) % int(dispatch.group(2)) == 0
 
 
+def test_barrier_bit_of_large_transfers(pkg, signals, torch_cuda, monkeypatch, capfd):
+    """Without dependencies a blit's dispatch packet has the barrier bit clear, as
+    the reference's has (amd_blit_kernel.cpp:870-882) -- except transfers of
+    4 MiB and more on an engine's own queue, which wait for the queue to drain.
+    An engine on a borrowed queue keeps the reference's packets; either default
+    can be changed."""
+    import re
+    torch = torch_cuda
+    n = 8 * MIB
+    a = torch.zeros(n, dtype=torch.uint8, device="cuda:0")
+    b = torch.zeros(n, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    monkeypatch.setenv("MI355_BLIT_LOG_PKTS", "1")
+
+    def barrier_bits(engine):
+        """barrier bit of the dispatch packets of a 64 KiB copy, an 8 MiB copy and an 8 MiB fill"""
+        out = []
+        for submit in (lambda c: engine.copy(b.data_ptr(), a.data_ptr(), 65536, completion=c),
+                       lambda c: engine.copy(b.data_ptr(), a.data_ptr(), n, completion=c),
+                       lambda c: engine.fill32(b.data_ptr(), 7, n // 4, completion=c)):
+            done = signals.create(1)
+            capfd.readouterr()
+            assert submit(done) == 0
+            assert engine.wait_signal(done) == 0
+            m = re.search(r"Dispatch Header = 0x[0-9a-f]+ \(type=2, barrier=(\d)", capfd.readouterr().err)
+            signals.destroy(done)
+            assert m
+            out.append(int(m.group(1)))
+        return out
+
+    own = pkg.aql.AqlBlit(0)
+    queue = pkg.aql.BorrowedQueue(0)
+    try:
+        assert barrier_bits(own) == [0, 1, 1]
+        assert own.set_large_transfer_barrier(False) == 0
+        assert barrier_bits(own) == [0, 0, 0]
+        borrowed = pkg.aql.AqlBlit(borrowed=queue)
+        try:
+            assert barrier_bits(borrowed) == [0, 0, 0]
+            assert borrowed.set_large_transfer_barrier(True) == 0
+            assert barrier_bits(borrowed) == [0, 1, 1]
+        finally:
+            borrowed.close()
+    finally:
+        own.close()
+        queue.close()
+
+
 def test_kernarg_ring_in_host_memory(pkg, capi, oracle, rand, torch_cuda, monkeypatch):
     """MI355_BLIT_HOST_KERNARGS=1 keeps every kernarg slot in host memory, as the
     reference does (amd_blit_kernel.cpp:565-569): a small copy, a copy of many

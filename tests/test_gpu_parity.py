@@ -1082,3 +1082,63 @@ def test_create_destroy_many(capi, pkg):
         pkg.aql.AqlBlit(1000)
     h = C.c_void_p()
     assert capi.load().mi355_blit_create(10_000, C.byref(h)) == capi.ERROR_INVALID_ARGUMENT
+
+
+@pytest.mark.gpu
+def test_engines_of_one_agent_share_one_code_object(pkg, oracle, rand, torch_cuda):
+    """Three engines on one agent -- the shape of GpuAgent's blits_[] slots, whose
+    BlitKernels all run the shaders the agent assembled once
+    (amd_gpu_agent.cpp:251-428) -- hold one executable between them, an owner's
+    own reference keeps it loaded while no engine exists, and it survives the
+    engines' destruction in any order: after each destroy the others still copy
+    correctly."""
+    torch = torch_cuda
+    aql = pkg.aql
+    lib = aql.load()
+    queue = aql.BorrowedQueue(0)
+    n = 3 * MIB + 5
+    host = rand(n + 64, 0xB1170077)
+    src = torch.from_numpy(host).to("cuda:0")
+    dst = torch.empty(n + 64, dtype=torch.uint8, device="cuda:0")
+
+    def copies_right(engine, seed):
+        dst.fill_(seed)
+        torch.cuda.synchronize()
+        assert engine.copy_sync(dst.data_ptr() + 9, src.data_ptr() + 3, n) == 0
+        want = np.full(n + 64, seed, dtype=np.uint8)
+        oracle.oracle_copy(want.ctypes.data + 9, host.ctypes.data + 3, n)
+        assert np.array_equal(dst.cpu().numpy(), want)
+
+    try:
+        a = aql.AqlBlit(borrowed=queue)
+        exe, users = a.code_object_info()
+        assert exe != 0 and users == 1
+        b = aql.AqlBlit(borrowed=queue)       # a second engine on the same queue
+        c = aql.AqlBlit(0)                    # and one on a queue of its own
+        assert b.code_object_info() == (exe, 3) and c.code_object_info() == (exe, 3)
+        own = C.c_void_p()
+        assert lib.mi355_aql_code_object_acquire(queue.agent, C.byref(own)) == 0
+        assert a.code_object_info() == (exe, 4)
+        for engine, seed in ((a, 1), (b, 2), (c, 3)):
+            copies_right(engine, seed)
+        b.close()
+        assert a.code_object_info() == (exe, 3)
+        copies_right(a, 4)
+        copies_right(c, 5)
+        a.close()
+        copies_right(c, 6)
+        c.close()
+        # only the owner's reference is left: a new engine finds the same executable
+        d = aql.AqlBlit(borrowed=queue)
+        assert d.code_object_info() == (exe, 2)
+        copies_right(d, 7)
+        d.close()
+        assert lib.mi355_aql_code_object_release(own) == 0
+        assert lib.mi355_aql_code_object_release(own) == pkg.capi.ERROR_INVALID_ARGUMENT   # already gone
+        e = aql.AqlBlit(borrowed=queue)       # loaded afresh
+        assert e.code_object_info()[1] == 1
+        copies_right(e, 8)
+        e.close()
+        assert lib.mi355_aql_code_object_acquire(0, C.byref(own)) == pkg.capi.ERROR_INVALID_ARGUMENT
+    finally:
+        queue.close()

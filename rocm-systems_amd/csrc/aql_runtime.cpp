@@ -11,10 +11,15 @@
 #include <cstring>
 #include <mutex>
 
+#include "aql_host_lock.h"
 #include "blit_plan.h"
 #include "mi355_blit_aql.h"
 
 namespace {
+
+using mi355::HostLockFns;
+using mi355::HostLockLatch;
+using mi355::ScopedHostLock;
 
 enum class Where { kHost, kHostUnknown, kGpu };
 
@@ -67,34 +72,17 @@ uint32_t route_of(bool src_is_host, bool dst_is_host) {
 // tiles for the shapes to differ, and a pointer lookup would only add latency.
 constexpr size_t kRouteLookupMinBytes = 1u << 20;
 
-// Locks [ptr, ptr+size) for the GPU when it is host memory the runtime does
-// not know (runtime.cpp:521-535); unlocks on destruction.
-class ScopedLock {
- public:
-  ScopedLock() = default;
-  ~ScopedLock() {
-    if (host_) hsa_amd_memory_unlock(host_);
-  }
-  int Lock(mi355_aql_t* h, const void* ptr, size_t size, void** agent_ptr) {
-    // a system that refuses to lock existing memory refuses every time
-    static std::atomic<bool> refused{false};
-    if (refused.load()) return MI355_BLIT_ERROR;
-    hsa_agent_t gpu;
-    gpu.handle = mi355_aql_gpu_agent(h);
-    void* mapped = nullptr;
-    hsa_status_t st = hsa_amd_memory_lock(const_cast<void*>(ptr), size, &gpu, 1, &mapped);
-    if (st != HSA_STATUS_SUCCESS) {
-      refused.store(true);
-      return static_cast<int>(st);
-    }
-    host_ = const_cast<void*>(ptr);
-    *agent_ptr = mapped;
-    return MI355_BLIT_SUCCESS;
-  }
-
- private:
-  void* host_ = nullptr;
-};
+// Host memory the runtime does not know is locked for the GPU
+// (runtime.cpp:521-535) through the runtime's own calls; which agents' systems
+// refuse that is remembered for the process (aql_host_lock.h).
+int runtime_lock(void* ptr, size_t size, uint64_t gpu_agent, void** mapped) {
+  hsa_agent_t gpu;
+  gpu.handle = gpu_agent;
+  return static_cast<int>(hsa_amd_memory_lock(ptr, size, &gpu, 1, mapped));
+}
+int runtime_unlock(void* ptr) { return static_cast<int>(hsa_amd_memory_unlock(ptr)); }
+const HostLockFns kRuntimeLock{runtime_lock, runtime_unlock};
+HostLockLatch g_lock_refused;
 
 // Host<->device copy through the engine's two GPU-visible bounce buffers, for
 // host memory that can neither be reached by the GPU nor locked: while the
@@ -183,17 +171,17 @@ int mi355_hsa_memory_copy(mi355_aql_t* h, void* dst, const void* src, size_t siz
   }
   // Same GPU, or GPU-CPU with the host side made visible to the GPU first.
   // Where existing host memory cannot be locked the copy is bounced instead.
-  ScopedLock lock_src, lock_dst;
+  ScopedHostLock lock_src(kRuntimeLock, g_lock_refused), lock_dst(kRuntimeLock, g_lock_refused);
   void* d = dst;
   const void* s = src;
   if (src_sys && !ps.gpu_can_access) {
     void* mapped = nullptr;
-    if (lock_src.Lock(h, src, size, &mapped) != MI355_BLIT_SUCCESS) return bounced_copy(h, dst, src, size, true);
+    if (lock_src.Lock(mi355_aql_gpu_agent(h), src, size, &mapped) != MI355_BLIT_SUCCESS) return bounced_copy(h, dst, src, size, true);
     s = mapped;
   }
   if (dst_sys && !pd.gpu_can_access) {
     void* mapped = nullptr;
-    if (lock_dst.Lock(h, dst, size, &mapped) != MI355_BLIT_SUCCESS) return bounced_copy(h, dst, src, size, false);
+    if (lock_dst.Lock(mi355_aql_gpu_agent(h), dst, size, &mapped) != MI355_BLIT_SUCCESS) return bounced_copy(h, dst, src, size, false);
     d = mapped;
   }
   // Waits for this copy's own completion signal, not for the queue to drain

@@ -21,6 +21,7 @@
 #include <vector>
 
 #include "../../oracle/blit_oracle.h"
+#include "aql_host_lock.h"
 #include "aql_wait.h"
 #include "blit_batch_host.h"
 #include "blit_plan.h"
@@ -502,9 +503,104 @@ void engine_policy_cases() {
 
 }  // namespace
 
+namespace {
+using namespace mi355;
+
+// The policy around hsa_amd_memory_lock (csrc/aql_host_lock.h), with the two
+// runtime calls injected: the branch that succeeds -- which the GPU boxes of
+// this pool never take, they refuse to lock existing memory -- must hand out
+// the mapped address and unlock the host pointer exactly once; a refusal that
+// speaks for the system is remembered for that agent only, one that speaks for
+// the pointer is not remembered at all (runtime.cpp:521-537).
+struct FakeLocker {
+  static int mode;      // status the next lock() answers with
+  static int locks, unlocks;
+  static void* last_unlocked;
+  static uint64_t last_agent;
+  static int lock(void* ptr, size_t, uint64_t agent, void** mapped) {
+    ++locks;
+    last_agent = agent;
+    if (mode != MI355_BLIT_SUCCESS) return mode;
+    *mapped = static_cast<char*>(ptr) + 0x1000;  // the GPU's address of the range differs from the host's
+    return MI355_BLIT_SUCCESS;
+  }
+  static int unlock(void* ptr) {
+    ++unlocks;
+    last_unlocked = ptr;
+    return MI355_BLIT_SUCCESS;
+  }
+};
+int FakeLocker::mode = 0, FakeLocker::locks = 0, FakeLocker::unlocks = 0;
+void* FakeLocker::last_unlocked = nullptr;
+uint64_t FakeLocker::last_agent = 0;
+
+void host_lock_cases() {
+  const HostLockFns fns{FakeLocker::lock, FakeLocker::unlock};
+  HostLockLatch latch;
+  char buffer[64];
+  const uint64_t gpu_a = 0x1111, gpu_b = 0x2222;
+  {
+    // success: mapped address out, one unlock of the host pointer at scope end
+    FakeLocker::mode = MI355_BLIT_SUCCESS;
+    void* mapped = nullptr;
+    {
+      ScopedHostLock l(fns, latch);
+      CHECK(l.Lock(gpu_a, buffer, sizeof buffer, &mapped) == MI355_BLIT_SUCCESS, "lock that succeeds");
+      CHECK(mapped == buffer + 0x1000 && FakeLocker::last_agent == gpu_a, "mapped address / agent");
+      CHECK(FakeLocker::unlocks == 0, "unlocked too early");
+      void* again = nullptr;
+      CHECK(l.Lock(gpu_a, buffer, sizeof buffer, &again) != MI355_BLIT_SUCCESS && FakeLocker::locks == 1,
+            "one range per object");
+    }
+    CHECK(FakeLocker::locks == 1 && FakeLocker::unlocks == 1 && FakeLocker::last_unlocked == buffer, "unlock exactly once");
+  }
+  {
+    // a refusal about this pointer: nothing unlocked, nothing remembered
+    FakeLocker::mode = MI355_BLIT_ERROR_INVALID_ARGUMENT;
+    void* mapped = nullptr;
+    {
+      ScopedHostLock l(fns, latch);
+      CHECK(l.Lock(gpu_a, buffer, sizeof buffer, &mapped) == MI355_BLIT_ERROR_INVALID_ARGUMENT, "status passed on");
+    }
+    CHECK(FakeLocker::unlocks == 1, "a failed lock must not unlock");
+    CHECK(!latch.refused(gpu_a), "a pointer's refusal was remembered");
+    FakeLocker::mode = MI355_BLIT_SUCCESS;
+    ScopedHostLock l(fns, latch);
+    CHECK(l.Lock(gpu_a, buffer, sizeof buffer, &mapped) == MI355_BLIT_SUCCESS && FakeLocker::locks == 3, "asked again");
+  }
+  CHECK(FakeLocker::unlocks == 2, "second unlock");
+  for (int status : {static_cast<int>(MI355_BLIT_ERROR_OUT_OF_RESOURCES), static_cast<int>(MI355_BLIT_ERROR)}) {
+    // the system's refusal: remembered, for that agent only
+    HostLockLatch fresh;
+    const int before = FakeLocker::locks;
+    FakeLocker::mode = status;
+    void* mapped = nullptr;
+    {
+      ScopedHostLock l(fns, fresh);
+      CHECK(l.Lock(gpu_a, buffer, sizeof buffer, &mapped) == status, "refusal passed on");
+    }
+    CHECK(fresh.refused(gpu_a) && !fresh.refused(gpu_b), "latched for the agent that was refused only");
+    FakeLocker::mode = MI355_BLIT_SUCCESS;
+    {
+      ScopedHostLock l(fns, fresh);
+      CHECK(l.Lock(gpu_a, buffer, sizeof buffer, &mapped) != MI355_BLIT_SUCCESS && FakeLocker::locks == before + 1,
+            "a refused agent is not asked again");
+    }
+    {
+      ScopedHostLock l(fns, fresh);
+      CHECK(l.Lock(gpu_b, buffer, sizeof buffer, &mapped) == MI355_BLIT_SUCCESS && FakeLocker::locks == before + 2,
+            "another agent is still asked");
+    }
+  }
+  CHECK(FakeLocker::unlocks == 4, "unlock count at the end: %d", FakeLocker::unlocks);
+}
+
+}  // namespace
+
 int main(int argc, char** argv) {
   wait_helper_cases();
   engine_policy_cases();
+  host_lock_cases();
   const long cases = argc > 1 ? std::atol(argv[1]) : 200000;
   for (long i = 0; i < cases; ++i) {
     one_copy_plan();

@@ -1111,32 +1111,35 @@ def test_engines_of_one_agent_share_one_code_object(pkg, oracle, rand, torch_cud
 
     try:
         a = aql.AqlBlit(borrowed=queue)
-        exe, users = a.code_object_info()
-        assert exe != 0 and users == 1
+        exe, base = a.code_object_info()
+        # other engines of this test session may be alive on the same agent: they hold the same executable
+        assert exe != 0 and base >= 1
         b = aql.AqlBlit(borrowed=queue)       # a second engine on the same queue
         c = aql.AqlBlit(0)                    # and one on a queue of its own
-        assert b.code_object_info() == (exe, 3) and c.code_object_info() == (exe, 3)
+        assert b.code_object_info() == (exe, base + 2) and c.code_object_info() == (exe, base + 2)
         own = C.c_void_p()
         assert lib.mi355_aql_code_object_acquire(queue.agent, C.byref(own)) == 0
-        assert a.code_object_info() == (exe, 4)
+        assert a.code_object_info() == (exe, base + 3)
         for engine, seed in ((a, 1), (b, 2), (c, 3)):
             copies_right(engine, seed)
         b.close()
-        assert a.code_object_info() == (exe, 3)
+        assert a.code_object_info() == (exe, base + 2)
         copies_right(a, 4)
         copies_right(c, 5)
         a.close()
         copies_right(c, 6)
         c.close()
-        # only the owner's reference is left: a new engine finds the same executable
+        # the owner's reference is left: a new engine finds the same executable
         d = aql.AqlBlit(borrowed=queue)
-        assert d.code_object_info() == (exe, 2)
+        assert d.code_object_info() == (exe, base + 1)
         copies_right(d, 7)
         d.close()
         assert lib.mi355_aql_code_object_release(own) == 0
-        assert lib.mi355_aql_code_object_release(own) == pkg.capi.ERROR_INVALID_ARGUMENT   # already gone
-        e = aql.AqlBlit(borrowed=queue)       # loaded afresh
-        assert e.code_object_info()[1] == 1
+        if base == 1:
+            # that was the last reference: the handle is gone, and the next engine loads the code afresh
+            assert lib.mi355_aql_code_object_release(own) == pkg.capi.ERROR_INVALID_ARGUMENT
+        e = aql.AqlBlit(borrowed=queue)
+        assert e.code_object_info()[1] == base
         copies_right(e, 8)
         e.close()
         assert lib.mi355_aql_code_object_acquire(0, C.byref(own)) == pkg.capi.ERROR_INVALID_ARGUMENT

@@ -48,7 +48,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=WARMUP_AFTER_IDLE)
     ap.add_argument("--workload", default="copy",
                     choices=["copy", "fill", "misaligned", "batch", "rect", "calib", "idle_series", "batch_layouts",
-                             "sustain"])
+                             "sustain", "rect_grid", "rect_check"])
     ap.add_argument("--bytes", type=int, default=GIB, help="transfer size of the copy/fill workloads")
     ap.add_argument("--rect", default="8192,131072,262144,0,0",
                     help="shape of the rect workload: rows,width,pitch[,source x,destination x] in bytes")
@@ -637,6 +637,52 @@ def sustain_series(r):
     return out
 
 
+RECT_GRID_WIDTHS_KIB = (2, 4, 8, 12, 16, 24, 32, 48, 64, 96, 128, 256)
+RECT_GRID_RATIOS = (2, 3, 4, 6, 8, 12, 16)
+# shapes off that grid, to check rules read from it: widths that are not on it at pitches 2.5 to 10 times the
+# width, odd widths at power-of-two pitches, pitches a line off a power of two, and a few of the grid's own
+RECT_CHECK_SHAPES_KIB = tuple((w, w * r) for w in (3, 5, 6, 10, 20, 40, 80, 160) for r in (2.5, 3.5, 5, 7, 10)) + (
+    (6, 16), (6, 32), (10, 32), (10, 64), (20, 64), (20, 128), (40, 128), (40, 256), (80, 256), (80, 512), (160, 512),
+    (20, 256), (40, 512), (16, 64.25), (32, 128.25), (64, 256.25), (128, 512.25), (8, 16.25), (32, 512.25), (16, 48.25),
+    (48, 192), (32, 192), (96, 384), (8, 16), (32, 512), (16, 256))
+
+
+def rect_grid(r, which):
+    """Where the region copy's heuristics stand: rows of whole cache lines,
+    512 MiB moved per launch (less where 12 GiB of surface do not hold it), each
+    shape as the library plans it and at eight forced combinations of store
+    policy (nt, sc1) and walk order (launch order, XCD runs of 144, 576 and 2304
+    units).  One JSON object per shape, GB/s of bytes read plus written."""
+    K = 1024
+    if which == "check":
+        pairs = [(int(w * K) // 128 * 128, int(p * K) // 128 * 128) for w, p in RECT_CHECK_SHAPES_KIB]
+    else:
+        pairs = [(w * K, w * K * ratio) for ratio in RECT_GRID_RATIOS for w in RECT_GRID_WIDTHS_KIB]
+    out = []
+    for width, pitch in pairs:
+        rows = min(512 * MIB // width, 12 * GIB // pitch)
+        fn, verify, algo, keep = make_rect(r, rows, width, pitch, 0, 0)
+        r.blit.set_tuning()
+        _, us = r.time_settled(fn, 12, settle_ms=15)
+        plan = r.blit.last_plan()
+        rec = {"width": width, "pitch": pitch, "rows": rows,
+               "planned": {"store_policy": plan.store_policy, "xcd_run": plan.xcd_run, "gbs": round(algo / us / 1e3)},
+               "forced_gbs": {}}
+        for store, name in ((2, "nt"), (3, "sc1")):
+            for run in (1, 144, 576, 2304):
+                r.blit.set_tuning(xcd_run=run, store_policy=store)
+                _, us = r.time_settled(fn, 12, settle_ms=5)
+                rec["forced_gbs"]["%s_run%d" % (name, run)] = round(algo / us / 1e3)
+        r.blit.set_tuning()
+        fn()
+        r.tstream.synchronize()
+        verify()
+        out.append(rec)
+        del fn, verify, keep
+        r.torch.cuda.empty_cache()
+    return out
+
+
 def small_copy_latency(r, sizes=(4096, 65536, MIB)):
     """Host-observed microseconds per blocking copy (submit -> completion seen),
     the way rocrtst times hsa_amd_memory_async_copy (memory_async_copy.cc:396-405)."""
@@ -1068,7 +1114,7 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus)
     # the clock sampler is a process of its own and is started before this one touches the GPU
-    main_flow = args.workload not in ("idle_series", "sustain", "batch_layouts")
+    main_flow = args.workload not in ("idle_series", "sustain", "batch_layouts", "rect_grid", "rect_check")
     sampler = SysfsSampler(0.002).start() if main_flow and not args.no_sample else None
     import torch
     import __graft_entry__ as entry
@@ -1083,6 +1129,12 @@ def main():
     nbytes = args.bytes
     if args.workload == "sustain":
         print(json.dumps(sustain_series(r)))
+        r.blit.close()
+        return
+    if args.workload in ("rect_grid", "rect_check"):
+        print(json.dumps({"metric": "region copies of whole-line rows: the plan against forced store policies and "
+                                    "walk orders", "unit": "GB/s",
+                          "shapes": rect_grid(r, "check" if args.workload == "rect_check" else "grid")}))
         r.blit.close()
         return
     if args.workload == "batch_layouts":

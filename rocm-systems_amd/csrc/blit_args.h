@@ -27,7 +27,9 @@ inline uint64_t magic_divisor(uint32_t d) { return d > 1 ? ~0ull / d + 1 : 0; }
 
 MI355_HOST_DEVICE inline uint32_t div_magic(uint32_t n, uint64_t magic) {
 #ifdef __HIP_DEVICE_COMPILE__
-  return magic ? static_cast<uint32_t>(__umul64hi(n, magic)) : n;
+  // a select, not a branch: the multiplication is cheaper than the jump
+  const uint32_t q = static_cast<uint32_t>(__umul64hi(n, magic));
+  return magic ? q : n;
 #else
   return magic ? static_cast<uint32_t>((static_cast<unsigned __int128>(n) * magic) >> 64) : n;
 #endif

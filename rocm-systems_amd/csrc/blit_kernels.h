@@ -170,10 +170,15 @@ MI355_DEVICE uint64_t global_wave(unsigned waves_per_wg) {
 // global_wave() of a launch whose workgroups take their work in runs per XCD
 // (xcd_workgroup): workgroups below x.full swap places among themselves, the
 // others keep theirs.  x.full == 0: launch order.
+// Written without a branch on purpose: the permutation is a dozen scalar
+// instructions, and with every field of x used unconditionally the compiler
+// fetches the whole argument block in one go at the kernel's entry instead of
+// in pieces behind each branch (three dependent scalar loads in front of a
+// wave's first data load became one).
 MI355_DEVICE uint64_t global_wave_xcd(unsigned waves_per_wg, const XcdRuns& x) {
-  uint32_t wg = workgroup_index();
-  if (wg < x.full) wg = xcd_workgroup(wg, x);
-  return wave_uniform(wg * waves_per_wg + thread_in_workgroup() / kWave);
+  const uint32_t wg = workgroup_index();
+  const uint32_t permuted = xcd_workgroup(wg, x);
+  return wave_uniform((wg < x.full ? permuted : wg) * waves_per_wg + thread_in_workgroup() / kWave);
 }
 
 template <int U, bool NTL, int NTS, bool SHIFT>
@@ -514,14 +519,20 @@ MI355_DEVICE void batch_copy_records_body(const BatchCopyArgs& a) {
   const unsigned lane = thread_in_workgroup() & (kWave - 1);
   const uint64_t wave = global_wave_xcd(a.waves_per_wg, a.xcd);
   const uint64_t n_waves = a.n_waves;
+  const unsigned ahead = a.prefetch_waves;
   for (uint64_t w = wave; w < total_chunks * SPLIT; w += n_waves) {
-    const unsigned q = static_cast<unsigned>(w % SPLIT);
-    const unsigned touched = touch_record_ahead(records, w, q, a.prefetch_waves, SPLIT, total_chunks, lane);
+    // The record first, then the data loads it describes, and only then the
+    // touch of the record ahead: nothing may stand between a wave's start and
+    // its data loads that does not have to (the touch is a predicated vector
+    // load, a block of its own to the compiler, and in front of the record's
+    // load it delayed that load by its whole length).
     const ChunkRecord rec = ld_uniform_record(records + w / SPLIT);
+    const unsigned q = static_cast<unsigned>(w % SPLIT);
     const unsigned v0 = q * (kChunkVecs / SPLIT);
     v4u x[U];
     unsigned e;
     record_load<U, NTL>(rec, v0, lane, x, e);
+    const unsigned touched = touch_record_ahead(records, w, q, ahead, SPLIT, total_chunks, lane);
     record_store<U, NTS>(rec, v0, lane, x, e);
     record_edges(rec, q == 0, q == SPLIT - 1, lane);
     keep_alive(touched);
@@ -607,12 +618,12 @@ MI355_DEVICE void batch_copy_lookup_body(const BatchLookupArgs& a) {
   for (uint64_t w = wave; w < total_chunks * SPLIT; w += n_waves) {
     const uint64_t c = w / SPLIT;
     const unsigned q = static_cast<unsigned>(w % SPLIT);
-    const unsigned touched = touch_record_ahead(records, w, q, a.copy.prefetch_waves, SPLIT, have, lane);
     const ChunkRecord rec = c < capacity ? ld_uniform_record(records + c) : lookup_record(a, static_cast<uint32_t>(c));
     const unsigned v0 = q * (kChunkVecs / SPLIT);
     v4u x[U];
     unsigned e;
     record_load<U, NTL>(rec, v0, lane, x, e);
+    const unsigned touched = touch_record_ahead(records, w, q, a.copy.prefetch_waves, SPLIT, have, lane);
     record_store<U, NTS>(rec, v0, lane, x, e);
     record_edges(rec, q == 0, q == SPLIT - 1, lane);
     keep_alive(touched);

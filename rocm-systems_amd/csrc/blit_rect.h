@@ -63,20 +63,25 @@ inline uint64_t rect_gcd(uint64_t a, uint64_t b) {
 }
 
 // Whether rows of whole cache lines are better written through L2 (sc1, the
-// linear copy's stores) than with non-temporal stores.  Measured on MI355X
-// over some 90 shapes of 0.125 to 1 GiB, rows of 128 bytes to 128 KiB at
-// pitches of 1.002 to 8 times the width, GB/s of bytes moved, sc1 against nt:
+// linear copy's stores) than with non-temporal stores.  Measured on MI355X, GB/s
+// of bytes moved, sc1 against nt, first over some 90 shapes (rows of 128 bytes
+// to 128 KiB at pitches of 1.002 to 8 times the width), then over a grid of 84
+// (rows of 2 to 256 KiB at 2, 3, 4, 6, 8, 12 and 16 times their width, each
+// policy at its best walk order, the worse of three processes):
 //  * rows under 1 KiB (a wave stores pieces of several rows): sc1 wins at
 //    every pitch, by 1 to 18 % (512-byte rows at a 2176-byte pitch 6956 against
 //    5891, 128-byte rows at 384 bytes 6812 against 5867);
 //  * rows of 1 KiB and more (every wave stores one contiguous KiB): sc1 wins by
-//    3 to 9 % when the pitch is a power of two (4 KiB rows at 8 KiB 6648 against
-//    6141) or a multiple of 128 KiB (128 KiB rows at 384 KiB 6572 against 6351),
-//    is level at multiples of 64 KiB, and loses by 4 to 20 % at any other pitch
-//    (2 KiB rows at 4352 bytes 5330 against 6384, 16 KiB rows at 68 KiB 5493
-//    against 6074, 128 KiB rows at 260 KiB 5775 against 6419), unless the rows
-//    nearly abut (a gap of up to 3 % of the pitch: 16 KiB rows at 16,640 bytes
-//    6531 against 6382).
+//    1 to 11 % at every pitch that is a power of two (4 KiB rows at 32 KiB 6580
+//    against 5930), and by 1 to 5 % at a multiple of 128 KiB when the width is a
+//    power of two as well (128 KiB rows at 384 KiB 6646 against 6324); at such a
+//    pitch rows of 12, 24, 48 or 96 KiB want nt by 6 to 12 % (48 KiB rows at
+//    384 KiB 5337 against 5999), and at odd multiples of 64 KiB every width does
+//    (32 KiB rows at 192 KiB 5377 against 5991).  At any other pitch sc1 loses by
+//    4 to 20 % (2 KiB rows at 4352 bytes 5330 against 6384, 16 KiB rows at
+//    68 KiB 5493 against 6074, 128 KiB rows at 260 KiB 5775 against 6419),
+//    unless the rows nearly abut (a gap of up to 3 % of the pitch: 16 KiB rows
+//    at 16,640 bytes 6531 against 6382).
 // The batched copy, whose chunks lie at arbitrary 256-byte boundaries, shows
 // the same preference for nt.  What the pitch changes is the order in which
 // the rows' lines reach the memory channels; the rule is what the measurements
@@ -84,7 +89,8 @@ inline uint64_t rect_gcd(uint64_t a, uint64_t b) {
 inline bool rect_whole_lines_write_through(uint64_t width, uint64_t dst_pitch) {
   if (width < 1024) return true;
   const uint64_t pow2_divisor = dst_pitch & (~dst_pitch + 1);
-  if (pow2_divisor == dst_pitch || pow2_divisor >= (64u << 10)) return true;
+  if (pow2_divisor == dst_pitch) return true;
+  if (pow2_divisor >= (128u << 10) && (width & (width - 1)) == 0) return true;
   return dst_pitch >= width && (dst_pitch - width) * 32 <= dst_pitch;
 }
 
@@ -112,6 +118,37 @@ inline bool rect_plain_rows_in_launch_order(uint64_t width, uint64_t dst_pitch, 
   const auto sparse = [width](uint64_t pitch) { return pitch * 3 >= width * 8 && pitch <= width * 8; };
   const auto dense_or_sparse = [width, sparse](uint64_t pitch) { return pitch == width || sparse(pitch); };
   return (sparse(dst_pitch) || sparse(src_pitch)) && dense_or_sparse(dst_pitch) && dense_or_sparse(src_pitch);
+}
+
+// The walk order of plain rows of a large region: units per XCD run, 1 for
+// launch order.  The window above first.  Beyond it, runs of 576 units, with
+// three exceptions for surfaces of one power-of-two pitch on both sides, taken
+// from a grid of 84 shapes (rows of 2 to 256 KiB at 2 to 16 times their width,
+// each at eight combinations of store policy and run length, the worse of three
+// processes) and checked on 66 other shapes in two more processes:
+//  * 8 KiB rows at 16 KiB: launch order (6520 against 5884 GB/s);
+//  * rows of 16 and 32 KiB at 16 times their width: launch order (6369 against
+//    5984, 6196 against 5130);
+//  * rows of 128 KiB and more at 512 KiB and more: runs four times as long
+//    (128 KiB rows at 512 KiB 6582 against 6267; 160 KiB rows 5978 against 5786).
+// With these and the store rule above the grid's shapes run 1.7 % under the best
+// combination found for each on average and at most 9.6 % (2 KiB rows at
+// 24 KiB), the other 66 shapes 2.2 % and 12.7 %; with runs of 576 everywhere
+// outside the window and stores written through at every multiple of 64 KiB,
+// 3.3 % and 20.8 %, 3.0 % and 15.9 %.  Launch order for rows with non-temporal
+// stores up to a few widths apart, which the grid suggested (+2 to +5 % at
+// exactly 3 times the width), lost 4 to 12 % on the other shapes (3 KiB rows at
+// 10.5 KiB 5381 against 5954, 16 KiB rows at 64.25 KiB 4614 against 5112) and
+// was not taken.
+inline uint32_t rect_plain_rows_run_units(uint64_t width, uint64_t dst_pitch, uint64_t src_pitch, uint64_t layers) {
+  const uint32_t run = kXcdRunBytes / 1024;
+  if (rect_plain_rows_in_launch_order(width, dst_pitch, src_pitch, layers)) return 1;
+  if (layers != 1 || dst_pitch != src_pitch || (dst_pitch & (dst_pitch - 1)) != 0) return run;
+  const uint64_t k = 1024;
+  if (width == 8 * k && dst_pitch == 2 * width) return 1;
+  if ((width == 16 * k || width == 32 * k) && dst_pitch == 16 * width) return 1;
+  if (width >= 128 * k && dst_pitch >= 512 * k) return 4 * run;
+  return run;
 }
 
 inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_offset, const mi355_pitched_ptr_t* src,
@@ -343,9 +380,14 @@ inline int plan_rect(const mi355_pitched_ptr_t* dst, const mi355_dim3_t* dst_off
   // Whole-line rows that are not plain go through the general path of the
   // kernel, where runs lose (347 us against 330 us).
   uint32_t run = 0;
-  if ((!whole_lines || plain_runs) && !link && out->total_bytes >= kXcdRunMinBytes &&
-      !(plain_runs && rect_plain_rows_in_launch_order(width, dp, sp, layers)))
+  if ((!whole_lines || plain_runs) && !link && out->total_bytes >= kXcdRunMinBytes) {
     run = static_cast<uint32_t>(kXcdRunBytes / (waves_per_wg * 1024 * unroll));
+    if (plain_runs) {
+      // in units of 1 KiB, which is what a workgroup of the default shape moves
+      const uint32_t units = rect_plain_rows_run_units(width, dp, sp, layers);
+      run = units <= 1 ? 0 : static_cast<uint32_t>(units / (waves_per_wg * unroll));
+    }
+  }
   out->xcd_run = plan_xcd_run(run, t);
   a.xcd = make_xcd_runs(out->grid, out->xcd_run);
   return MI355_BLIT_SUCCESS;

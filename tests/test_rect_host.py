@@ -345,16 +345,18 @@ def test_plan_rect_slots_follow_row_alignment(capi_host):
 
 def test_plan_rect_whole_line_rows_store_policy_follows_the_pitch(capi_host):
     """Rows of whole cache lines are written through L2 when they are under
-    1 KiB, or when the destination pitch is a power of two, a multiple of
-    64 KiB or within 3 % of the width; at any other pitch their stores are
-    non-temporal (rect_whole_lines_write_through)."""
+    1 KiB, or when the destination pitch is a power of two, or a multiple of
+    128 KiB while the width is a power of two, or within 3 % of the width; at
+    any other pitch their stores are non-temporal
+    (rect_whole_lines_write_through)."""
     base_d, base_s = 0x7f0000000000, 0x7f1000000000
     K = 1024
     WT, NT = capi_host.STORE_AGENT_WT, capi_host.STORE_NT
     cases = [
         # width, destination pitch, rows, expected
         (128 * K, 256 * K, 8192, WT), (128 * K, 260 * K, 8192, NT), (128 * K, 384 * K, 8192, WT),
-        (128 * K, 192 * K, 8192, WT), (128 * K, 160 * K, 8192, NT), (128 * K, 132 * K, 8192, WT),
+        (128 * K, 192 * K, 8192, NT), (128 * K, 160 * K, 8192, NT), (128 * K, 132 * K, 8192, WT),
+        (48 * K, 384 * K, 16384, NT), (96 * K, 384 * K, 8192, NT), (32 * K, 192 * K, 32768, NT), (64 * K, 768 * K, 8192, WT),
         (128 * K, 136 * K + 128, 8192, NT),
         (16 * K, 16 * K + 256, 65536, WT), (16 * K, 20 * K, 65536, NT), (16 * K, 32 * K, 65536, WT),
         (2 * K, 4 * K, 262144, WT), (2 * K, 4352, 262144, NT), (2 * K, 2304, 262144, NT),
@@ -383,28 +385,38 @@ def test_plan_rect_whole_line_rows_store_policy_follows_the_pitch(capi_host):
 
 
 def test_plan_rect_plain_rows_order_follows_the_pitches(capi_host):
-    """Plain rows of a large region run in XCD runs of 576 units, except in the
-    narrow window where launch order was measured to win: both pitches powers of
-    two, rows of 4 KiB or a multiple of 8 KiB up to 48 KiB that take up three
-    eighths of a pitch or less (but at least an eighth), one layer
-    (rect_plain_rows_in_launch_order)."""
+    """Plain rows of a large region run in XCD runs of 576 units, except where
+    launch order or longer runs were measured to win
+    (rect_plain_rows_in_launch_order, rect_plain_rows_run_units): both pitches
+    powers of two and rows of 4 KiB or a multiple of 8 KiB up to 48 KiB that take
+    up an eighth to three eighths of a pitch; and, for surfaces of one
+    power-of-two pitch, 8 KiB rows at 16 KiB and rows of 16 or 32 KiB at 16 times
+    their width (launch order) and rows of 128 KiB and more at 512 KiB and more
+    (runs of 2304)."""
     base_d, base_s = 0x7f0000000000, 0x7f1000000000
     K = 1024
     GIB = 1 << 30
     cases = [
-        # width, destination pitch, source pitch, launch order?
-        (32 * K, 128 * K, 128 * K, True), (32 * K, 256 * K, 256 * K, True), (32 * K, 64 * K, 64 * K, False),
-        (32 * K, 512 * K, 512 * K, False), (32 * K, 128 * K, 256 * K, True), (32 * K, 32 * K, 128 * K, True),
-        (32 * K, 128 * K, 32 * K, True), (32 * K, 128 * K + 256, 128 * K, False), (32 * K, 128 * K, 128 * K + 256, False),
-        (4 * K, 16 * K, 16 * K, True), (4 * K, 8 * K, 8 * K, False), (8 * K, 32 * K, 32 * K, True),
-        (12 * K, 64 * K, 64 * K, False), (24 * K, 64 * K, 64 * K, True), (48 * K, 128 * K, 128 * K, True),
-        (64 * K, 256 * K, 256 * K, False), (2 * K, 8 * K, 8 * K, False), (128 * K, 512 * K, 512 * K, False),
+        # width, destination pitch, source pitch, units per run (0: launch order)
+        (32 * K, 128 * K, 128 * K, 0), (32 * K, 256 * K, 256 * K, 0), (32 * K, 64 * K, 64 * K, 576),
+        (32 * K, 512 * K, 512 * K, 0), (32 * K, 128 * K, 256 * K, 0), (32 * K, 32 * K, 128 * K, 0),
+        (32 * K, 128 * K, 32 * K, 0), (32 * K, 128 * K + 256, 128 * K, 576), (32 * K, 128 * K, 128 * K + 256, 576),
+        (4 * K, 16 * K, 16 * K, 0), (4 * K, 8 * K, 8 * K, 576), (8 * K, 32 * K, 32 * K, 0),
+        (12 * K, 64 * K, 64 * K, 576), (24 * K, 64 * K, 64 * K, 0), (48 * K, 128 * K, 128 * K, 0),
+        (64 * K, 256 * K, 256 * K, 576), (2 * K, 8 * K, 8 * K, 576), (128 * K, 512 * K, 512 * K, 2304),
+        (8 * K, 16 * K, 16 * K, 0), (16 * K, 256 * K, 256 * K, 0), (4 * K, 64 * K, 64 * K, 576),
+        (256 * K, 1024 * K, 1024 * K, 2304), (128 * K, 256 * K, 256 * K, 576),
+        # any pitch that is not a power of two: runs of 576
+        (128 * K, 384 * K, 384 * K, 576), (128 * K, 768 * K, 768 * K, 576), (64 * K, 384 * K, 384 * K, 576),
+        (2 * K, 6 * K, 6 * K, 576), (4 * K, 12 * K, 12 * K, 576), (32 * K, 96 * K, 96 * K, 576),
+        (48 * K, 384 * K, 384 * K, 576), (12 * K, 192 * K, 192 * K, 576), (128 * K, 260 * K, 260 * K, 576),
+        (16 * K, 68 * K, 68 * K, 576),
     ]
-    for width, dp, sp, order in cases:
-        rows = GIB // width
+    for width, dp, sp, units in cases:
+        rows = min(GIB // width, (12 * GIB) // dp)
         st, p = capi_host.plan_rect((base_d, dp, 0), (0, 0, 0), (base_s, sp, 0), (0, 0, 0), (width, rows, 1))
         assert st == SUCCESS and p.plain_rows == 1 and p.wg_size == 64, (width, dp, sp)
-        assert p.xcd_run == (0 if order else 576), (width, dp, sp, p.xcd_run)
+        assert p.xcd_run == units, (width, dp, sp, p.xcd_run)
     # x offsets change nothing; several layers, a small region and tuning do
     st, p = capi_host.plan_rect((base_d, 128 * K, 0), (4096, 0, 0), (base_s, 128 * K, 0), (8192, 0, 0), (32 * K, 32768, 1))
     assert st == SUCCESS and (p.plain_rows, p.xcd_run) == (1, 0)

@@ -48,7 +48,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=WARMUP_AFTER_IDLE)
     ap.add_argument("--workload", default="copy",
                     choices=["copy", "fill", "misaligned", "batch", "rect", "calib", "idle_series", "batch_layouts",
-                             "sustain", "rect_grid", "rect_check"])
+                             "sustain", "pieces", "rect_grid", "rect_check", "misaligned_classes"])
     ap.add_argument("--bytes", type=int, default=GIB, help="transfer size of the copy/fill workloads")
     ap.add_argument("--rect", default="8192,131072,262144,0,0",
                     help="shape of the rect workload: rows,width,pitch[,source x,destination x] in bytes")
@@ -147,8 +147,11 @@ class SysfsSampler:
 
     def start(self):
         import subprocess
+        # the sampler is no part of what a profiler wrapped around this process should see
+        env = {k: v for k, v in os.environ.items()
+               if k != "LD_PRELOAD" and not k.startswith(("ROCP", "ROCPROF", "HSA_TOOLS"))}
         self.proc = subprocess.Popen([sys.executable, "-c", SAMPLER_SOURCE, str(self.period)], stdout=subprocess.PIPE,
-                                     stderr=subprocess.DEVNULL, text=True)
+                                     stderr=subprocess.DEVNULL, text=True, env=env)
         return self
 
     def stop(self):
@@ -594,12 +597,13 @@ def misaligned_figures(r, pkg):
 
 def sustain_series(r):
     """Whether a long transfer is slower per byte than a short one, and why: in
-    one process, back-to-back aligned copies of 1 GiB (272 launches), of 4 GiB
-    (68 launches: the same bytes, the same ~86 ms of load) and of 1 GiB again,
-    each series after a second without work, every launch timed by an event
-    behind it, with the clocks the driver reports sampled every millisecond.
-    Under `rocprofv3 --kernel-trace` the trace holds the kernels' own durations
-    for the same launches."""
+    one process, back-to-back aligned copies of 1 GiB (272 commands), of 4 GiB
+    as a single launch (68 commands: the same bytes, the same ~86 ms of load),
+    of 4 GiB the way the library submits it (eight launches of 512 MiB a
+    command) and of 1 GiB again, each series after a second without work, every
+    command timed by an event behind it, with the clocks the driver reports
+    sampled every millisecond.  Under `rocprofv3 --kernel-trace` the trace holds
+    the kernels' own durations for the same launches."""
     torch = r.torch
     top = 4 * GIB
     src = r.device_bytes(top + 64, seed=0xB1170003)
@@ -608,9 +612,10 @@ def sustain_series(r):
     out = {"metric": "pace of back-to-back aligned copies, 1 GiB against 4 GiB", "unit": "us per GiB", "series": []}
     sampler = SysfsSampler(0.001).start()
     windows = []
-    for gib, launches in ((1, 272), (4, 68), (1, 272)):
+    for gib, launches, one_launch in ((1, 272, False), (4, 68, True), (4, 68, False), (1, 272, False)):
         n = gib * GIB
         fn = lambda: r.check(r.blit.copy(D, S, n, r.stream), "copy")
+        r.blit.set_tuning(copy_piece_mib=1) if one_launch else r.blit.set_tuning()
         r.tstream.synchronize()
         torch.cuda.synchronize()
         time.sleep(1.0)
@@ -623,11 +628,12 @@ def sustain_series(r):
         def mean(v):
             return round(sum(v) / len(v), 2)
         out["series"].append({
-            "copy_GiB": gib, "launches": launches,
+            "copy_GiB": gib, "commands": launches, "launches_per_command": r.blit.last_plan().pieces,
             "us_per_GiB_by_quarter_of_the_series": [mean(per_gib[i * k:(i + 1) * k]) for i in range(4)],
             "us_per_GiB_last_half": mean(per_gib[launches // 2:]),
             "us_per_GiB_min": round(min(per_gib), 2),
             "us_per_launch": [round(u, 1) for u in us]})
+    r.blit.set_tuning()
     sampler.stop()
     for series, (t0, t1) in zip(out["series"], windows):
         series["sysfs_columns"] = ["ms since first launch"] + sampler.columns()
@@ -635,6 +641,78 @@ def sustain_series(r):
     so, do = (-src.data_ptr()) % 256, (-dst.data_ptr()) % 256
     assert torch.equal(dst[do:do + top], src[so:so + top]), "4 GiB copy differs"
     return out
+
+
+def piece_sweep(r, rounds=3):
+    """What cutting a long copy into consecutive launches is worth: copies of 1 to
+    8 GiB, aligned and at byte offsets (3, 9), each as one launch and in pieces
+    of 2 GiB down to 128 MiB (the tuning field copy_piece_mib), through the
+    library's own entry point.  Every configuration is timed `rounds` times in
+    rotation, 24 GiB of copies a time behind a settle burst; the figure is the
+    median, in microseconds per GiB, from events on the launch stream."""
+    torch = r.torch
+    top = 8 * GIB
+    src = r.device_bytes(top + 64, seed=0xB1170003)
+    dst = r.device_bytes(top + 64)
+    S, D = aligned_ptr(src), aligned_ptr(dst)
+    cases = []
+    for gib in (1, 2, 4, 8):
+        for s_off, d_off in ((0, 0), (3, 9)):
+            if (s_off, d_off) != (0, 0) and gib not in (1, 4):
+                continue
+            for piece_mib in (1, 2048, 1024, 512, 256, 128):
+                if piece_mib != 1 and piece_mib >= gib * 1024:
+                    continue
+                cases.append({"copy_GiB": gib, "offsets": [s_off, d_off], "copy_piece_mib": piece_mib, "us_per_GiB": []})
+    for _ in range(rounds):
+        for c in cases:
+            n = c["copy_GiB"] * GIB - 64
+            s_off, d_off = c["offsets"]
+            fn = lambda: r.check(r.blit.copy(D + d_off, S + s_off, n, r.stream), "copy")
+            r.blit.set_tuning(copy_piece_mib=c["copy_piece_mib"])
+            _, us = r.time_settled(fn, max(3, 24 // c["copy_GiB"]), settle_ms=30.0, warmup=2)
+            c["launches"] = r.blit.last_plan().pieces
+            c["us_per_GiB"].append(round(us * GIB / n, 2))
+    r.blit.set_tuning()
+    for c in cases:
+        c["median"] = sorted(c["us_per_GiB"])[len(c["us_per_GiB"]) // 2]
+    # what the library does by itself
+    default = []
+    for gib in (1, 2, 4, 8):
+        n = gib * GIB - 64
+        fn = lambda: r.check(r.blit.copy(D, S, n, r.stream), "copy")
+        _, us = r.time_settled(fn, max(3, 24 // gib), settle_ms=30.0, warmup=2)
+        default.append({"copy_GiB": gib, "launches": r.blit.last_plan().pieces, "us_per_GiB": round(us * GIB / n, 2)})
+    # where a single long launch loses: single launches of 1 and 4 GiB timed one by one, back to back and with the
+    # stream drained and the host asleep between them; and the 4 GiB launch in launch order and with other run lengths
+    def one_by_one(n, launches, gap_s, **tuning):
+        r.blit.set_tuning(copy_piece_mib=1, **tuning)
+        fn = lambda: r.check(r.blit.copy(D, S, n, r.stream), "copy")
+        r.settle(fn, 30.0)
+        ev = []
+        for _ in range(launches):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(r.tstream)
+            fn()
+            e1.record(r.tstream)
+            ev.append((e0, e1))
+            if gap_s is not None:
+                r.tstream.synchronize()
+                time.sleep(gap_s)
+        r.tstream.synchronize()
+        us = sorted(a.elapsed_time(b) * 1e3 * GIB / n for a, b in ev)
+        return {"median": round(us[len(us) // 2], 2), "min": round(us[0], 2), "max": round(us[-1], 2)}
+    single = []
+    for gib in (1, 4):
+        for gap_ms in (None, 0.5, 5.0):
+            single.append({"copy_GiB": gib, "idle_ms_between_launches": gap_ms,
+                           "us_per_GiB": one_by_one(gib * GIB, 48 // gib, None if gap_ms is None else gap_ms * 1e-3)})
+    orders = [{"copy_GiB": 4, "xcd_run": x, "us_per_GiB": one_by_one(4 * GIB, 12, None, xcd_run=x)}
+              for x in (1, 288, 576, 1152, 4608)]
+    r.blit.set_tuning()
+    so, do = (-src.data_ptr()) % 256, (-dst.data_ptr()) % 256
+    assert torch.equal(dst[do:do + top - 64], src[so:so + top - 64]), "8 GiB copy differs"
+    return {"cases": cases, "default": default, "single_launches": single, "single_launch_walk_orders": orders}
 
 
 RECT_GRID_WIDTHS_KIB = (2, 4, 8, 12, 16, 24, 32, 48, 64, 96, 128, 256)
@@ -1114,7 +1192,8 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus)
     # the clock sampler is a process of its own and is started before this one touches the GPU
-    main_flow = args.workload not in ("idle_series", "sustain", "batch_layouts", "rect_grid", "rect_check")
+    main_flow = args.workload not in ("idle_series", "sustain", "pieces", "batch_layouts", "rect_grid", "rect_check",
+                                      "misaligned_classes")
     sampler = SysfsSampler(0.002).start() if main_flow and not args.no_sample else None
     import torch
     import __graft_entry__ as entry
@@ -1129,6 +1208,17 @@ def main():
     nbytes = args.bytes
     if args.workload == "sustain":
         print(json.dumps(sustain_series(r)))
+        r.blit.close()
+        return
+    if args.workload == "pieces":
+        print(json.dumps({"metric": "pace of long D2D copies as one launch and cut into pieces", "unit": "us per GiB",
+                          **piece_sweep(r)}))
+        r.blit.close()
+        return
+    if args.workload == "misaligned_classes":
+        print(json.dumps({"metric": "misaligned D2D copy: one offset pair per class at 1 GiB - 64 B, a length sweep at "
+                                    "(3, 9), the blocking 4 KiB copy", "unit": "us per launch / GB/s",
+                          "misaligned": misaligned_figures(r, pkg)}))
         r.blit.close()
         return
     if args.workload in ("rect_grid", "rect_check"):

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define MI355_BLIT_ABI_VERSION 3
+#define MI355_BLIT_ABI_VERSION 4
 
 /* Same numeric values as HSA_STATUS_* (inc/hsa.h). */
 enum {
@@ -82,7 +82,10 @@ typedef struct {
                            sent the last mi355_hsa_amd_memory_async_copy to;
                            0 when no such call has been judged.  Reported by
                            mi355_aql_last_launch_info only */
-  uint32_t reserved;
+  uint32_t pieces;      /* launches the command was cut into: 1, or more for a
+                           copy of 1.5 GiB and beyond within the device, which is
+                           submitted as consecutive copies of at most 512 MiB
+                           (the other fields then describe the last of them) */
 } mi355_blit_plan_t;
 
 /* The engine choice of GpuAgent::GetBlitObject for an asynchronous copy within
@@ -144,6 +147,9 @@ typedef struct {
   uint32_t batch_staging;  /* batches of host-resident descriptors: 0 = heuristic, 1 = the host
                               walks the descriptors, 2 = they are staged as they are and the
                               GPU does the prefix sum */
+  uint32_t copy_piece_mib; /* copies within the device: 0 = heuristic (pieces of 512 MiB from
+                              1.5 GiB on), 1 = always one launch, N > 1 = a copy of more than
+                              N MiB goes out in pieces of N MiB */
 } mi355_blit_tuning_t;
 
 /* One element of a batched submission.  No counterpart in the reference. */
@@ -386,6 +392,14 @@ int mi355_blit_plan_fill(uint64_t ptr, uint64_t num_dwords, uint32_t num_cus,
 /* mi355_blit_plan_copy for a route other than within the device. */
 int mi355_blit_plan_copy_route(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t num_cus,
                                const mi355_blit_tuning_t* tuning, uint32_t route, mi355_blit_plan_t* out);
+
+/* How a copy of `bytes` is cut into consecutive launches (no counterpart in the
+ * reference, whose copy is one dispatch of a fixed grid that strides over any
+ * size, amd_blit_kernel.cpp:796-813): returns the number of launches, at most
+ * max_pieces, and writes the bytes of each but the last.  1 below 1.5 GiB and
+ * for routes over the bus; tuning (may be NULL) can say otherwise. */
+uint32_t mi355_blit_plan_copy_pieces(uint64_t bytes, uint32_t route, uint32_t max_pieces,
+                                     const mi355_blit_tuning_t* tuning, uint64_t* piece_bytes);
 
 /* Installs overrides used by every later command on the handle (NULL clears).
  * For tuning sweeps; replaces the reference's string-parsed kernel parameters

@@ -39,7 +39,7 @@ class Plan(C.Structure):
         ("byte_shift", C.c_uint32), ("lead_vecs", C.c_uint32),
         ("head_bytes", C.c_uint64), ("body_vecs", C.c_uint64), ("tail_bytes", C.c_uint64),
         ("xcd_run", C.c_uint32), ("route", C.c_uint32),
-        ("reference_engine", C.c_uint32), ("reserved", C.c_uint32),
+        ("reference_engine", C.c_uint32), ("pieces", C.c_uint32),
     ]
 
     def as_dict(self):
@@ -50,7 +50,7 @@ class Tuning(C.Structure):
     _fields_ = [
         ("wg_size", C.c_uint32), ("unroll", C.c_uint32), ("max_grid", C.c_uint32),
         ("nt_load", C.c_uint32), ("store_policy", C.c_uint32), ("xcd_run", C.c_uint32),
-        ("batch_prefetch", C.c_uint32), ("batch_staging", C.c_uint32),
+        ("batch_prefetch", C.c_uint32), ("batch_staging", C.c_uint32), ("copy_piece_mib", C.c_uint32),
     ]
 
 
@@ -119,6 +119,8 @@ SIGNATURES = {
                                              C.POINTER(Tuning), C.c_uint32, C.POINTER(Plan)]),
     "mi355_blit_plan_fill": (C.c_int, [C.c_uint64, C.c_uint64, C.c_uint32,
                                        C.POINTER(Tuning), C.POINTER(Plan)]),
+    "mi355_blit_plan_copy_pieces": (C.c_uint32, [C.c_uint64, C.c_uint32, C.c_uint32, C.POINTER(Tuning),
+                                                 C.POINTER(C.c_uint64)]),
     "mi355_blit_set_tuning": (C.c_int, [C.c_void_p, C.POINTER(Tuning)]),
     "mi355_blit_num_cus": (C.c_int, [C.c_void_p]),
     "mi355_blit_stream": (C.c_void_p, [C.c_void_p]),
@@ -257,6 +259,14 @@ def plan_copy(dst, src, nbytes, num_cus=256, tuning=None, route=None):
     else:
         st = load().mi355_blit_plan_copy(dst, src, nbytes, num_cus, t, C.byref(p))
     return st, p
+
+
+def plan_copy_pieces(nbytes, route=0, max_pieces=32, tuning=None):
+    """(launches, bytes of each but the last) for a copy of nbytes."""
+    piece = C.c_uint64()
+    t = C.byref(tuning) if tuning is not None else None
+    n = load().mi355_blit_plan_copy_pieces(nbytes, route, max_pieces, t, C.byref(piece))
+    return n, piece.value
 
 
 def plan_rect(dst, dst_offset, src, src_offset, extent, tuning=None, route=None):

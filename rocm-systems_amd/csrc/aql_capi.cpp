@@ -934,21 +934,41 @@ int mi355_aql_copy_route(mi355_aql_t* h, void* dst, const void* src, size_t byte
   if (!h || !dst || !src || (num_deps && !dep_signals) || route > MI355_BLIT_ROUTE_DEVICE_TO_HOST)
     return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   if (h->queue_error.load()) return MI355_BLIT_ERROR;
-  mi355_blit_plan_t p;
-  const Kernel* k = nullptr;
-  CopyArgs a{};
+  const uint32_t nb = barrier_packets(num_deps);
+  // One dispatch, or several for a copy of several GiB (copy_pieces) where the
+  // engine shapes large transfers (its own queue, or asked to): every piece after
+  // the first carries the barrier bit, which is the point of cutting.
+  struct Piece {
+    mi355_blit_plan_t p;
+    const Kernel* k;
+    CopyArgs a;
+  };
+  Piece piece[kCopyMaxPieces];
+  uint32_t pieces = 0;
   {
     std::lock_guard<std::mutex> g(h->lock);
     if (bytes) {
-      int rc = plan_copy(reinterpret_cast<uint64_t>(dst), reinterpret_cast<uint64_t>(src), bytes, h->num_cus,
-                         h->has_tuning ? &h->tuning : nullptr, &p, route);
-      if (rc != MI355_BLIT_SUCCESS) return rc;
-      k = find_copy(h, p);
-      if (!k) return MI355_BLIT_ERROR;
-      h->last_plan = p;
+      const uint32_t room = h->queue->size / 2 > nb ? h->queue->size / 2 - nb : 1;
+      uint64_t piece_bytes;
+      pieces = copy_pieces(bytes, route, h->serialise_large.load() ? room : 1, h->has_tuning ? &h->tuning : nullptr,
+                           &piece_bytes);
+      for (uint32_t i = 0; i < pieces; ++i) {
+        const uint64_t off = i * piece_bytes;
+        const uint64_t n = bytes - off < piece_bytes ? bytes - off : piece_bytes;
+        uint8_t* d = static_cast<uint8_t*>(dst) + off;
+        const uint8_t* s = static_cast<const uint8_t*>(src) + off;
+        Piece& q = piece[i];
+        int rc = plan_copy(reinterpret_cast<uint64_t>(d), reinterpret_cast<uint64_t>(s), n, h->num_cus,
+                           h->has_tuning ? &h->tuning : nullptr, &q.p, route);
+        if (rc != MI355_BLIT_SUCCESS) return rc;
+        q.k = find_copy(h, q.p);
+        if (!q.k) return MI355_BLIT_ERROR;
+        q.a = make_copy_args(q.p, d, s, n);
+      }
+      h->last_plan = piece[pieces - 1].p;
+      h->last_plan.pieces = pieces;
     }
   }
-  const uint32_t nb = barrier_packets(num_deps);
   if (bytes == 0) {
     // nothing to move: the dependencies and the completion ride on barriers
     const uint32_t n = nb ? nb : 1;
@@ -963,8 +983,7 @@ int mi355_aql_copy_route(mi355_aql_t* h, void* dst, const void* src, size_t byte
     release_write_index(h, index, n);
     return MI355_BLIT_SUCCESS;
   }
-  a = make_copy_args(p, dst, src, bytes);
-  const uint32_t total = nb + 1;
+  const uint32_t total = nb + pieces;
   uint64_t index;
   {
     std::lock_guard<std::mutex> r(h->reservation_lock);
@@ -974,8 +993,17 @@ int mi355_aql_copy_route(mi355_aql_t* h, void* dst, const void* src, size_t byte
   write_barriers(h, index, dep_signals, num_deps, nb, 0, false);
   // Barrier bit clear, as in the reference: consecutive blits may overlap
   // unless linked by signals.  After dependency barriers the bit is set so
-  // that the copy cannot start before them.
-  write_dispatch(h, index + nb, *k, &a, sizeof(a), p.grid, p.wg_size, completion_signal, nb != 0 || serialise(h, bytes));
+  // that the copy cannot start before them.  The completion signal goes on the
+  // last piece, which the barrier bit orders behind the others.
+  for (uint32_t i = 0; i < pieces; ++i) {
+    const Piece& q = piece[i];
+    const Chain chain = pieces == 1 ? Chain::kAlone
+                        : i == 0 ? Chain::kFirst
+                        : i + 1 == pieces ? Chain::kLast
+                                          : Chain::kMiddle;
+    write_dispatch(h, index + nb + i, *q.k, &q.a, sizeof(q.a), q.p.grid, q.p.wg_size,
+                   i + 1 == pieces ? completion_signal : 0, i != 0 || nb != 0 || serialise(h, bytes), chain);
+  }
   release_write_index(h, index, total);
   return MI355_BLIT_SUCCESS;
 }

@@ -363,6 +363,12 @@ int mi355_blit_plan_fill(uint64_t ptr, uint64_t num_dwords, uint32_t num_cus,
   return plan_fill(ptr, num_dwords, num_cus, tuning, out);
 }
 
+uint32_t mi355_blit_plan_copy_pieces(uint64_t bytes, uint32_t route, uint32_t max_pieces,
+                                     const mi355_blit_tuning_t* tuning, uint64_t* piece_bytes) {
+  uint64_t unused;
+  return copy_pieces(bytes, route, max_pieces, tuning, piece_bytes ? piece_bytes : &unused);
+}
+
 uint64_t mi355_policy_force_sdma_size(void) { return policy_force_sdma_size(); }
 
 uint32_t mi355_policy_same_gpu_engine(uint64_t size, uint64_t force_sdma_size) {
@@ -465,16 +471,26 @@ int mi355_blit_copy_route(mi355_blit_t* h, void* dst, const void* src, size_t by
   std::lock_guard<std::mutex> g(h->lock);
   DeviceScope scope(h->device);
   if (scope.err != hipSuccess) return status_of(scope.err);
-  mi355_blit_plan_t p;
-  int rc = plan_copy(reinterpret_cast<uint64_t>(dst), reinterpret_cast<uint64_t>(src), bytes,
-                     h->num_cus, h->has_tuning ? &h->tuning : nullptr, &p, route);
-  if (rc != MI355_BLIT_SUCCESS) return rc;
-  copy_kernel_t k = select_copy_kernel(p);
-  if (!k) return MI355_BLIT_ERROR;
-  const CopyArgs a = make_copy_args(p, dst, src, bytes);
   hipStream_t s = stream ? static_cast<hipStream_t>(stream) : h->stream;
-  hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
-  BLIT_HIP(hipGetLastError());
+  // one launch, or several for a copy of several GiB (copy_pieces)
+  uint64_t piece_bytes;
+  const uint32_t pieces = copy_pieces(bytes, route, kCopyMaxPieces, h->has_tuning ? &h->tuning : nullptr, &piece_bytes);
+  mi355_blit_plan_t p;
+  for (uint32_t i = 0; i < pieces; ++i) {
+    const uint64_t off = i * piece_bytes;
+    const uint64_t n = bytes - off < piece_bytes ? bytes - off : piece_bytes;
+    uint8_t* d = static_cast<uint8_t*>(dst) + off;
+    const uint8_t* sp = static_cast<const uint8_t*>(src) + off;
+    int rc = plan_copy(reinterpret_cast<uint64_t>(d), reinterpret_cast<uint64_t>(sp), n, h->num_cus,
+                       h->has_tuning ? &h->tuning : nullptr, &p, route);
+    if (rc != MI355_BLIT_SUCCESS) return rc;
+    copy_kernel_t k = select_copy_kernel(p);
+    if (!k) return MI355_BLIT_ERROR;
+    const CopyArgs a = make_copy_args(p, d, sp, n);
+    hipLaunchKernelGGL(k, dim3(p.grid), dim3(p.wg_size), 0, s, a);
+    BLIT_HIP(hipGetLastError());
+  }
+  p.pieces = pieces;
   h->last_plan = p;
   return ledger_record(h, s, bytes);
 }

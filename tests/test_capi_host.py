@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol(capi_host):
 
 def test_abi_version_and_status_strings(capi_host):
     lib = capi_host.load()
-    assert lib.mi355_blit_abi_version() == 3
+    assert lib.mi355_blit_abi_version() == 4
     assert lib.mi355_blit_status_string(0) == b"success"
     assert lib.mi355_blit_status_string(capi_host.ERROR_INVALID_ARGUMENT) == b"invalid argument"
     assert lib.mi355_blit_status_string(12345) == b"unknown status"
@@ -44,7 +44,7 @@ def test_abi_version_and_status_strings(capi_host):
 def test_struct_layouts_match_header(capi_host):
     assert C.sizeof(capi_host.Plan) == 8 * 4 + 3 * 8 + 4 * 4
     assert capi_host.Plan.lead_vecs.offset == 28
-    assert C.sizeof(capi_host.Tuning) == 32
+    assert C.sizeof(capi_host.Tuning) == 36
     assert C.sizeof(capi_host.Desc) == 24
 
 
@@ -187,6 +187,41 @@ def test_plan_copy_routes_across_the_host_link(capi_host):
     assert st == 0 and p.grid == 512
     st, p = capi_host.plan_copy(dst, src, 1 << 30, route=3)
     assert st == capi_host.ERROR_INVALID_ARGUMENT
+
+
+def test_copies_of_several_gib_are_cut_into_pieces(capi_host):
+    """Within the device a copy of 1.5 GiB or more goes out as consecutive copies
+    of at most 512 MiB (a multiple of 1 MiB each, so every piece keeps the
+    alignment of the whole), at most 32 of them and at most what the submission
+    path has room for; the pieces tile the copy exactly.  Smaller copies and
+    copies over the bus stay one launch."""
+    MIB, GIB = 1 << 20, 1 << 30
+    for n in (0, 1, GIB, 1536 * MIB - 1):
+        assert capi_host.plan_copy_pieces(n) == (1, n)
+    for route in (capi_host.ROUTE_HOST_TO_DEVICE, capi_host.ROUTE_DEVICE_TO_HOST):
+        assert capi_host.plan_copy_pieces(8 * GIB, route) == (1, 8 * GIB)
+    assert capi_host.plan_copy_pieces(1536 * MIB) == (3, 512 * MIB)
+    assert capi_host.plan_copy_pieces(2 * GIB) == (4, 512 * MIB)
+    assert capi_host.plan_copy_pieces(4 * GIB) == (8, 512 * MIB)
+    assert capi_host.plan_copy_pieces(4 * GIB, max_pieces=4) == (4, GIB)
+    assert capi_host.plan_copy_pieces(4 * GIB, max_pieces=1) == (1, 4 * GIB)
+    assert capi_host.plan_copy_pieces(4 * GIB, max_pieces=0) == (1, 4 * GIB)
+    for n in (1536 * MIB + 1, 2 * GIB - 1, 3 * GIB + 12345, 16 * GIB, 16 * GIB + 7, 33 * GIB + 3, 200 * GIB):
+        for cap in (32, 7, 2):
+            count, piece = capi_host.plan_copy_pieces(n, max_pieces=cap)
+            assert 2 <= count <= cap and piece % MIB == 0
+            assert (count - 1) * piece < n <= count * piece
+            if n <= cap * 512 * MIB:
+                assert piece <= 512 * MIB
+            # no piece is a sliver beside the others unless the size says so
+            assert piece - (n - (count - 1) * piece) < count * MIB
+    # tuning: never, or pieces of a given size for anything larger
+    T = capi_host.Tuning
+    assert capi_host.plan_copy_pieces(64 * GIB, tuning=T(copy_piece_mib=1)) == (1, 64 * GIB)
+    assert capi_host.plan_copy_pieces(64 * MIB, tuning=T(copy_piece_mib=64)) == (1, 64 * MIB)
+    assert capi_host.plan_copy_pieces(64 * MIB + 1, tuning=T(copy_piece_mib=64)) == (2, 33 * MIB)
+    assert capi_host.plan_copy_pieces(GIB, tuning=T(copy_piece_mib=256)) == (4, 256 * MIB)
+    assert capi_host.plan_copy_pieces(GIB, capi_host.ROUTE_HOST_TO_DEVICE, tuning=T(copy_piece_mib=256)) == (1, GIB)
 
 
 def test_plan_fill_invariants(capi_host):

@@ -134,13 +134,19 @@ def test_copy_4gib_properties(capi, blit, oracle, rand, torch_cuda):
         assert oracle.oracle_fnv1a64(got.ctypes.data, 1 << 16) == want_hash
     p = blit.last_plan()
     assert p.grid * (p.wg_size // 64) >= -(-p.body_vecs // (64 * p.unroll))
+    # eight launches of 512 MiB, except on a queue the engine does not own
+    assert p.pieces == (1 if getattr(blit, "borrowed", None) is not None else 8)
 
 
-def test_copy_and_fill_beyond_the_largest_grid(capi, blit, oracle, rand, torch_cuda):
-    """33 GiB: more 1 KiB tiles than a grid can have workgroups (an AQL packet
-    counts work-items in 32 bits), so the grid is capped and waves take a
-    second tile.  Same properties as at 4 GiB, compared on the device in 1 GiB
-    slices, with the slices around the wrap of the grid also hashed on the host."""
+def test_copy_and_fill_beyond_the_largest_grid(capi, fresh_tuning, oracle, rand, torch_cuda):
+    """33 GiB, twice.  As one launch (the tuning asks for it; a borrowed queue
+    gets one anyway) it has more 1 KiB tiles than a grid can have workgroups (an
+    AQL packet counts work-items in 32 bits), so the grid is capped and waves
+    take a second tile.  By default it goes out in 32 pieces of a little over
+    1 GiB.  Same properties as at 4 GiB, compared on the device in 1 GiB slices,
+    with the 64 MiB blocks around the wrap of the grid, or around the seams
+    between pieces, also compared on the host."""
+    blit = fresh_tuning
     torch = torch_cuda
     gib = 1 << 30
     n = 33 * gib + 12345 * 16
@@ -156,22 +162,38 @@ def test_copy_and_fill_beyond_the_largest_grid(capi, blit, oracle, rand, torch_c
         src.view[lo:lo + m].copy_(block_dev[:m])
     torch.cuda.synchronize()
     dst = Arena(torch, n + 2 * GUARD, fill=GUARD_BYTE)
-    check_ok(capi, blit.copy(dst.base + GUARD, src.base, n), "copy")
-    check_ok(capi, blit.synchronize(), "synchronize")
-    p = blit.last_plan()
-    tiles = -(-(p.body_vecs + p.lead_vecs) // (64 * p.unroll))
-    waves = p.grid * (p.wg_size // 64)
-    assert waves < tiles, "the case is meant to cap the grid: %s" % p.as_dict()
-    assert bool((dst.view[:GUARD] == GUARD_BYTE).all()) and bool((dst.view[GUARD + n:] == GUARD_BYTE).all())
-    for lo in range(0, n, gib):
-        m = min(gib, n - lo)
-        assert torch.equal(dst.view[GUARD + lo:GUARD + lo + m], src.view[lo:lo + m]), "slice at %d GiB differs" % (lo >> 30)
     want = np.empty(blk, dtype=np.uint8)
     oracle.oracle_copy(want.ctypes.data, block_host.ctypes.data, blk)
-    wrap = waves * 64 * p.unroll * 16 // blk      # the 64 MiB block in which the second round of tiles starts
-    for i in (0, wrap - 1, wrap, wrap + 1, n // blk - 1):
-        got = dst.host(GUARD + i * blk, GUARD + (i + 1) * blk)
-        assert np.array_equal(got, want), "block %d differs" % i
+    borrowed = getattr(blit, "borrowed", None) is not None
+    for one_launch in (True, False):
+        if one_launch:
+            blit.set_tuning(copy_piece_mib=1)
+        else:
+            blit.set_tuning()
+            dst.fill(0, n + 2 * GUARD, GUARD_BYTE)
+        check_ok(capi, blit.copy(dst.base + GUARD, src.base, n), "copy")
+        check_ok(capi, blit.synchronize(), "synchronize")
+        p = blit.last_plan()
+        if one_launch or borrowed:
+            assert p.pieces == 1
+            tiles = -(-(p.body_vecs + p.lead_vecs) // (64 * p.unroll))
+            waves = p.grid * (p.wg_size // 64)
+            assert waves < tiles, "the case is meant to cap the grid: %s" % p.as_dict()
+            wrap = waves * 64 * p.unroll * 16 // blk      # the 64 MiB block in which the second round of tiles starts
+            blocks = (0, wrap - 1, wrap, wrap + 1, n // blk - 1)
+        else:
+            count, piece = capi.plan_copy_pieces(n)
+            assert p.pieces == count == 32 and gib < piece < gib + 64 * MIB
+            # a seam lies inside block k * piece // blk
+            blocks = sorted({0, n // blk - 1} | {k * piece // blk for k in (1, 2, 16, 31)})
+        assert bool((dst.view[:GUARD] == GUARD_BYTE).all()) and bool((dst.view[GUARD + n:] == GUARD_BYTE).all())
+        for lo in range(0, n, gib):
+            m = min(gib, n - lo)
+            assert torch.equal(dst.view[GUARD + lo:GUARD + lo + m], src.view[lo:lo + m]), \
+                "slice at %d GiB differs (one launch: %s)" % (lo >> 30, one_launch)
+        for i in blocks:
+            got = dst.host(GUARD + i * blk, GUARD + (i + 1) * blk)
+            assert np.array_equal(got, want), "block %d differs (one launch: %s)" % (i, one_launch)
     del src
     torch.cuda.empty_cache()
     # the fill, over what the copy left
@@ -322,6 +344,7 @@ def test_copy_8gib_grid_limits(capi, blit, torch_cuda):
     assert bool((dst.view[GUARD + 5 + n - 16:] == GUARD_BYTE).all())
     p = blit.last_plan()
     assert p.grid * p.wg_size < 2 ** 31
+    assert p.pieces == (1 if getattr(blit, "borrowed", None) is not None else 16)
 
 
 # ------------------------------------------------------------------------- fill

@@ -518,6 +518,14 @@ def _make_batch(capi, rng, src, dst, n, min_len=64, max_len=256 << 10):
     return descs, lens, offs, so, do, total
 
 
+class _Window:
+    """An arena from `offset` on, for _make_batch."""
+
+    def __init__(self, arena, offset):
+        self.base = arena.base + offset
+        self.nbytes = arena.nbytes - offset
+
+
 def _grid_chunks(p):
     """Chunks a batch launch has waves for: four waves to a 4 KiB chunk."""
     return p.grid * (p.wg_size // 64) // (4 // p.unroll)
@@ -990,6 +998,82 @@ def test_batch_back_to_back_reuses_staging(capi, blit, oracle, arenas):
     for i in range(200):
         oracle.oracle_copy(want2.ctypes.data + int(o1[i] + e1[i]), src_host.ctypes.data + int(o1[i] + s1[i]), int(l1[i]))
     assert np.array_equal(dst.host(shift, shift + t1), want2)
+
+
+@pytest.mark.parametrize("queue", ["own", "borrowed"])
+def test_batches_with_signals_between_other_commands(capi, pkg, oracle, arenas, queue):
+    """Host-descriptor batches on an AQL engine, back to back and growing (the
+    staging and record buffers are replaced on the way), with and without the
+    caller's completion signal, one held back by a dependency signal, with a
+    linear copy and a device-resident batch in between.  Every batch has a
+    stretch of the destination of its own; all are compared with the oracle at
+    the end, and the held batch must not have finished before its dependency
+    was released."""
+    import time
+    src, src_host, dst = arenas
+    pkg.aql.load()
+    sig = pkg.aql.HsaSignals()
+    borrowed = pkg.aql.BorrowedQueue(0, packets=64) if queue == "borrowed" else None
+    eng = pkg.aql.AqlBlit(borrowed=borrowed) if borrowed is not None else pkg.aql.AqlBlit(0)
+    made = []
+    try:
+        rng = np.random.default_rng(0xB11705EC)
+        dst.fill(0, dst.nbytes, GUARD_BYTE)
+        want = np.full(dst.nbytes, GUARD_BYTE, dtype=np.uint8)
+        at = 0
+        keep = []
+
+        def batch(n, max_len, on_device=False, **kw):
+            nonlocal at
+            descs, lens, offs, so, do, total = _make_batch(capi, rng, _Window(src, at), _Window(dst, at), n, max_len=max_len)
+            for i in range(n):
+                oracle.oracle_copy(want.ctypes.data + at + int(offs[i] + do[i]),
+                                   src_host.ctypes.data + at + int(offs[i] + so[i]), int(lens[i]))
+            if on_device:
+                dev = src.torch.from_numpy(np.frombuffer(descs, dtype=np.uint8).copy()).to("cuda:0")
+                src.torch.cuda.synchronize()
+                keep.append(dev)
+                check_ok(capi, eng.copy_batch(dev.data_ptr(), n, on_device=True, **kw), "copy_batch")
+            else:
+                keep.append(descs)
+                check_ok(capi, eng.copy_batch(descs, n, **kw), "copy_batch")
+            at += (total + 255) // 256 * 256
+
+        for n, max_len in ((40, 4096), (300, 64 << 10), (5, 1 << 20), (3000, 8 << 10), (700, 32 << 10)):
+            batch(n, max_len)
+        done = sig.create(1)
+        made.append(done)
+        batch(200, 16 << 10, completion=done)
+        sig.wait_below_one(done)
+        n_lin = 3 * MIB + 5
+        check_ok(capi, eng.copy(dst.base + at + 7, src.base + at + 2, n_lin), "copy")
+        oracle.oracle_copy(want.ctypes.data + at + 7, src_host.ctypes.data + at + 2, n_lin)
+        at += (n_lin + 7 + 255) // 256 * 256 + 256
+        batch(100, 128 << 10)
+        dep, held = sig.create(1), sig.create(1)
+        made += [dep, held]
+        batch(150, 32 << 10, deps=[dep], completion=held)
+        batch(60, 8 << 10)          # queued behind the held one
+        time.sleep(0.05)
+        assert sig.load(held) == 1, "a batch ran before its dependency was released"
+        sig.store(dep, 0)
+        sig.wait_below_one(held)
+        batch(120, 16 << 10, on_device=True)
+        batch(90, 64 << 10)
+        check_ok(capi, eng.synchronize(), "synchronize")
+        assert at <= dst.nbytes
+        got = dst.host(0, at)
+        if not np.array_equal(got, want[:at]):
+            bad = np.nonzero(got != want[:at])[0]
+            raise AssertionError("%d bytes differ, first at %d of %d" % (bad.size, bad[0], at))
+        assert eng.pending_bytes() == 0
+    finally:
+        for s_ in made:
+            sig.destroy(s_)
+        eng.close()
+        if borrowed is not None:
+            assert borrowed.errors == []
+            borrowed.close()
 
 
 # ---------------------------------------------------------- API edge behaviour

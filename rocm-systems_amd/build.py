@@ -19,6 +19,7 @@ ROCR_TEST = os.path.join(LIB_DIR, "test_rocr_blit")
 ORACLE_LIB = os.path.join(ORACLE_DIR, "libblit_oracle.so")
 HOST_LOGIC_TEST = os.path.join(LIB_DIR, "test_host_logic")
 KERNELS_ON_CPU_TEST = os.path.join(LIB_DIR, "test_kernels_on_cpu")
+XCD_PROGRESS = os.path.join(LIB_DIR, "xcd_progress")
 
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
@@ -138,13 +139,25 @@ def build_oracle():
     return ORACLE_LIB
 
 
+def build_xcd_progress():
+    """GPU diagnostic: the XCD every workgroup of a launch runs on and how far
+    apart the XCDs drift in one long copy (tests/cpp/xcd_progress.hip)."""
+    src = os.path.join(ROOT, "tests", "cpp", "xcd_progress.hip")
+    if not os.path.exists(src):
+        return None
+    os.makedirs(LIB_DIR, exist_ok=True)
+    flags = [f for f in HIPCC_FLAGS if f != "-fPIC"]
+    _run([_hipcc()] + flags + ["-I", INCLUDE, "-I", CSRC, "-o", XCD_PROGRESS, src])
+    return XCD_PROGRESS
+
+
 def build_all():
     out = [build_blit(), build_aql()]
     r = build_rocr_adapter()
     if r:
         out.append(r)
     out.append(build_oracle())
-    for t in (build_rocr_test(), build_host_logic_test(), build_kernels_on_cpu_test()):
+    for t in (build_rocr_test(), build_host_logic_test(), build_kernels_on_cpu_test(), build_xcd_progress()):
         if t:
             out.append(t)
     return out

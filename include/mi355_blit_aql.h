@@ -204,7 +204,9 @@ uint64_t mi355_aql_pending_bytes(mi355_aql_t* h);
 
 /* Replaces BlitKernel::EnableProfiling (amd_blit_kernel.cpp:839-842): sets the
  * queue's profiling bit, after which the packet processor writes start and end
- * timestamps into each completion signal. */
+ * timestamps into each completion signal.  While it is on, a copy of 1.5 GiB
+ * or more is not cut into pieces (mi355_aql_copy): the stamps are those of one
+ * dispatch, and they are to cover the command. */
 int mi355_aql_enable_profiling(mi355_aql_t* h, int enable);
 
 /* Start and end of the command whose completion signal is given, as stamped

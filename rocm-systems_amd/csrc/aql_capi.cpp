@@ -173,6 +173,9 @@ struct mi355_aql {
   // Transfers of 4 MiB and more carry the barrier bit (serialise()): set for an
   // engine on a queue of its own, clear on a borrowed queue.
   std::atomic<bool> serialise_large{false};
+  // mi355_aql_enable_profiling: the packet processor stamps a dispatch's
+  // completion signal, so a command whose times are asked for stays one dispatch.
+  std::atomic<bool> profiling{false};
   std::atomic<bool> queue_error{false};
 
   // batched path: two staging buffers used alternately, device buffers.  The
@@ -908,6 +911,7 @@ int mi355_aql_set_large_transfer_barrier(mi355_aql_t* h, int enable) {
 int mi355_aql_enable_profiling(mi355_aql_t* h, int enable) {
   if (!h) return MI355_BLIT_ERROR_INVALID_ARGUMENT;
   AQL_HSA(hsa_amd_profiling_set_profiler_enabled(h->queue, enable ? 1 : 0));
+  h->profiling.store(enable != 0);
   return MI355_BLIT_SUCCESS;
 }
 
@@ -950,8 +954,8 @@ int mi355_aql_copy_route(mi355_aql_t* h, void* dst, const void* src, size_t byte
     if (bytes) {
       const uint32_t room = h->queue->size / 2 > nb ? h->queue->size / 2 - nb : 1;
       uint64_t piece_bytes;
-      pieces = copy_pieces(bytes, route, h->serialise_large.load() ? room : 1, h->has_tuning ? &h->tuning : nullptr,
-                           &piece_bytes);
+      const bool cut = h->serialise_large.load() && !h->profiling.load();
+      pieces = copy_pieces(bytes, route, cut ? room : 1, h->has_tuning ? &h->tuning : nullptr, &piece_bytes);
       for (uint32_t i = 0; i < pieces; ++i) {
         const uint64_t off = i * piece_bytes;
         const uint64_t n = bytes - off < piece_bytes ? bytes - off : piece_bytes;

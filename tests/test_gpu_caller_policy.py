@@ -226,6 +226,53 @@ def test_barrier_bit_of_large_transfers(pkg, signals, torch_cuda, monkeypatch, c
         queue.close()
 
 
+def test_long_copies_go_out_in_pieces_except_where_they_must_not(pkg, signals, torch_cuda):
+    """A copy of 1.5 GiB or more within the device is several dispatches on an
+    engine's own queue (the completion signal on the last), one on a borrowed
+    queue unless asked otherwise, and one while the queue's profiling is on, so
+    that the stamps in the completion signal cover the whole command."""
+    torch = torch_cuda
+    n = 2 << 30
+    a = torch.empty(n + 64, dtype=torch.uint8, device="cuda:0")
+    b = torch.zeros(n + 64, dtype=torch.uint8, device="cuda:0")
+    a.view(torch.int32)[:n // 4].copy_(torch.arange(n // 4, dtype=torch.int32, device="cuda:0"))
+    torch.cuda.synchronize()
+
+    def run(engine, want_pieces):
+        b.zero_()
+        torch.cuda.synchronize()
+        done = signals.create(1)
+        assert engine.copy(b.data_ptr() + 5, a.data_ptr() + 1, n - 16, completion=done) == 0
+        assert engine.wait_signal(done) == 0
+        assert signals.load(done) == 0
+        # the signal says the whole copy is done, not a piece of it
+        assert torch.equal(b[5:5 + n - 16], a[1:1 + n - 16])
+        assert engine.last_plan().pieces == want_pieces
+        return done
+
+    own = pkg.aql.AqlBlit(0)
+    queue = pkg.aql.BorrowedQueue(0)
+    try:
+        signals.destroy(run(own, 4))
+        assert own.enable_profiling(True) == 0
+        done = run(own, 1)
+        us = own.command_time_us(done)
+        signals.destroy(done)
+        assert 500.0 < us < 1500.0, us        # 2 GiB at 6-7 TB/s is 620-720 us: the whole command, not a quarter
+        assert own.enable_profiling(False) == 0
+        signals.destroy(run(own, 4))
+        borrowed = pkg.aql.AqlBlit(borrowed=queue)
+        try:
+            signals.destroy(run(borrowed, 1))
+            assert borrowed.set_large_transfer_barrier(True) == 0
+            signals.destroy(run(borrowed, 4))
+        finally:
+            borrowed.close()
+    finally:
+        own.close()
+        queue.close()
+
+
 def test_kernarg_ring_in_host_memory(pkg, capi, oracle, rand, torch_cuda, monkeypatch):
     """MI355_BLIT_HOST_KERNARGS=1 keeps every kernarg slot in host memory, as the
     reference does (amd_blit_kernel.cpp:565-569): a small copy, a copy of many

@@ -376,6 +376,10 @@ std::vector<uint64_t> batch_lengths(unsigned which, bool quick) {
     v.insert(v.end(), 130, 0);
     v.push_back(9);
     v.push_back(262144 + 4096 - 17);
+  } else if (which == 4) {
+    // more than 1024 copies: the prefix sum's first level has several workgroups
+    const unsigned n = quick ? 1100 : 2600;
+    for (unsigned i = 0; i < n; ++i) v.push_back(below(7) == 0 ? 0 : 1 + below(i % 50 == 0 ? 9000 : 300));
   } else {
     const unsigned n = quick ? 150 : 700;
     for (unsigned i = 0; i < n; ++i) {
@@ -561,6 +565,11 @@ void batches(bool quick) {
         t.xcd_run = percent == 40 ? 2 : 0;
         batch_device(which, percent, t, quick);
       }
+  }
+  for (unsigned percent : {40u, 100u}) {
+    if (index++ % g_shards != g_shard) continue;
+    mi355_blit_tuning_t t{};
+    batch_device(4, percent, t, quick);
   }
 }
 

@@ -209,14 +209,24 @@ class Runner:
         for _ in range(steps):
             fn()
         e1.record(self.tstream)
+        t_issued = time.perf_counter()
         # the host watches for the closing event instead of sleeping on it: a blocked wait's wake-up is a few
         # tens of microseconds of a 6 ms region; the synchronisation behind it then returns at once
         while not e1.query():
             pass
-        self.tstream.synchronize()
+        t_seen = time.perf_counter()
+        # one device-wide synchronisation closes the region (it covers the launch stream; a stream synchronisation
+        # in front of it cost another 15-20 us of host time on a device that is already idle)
         torch.cuda.synchronize()
         t1 = time.perf_counter()
-        return t1 - t0, e0.elapsed_time(e1) * 1e3 / steps
+        device_us = e0.elapsed_time(e1) * 1e3
+        # where the wall clock's microseconds beyond the device's own lie
+        self.last_wall_breakdown_us = {
+            "all_steps_issued_after": round((t_issued - t0) * 1e6, 1),
+            "closing_event_seen_after": round((t_seen - t0) * 1e6, 1),
+            "synchronisation_returned_after": round((t1 - t0) * 1e6, 1),
+            "device_first_to_last_event": round(device_us, 1)}
+        return t1 - t0, device_us / steps
 
     def settle(self, fn, min_ms):
         """Back-to-back launches of the workload until min_ms of them have run:
@@ -1274,6 +1284,7 @@ def main():
     settle_launches, settle_ms = r.settle(fn, args.settle_ms) if args.settle_ms > 0 else (0, 0.0)
     t_timed = time.perf_counter()
     wall, dev_us = r.time_launches(fn, args.steps, args.warmup)
+    wall_breakdown = r.last_wall_breakdown_us
     t_replica = time.perf_counter()
     replica = r.time_each(fn, max(args.steps, 5), 0)
     t_end = time.perf_counter()
@@ -1288,13 +1299,18 @@ def main():
                                          "one_by_one": [round((t_replica - t_first) * 1e3, 1),
                                                         round((t_end - t_first) * 1e3, 1)]},
         "us_per_launch_one_by_one": [round(u, 1) for u in replica],
+        "wall_clock_us_since_timing_began": wall_breakdown,
         "sysfs_columns": (["ms since first launch"] + sampler.columns()) if sampler else None,
         "sysfs_changes": sampler.changes(t_first, t_end) if sampler else None,
         "what": "the device is brought to its sustained state by settle_ms of back-to-back launches of the workload "
                 "itself (BASELINE asks for the rate a transfer sustains), then W warm-up and K timed launches follow "
                 "without a gap: `value` is bytes over the host's wall clock around the K launches, roofline.kernel_us "
                 "the HIP events around the same K launches.  us_per_launch_one_by_one are the next K launches, an "
-                "event between every two (each figure includes the event's few microseconds of queue time)",
+                "event between every two (each figure includes the event's few microseconds of queue time).  "
+                "wall_clock_us_since_timing_began says where the wall clock's microseconds beyond the device's own "
+                "lie: when the host had issued the K steps, when it saw the closing event complete, when the "
+                "synchronisation that closes the region had returned (the end of `value`'s clock), and the device's "
+                "time between the events around the K steps",
     }
     if not args.no_verify:
         verify()
